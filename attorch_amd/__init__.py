@@ -1,0 +1,12 @@
+"""
+MI355X-native implementation of attorch's layer-kernel hot path.
+
+The public names match attorch's (Linear, LayerNorm, RMSNorm, Softmax, LogSoftmax, Softmin,
+CrossEntropyLoss, Conv2d, BatchNorm2d and their autograd Functions), so
+`import attorch_amd as attorch` is a drop-in for that path.  All compute happens in
+hand-written gfx950 HIP kernels behind the C ABI declared in include/attorch_hip.h.
+"""
+
+from .norms import LayerNorm, LayerNormAutoGrad, RMSNorm, RMSNormAutoGrad
+from .softmax import LogSoftmax, Softmax, SoftmaxAutoGrad, Softmin
+from .utils import get_output_dtype

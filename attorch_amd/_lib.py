@@ -1,0 +1,114 @@
+"""
+ctypes binding of libattorch_hip.so, the C-ABI library holding the gfx950 kernels.
+
+The library is the only compute backend: if it cannot be loaded the first call raises,
+there is no fallback path.  Prototypes mirror include/attorch_hip.h one to one.
+"""
+
+import ctypes
+from ctypes import c_float, c_int, c_int64, c_void_p
+from pathlib import Path
+from typing import Optional
+
+import torch
+from torch import Tensor
+
+LIB_PATH = Path(__file__).resolve().parent / 'lib' / 'libattorch_hip.so'
+
+DTYPE_IDS = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+P, I, L, F = c_void_p, c_int, c_int64, c_float
+
+# name -> (restype, argtypes); the order is the order of include/attorch_hip.h
+PROTOTYPES = {
+    'at_version': (I, []),
+    'at_error_string': (ctypes.c_char_p, [I]),
+    'at_rms_norm_fwd': (I, [P, P, P, P, L, L, L, L, F, I, I, I, P]),
+    'at_rms_norm_bwd': (I, [P, P, P, P, P, P, P, L, L, L, L, L, L, I, I, I, I, P]),
+    'at_norm_bwd_workspace_bytes': (L, [L, L, I]),
+    'at_layer_norm_fwd': (I, [P, P, P, P, P, P, L, L, L, L, F, I, I, I, P]),
+    'at_layer_norm_bwd': (I, [P, P, P, P, P, P, P, P, P, L, L, L, L, L, L, I, I, I, I, P]),
+    'at_softmax_fwd': (I, [P, P, L, L, L, L, I, I, I, I, P]),
+    'at_softmax_bwd': (I, [P, P, P, L, L, L, L, L, I, I, I, I, I, P]),
+}
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def load() -> ctypes.CDLL:
+    """
+    Loads the shared library once and declares every prototype.
+
+    Raises:
+        RuntimeError: The library has not been built or misses an entry point.
+    """
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise RuntimeError(f'{LIB_PATH} is missing: build it with `python -m attorch_amd.build` '
+                           '(the HIP library is the only backend, there is no fallback)')
+    lib = ctypes.CDLL(str(LIB_PATH))
+    for name, (restype, argtypes) in PROTOTYPES.items():
+        try:
+            fn = getattr(lib, name)
+        except AttributeError as err:
+            raise RuntimeError(f'{LIB_PATH} does not export {name}; rebuild it') from err
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def check(code: int, what: str) -> None:
+    """
+    Converts a non-zero return code of the library into a RuntimeError.
+    """
+    if code != 0:
+        msg = load().at_error_string(code).decode()
+        raise RuntimeError(f'{what} failed with code {code}: {msg}')
+
+
+def ptr(tensor: Optional[Tensor]) -> Optional[int]:
+    """
+    Device address of a tensor, None for an absent optional.
+    """
+    return None if tensor is None else tensor.data_ptr()
+
+
+def dtype_id(dtype: torch.dtype) -> int:
+    """
+    AT_DTYPE_* id of a torch dtype.
+    """
+    try:
+        return DTYPE_IDS[dtype]
+    except KeyError:
+        raise RuntimeError(f'dtype {dtype} is not supported; use float32, float16 or bfloat16') from None
+
+
+def stream_of(tensor: Tensor) -> int:
+    """
+    Raw hipStream_t of the current PyTorch stream on the tensor's device.
+    """
+    return torch.cuda.current_stream(tensor.device).cuda_stream
+
+
+def require_gpu(tensor: Tensor, what: str) -> None:
+    """
+    The kernels only run on the GPU: refuse host tensors loudly instead of falling back.
+    """
+    if not tensor.is_cuda:
+        raise RuntimeError(f'{what}: expected a tensor on a HIP device (device type "cuda"), '
+                           f'received one on {tensor.device}; there is no CPU path')
+
+
+def rows(tensor: Tensor) -> Tensor:
+    """
+    Returns the tensor as a [rows, feat] matrix with unit stride along feat.
+    """
+    if tensor.ndim == 1:
+        tensor = tensor.unsqueeze(0)
+    tensor = tensor.flatten(0, -2) if tensor.ndim != 2 else tensor
+    if tensor.stride(-1) != 1 or (tensor.shape[0] > 1 and tensor.stride(0) < tensor.shape[1]):
+        tensor = tensor.contiguous()
+    return tensor

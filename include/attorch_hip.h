@@ -1,0 +1,171 @@
+/*
+ * libattorch_hip — C ABI of the MI355X (gfx950) kernels behind the attorch layer API.
+ *
+ * The reference (BobMcDear/attorch) has no FFI: its device boundary is the Triton launch
+ * `kernel[grid](tensor pointers, dims, strides, constexpr flags)` inside each
+ * torch.autograd.Function.  Every entry point below replaces one such launch (or the torch
+ * call the reference delegates to) and keeps its argument meaning; the reference site is
+ * cited above each declaration as attorch/<file>:<lines>.
+ *
+ * Rules common to every entry point
+ *   - all pointers are device pointers; the caller allocates every output and every
+ *     workspace (the library never allocates, frees or keeps device memory)
+ *   - "nullable" pointers are null exactly where the reference passes None
+ *   - tensors are row-major with unit stride in the last dimension; row strides are given
+ *     in elements
+ *   - dtype arguments take AT_DTYPE_*; arithmetic is always fp32
+ *   - the work is enqueued on `stream` (a hipStream_t, null = default stream); no call
+ *     synchronises the device
+ *   - return value: 0 on success, > 0 a hipError_t from the launch, < 0 an AT_ERR_* argument
+ *     error (checked before any device call, so argument errors are reported without a GPU)
+ *   - results are bit-reproducible: no floating-point atomics are used anywhere
+ */
+#ifndef ATTORCH_HIP_H
+#define ATTORCH_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AT_OK 0
+#define AT_ERR_NULL (-1)        /* a required pointer is null */
+#define AT_ERR_DIM (-2)         /* a dimension or stride is out of range */
+#define AT_ERR_DTYPE (-3)       /* unknown dtype or unsupported dtype combination */
+#define AT_ERR_ACT (-4)         /* unknown activation id */
+#define AT_ERR_WORKSPACE (-5)   /* workspace missing or too small */
+#define AT_ERR_ALIGN (-6)       /* pointer or stride alignment the kernel cannot serve */
+#define AT_ERR_UNSUPPORTED (-7) /* valid arguments, configuration not implemented */
+
+#define AT_DTYPE_F32 0
+#define AT_DTYPE_F16 1
+#define AT_DTYPE_BF16 2
+
+/* Activation ids: the strings accepted by attorch/linear_layer.py:42-49 and dispatched by
+ * apply_act_func / apply_act_func_grad, attorch/act_kernels.py:631-837. */
+#define AT_ACT_NONE 0
+#define AT_ACT_SIGMOID 1
+#define AT_ACT_LOGSIGMOID 2
+#define AT_ACT_TANH 3
+#define AT_ACT_RELU 4
+#define AT_ACT_GELU 5
+#define AT_ACT_GELUAPPROX 6
+#define AT_ACT_SILU 7
+#define AT_ACT_RELU6 8
+#define AT_ACT_HARDSIGMOID 9
+#define AT_ACT_HARDTANH 10
+#define AT_ACT_HARDSWISH 11
+#define AT_ACT_SELU 12
+#define AT_ACT_MISH 13
+#define AT_ACT_SOFTPLUS 14
+#define AT_ACT_SOFTSIGN 15
+#define AT_ACT_TANHSHRINK 16
+#define AT_ACT_LEAKY_RELU 17
+#define AT_ACT_ELU 18
+#define AT_ACT_CELU 19
+#define AT_ACT_HARDSHRINK 20
+#define AT_ACT_SOFTSHRINK 21
+#define AT_ACT_COUNT 22
+
+typedef void* at_stream_t;
+
+/* Library version (major * 10000 + minor * 100 + patch). */
+int at_version(void);
+
+/* Static description of a return code of this library (never null). */
+const char* at_error_string(int code);
+
+/* ------------------------------------------------------------------------------------------
+ * RMSNorm — replaces rms_norm_forward_kernel / rms_norm_backward_kernel,
+ * attorch/rms_norm_kernels.py:21-88 and :98-193, launched from attorch/rms_norm_layer.py:68-75
+ * and :114-124.
+ *   fwd: inv_rms = rsqrt(sum(x^2)/feat + eps); y = x * inv_rms (* weight)
+ *   bwd: g = weight*dy; dx = inv_rms*(g - x*sum(x*g)*inv_rms^2/feat); weight_grad = sum_rows dy*x*inv_rms
+ * weight (nullable) = scale_by_weight False; inv_rms (nullable in fwd) = save_stats False.
+ * weight_grad is fp32 [feat] and is the finished column sum (the reference writes per-program
+ * partial rows and sums them with torch, rms_norm_layer.py:126-127; here the partial rows live in
+ * `workspace`, at least at_norm_bwd_workspace_bytes(batch, feat, 1) bytes, and are reduced by a
+ * second launch in fixed order).
+ * ------------------------------------------------------------------------------------------ */
+int at_rms_norm_fwd(const void* x, const void* weight, float* inv_rms, void* y,
+                    int64_t batch, int64_t feat, int64_t x_stride, int64_t y_stride, float eps,
+                    int x_dtype, int weight_dtype, int y_dtype, at_stream_t stream);
+
+int at_rms_norm_bwd(const void* dy, const void* x, const float* inv_rms, const void* weight,
+                    void* dx, float* weight_grad, void* workspace, int64_t workspace_bytes,
+                    int64_t batch, int64_t feat, int64_t dy_stride, int64_t x_stride,
+                    int64_t dx_stride, int dy_dtype, int x_dtype, int weight_dtype, int dx_dtype,
+                    at_stream_t stream);
+
+/* Bytes of workspace the norm backward kernels need for `n_param_grads` (1 = weight only,
+ * 2 = weight and bias) fp32 parameter gradients; 0 when n_param_grads is 0. */
+int64_t at_norm_bwd_workspace_bytes(int64_t batch, int64_t feat, int n_param_grads);
+
+/* ------------------------------------------------------------------------------------------
+ * LayerNorm — replaces layer_norm_forward_kernel / layer_norm_backward_kernel,
+ * attorch/layer_norm_kernels.py:21-101 and :111-224, launched from
+ * attorch/layer_norm_layer.py:77-85 and :137-148 (+ the torch sums at :150-153).
+ *   fwd: mean = sum(x)/feat; inv_std = rsqrt(sum((x-mean)^2)/feat + eps);
+ *        y = (x-mean)*inv_std (* weight (+ bias))
+ *   bwd: xh = (x-mean)*inv_std; g = weight*dy;
+ *        dx = inv_std*(g - xh*mean(xh*g) - mean(g)); weight_grad = sum_rows dy*xh; bias_grad = sum_rows dy
+ * bias is ignored when weight is null (layer_norm_layer.py:60). mean/inv_std nullable in fwd.
+ * ------------------------------------------------------------------------------------------ */
+int at_layer_norm_fwd(const void* x, const void* weight, const void* bias, float* mean,
+                      float* inv_std, void* y, int64_t batch, int64_t feat, int64_t x_stride,
+                      int64_t y_stride, float eps, int x_dtype, int weight_dtype, int y_dtype,
+                      at_stream_t stream);
+
+int at_layer_norm_bwd(const void* dy, const void* x, const float* mean, const float* inv_std,
+                      const void* weight, void* dx, float* weight_grad, float* bias_grad,
+                      void* workspace, int64_t workspace_bytes, int64_t batch, int64_t feat,
+                      int64_t dy_stride, int64_t x_stride, int64_t dx_stride, int dy_dtype,
+                      int x_dtype, int weight_dtype, int dx_dtype, at_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Softmax / LogSoftmax / Softmin over the last dimension — replaces softmax_forward_kernel /
+ * softmax_backward_kernel, attorch/softmax_kernels.py:43-103 and :113-181, launched from
+ * attorch/softmax_layers.py:50-52 and :82-86.  neg = softmin, log = log-softmax.
+ *   bwd (from the saved OUTPUT y): softmax dx = y*(dy - sum(dy*y)); log dx = dy - exp(y)*sum(dy);
+ *   negated when neg.
+ * ------------------------------------------------------------------------------------------ */
+int at_softmax_fwd(const void* x, void* y, int64_t batch, int64_t feat, int64_t x_stride,
+                   int64_t y_stride, int neg, int log, int x_dtype, int y_dtype, at_stream_t stream);
+
+int at_softmax_bwd(const void* dy, const void* y, void* dx, int64_t batch, int64_t feat,
+                   int64_t dy_stride, int64_t y_stride, int64_t dx_stride, int neg, int log,
+                   int dy_dtype, int y_dtype, int dx_dtype, at_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Cross entropy (mean reduction, optional class weights, ignore_index) — replaces
+ * cross_entropy_loss_forward_kernel / cross_entropy_loss_backward_kernel,
+ * attorch/cross_entropy_loss_kernels.py:21-86 and :96-172, the torch sums at
+ * attorch/cross_entropy_loss_layer.py:76-80, and adds ignore_index (absent upstream, :144).
+ * One pass over the logits produces the loss and, when dlogits is non-null, the gradient for an
+ * upstream gradient of 1:  dlogits = (softmax - onehot(target)) * w[target] / denom, with
+ * denom = sum of w[target] over kept rows (or the kept-row count when weight is null).
+ * Rows whose target equals ignore_index — or lies outside [0, feat) — contribute nothing and
+ * get an all-zero gradient row. loss is one element of out_dtype; workspace needs
+ * at_cross_entropy_workspace_bytes(batch) bytes; on return workspace[0] (fp32) holds denom.
+ * at_cross_entropy_scale_grad multiplies dlogits in place by the upstream gradient, read on
+ * the device as one element of grad_dtype (cross_entropy_loss_kernels.py:155); it returns
+ * without touching memory when that value is exactly 1.
+ * ------------------------------------------------------------------------------------------ */
+int64_t at_cross_entropy_workspace_bytes(int64_t batch);
+
+int at_cross_entropy_fwd_bwd(const void* logits, const int64_t* target, const void* weight,
+                             void* loss, void* dlogits, void* workspace, int64_t workspace_bytes,
+                             int64_t batch, int64_t feat, int64_t logits_stride,
+                             int64_t dlogits_stride, int64_t ignore_index, int logits_dtype,
+                             int weight_dtype, int out_dtype, at_stream_t stream);
+
+int at_cross_entropy_scale_grad(void* dlogits, const void* output_grad, int64_t batch,
+                                int64_t feat, int64_t dlogits_stride, int dlogits_dtype,
+                                int grad_dtype, at_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* ATTORCH_HIP_H */
