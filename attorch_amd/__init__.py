@@ -7,6 +7,7 @@ CrossEntropyLoss, Conv2d, BatchNorm2d and their autograd Functions), so
 hand-written gfx950 HIP kernels behind the C ABI declared in include/attorch_hip.h.
 """
 
+from .cross_entropy import CrossEntropyLoss, CrossEntropyLossAutoGrad
 from .norms import LayerNorm, LayerNormAutoGrad, RMSNorm, RMSNormAutoGrad
 from .softmax import LogSoftmax, Softmax, SoftmaxAutoGrad, Softmin
 from .utils import get_output_dtype

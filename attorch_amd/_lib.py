@@ -30,6 +30,9 @@ PROTOTYPES = {
     'at_layer_norm_bwd': (I, [P, P, P, P, P, P, P, P, P, L, L, L, L, L, L, I, I, I, I, P]),
     'at_softmax_fwd': (I, [P, P, L, L, L, L, I, I, I, I, P]),
     'at_softmax_bwd': (I, [P, P, P, L, L, L, L, L, I, I, I, I, I, P]),
+    'at_cross_entropy_workspace_bytes': (L, [L]),
+    'at_cross_entropy_fwd_bwd': (I, [P, P, P, P, P, P, L, L, L, L, L, L, I, I, I, P]),
+    'at_cross_entropy_scale_grad': (I, [P, P, L, L, L, I, I, P]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

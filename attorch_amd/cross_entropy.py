@@ -1,0 +1,137 @@
+"""
+Cross entropy loss with PyTorch autodiff support, running on the fused gfx950 kernel.
+
+API mirrors attorch/cross_entropy_loss_layer.py (mean reduction only, no label smoothing,
+optional class weights) and adds what the reference lacks: ignore_index.  The forward pass
+reads the logits once and produces both the loss and, when the logits require a gradient,
+the gradient for an upstream gradient of one; backward only rescales it.
+"""
+
+from typing import Any, Optional, Tuple
+
+import torch
+from torch import Tensor
+from torch import nn
+
+from . import _lib
+from .utils import get_output_dtype
+
+
+class CrossEntropyLossAutoGrad(torch.autograd.Function):
+    """
+    Autodiff for cross entropy loss (attorch/cross_entropy_loss_layer.py:20-121).
+    """
+    @staticmethod
+    def forward(
+        ctx: Any,
+        input: Tensor,
+        target: Tensor,
+        weight: Optional[Tensor] = None,
+        ignore_index: int = -100,
+        ) -> Tensor:
+        """
+        Mean cross entropy of the logits against class indices.
+
+        Args:
+            input: Logits of shape [batch_dim, feat_dim].
+            target: Class indices of shape [batch_dim] (int64).
+            weight: Optional class weights of shape [feat_dim]; the mean is then weighted.
+            ignore_index: Rows with this target contribute neither loss nor gradient.
+
+        Returns:
+            Scalar loss, float32 under autocast and the input dtype otherwise.
+        """
+        assert input.ndim == 2, f'Inputs of rank other than 2 not valid'
+        assert len(input) == len(target), \
+            f'Incompatible input shape ({input.shape}) and target shape ({target.shape})'
+        assert weight is None or len(weight) == input.shape[1], \
+            f'Dimensionality of weight vector ({len(weight)}) and input features ({input.shape[1]}) not equal'
+
+        _lib.require_gpu(input, 'CrossEntropyLoss')
+        lib = _lib.load()
+        batch_dim, feat_dim = input.shape
+        output_dtype = get_output_dtype(input.dtype, autocast='fp32')
+
+        logits = input if input.stride(1) == 1 and input.stride(0) >= feat_dim else input.contiguous()
+        target_k = target.to(torch.int64).contiguous()
+        weight_k = None if weight is None else weight.contiguous()
+        output = torch.empty((), dtype=output_dtype, device=input.device)
+        input_grad = (torch.empty((batch_dim, feat_dim), dtype=output_dtype, device=input.device)
+                      if input.requires_grad else None)
+        workspace_bytes = lib.at_cross_entropy_workspace_bytes(batch_dim)
+        workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=input.device)
+
+        with torch.cuda.device_of(input):
+            _lib.check(lib.at_cross_entropy_fwd_bwd(
+                _lib.ptr(logits), _lib.ptr(target_k), _lib.ptr(weight_k), _lib.ptr(output),
+                _lib.ptr(input_grad), _lib.ptr(workspace), workspace_bytes, batch_dim, feat_dim,
+                logits.stride(0), feat_dim, ignore_index, _lib.dtype_id(logits.dtype),
+                _lib.dtype_id(weight_k.dtype) if weight_k is not None else 0,
+                _lib.dtype_id(output_dtype), _lib.stream_of(input)), 'at_cross_entropy_fwd_bwd')
+
+        ctx.output_dtype = output_dtype
+        if input.requires_grad:
+            ctx.save_for_backward(input_grad)
+
+        return output
+
+    @staticmethod
+    def backward(
+        ctx: Any,
+        output_grad: Tensor,
+        ) -> Tuple[Optional[Tensor], ...]:
+        """
+        Gradient of the logits: the one computed in forward, times the upstream gradient
+        (read on the device; nothing is rewritten when it is exactly one).
+        """
+        lib = _lib.load()
+        (input_grad,) = ctx.saved_tensors
+        batch_dim, feat_dim = input_grad.shape
+        output_grad = output_grad.contiguous()
+        if output_grad.dtype not in _lib.DTYPE_IDS:
+            output_grad = output_grad.float()
+
+        with torch.cuda.device_of(input_grad):
+            _lib.check(lib.at_cross_entropy_scale_grad(
+                _lib.ptr(input_grad), _lib.ptr(output_grad), batch_dim, feat_dim,
+                input_grad.stride(0), _lib.dtype_id(input_grad.dtype),
+                _lib.dtype_id(output_grad.dtype), _lib.stream_of(input_grad)),
+                'at_cross_entropy_scale_grad')
+
+        return input_grad, None, None, None
+
+
+class CrossEntropyLoss(nn.CrossEntropyLoss):
+    """
+    Mean cross entropy between logits and class indices, optionally weighted per class.
+    See also base class; mirrors attorch/cross_entropy_loss_layer.py:124-170 and
+    additionally honours ignore_index.
+
+    Args:
+        reduction: Only 'mean' is supported.
+        size_average: Deprecated torch argument, forwarded to the base class.
+        reduce: Deprecated torch argument, forwarded to the base class.
+        weight: Optional class weights of shape [feat_dim].
+        ignore_index: Target value whose rows are ignored.
+        label_smoothing: Must be 0.
+    """
+    def __init__(
+        self,
+        reduction: str = 'mean',
+        size_average: Optional[bool] = None,
+        reduce: Optional[bool] = None,
+        weight: Optional[Tensor] = None,
+        ignore_index: int = -100,
+        label_smoothing: float = 0.0,
+        ) -> None:
+        super().__init__(weight, size_average, ignore_index, reduce,
+                         reduction, label_smoothing)
+
+        if self.reduction != 'mean':
+            raise RuntimeError('Cross entropy only supports averaging the loss.')
+
+        if label_smoothing > 0.0:
+            raise RuntimeError('Cross entropy does not support label smoothing.')
+
+    def forward(self, input: Tensor, target: Tensor) -> Tensor:
+        return CrossEntropyLossAutoGrad.apply(input, target, self.weight, self.ignore_index)

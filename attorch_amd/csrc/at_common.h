@@ -104,6 +104,73 @@ __device__ __forceinline__ void store_scalar_f32(void* __restrict__ p, int dt, i
   else reinterpret_cast<bf16_t*>(p)[idx] = from_f32<bf16_t>(v);
 }
 
+// ---- packed access to raw 32-bit words (keeps register-cached rows packed) ----
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+template <typename T> struct Word;   // view of one 32-bit register holding 1 (fp32) or 2 elements
+template <> struct Word<float> {
+  static constexpr int N = 1;
+  static constexpr uint32_t kNegInf = 0xff800000u;
+  template <int K> static __device__ __forceinline__ float get(uint32_t w) { return __uint_as_float(w); }
+  static __device__ __forceinline__ uint32_t pack(float a, float) { return __float_as_uint(a); }
+};
+template <> struct Word<f16_t> {
+  static constexpr int N = 2;
+  static constexpr uint32_t kNegInf = 0xfc00fc00u;
+  template <int K> static __device__ __forceinline__ float get(uint32_t w) {
+    const f16x2_t h = __builtin_bit_cast(f16x2_t, w);
+    return static_cast<float>(K == 0 ? h.x : h.y);
+  }
+  static __device__ __forceinline__ uint32_t pack(float a, float b) {
+    f16x2_t h;
+    h.x = static_cast<f16_t>(a);
+    h.y = static_cast<f16_t>(b);
+    return __builtin_bit_cast(uint32_t, h);
+  }
+};
+template <> struct Word<bf16_t> {
+  static constexpr int N = 2;
+  static constexpr uint32_t kNegInf = 0xff80ff80u;
+  template <int K> static __device__ __forceinline__ float get(uint32_t w) {
+    return __uint_as_float(K == 0 ? (w << 16) : (w & 0xffff0000u));
+  }
+  static __device__ __forceinline__ uint32_t pack(float a, float b) {
+    bf16x2_t h;
+    h.x = static_cast<bf16_t>(a);
+    h.y = static_cast<bf16_t>(b);
+    return __builtin_bit_cast(uint32_t, h);
+  }
+};
+
+// Widens the 16 / sizeof(T) elements of a raw 128-bit vector.
+template <typename T>
+__device__ __forceinline__ void unpack16(const uint4& r, float (&f)[16 / sizeof(T)]) {
+  const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if constexpr (Word<T>::N == 1) f[i] = Word<T>::template get<0>(w[i]);
+    else { f[2 * i] = Word<T>::template get<0>(w[i]); f[2 * i + 1] = Word<T>::template get<1>(w[i]); }
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ uint4 pack16(const float (&f)[16 / sizeof(T)]) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if constexpr (Word<T>::N == 1) w[i] = Word<T>::pack(f[i], 0.f);
+    else w[i] = Word<T>::pack(f[2 * i], f[2 * i + 1]);
+  }
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// Optimisation barrier on a register-resident 128-bit value: the compiler must treat it as
+// modified, so values derived from it earlier (e.g. widened copies) are not kept alive.
+__device__ __forceinline__ void keep_raw(uint4& v) {
+  asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w));
+}
+
 // ---- reductions over a group of `group` consecutive lanes (power of two, <= 1024) ----
 struct SumOp { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
 struct MaxOp { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };

@@ -1,0 +1,323 @@
+// Cross entropy with mean reduction, optional class weights and ignore_index: loss and the
+// gradient of the logits from ONE pass over the logits.
+//
+// HBM-bound: the algorithmic traffic is one read of the logits and one write of the gradient.
+// One 512-lane workgroup owns a row and keeps it in registers as raw 128-bit vectors
+// (CACHE_VECS per lane), so the three sweeps the math needs (max, sum of exponentials,
+// gradient) cost a single read.  Rows need not be 16-byte aligned (a vocabulary of 50257
+// fp16 logits makes every other row start on an odd element): a row is addressed through
+// the 16-byte grid of its own address space, interior vectors move with 128-bit accesses and
+// only the first and last vector of a row fall back to guarded element accesses.  The
+// gradient row must sit at the same phase of the 16-byte grid as the logits row for this
+// path; anything else (or a different gradient dtype) takes the streaming kernel.
+#include <type_traits>
+
+#include "at_common.h"
+
+namespace at_hip {
+namespace {
+
+constexpr int kCeBlock = 512;
+
+__device__ __forceinline__ bool target_kept(int64_t t, int64_t ignore_index, int feat) {
+  return t != ignore_index && t >= 0 && t < feat;
+}
+
+// denom = sum over kept rows of weight[target] (or the kept-row count).  Single workgroup so
+// the summation order is fixed.
+__global__ __launch_bounds__(1024) void ce_denominator_kernel(
+    const int64_t* __restrict__ target, const void* __restrict__ weight, int wdt,
+    float* __restrict__ denom_out, int64_t batch, int feat, int64_t ignore_index) {
+  __shared__ float scratch[16];
+  float s = 0.f;
+  for (int64_t i = threadIdx.x; i < batch; i += blockDim.x) {
+    const int64_t t = target[i];
+    if (target_kept(t, ignore_index, feat)) s += weight ? load_scalar_f32(weight, wdt, t) : 1.f;
+  }
+  s = group_reduce(s, (int)blockDim.x, scratch, SumOp(), 0.f);
+  if (threadIdx.x == 0) denom_out[0] = s;
+}
+
+__global__ __launch_bounds__(1024) void ce_finalize_kernel(
+    const float* __restrict__ row_loss, const float* __restrict__ denom, void* __restrict__ loss,
+    int out_dt, int64_t batch) {
+  __shared__ float scratch[16];
+  float s = 0.f;
+  for (int64_t i = threadIdx.x; i < batch; i += blockDim.x) s += row_loss[i];
+  s = group_reduce(s, (int)blockDim.x, scratch, SumOp(), 0.f);
+  if (threadIdx.x == 0) store_scalar_f32(loss, out_dt, 0, s / denom[0]);
+}
+
+// Register-cached row kernel.  T is the dtype of both the logits and the gradient.
+// A row is split into "interior" 16-byte vectors (fully inside the row, 128-bit accesses) and
+// at most 7 + 7 "edge" elements before the first and after the last interior vector, each
+// owned by one of the first 16 lanes and moved with element accesses.
+template <typename T, int CACHE_VECS>
+__global__ __launch_bounds__(kCeBlock, 4) void ce_row_kernel(
+    const T* __restrict__ logits, const int64_t* __restrict__ target, const void* __restrict__ weight,
+    int wdt, const float* __restrict__ denom, float* __restrict__ row_loss, T* __restrict__ dlogits,
+    int feat, int64_t xs, int64_t ds, int64_t ignore_index) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  __shared__ float scratch[16];
+  const int tid = threadIdx.x;
+  const int64_t row = blockIdx.x;
+  const T* xr = logits + row * xs;
+  T* dr = dlogits ? dlogits + row * ds : nullptr;
+  const int off = (int)((reinterpret_cast<uintptr_t>(xr) & 15u) / sizeof(T));
+  const int head_n = off ? (VEC - off < feat ? VEC - off : feat) : 0;  // row elements [0, head_n)
+  const int n_int = (feat - head_n) / VEC;                             // interior vectors
+  const int tail0 = head_n + n_int * VEC;                              // row elements [tail0, feat)
+  const uint4* xv = reinterpret_cast<const uint4*>(xr + head_n);       // 16-byte aligned
+  uint4* dv = dr ? reinterpret_cast<uint4*>(dr + head_n) : nullptr;    // same phase (host check)
+  // edge element owned by this lane, -1 if none
+  const int edge = tid < 8 ? (tid < head_n ? tid : -1)
+                           : (tid < 16 && tail0 + tid - 8 < feat ? tail0 + tid - 8 : -1);
+  const int64_t t = target[row];
+  const bool kept = target_kept(t, ignore_index, feat);
+
+  if (!kept) {
+    if (tid == 0) row_loss[row] = 0.f;
+    if (dr) {
+      for (int v = tid; v < n_int; v += kCeBlock) dv[v] = make_uint4(0, 0, 0, 0);
+      if (edge >= 0) dr[edge] = from_f32<T>(0.f);
+    }
+    return;
+  }
+
+  uint4 cache[CACHE_VECS];
+#pragma unroll
+  for (int i = 0; i < CACHE_VECS; ++i) {
+    const int v = tid + i * kCeBlock;
+    constexpr uint32_t P = Word<T>::kNegInf;
+    cache[i] = v < n_int ? xv[v] : make_uint4(P, P, P, P);
+  }
+  const float edge_x = edge >= 0 ? to_f32(xr[edge]) : -INFINITY;
+
+  float m = edge_x;
+#pragma unroll
+  for (int i = 0; i < CACHE_VECS; ++i) {
+    float f[VEC];
+    unpack16<T>(cache[i], f);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) m = fmaxf(m, f[j]);
+  }
+  m = group_reduce(m, kCeBlock, scratch, MaxOp(), -INFINITY);
+  // Keep the row cached as raw data: without this the compiler may keep widened fp32 copies
+  // of every element alive across the sweeps.
+#pragma unroll
+  for (int i = 0; i < CACHE_VECS; ++i) keep_raw(cache[i]);
+
+  float s = __expf(edge_x - m);
+#pragma unroll
+  for (int i = 0; i < CACHE_VECS; ++i) {
+    float f[VEC];
+    unpack16<T>(cache[i], f);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) s += __expf(f[j] - m);   // exp(-inf) = 0 for the padding
+  }
+  s = group_reduce(s, kCeBlock, scratch, SumOp(), 0.f);
+#pragma unroll
+  for (int i = 0; i < CACHE_VECS; ++i) keep_raw(cache[i]);
+
+  const float wt = weight ? load_scalar_f32(weight, wdt, t) : 1.f;
+  if (tid == 0) row_loss[row] = (__logf(s) - to_f32(xr[t]) + m) * wt;
+  if (!dr) return;
+
+  const float scale = wt / denom[0];
+  const float k = scale / s;
+  const int tv = (int)t - head_n;  // target position relative to the first interior element
+#pragma unroll
+  for (int i = 0; i < CACHE_VECS; ++i) {
+    const int v = tid + i * kCeBlock;
+    if (v < n_int) {
+      float f[VEC];
+      unpack16<T>(cache[i], f);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        f[j] = __expf(f[j] - m) * k;
+        if (v * VEC + j == tv) f[j] -= scale;
+      }
+      dv[v] = pack16<T>(f);
+    }
+  }
+  if (edge >= 0) {
+    float g = __expf(edge_x - m) * k;
+    if (edge == (int)t) g -= scale;
+    dr[edge] = from_f32<T>(g);
+  }
+}
+
+// Streaming kernel: any dtypes, any alignment, any width; the row is read twice (online
+// max / sum of exponentials, then the gradient), element accesses only.
+template <typename T, typename TO>
+__global__ __launch_bounds__(1024) void ce_row_stream_kernel(
+    const T* __restrict__ logits, const int64_t* __restrict__ target, const void* __restrict__ weight,
+    int wdt, const float* __restrict__ denom, float* __restrict__ row_loss, TO* __restrict__ dlogits,
+    int feat, int64_t xs, int64_t ds, int64_t ignore_index) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  const T* xr = logits + row * xs;
+  TO* dr = dlogits ? dlogits + row * ds : nullptr;
+  const int64_t t = target[row];
+  const bool kept = target_kept(t, ignore_index, feat);
+  if (!kept) {
+    if (threadIdx.x == 0) row_loss[row] = 0.f;
+    if (dr)
+      for (int c = threadIdx.x; c < feat; c += blockDim.x) dr[c] = from_f32<TO>(0.f);
+    return;
+  }
+  float m = -INFINITY;
+  for (int c = threadIdx.x; c < feat; c += blockDim.x) m = fmaxf(m, to_f32(xr[c]));
+  m = group_reduce(m, (int)blockDim.x, scratch, MaxOp(), -INFINITY);
+  float s = 0.f;
+  for (int c = threadIdx.x; c < feat; c += blockDim.x) s += __expf(to_f32(xr[c]) - m);
+  s = group_reduce(s, (int)blockDim.x, scratch, SumOp(), 0.f);
+  const float wt = weight ? load_scalar_f32(weight, wdt, t) : 1.f;
+  if (threadIdx.x == 0) row_loss[row] = (__logf(s) - to_f32(xr[t]) + m) * wt;
+  if (!dr) return;
+  const float scale = wt / denom[0];
+  const float k = scale / s;
+  for (int c = threadIdx.x; c < feat; c += blockDim.x) {
+    float g = __expf(to_f32(xr[c]) - m) * k;
+    if (c == (int)t) g -= scale;
+    dr[c] = from_f32<TO>(g);
+  }
+}
+
+// In-place scale of a [batch, feat] gradient by a device scalar; nothing is touched when the
+// scalar is exactly 1.
+template <typename T>
+__global__ void ce_scale_kernel(T* __restrict__ d, const void* __restrict__ g_ptr, int gdt,
+                                int64_t batch, int feat, int64_t ds) {
+  const float g = load_scalar_f32(g_ptr, gdt, 0);
+  if (g == 1.0f) return;
+  const int64_t total = batch * (int64_t)feat;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int64_t r = i / feat, c = i - r * feat;
+    T* p = d + r * ds + c;
+    *p = from_f32<T>(to_f32(*p) * g);
+  }
+}
+
+template <typename T>
+__global__ void ce_scale_flat_kernel(T* __restrict__ d, const void* __restrict__ g_ptr, int gdt,
+                                     int64_t total) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  const float g = load_scalar_f32(g_ptr, gdt, 0);
+  if (g == 1.0f) return;
+  // d is 16-byte aligned (checked by the host); vectors first, then the tail.
+  const int64_t nvec = total / VEC;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += stride) {
+    float f[VEC];
+    load_f32<T, VEC>(d + v * VEC, f);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) f[j] *= g;
+    store_f32<T, VEC>(d + v * VEC, f);
+  }
+  if (blockIdx.x == 0)
+    for (int64_t i = nvec * VEC + threadIdx.x; i < total; i += blockDim.x)
+      d[i] = from_f32<T>(to_f32(d[i]) * g);
+}
+
+template <typename F>
+inline int dispatch_one(int dt, F&& f) {
+  if (dt == AT_DTYPE_F32) return f((float*)0);
+  if (dt == AT_DTYPE_F16) return f((f16_t*)0);
+  if (dt == AT_DTYPE_BF16) return f((bf16_t*)0);
+  return AT_ERR_DTYPE;
+}
+
+}  // namespace
+}  // namespace at_hip
+
+using namespace at_hip;
+
+extern "C" {
+
+int64_t at_cross_entropy_workspace_bytes(int64_t batch) {
+  if (batch < 0) return 0;
+  return (4 + batch) * (int64_t)sizeof(float);
+}
+
+int at_cross_entropy_fwd_bwd(const void* logits, const int64_t* target, const void* weight, void* loss,
+                             void* dlogits, void* workspace, int64_t workspace_bytes, int64_t batch,
+                             int64_t feat, int64_t logits_stride, int64_t dlogits_stride,
+                             int64_t ignore_index, int logits_dtype, int weight_dtype, int out_dtype,
+                             at_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (!logits || !target || !loss) return AT_ERR_NULL;
+  if (!dtype_valid(logits_dtype) || !dtype_valid(out_dtype) || (weight && !dtype_valid(weight_dtype)))
+    return AT_ERR_DTYPE;
+  if (!(out_dtype == logits_dtype || out_dtype == AT_DTYPE_F32)) return AT_ERR_DTYPE;
+  if (batch <= 0 || feat <= 0 || feat > ((int64_t)1 << 30)) return AT_ERR_DIM;
+  if (logits_stride < feat || (dlogits && dlogits_stride < feat)) return AT_ERR_DIM;
+  if (!workspace || workspace_bytes < at_cross_entropy_workspace_bytes(batch)) return AT_ERR_WORKSPACE;
+  if ((reinterpret_cast<uintptr_t>(workspace) & 3u) != 0) return AT_ERR_ALIGN;
+
+  float* denom = (float*)workspace;
+  float* row_loss = denom + 4;
+  hipLaunchKernelGGL(ce_denominator_kernel, dim3(1), dim3(1024), 0, stream, target, weight, weight_dtype,
+                     denom, batch, (int)feat, ignore_index);
+
+  const int es = dtype_size(logits_dtype);
+  const int vec = 16 / es;
+  const int64_t max_vecs = cdiv64(feat, vec);
+  const bool same_phase =
+      !dlogits || (((reinterpret_cast<uintptr_t>(dlogits) ^ reinterpret_cast<uintptr_t>(logits)) & 15u) == 0 &&
+                   ((dlogits_stride - logits_stride) * es) % 16 == 0);
+  const bool cached = out_dtype == logits_dtype && same_phase && max_vecs <= (int64_t)kCeBlock * 16 &&
+                      (reinterpret_cast<uintptr_t>(logits) % es) == 0;
+
+  int rc = dispatch_one(logits_dtype, [&](auto* tp) -> int {
+    typedef std::remove_pointer_t<decltype(tp)> T;
+    if (cached) {
+      const int per_lane = (int)cdiv64(max_vecs, kCeBlock);
+#define AT_CE_LAUNCH(CV)                                                                          \
+  hipLaunchKernelGGL((ce_row_kernel<T, CV>), dim3((unsigned)batch), dim3(kCeBlock), 0, stream,    \
+                     (const T*)logits, target, weight, weight_dtype, denom, row_loss, (T*)dlogits, \
+                     (int)feat, logits_stride, dlogits_stride, ignore_index)
+      if (per_lane <= 2) AT_CE_LAUNCH(2);
+      else if (per_lane <= 4) AT_CE_LAUNCH(4);
+      else if (per_lane <= 8) AT_CE_LAUNCH(8);
+      else AT_CE_LAUNCH(16);
+#undef AT_CE_LAUNCH
+    } else if (out_dtype == logits_dtype) {
+      hipLaunchKernelGGL((ce_row_stream_kernel<T, T>), dim3((unsigned)batch), dim3(1024), 0, stream,
+                         (const T*)logits, target, weight, weight_dtype, denom, row_loss, (T*)dlogits,
+                         (int)feat, logits_stride, dlogits_stride, ignore_index);
+    } else {
+      hipLaunchKernelGGL((ce_row_stream_kernel<T, float>), dim3((unsigned)batch), dim3(1024), 0, stream,
+                         (const T*)logits, target, weight, weight_dtype, denom, row_loss, (float*)dlogits,
+                         (int)feat, logits_stride, dlogits_stride, ignore_index);
+    }
+    return launch_status();
+  });
+  if (rc) return rc;
+  hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(1024), 0, stream, row_loss, denom, loss, out_dtype,
+                     batch);
+  return launch_status();
+}
+
+int at_cross_entropy_scale_grad(void* dlogits, const void* output_grad, int64_t batch, int64_t feat,
+                                int64_t dlogits_stride, int dlogits_dtype, int grad_dtype,
+                                at_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (!dlogits || !output_grad) return AT_ERR_NULL;
+  if (!dtype_valid(dlogits_dtype) || !dtype_valid(grad_dtype)) return AT_ERR_DTYPE;
+  if (batch <= 0 || feat <= 0 || dlogits_stride < feat) return AT_ERR_DIM;
+  const int blocks = device_cu_count() * 8;
+  return dispatch_one(dlogits_dtype, [&](auto* tp) -> int {
+    typedef std::remove_pointer_t<decltype(tp)> T;
+    if (dlogits_stride == feat && aligned16(dlogits))
+      hipLaunchKernelGGL((ce_scale_flat_kernel<T>), dim3(blocks), dim3(256), 0, stream, (T*)dlogits,
+                         output_grad, grad_dtype, batch * feat);
+    else
+      hipLaunchKernelGGL((ce_scale_kernel<T>), dim3(blocks), dim3(256), 0, stream, (T*)dlogits, output_grad,
+                         grad_dtype, batch, (int)feat, dlogits_stride);
+    return launch_status();
+  });
+}
+
+}  // extern "C"
