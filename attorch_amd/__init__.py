@@ -8,6 +8,7 @@ hand-written gfx950 HIP kernels behind the C ABI declared in include/attorch_hip
 """
 
 from .cross_entropy import CrossEntropyLoss, CrossEntropyLossAutoGrad
+from .linear import Linear, LinearAutoGrad
 from .norms import LayerNorm, LayerNormAutoGrad, RMSNorm, RMSNormAutoGrad
 from .softmax import LogSoftmax, Softmax, SoftmaxAutoGrad, Softmin
 from .utils import get_output_dtype

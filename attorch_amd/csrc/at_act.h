@@ -1,0 +1,95 @@
+// The 21 activation functions accepted by the Linear / BatchNorm epilogues and their
+// derivatives, as fp32 device functions (formulas of attorch/act_kernels.py:13-628; the
+// piecewise ones keep the reference's <= / < choices at the joints so gradients agree at the
+// boundary points attorch's tests probe).  tanh is 2*sigmoid(2x) - 1 as in the reference (:81).
+#pragma once
+
+#include "at_common.h"
+
+namespace at_hip {
+
+inline bool act_valid(int act) { return act >= AT_ACT_NONE && act < AT_ACT_COUNT; }
+inline bool act_needs_param(int act) { return act >= AT_ACT_LEAKY_RELU && act <= AT_ACT_SOFTSHRINK; }
+
+__device__ __forceinline__ float act_sigmoid(float x) { return 1.f / (1.f + __expf(-x)); }
+__device__ __forceinline__ float act_tanh(float x) { return 2.f * act_sigmoid(2.f * x) - 1.f; }
+
+// erf by Abramowitz & Stegun 7.1.26 (absolute error < 1.5e-7): small enough to inline into the
+// fully unrolled GEMM epilogue, which the libm erff is not.
+__device__ __forceinline__ float act_erf(float x) {
+  const float ax = fabsf(x);
+  const float t = 1.f / (1.f + 0.3275911f * ax);
+  const float poly = ((((1.061405429f * t - 1.453152027f) * t + 1.421413741f) * t - 0.284496736f) * t +
+                      0.254829592f) * t;
+  return copysignf(1.f - poly * __expf(-ax * ax), x);
+}
+
+constexpr float kSeluScale = 1.0507009873554804934193349852946f;
+constexpr float kSeluAlpha = 1.6732632423543772848170429916717f;
+
+__device__ __forceinline__ float act_forward(int act, float x, float p) {
+  switch (act) {
+    case AT_ACT_SIGMOID: return act_sigmoid(x);
+    case AT_ACT_LOGSIGMOID: return __logf(act_sigmoid(x));
+    case AT_ACT_TANH: return act_tanh(x);
+    case AT_ACT_RELU: return fmaxf(0.f, x);
+    case AT_ACT_GELU: return 0.5f * (1.f + act_erf(0.707106781f * x)) * x;
+    case AT_ACT_GELUAPPROX: return 0.5f * (1.f + act_tanh(0.7978845608f * x * (1.f + 0.044715f * x * x))) * x;
+    case AT_ACT_SILU: return x * act_sigmoid(x);
+    case AT_ACT_RELU6: return fminf(fmaxf(0.f, x), 6.f);
+    case AT_ACT_HARDSIGMOID: return fmaxf(0.f, fminf(1.f, x / 6.f + 0.5f));
+    case AT_ACT_HARDTANH: return fmaxf(-1.f, fminf(1.f, x));
+    case AT_ACT_HARDSWISH: return x * fminf(fmaxf(0.f, x + 3.f), 6.f) / 6.f;
+    case AT_ACT_SELU: return kSeluScale * (fmaxf(0.f, x) + fminf(0.f, kSeluAlpha * (__expf(x) - 1.f)));
+    case AT_ACT_MISH: return x * act_tanh(__logf(1.f + __expf(x)));
+    case AT_ACT_SOFTPLUS: return __logf(1.f + __expf(x));
+    case AT_ACT_SOFTSIGN: return x / (1.f + fabsf(x));
+    case AT_ACT_TANHSHRINK: return x - act_tanh(x);
+    case AT_ACT_LEAKY_RELU: return fmaxf(0.f, x) + p * fminf(0.f, x);
+    case AT_ACT_ELU: return x <= 0.f ? p * (__expf(x) - 1.f) : x;
+    case AT_ACT_CELU: return fmaxf(0.f, x) + fminf(0.f, p * (__expf(x / p) - 1.f));
+    case AT_ACT_HARDSHRINK: return fabsf(x) <= p ? 0.f : x;
+    case AT_ACT_SOFTSHRINK: return x > p ? x - p : (x < -p ? x + p : 0.f);
+    default: return x;
+  }
+}
+
+__device__ __forceinline__ float act_derivative(int act, float x, float p) {
+  switch (act) {
+    case AT_ACT_SIGMOID: { const float s = act_sigmoid(x); return s * (1.f - s); }
+    case AT_ACT_LOGSIGMOID: return 1.f / (1.f + __expf(x));
+    case AT_ACT_TANH: { const float t = act_tanh(x); return 1.f - t * t; }
+    case AT_ACT_RELU: return x <= 0.f ? 0.f : 1.f;
+    case AT_ACT_GELU: {
+      const float cdf = 0.5f * (1.f + act_erf(0.707106781f * x));
+      return 0.39894228f * __expf(-0.5f * x * x) * x + cdf;
+    }
+    case AT_ACT_GELUAPPROX: {
+      const float t = act_tanh(0.7978845608f * x * (1.f + 0.044715f * x * x));
+      return 0.5f * (1.f + t + x * (1.f - t * t) * 0.7978845608f * (1.f + 3.f * 0.044715f * x * x));
+    }
+    case AT_ACT_SILU: { const float s = act_sigmoid(x); return s * (x * (1.f - s) + 1.f); }
+    case AT_ACT_RELU6: return (0.f < x && x < 6.f) ? 1.f : 0.f;
+    case AT_ACT_HARDSIGMOID: return (-3.f < x && x < 3.f) ? (1.f / 6.f) : 0.f;
+    case AT_ACT_HARDTANH: return (-1.f < x && x < 1.f) ? 1.f : 0.f;
+    case AT_ACT_HARDSWISH: return x < -3.f ? 0.f : (x <= 3.f ? x / 3.f + 0.5f : 1.f);
+    case AT_ACT_SELU: return kSeluScale * (x <= 0.f ? kSeluAlpha * __expf(x) : 1.f);
+    case AT_ACT_MISH: {
+      if (x > 20.f) return 1.f;  // the ratio is 1 to fp32 precision and exp(4x) would overflow
+      const float e = __expf(x);
+      const float d = e * (e + 2.f) + 2.f;
+      return e * (e * ((4.f * x + 6.f) + e * (e + 4.f)) + 4.f * (x + 1.f)) / (d * d);
+    }
+    case AT_ACT_SOFTPLUS: return act_sigmoid(x);
+    case AT_ACT_SOFTSIGN: { const float d = 1.f + fabsf(x); return 1.f / (d * d); }
+    case AT_ACT_TANHSHRINK: { const float t = act_tanh(x); return t * t; }
+    case AT_ACT_LEAKY_RELU: return x <= 0.f ? p : 1.f;
+    case AT_ACT_ELU: return x <= 0.f ? p * __expf(x) : 1.f;
+    case AT_ACT_CELU: return x <= 0.f ? __expf(x / p) : 1.f;
+    case AT_ACT_HARDSHRINK:
+    case AT_ACT_SOFTSHRINK: return fabsf(x) <= p ? 0.f : 1.f;
+    default: return 1.f;
+  }
+}
+
+}  // namespace at_hip

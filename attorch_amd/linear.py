@@ -1,0 +1,224 @@
+"""
+Linear layer with fused bias and activation with PyTorch autodiff support, running on the
+gfx950 MFMA GEMM kernels.
+
+API mirrors attorch/linear_layer.py: the weight is stored [in_features, out_features], the
+forward pass fuses bias + activation (saving the pre-activation only when a gradient is
+needed), and backward returns gradients for (input, weight, bias, act_func).  Unlike the
+reference, the two backward matrix products and the bias column sum also run on this
+library's kernels instead of torch's.
+"""
+
+from typing import Any, Optional, Tuple
+
+import torch
+from torch import Tensor
+from torch import nn
+
+from . import _lib
+from .act import act_id, parse_act_func
+from .utils import get_output_dtype
+
+
+def _matrix(tensor: Tensor) -> Tensor:
+    """
+    2D view with unit inner stride (copies only when the layout requires it).
+    """
+    if tensor.stride(-1) != 1 or (tensor.shape[0] > 1 and tensor.stride(0) < tensor.shape[1]):
+        tensor = tensor.contiguous()
+    return tensor
+
+
+class LinearAutoGrad(torch.autograd.Function):
+    """
+    Autodiff for linear layer (attorch/linear_layer.py:19-161).
+    """
+    @staticmethod
+    def forward(
+        ctx: Any,
+        input: Tensor,
+        weight: Tensor,
+        bias: Optional[Tensor] = None,
+        act_func: Optional[str] = None,
+        ) -> Tensor:
+        """
+        Linearly transforms the input using weights, optionally adding bias
+        and fusing an activation function.
+
+        Args:
+            input: Input of shape [..., in_feat_dim].
+            weight: Weights of shape [in_feat_dim, out_feat_dim].
+            bias: Optional bias of shape [out_feat_dim].
+            act_func: Activation name, None for identity: 'sigmoid', 'logsigmoid', 'tanh',
+                'relu', 'gelu', 'geluapprox', 'silu', 'relu6', 'hardsigmoid', 'hardtanh',
+                'hardswish', 'selu', 'mish', 'softplus', 'softsign', 'tanhshrink',
+                'leaky_relu_PARAM', 'elu_PARAM', 'celu_PARAM', 'hardshrink_PARAM',
+                'softshrink_PARAM'.
+
+        Returns:
+            Transformed input of shape [..., out_feat_dim].
+        """
+        assert weight.ndim == 2, \
+            f'Weights must be 2D, received shape {weight.shape}'
+        assert bias is None or bias.ndim == 1, \
+            f'Bias must be 1D, received shape {bias.shape}'
+
+        assert input.shape[-1] == weight.shape[0], \
+            f'Incompatible input ({input.shape}) and weights ({weight.shape}) shape'
+        assert bias is None or weight.shape[1] == bias.shape[0], \
+            f'Incompatible weights ({weight.shape}) and bias ({bias.shape}) shape'
+
+        _lib.require_gpu(input, 'Linear')
+        lib = _lib.load()
+        act_func, param = parse_act_func(act_func)
+        act = act_id(act_func, param)
+
+        flattened_input = input.flatten(0, -2)
+        batch_dim, in_feat_dim = flattened_input.shape
+        _, out_feat_dim = weight.shape
+
+        requires_grad = (input.requires_grad or
+                         weight.requires_grad or
+                         (bias is not None and bias.requires_grad))
+        save_pre_act = requires_grad and (act_func is not None)
+
+        output_dtype = get_output_dtype(input.dtype, autocast='fp16')
+        # Under autocast the operands are rounded to the low-precision dtype before the
+        # product (linear_kernels.py:161-163); otherwise input and weight share a dtype.
+        compute_dtype = output_dtype if output_dtype != input.dtype else input.dtype
+        input_k = _matrix(flattened_input.to(compute_dtype))
+        weight_k = _matrix(weight.to(compute_dtype))
+        bias_k = None if bias is None else bias.contiguous()
+        if bias_k is not None and output_dtype != input.dtype:
+            bias_k = bias_k.to(output_dtype)
+
+        output = torch.empty((batch_dim, out_feat_dim), device=input.device, dtype=output_dtype)
+        pre_act = torch.empty_like(output) if save_pre_act else output
+
+        with torch.cuda.device_of(input):
+            _lib.check(lib.at_linear_fwd(
+                _lib.ptr(input_k), _lib.ptr(weight_k), _lib.ptr(bias_k), _lib.ptr(pre_act),
+                _lib.ptr(output), batch_dim, in_feat_dim, out_feat_dim, input_k.stride(0),
+                weight_k.stride(0), pre_act.stride(0), output.stride(0), act,
+                0.0 if param is None else param, _lib.dtype_id(compute_dtype),
+                _lib.dtype_id(bias_k.dtype) if bias_k is not None else 0,
+                _lib.dtype_id(output_dtype), _lib.stream_of(input)), 'at_linear_fwd')
+
+        ctx.param = param
+        ctx.act_func = act_func
+        ctx.act = act
+        ctx.bias_requires_grad = False if bias is None else bias.requires_grad
+        ctx.output_dtype = output_dtype
+        if requires_grad:
+            ctx.save_for_backward(input, pre_act if save_pre_act else None, weight)
+
+        return output.view(*input.shape[:-1], out_feat_dim)
+
+    @staticmethod
+    def backward(
+        ctx: Any,
+        output_grad: Tensor,
+        ) -> Tuple[Optional[Tensor], ...]:
+        """
+        Gradients of the linear layer with respect to input, weight and bias.
+        """
+        lib = _lib.load()
+        input, pre_act, weight = ctx.saved_tensors
+        output_dtype = ctx.output_dtype
+        device = input.device
+
+        output_grad = _matrix(output_grad.flatten(0, -2))
+        flattened_input = input.flatten(0, -2)
+        batch_dim, in_feat_dim = flattened_input.shape
+        _, out_feat_dim = weight.shape
+        stream = _lib.stream_of(input)
+
+        with torch.cuda.device_of(input):
+            if ctx.act_func is None:
+                pre_act_grad = output_grad
+            else:
+                pre_act_grad = torch.empty((batch_dim, out_feat_dim), dtype=pre_act.dtype,
+                                           device=device)
+                _lib.check(lib.at_act_bwd(
+                    _lib.ptr(output_grad), _lib.ptr(pre_act), _lib.ptr(pre_act_grad),
+                    batch_dim, out_feat_dim, output_grad.stride(0), pre_act.stride(0),
+                    pre_act_grad.stride(0), ctx.act, 0.0 if ctx.param is None else ctx.param,
+                    _lib.dtype_id(output_grad.dtype), _lib.dtype_id(pre_act.dtype), stream),
+                    'at_act_bwd')
+
+            # The products run in the output dtype, as under the reference's
+            # torch.autocast(dtype=output_dtype) block (linear_layer.py:152-155).
+            grad_mm = _matrix(pre_act_grad.to(output_dtype))
+            input_grad = weight_grad = bias_grad = None
+            if input.requires_grad:
+                weight_mm = _matrix(weight.to(output_dtype))
+                input_grad = torch.empty((batch_dim, in_feat_dim), dtype=output_dtype, device=device)
+                _lib.check(lib.at_linear_bwd_input(
+                    _lib.ptr(grad_mm), _lib.ptr(weight_mm), _lib.ptr(input_grad), batch_dim,
+                    in_feat_dim, out_feat_dim, grad_mm.stride(0), weight_mm.stride(0),
+                    input_grad.stride(0), _lib.dtype_id(output_dtype),
+                    _lib.dtype_id(output_dtype), stream), 'at_linear_bwd_input')
+                input_grad = input_grad.view_as(input)
+            if weight.requires_grad:
+                input_mm = _matrix(flattened_input.to(output_dtype))
+                weight_grad = torch.empty((in_feat_dim, out_feat_dim), dtype=output_dtype,
+                                          device=device)
+                if batch_dim == 0:
+                    weight_grad.zero_()
+                else:
+                    _lib.check(lib.at_linear_bwd_weight(
+                        _lib.ptr(input_mm), _lib.ptr(grad_mm), _lib.ptr(weight_grad), batch_dim,
+                        in_feat_dim, out_feat_dim, input_mm.stride(0), grad_mm.stride(0),
+                        weight_grad.stride(0), _lib.dtype_id(output_dtype),
+                        _lib.dtype_id(output_dtype), stream), 'at_linear_bwd_weight')
+            if ctx.bias_requires_grad:
+                bias_grad = torch.empty(out_feat_dim, dtype=pre_act_grad.dtype, device=device)
+                if batch_dim == 0:
+                    bias_grad.zero_()
+                else:
+                    workspace_bytes = lib.at_colsum_workspace_bytes(batch_dim, out_feat_dim)
+                    workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=device)
+                    _lib.check(lib.at_colsum(
+                        _lib.ptr(pre_act_grad), _lib.ptr(bias_grad), _lib.ptr(workspace),
+                        workspace_bytes, batch_dim, out_feat_dim, pre_act_grad.stride(0),
+                        _lib.dtype_id(pre_act_grad.dtype), _lib.dtype_id(bias_grad.dtype), stream),
+                        'at_colsum')
+
+        # One gradient (or None) per forward argument.
+        return input_grad, weight_grad, bias_grad, None
+
+
+class Linear(nn.Linear):
+    """
+    Linearly transforms the input using weights, optionally adding bias
+    and fusing an activation function.
+    See also base class; mirrors attorch/linear_layer.py:164-205.
+
+    Note: the weight matrix of this module has shape [in_features, out_features], not
+    torch's [out_features, in_features].
+
+    Args:
+        in_features: Number of input features.
+        out_features: Number of output features.
+        bias: Flag for additive bias.
+        act_func: Name of activation function to apply, with None for identity
+            (see LinearAutoGrad.forward for the options).
+        device: Device to use.
+        dtype: Dtype of layer.
+    """
+    def __init__(
+        self,
+        in_features: int,
+        out_features: int,
+        bias: bool = True,
+        act_func: Optional[str] = None,
+        device: Any = 'cuda',
+        dtype: torch.dtype = torch.float32,
+        ) -> None:
+        super().__init__(in_features, out_features, bias, device, dtype)
+        self.weight = nn.Parameter(self.weight.T.contiguous())
+        self.act_func = act_func
+
+    def forward(self, input: Tensor) -> Tensor:
+        return LinearAutoGrad.apply(input, self.weight, self.bias,
+                                    self.act_func)

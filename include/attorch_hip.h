@@ -164,6 +164,52 @@ int at_cross_entropy_scale_grad(void* dlogits, const void* output_grad, int64_t 
                                 int64_t feat, int64_t dlogits_stride, int dlogits_dtype,
                                 int grad_dtype, at_stream_t stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Linear — replaces linear_forward_kernel, attorch/linear_kernels.py:59-188 (launched from
+ * attorch/linear_layer.py:90-98), act_func_backward_kernel, attorch/act_kernels.py:888-927
+ * (launched from linear_layer.py:144-146 and batch_norm_layer.py:204-206), and the torch calls
+ * at linear_layer.py:152-156 (two matmuls and a column sum).
+ *   fwd:  output = act(input @ weight + bias), weight is [in_feat, out_feat] (row stride
+ *         weight_stride); fp32 accumulation; when act != AT_ACT_NONE and pre_act is non-null
+ *         (and != output) the accumulator is also stored there before the activation
+ *         (save_pre_act).  bias nullable (add_bias False).  in_dtype is the dtype of input and
+ *         weight; bias may have its own dtype.
+ *   bwd_input:  input_grad[batch, in_feat]   = pre_act_grad[batch, out_feat] @ weight^T
+ *   bwd_weight: weight_grad[in_feat, out_feat] = input^T @ pre_act_grad
+ *   act_bwd:    input_grad = output_grad * act'(input) over a [rows, cols] matrix (a flat
+ *               tensor is rows = 1); input_grad has input's dtype (linear_layer.py:138).
+ *   colsum:     out[cols] = sum over rows (bias gradient, linear_layer.py:156); workspace of
+ *               at_colsum_workspace_bytes(rows, cols) bytes; fixed summation order.
+ * 16-bit operands whose pointers and strides are 16-byte aligned (and K, plus the contiguous
+ * extent of a transposed operand, a multiple of 8) run on the 256x256x64 MFMA kernel; any
+ * other case (fp32, odd sizes, small problems) runs on the generic fp32-MFMA kernel.
+ * ------------------------------------------------------------------------------------------ */
+int at_linear_fwd(const void* input, const void* weight, const void* bias, void* pre_act,
+                  void* output, int64_t batch, int64_t in_feat, int64_t out_feat,
+                  int64_t input_stride, int64_t weight_stride, int64_t pre_act_stride,
+                  int64_t output_stride, int act, float param, int in_dtype, int bias_dtype,
+                  int out_dtype, at_stream_t stream);
+
+int at_linear_bwd_input(const void* pre_act_grad, const void* weight, void* input_grad,
+                        int64_t batch, int64_t in_feat, int64_t out_feat, int64_t grad_stride,
+                        int64_t weight_stride, int64_t input_grad_stride, int in_dtype,
+                        int out_dtype, at_stream_t stream);
+
+int at_linear_bwd_weight(const void* input, const void* pre_act_grad, void* weight_grad,
+                         int64_t batch, int64_t in_feat, int64_t out_feat, int64_t input_stride,
+                         int64_t grad_stride, int64_t weight_grad_stride, int in_dtype,
+                         int out_dtype, at_stream_t stream);
+
+int at_act_bwd(const void* output_grad, const void* input, void* input_grad, int64_t rows,
+               int64_t cols, int64_t output_grad_stride, int64_t input_stride,
+               int64_t input_grad_stride, int act, float param, int grad_dtype, int input_dtype,
+               at_stream_t stream);
+
+int64_t at_colsum_workspace_bytes(int64_t rows, int64_t cols);
+
+int at_colsum(const void* x, void* out, void* workspace, int64_t workspace_bytes, int64_t rows,
+              int64_t cols, int64_t x_stride, int x_dtype, int out_dtype, at_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
