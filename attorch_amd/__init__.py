@@ -7,6 +7,8 @@ CrossEntropyLoss, Conv2d, BatchNorm2d and their autograd Functions), so
 hand-written gfx950 HIP kernels behind the C ABI declared in include/attorch_hip.h.
 """
 
+from .batch_norm import BatchNorm1d, BatchNorm2d, BatchNormAutoGrad
+from .conv import Conv1d, Conv2d, Conv2dAutoGrad
 from .cross_entropy import CrossEntropyLoss, CrossEntropyLossAutoGrad
 from .linear import Linear, LinearAutoGrad
 from .norms import LayerNorm, LayerNormAutoGrad, RMSNorm, RMSNormAutoGrad

@@ -1,0 +1,261 @@
+"""
+2D (and 1D) convolution with PyTorch autodiff support, running on the gfx950 implicit-GEMM
+kernels.
+
+API mirrors attorch/conv_layer.py: Conv2dAutoGrad.apply(input, weight, bias, stride_height,
+stride_width, padding_height, padding_width, groups) and Conv1d / Conv2d modules (zero
+padding, no dilation).  Unlike the reference, the backward pass (input gradient, weight
+gradient, bias gradient) also runs on this library's kernels instead of torch.nn.grad.
+"""
+
+from typing import Any, Optional, Tuple, Union
+
+import torch
+from torch import Tensor
+from torch import nn
+
+from . import _lib
+from .utils import get_output_dtype
+
+
+def conv2d_output_size(
+    in_size: int,
+    kernel_size: int,
+    stride: int,
+    padding: int,
+    ) -> int:
+    """
+    Output size of a convolution along one dimension (attorch/conv_layer.py:18-36).
+
+    Args:
+        in_size: Input size.
+        kernel_size: Kernel size.
+        stride: Stride.
+        padding: Padding on each side.
+
+    Returns:
+        Output size.
+    """
+    return (in_size + 2 * padding - kernel_size) // stride + 1
+
+
+class Conv2dAutoGrad(torch.autograd.Function):
+    """
+    Autodiff for 2D convolutional layer (attorch/conv_layer.py:39-164).
+    """
+    @staticmethod
+    def forward(
+        ctx: Any,
+        input: Tensor,
+        weight: Tensor,
+        bias: Optional[Tensor] = None,
+        stride_height: int = 1,
+        stride_width: int = 1,
+        padding_height: int = 1,
+        padding_width: int = 1,
+        groups: int = 1,
+        ) -> Tensor:
+        """
+        2D-convolves over the input using weights, optionally adding bias.
+
+        Args:
+            input: Input of shape [batch_dim, in_feat_dim, in_height, in_width].
+            weight: Weights of shape [out_feat_dim, in_feat_dim / groups, kernel_height, kernel_width].
+            bias: Optional bias of shape [out_feat_dim].
+            stride_height: Stride over the height.
+            stride_width: Stride over the width.
+            padding_height: Zero padding on each side of the height.
+            padding_width: Zero padding on each side of the width.
+            groups: Number of groups.
+
+        Returns:
+            Output of shape [batch_dim, out_feat_dim, out_height, out_width].
+        """
+        assert weight.ndim == 4, \
+            f'Weights must be 4D, received shape {weight.shape}'
+        assert bias is None or bias.ndim == 1, \
+            f'Bias must be 1D, received shape {bias.shape}'
+
+        assert input.shape[1] == groups * weight.shape[1], \
+            f'Incompatible input ({input.shape}) and weights ({weight.shape}) shape with {groups} groups'
+        assert bias is None or weight.shape[0] == bias.shape[0], \
+            f'Incompatible weights ({weight.shape}) and bias ({bias.shape}) shape'
+
+        _lib.require_gpu(input, 'Conv2d')
+        lib = _lib.load()
+        batch_dim, in_feat_dim, in_height, in_width = input.shape
+        out_feat_dim, _, kernel_height, kernel_width = weight.shape
+        out_height = conv2d_output_size(in_height, kernel_height,
+                                        stride_height, padding_height)
+        out_width = conv2d_output_size(in_width, kernel_width,
+                                       stride_width, padding_width)
+
+        output_dtype = get_output_dtype(input.dtype, autocast='fp16')
+        # Under autocast the operands are rounded to the low-precision dtype first
+        # (conv_kernels.py:191-193).
+        input_k = input.to(output_dtype).contiguous()
+        weight_k = weight.to(output_dtype).contiguous()
+        bias_k = None if bias is None else bias.to(output_dtype).contiguous()
+        output = torch.empty((batch_dim, out_feat_dim, out_height, out_width),
+                             device=input.device, dtype=output_dtype)
+        dims = (batch_dim, in_feat_dim, in_height, in_width, out_feat_dim, out_height, out_width,
+                kernel_height, kernel_width, stride_height, stride_width,
+                padding_height, padding_width, groups)
+
+        with torch.cuda.device_of(input):
+            _lib.check(lib.at_conv2d_fwd(
+                _lib.ptr(input_k), _lib.ptr(weight_k), _lib.ptr(bias_k), _lib.ptr(output), *dims,
+                _lib.dtype_id(output_dtype), _lib.dtype_id(output_dtype),
+                _lib.dtype_id(output_dtype), _lib.stream_of(input)), 'at_conv2d_fwd')
+
+        requires_grad = (input.requires_grad or
+                         weight.requires_grad or
+                         (bias is not None and bias.requires_grad))
+        ctx.dims = dims
+        ctx.bias_requires_grad = False if bias is None else bias.requires_grad
+        ctx.output_dtype = output_dtype
+        if requires_grad:
+            ctx.save_for_backward(input, weight)
+
+        return output
+
+    @staticmethod
+    def backward(
+        ctx: Any,
+        output_grad: Tensor,
+        ) -> Tuple[Optional[Tensor], ...]:
+        """
+        Gradients of the convolution with respect to input, weight and bias, all in the
+        output dtype (attorch/conv_layer.py:147-162).
+        """
+        lib = _lib.load()
+        input, weight = ctx.saved_tensors
+        output_dtype = ctx.output_dtype
+        device = input.device
+        dims = ctx.dims
+        (batch_dim, in_feat_dim, _, _, out_feat_dim, out_height, out_width,
+         kernel_height, kernel_width, _, _, _, _, groups) = dims
+        output_grad = output_grad.to(output_dtype).contiguous()
+        stream = _lib.stream_of(input)
+        dtype = _lib.dtype_id(output_dtype)
+
+        input_grad = weight_grad = bias_grad = None
+        with torch.cuda.device_of(input):
+            if input.requires_grad:
+                weight_k = weight.to(output_dtype).contiguous()
+                input_grad = torch.empty(input.shape, dtype=output_dtype, device=device)
+                _lib.check(lib.at_conv2d_bwd_input(
+                    _lib.ptr(output_grad), _lib.ptr(weight_k), _lib.ptr(input_grad), *dims,
+                    dtype, stream), 'at_conv2d_bwd_input')
+            if weight.requires_grad:
+                input_k = input.to(output_dtype).contiguous()
+                weight_grad = torch.empty(weight.shape, dtype=output_dtype, device=device)
+                workspace_bytes = lib.at_conv2d_bwd_weight_workspace_bytes(
+                    out_feat_dim, in_feat_dim // groups, kernel_height, kernel_width)
+                workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=device)
+                _lib.check(lib.at_conv2d_bwd_weight(
+                    _lib.ptr(output_grad), _lib.ptr(input_k), _lib.ptr(weight_grad),
+                    _lib.ptr(workspace), workspace_bytes, *dims, dtype, stream),
+                    'at_conv2d_bwd_weight')
+            if ctx.bias_requires_grad:
+                bias_grad = torch.empty(out_feat_dim, dtype=output_dtype, device=device)
+                _lib.check(lib.at_channel_sum(
+                    _lib.ptr(output_grad), _lib.ptr(bias_grad), batch_dim, out_feat_dim,
+                    out_height * out_width, dtype, dtype, stream), 'at_channel_sum')
+
+        return input_grad, weight_grad, bias_grad, None, None, None, None, None
+
+
+class Conv1d(nn.Conv1d):
+    """
+    1D-convolves over the input using weights, optionally adding bias.
+    See also base class; mirrors attorch/conv_layer.py:167-220.
+
+    Args:
+        in_channels: Number of input channels.
+        out_channels: Number of output channels.
+        kernel_size: Kernel size.
+        stride: Stride of kernel.
+        padding: Padding applied to the input.
+        dilation: Dilation of kernel. Only 1 is supported.
+        groups: Number of groups for the convolution.
+        bias: Flag for additive bias.
+        padding_mode: Padding mode. Only 'zeros' is supported.
+        device: Device to use.
+        dtype: Dtype of layer.
+    """
+    def __init__(
+        self,
+        in_channels: int,
+        out_channels: int,
+        kernel_size: int,
+        stride: int = 1,
+        padding: int = 0,
+        dilation: int = 1,
+        groups: int = 1,
+        bias: bool = True,
+        padding_mode: str = 'zeros',
+        device: Any = 'cuda',
+        dtype: torch.dtype = torch.float32,
+        ) -> None:
+        super().__init__(in_channels, out_channels, kernel_size, stride, padding,
+                         dilation, groups, bias, padding_mode, device, dtype)
+
+        if self.dilation != (1,):
+            raise RuntimeError('Convolutional layer only supports dilation of 1.')
+
+        if self.padding_mode != 'zeros':
+            raise RuntimeError("Convolutional layer only support 'zeros' padding mode.")
+
+    def forward(self, input: Tensor) -> Tensor:
+        return Conv2dAutoGrad.apply(input.unsqueeze(-1), self.weight.unsqueeze(-1),
+                                    self.bias,
+                                    *self.stride, 1, *self.padding, 0,
+                                    self.groups).squeeze(-1)
+
+
+class Conv2d(nn.Conv2d):
+    """
+    2D-convolves over the input using weights, optionally adding bias.
+    See also base class; mirrors attorch/conv_layer.py:223-278.
+
+    Args:
+        in_channels: Number of input channels.
+        out_channels: Number of output channels.
+        kernel_size: Kernel size.
+        stride: Stride of kernel.
+        padding: Padding applied to the input.
+        dilation: Dilation of kernel. Only 1 and (1, 1) are supported.
+        groups: Number of groups for the convolution.
+        bias: Flag for additive bias.
+        padding_mode: Padding mode. Only 'zeros' is supported.
+        device: Device to use.
+        dtype: Dtype of layer.
+    """
+    def __init__(
+        self,
+        in_channels: int,
+        out_channels: int,
+        kernel_size: Union[int, Tuple[int, int]],
+        stride: Union[int, Tuple[int, int]] = 1,
+        padding: Union[int, Tuple[int, int]] = 0,
+        dilation: Union[int, Tuple[int, int]] = 1,
+        groups: int = 1,
+        bias: bool = True,
+        padding_mode: str = 'zeros',
+        device: Any = 'cuda',
+        dtype: torch.dtype = torch.float32,
+        ) -> None:
+        super().__init__(in_channels, out_channels, kernel_size, stride, padding,
+                         dilation, groups, bias, padding_mode, device, dtype)
+
+        if self.dilation != (1, 1):
+            raise RuntimeError('Convolutional layer only supports dilation of 1 and (1, 1).')
+
+        if self.padding_mode != 'zeros':
+            raise RuntimeError("Convolutional layer only support 'zeros' padding mode.")
+
+    def forward(self, input: Tensor) -> Tensor:
+        return Conv2dAutoGrad.apply(input, self.weight, self.bias,
+                                    *self.stride, *self.padding,
+                                    self.groups)

@@ -1,0 +1,372 @@
+// 2D convolution (NCHW, zero padding, stride, groups, no dilation) as implicit GEMM: forward,
+// input gradient and weight gradient.
+//
+// The im2col matrix is never materialised: the operand tiles are gathered straight from the
+// NCHW tensors into LDS, multiplied with fp32-accumulating MFMA (v_mfma_f32_32x32x2f32) in
+// 64x64 output tiles, and scattered back to NCHW.
+//   forward      : Y[(n,oh,ow), co]   = sum_{c,kh,kw} X[n,c,oh*s-p+kh,ow*s-p+kw] * W[co,c,kh,kw]
+//   input grad   : dX[(n,ih,iw), c]   = sum_{co,kh,kw} dY[n,co,(ih+p-kh)/s,(iw+p-kw)/s] * W[co,c,kh,kw]
+//   weight grad  : dW[co, (c,kh,kw)]  = sum_{n,oh,ow} dY[n,co,oh,ow] * X[n,c,oh*s-p+kh,ow*s-p+kw]
+// The weight gradient contracts over batch x space, so it is split over many workgroups that
+// write fp32 partial tiles, summed by a second launch in fixed order.
+#include <type_traits>
+
+#include "at_common.h"
+
+namespace at_hip {
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+enum ConvMode { kConvFwd = 0, kConvDx = 1, kConvDw = 2 };
+
+struct ConvArgs {
+  const void* a;     // fwd: X, dx: dY, dw: dY
+  const void* b;     // fwd: W, dx: W,  dw: X
+  void* out;         // fwd: Y, dx: dX, dw: fp32 partials
+  const void* bias;  // fwd only, nullable
+  int bias_dt;
+  int N, C, H, W, O, KH, KW, OH, OW, sh, sw, ph, pw, groups;
+  int Cg, Og;        // channels per group (input / output)
+  int64_t M, K;      // GEMM rows and contraction length
+  int cols;          // GEMM columns
+  int64_t k_per_split;
+};
+
+constexpr int TM = 64, TN = 64, TK = 16;
+
+template <int MODE, typename TI, typename TO>
+__global__ __launch_bounds__(256) void conv_gemm_kernel(ConvArgs g) {
+  __shared__ float sa[TK][TM + 1];
+  __shared__ float sb[TK][TN + 1];
+  const TI* __restrict__ A = reinterpret_cast<const TI*>(g.a);
+  const TI* __restrict__ B = reinterpret_cast<const TI*>(g.b);
+  const int grp = blockIdx.z;
+  const int nbn = (g.cols + TN - 1) / TN;
+  const int64_t m0 = (int64_t)(blockIdx.x / nbn) * TM;
+  const int n0 = (blockIdx.x % nbn) * TN;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int KK = g.KH * g.KW;
+
+  int64_t k_begin = 0, k_end = g.K;
+  if (MODE == kConvDw) {
+    k_begin = (int64_t)blockIdx.y * g.k_per_split;
+    k_end = k_begin + g.k_per_split < g.K ? k_begin + g.k_per_split : g.K;
+  }
+
+  // Per-thread tile coordinates.  For fwd/dx the m index (fast across lanes, contiguous in
+  // memory along the image row) is fixed per thread; its decomposition is hoisted.
+  const int mm_fast = threadIdx.x & 63, kk_slow = threadIdx.x >> 6;   // e = tid + 256 i -> kk = kk_slow + 4 i
+  const int kk_fast = threadIdx.x & 15, xx_slow = threadIdx.x >> 4;   // e = tid + 256 i -> xx = xx_slow + 16 i
+
+  int a_n = 0, a_p = 0, a_q = 0;  // (n, oh, ow) for fwd, (n, ih, iw) for dx
+  bool a_row_ok = false;
+  if (MODE != kConvDw) {
+    const int64_t m = m0 + mm_fast;
+    a_row_ok = m < g.M;
+    const int pw_ = MODE == kConvFwd ? g.OW : g.W, ph_ = MODE == kConvFwd ? g.OH : g.H;
+    const int64_t t = a_row_ok ? m : 0;
+    a_q = (int)(t % pw_);
+    a_p = (int)((t / pw_) % ph_);
+    a_n = (int)(t / ((int64_t)pw_ * ph_));
+  }
+
+  f32x16 acc;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+
+  for (int64_t k0 = k_begin; k0 < k_end; k0 += TK) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      // ---- A tile ----
+      if (MODE == kConvFwd) {
+        const int kk = kk_slow + 4 * i;
+        const int64_t k = k0 + kk;
+        float v = 0.f;
+        if (a_row_ok && k < k_end) {
+          const int c = (int)(k / KK), r = (int)(k % KK), kh = r / g.KW, kw = r % g.KW;
+          const int ih = a_p * g.sh - g.ph + kh, iw = a_q * g.sw - g.pw + kw;
+          if (ih >= 0 && ih < g.H && iw >= 0 && iw < g.W)
+            v = to_f32(A[(((int64_t)a_n * g.C + grp * g.Cg + c) * g.H + ih) * g.W + iw]);
+        }
+        sa[kk][mm_fast] = v;
+      } else if (MODE == kConvDx) {
+        const int kk = kk_slow + 4 * i;
+        const int64_t k = k0 + kk;
+        float v = 0.f;
+        if (a_row_ok && k < k_end) {
+          const int co = (int)(k / KK), r = (int)(k % KK), kh = r / g.KW, kw = r % g.KW;
+          const int th = a_p + g.ph - kh, tw = a_q + g.pw - kw;
+          if (th >= 0 && tw >= 0 && th % g.sh == 0 && tw % g.sw == 0) {
+            const int oh = th / g.sh, ow = tw / g.sw;
+            if (oh < g.OH && ow < g.OW)
+              v = to_f32(A[(((int64_t)a_n * g.O + grp * g.Og + co) * g.OH + oh) * g.OW + ow]);
+          }
+        }
+        sa[kk][mm_fast] = v;
+      } else {
+        // dw: A(co, k) = dY[n, co, oh, ow], k = (n, oh, ow) contiguous over (oh, ow)
+        const int kk = kk_fast, mm = xx_slow + 16 * i;
+        const int64_t k = k0 + kk;
+        const int co = (int)m0 + mm;
+        float v = 0.f;
+        if (co < g.Og && k < k_end) {
+          const int64_t hw = (int64_t)g.OH * g.OW;
+          const int64_t n = k / hw, r = k % hw;
+          v = to_f32(A[(n * g.O + grp * g.Og + co) * hw + r]);
+        }
+        sa[kk][mm] = v;
+      }
+      // ---- B tile ----
+      if (MODE == kConvFwd) {
+        // B(k, co) = W[co, k], contiguous over k
+        const int kk = kk_fast, nn = xx_slow + 16 * i;
+        const int64_t k = k0 + kk;
+        const int co = n0 + nn;
+        sb[kk][nn] = (co < g.Og && k < k_end) ? to_f32(B[((int64_t)grp * g.Og + co) * g.K + k]) : 0.f;
+      } else if (MODE == kConvDx) {
+        // B(k = (co, kh, kw), c) = W[co, c, kh, kw]
+        const int kk = kk_fast, nn = xx_slow + 16 * i;
+        const int64_t k = k0 + kk;
+        const int c = n0 + nn;
+        float v = 0.f;
+        if (c < g.Cg && k < k_end) {
+          const int co = (int)(k / KK), r = (int)(k % KK);
+          v = to_f32(B[(((int64_t)grp * g.Og + co) * g.Cg + c) * KK + r]);
+        }
+        sb[kk][nn] = v;
+      } else {
+        // dw: B(k = (n, oh, ow), j = (c, kh, kw)) = X[n, c, oh*s-p+kh, ow*s-p+kw]
+        const int kk = kk_fast, nn = xx_slow + 16 * i;
+        const int64_t k = k0 + kk;
+        const int j = n0 + nn;
+        float v = 0.f;
+        if (j < g.cols && k < k_end) {
+          const int c = j / KK, r = j % KK, kh = r / g.KW, kw = r % g.KW;
+          const int ow = (int)(k % g.OW), oh = (int)((k / g.OW) % g.OH);
+          const int64_t n = k / ((int64_t)g.OW * g.OH);
+          const int ih = oh * g.sh - g.ph + kh, iw = ow * g.sw - g.pw + kw;
+          if (ih >= 0 && ih < g.H && iw >= 0 && iw < g.W)
+            v = to_f32(B[((n * g.C + grp * g.Cg + c) * g.H + ih) * g.W + iw]);
+        }
+        sb[kk][nn] = v;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < TK; ks += 2) {
+      const float av = sa[ks + (lane >> 5)][wm * 32 + (lane & 31)];
+      const float bv = sb[ks + (lane >> 5)][wn * 32 + (lane & 31)];
+      // fwd / dx outputs are contiguous along m, so the operands are swapped there: a lane then
+      // owns one m (lane % 32) and 16 columns, and 32 consecutive lanes store consecutive addresses
+      acc = MODE == kConvDw ? __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc, 0, 0, 0)
+                            : __builtin_amdgcn_mfma_f32_32x32x2f32(bv, av, acc, 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+  // acc[r] belongs to (row, column) = (sub, lane % 32) for dw and (lane % 32, sub) otherwise,
+  // with sub = (r/4)*8 + (lane/32)*4 + r%4.
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int sub = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+    const int64_t m = m0 + wm * 32 + (MODE == kConvDw ? sub : (lane & 31));
+    const int col = n0 + wn * 32 + (MODE == kConvDw ? (lane & 31) : sub);
+    if (m >= g.M || col >= g.cols) continue;
+    const float v = acc[r];
+    if (MODE == kConvFwd) {
+      const int ow = (int)(m % g.OW), oh = (int)((m / g.OW) % g.OH);
+      const int64_t n = m / ((int64_t)g.OW * g.OH);
+      const int co = grp * g.Og + col;
+      const float bb = g.bias ? load_scalar_f32(g.bias, g.bias_dt, co) : 0.f;
+      reinterpret_cast<TO*>(g.out)[((n * g.O + co) * g.OH + oh) * g.OW + ow] = from_f32<TO>(v + bb);
+    } else if (MODE == kConvDx) {
+      const int iw = (int)(m % g.W), ih = (int)((m / g.W) % g.H);
+      const int64_t n = m / ((int64_t)g.W * g.H);
+      reinterpret_cast<TO*>(g.out)[((n * g.C + grp * g.Cg + col) * g.H + ih) * g.W + iw] = from_f32<TO>(v);
+    } else {
+      // partial [split][O][cols]
+      float* part = reinterpret_cast<float*>(g.out);
+      part[((int64_t)blockIdx.y * g.O + grp * g.Og + m) * g.cols + col] = v;
+    }
+  }
+}
+
+template <typename TO>
+__global__ void conv_dw_reduce_kernel(const float* __restrict__ part, TO* __restrict__ out, int splits,
+                                      int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  float s = 0.f;
+  for (int p = 0; p < splits; ++p) s += part[(int64_t)p * total + i];
+  out[i] = from_f32<TO>(s);
+}
+
+// Per-channel sum over batch and space of a [N, C, S] tensor (bias gradient).
+template <typename T>
+__global__ __launch_bounds__(256) void channel_sum_kernel(const T* __restrict__ x, void* __restrict__ out,
+                                                         int out_dt, int64_t N, int C, int64_t S) {
+  __shared__ float smem[16];
+  const int c = blockIdx.x;
+  float s = 0.f;
+  for (int64_t n = 0; n < N; ++n) {
+    const T* plane = x + (n * C + c) * S;
+    for (int64_t i = threadIdx.x; i < S; i += 256) s += to_f32(plane[i]);
+  }
+  s = group_reduce(s, 256, smem, SumOp(), 0.f);
+  if (threadIdx.x == 0) store_scalar_f32(out, out_dt, c, s);
+}
+
+template <typename F>
+inline int dispatch_dtype(int dt, F&& f) {
+  if (dt == AT_DTYPE_F32) return f((float*)0);
+  if (dt == AT_DTYPE_F16) return f((f16_t*)0);
+  if (dt == AT_DTYPE_BF16) return f((bf16_t*)0);
+  return AT_ERR_DTYPE;
+}
+
+struct ConvShape {
+  int64_t N, C, H, W, O, KH, KW, sh, sw, ph, pw, groups;
+  int64_t OH, OW;
+};
+
+inline int check_shape(const ConvShape& s) {
+  if (s.N <= 0 || s.C <= 0 || s.H <= 0 || s.W <= 0 || s.O <= 0 || s.KH <= 0 || s.KW <= 0) return AT_ERR_DIM;
+  if (s.sh <= 0 || s.sw <= 0 || s.ph < 0 || s.pw < 0 || s.groups <= 0) return AT_ERR_DIM;
+  if (s.C % s.groups || s.O % s.groups) return AT_ERR_DIM;
+  if (s.OH <= 0 || s.OW <= 0) return AT_ERR_DIM;
+  if (s.OH != (s.H + 2 * s.ph - s.KH) / s.sh + 1 || s.OW != (s.W + 2 * s.pw - s.KW) / s.sw + 1) return AT_ERR_DIM;
+  const int64_t lim = INT32_MAX;
+  if (s.N > lim || s.C > lim || s.H > lim || s.W > lim || s.O > lim || s.C / s.groups * s.KH * s.KW > lim ||
+      s.O / s.groups * s.KH * s.KW > lim)
+    return AT_ERR_DIM;
+  return AT_OK;
+}
+
+inline ConvArgs base_args(const ConvShape& s) {
+  ConvArgs g{};
+  g.N = (int)s.N; g.C = (int)s.C; g.H = (int)s.H; g.W = (int)s.W; g.O = (int)s.O; g.KH = (int)s.KH;
+  g.KW = (int)s.KW; g.OH = (int)s.OH; g.OW = (int)s.OW; g.sh = (int)s.sh; g.sw = (int)s.sw; g.ph = (int)s.ph;
+  g.pw = (int)s.pw; g.groups = (int)s.groups; g.Cg = (int)(s.C / s.groups); g.Og = (int)(s.O / s.groups);
+  return g;
+}
+
+constexpr int kDwMaxSplits = 512;
+
+inline int dw_splits(const ConvShape& s) {
+  const int64_t K = s.N * s.OH * s.OW;
+  const int64_t tiles = cdiv64(s.O / s.groups, TM) * cdiv64(s.C / s.groups * s.KH * s.KW, TN) * s.groups;
+  int64_t want = cdiv64((int64_t)device_cu_count() * 4, tiles);
+  const int64_t max_by_k = cdiv64(K, 4 * TK);
+  if (want > max_by_k) want = max_by_k;
+  if (want > kDwMaxSplits) want = kDwMaxSplits;
+  if (want < 1) want = 1;
+  return (int)want;
+}
+
+}  // namespace
+}  // namespace at_hip
+
+using namespace at_hip;
+
+extern "C" {
+
+int at_conv2d_fwd(const void* input, const void* weight, const void* bias, void* output, int64_t batch,
+                  int64_t in_feat, int64_t in_height, int64_t in_width, int64_t out_feat, int64_t out_height,
+                  int64_t out_width, int64_t kernel_height, int64_t kernel_width, int64_t stride_height,
+                  int64_t stride_width, int64_t padding_height, int64_t padding_width, int64_t groups,
+                  int in_dtype, int bias_dtype, int out_dtype, at_stream_t stream) {
+  if (!input || !weight || !output) return AT_ERR_NULL;
+  if (!dtype_valid(in_dtype) || !dtype_valid(out_dtype) || (bias && !dtype_valid(bias_dtype))) return AT_ERR_DTYPE;
+  const ConvShape s{batch, in_feat, in_height, in_width, out_feat, kernel_height, kernel_width, stride_height,
+                    stride_width, padding_height, padding_width, groups, out_height, out_width};
+  int rc = check_shape(s);
+  if (rc) return rc;
+  ConvArgs g = base_args(s);
+  g.a = input; g.b = weight; g.out = output; g.bias = bias; g.bias_dt = bias_dtype;
+  g.M = s.N * s.OH * s.OW; g.K = (int64_t)g.Cg * g.KH * g.KW; g.cols = g.Og;
+  const dim3 grid((unsigned)(cdiv64(g.M, TM) * cdiv64(g.cols, TN)), 1, (unsigned)g.groups);
+  return dispatch_dtype(in_dtype, [&](auto* ti) -> int {
+    typedef std::remove_pointer_t<decltype(ti)> TI;
+    return dispatch_dtype(out_dtype, [&](auto* to) -> int {
+      typedef std::remove_pointer_t<decltype(to)> TO;
+      hipLaunchKernelGGL((conv_gemm_kernel<kConvFwd, TI, TO>), grid, dim3(256), 0, (hipStream_t)stream, g);
+      return launch_status();
+    });
+  });
+}
+
+int at_conv2d_bwd_input(const void* output_grad, const void* weight, void* input_grad, int64_t batch,
+                        int64_t in_feat, int64_t in_height, int64_t in_width, int64_t out_feat,
+                        int64_t out_height, int64_t out_width, int64_t kernel_height, int64_t kernel_width,
+                        int64_t stride_height, int64_t stride_width, int64_t padding_height,
+                        int64_t padding_width, int64_t groups, int dtype, at_stream_t stream) {
+  if (!output_grad || !weight || !input_grad) return AT_ERR_NULL;
+  if (!dtype_valid(dtype)) return AT_ERR_DTYPE;
+  const ConvShape s{batch, in_feat, in_height, in_width, out_feat, kernel_height, kernel_width, stride_height,
+                    stride_width, padding_height, padding_width, groups, out_height, out_width};
+  int rc = check_shape(s);
+  if (rc) return rc;
+  ConvArgs g = base_args(s);
+  g.a = output_grad; g.b = weight; g.out = input_grad;
+  g.M = s.N * s.H * s.W; g.K = (int64_t)g.Og * g.KH * g.KW; g.cols = g.Cg;
+  const dim3 grid((unsigned)(cdiv64(g.M, TM) * cdiv64(g.cols, TN)), 1, (unsigned)g.groups);
+  return dispatch_dtype(dtype, [&](auto* tp) -> int {
+    typedef std::remove_pointer_t<decltype(tp)> T;
+    hipLaunchKernelGGL((conv_gemm_kernel<kConvDx, T, T>), grid, dim3(256), 0, (hipStream_t)stream, g);
+    return launch_status();
+  });
+}
+
+int64_t at_conv2d_bwd_weight_workspace_bytes(int64_t out_feat, int64_t in_feat_per_group, int64_t kernel_height,
+                                             int64_t kernel_width) {
+  if (out_feat <= 0 || in_feat_per_group <= 0 || kernel_height <= 0 || kernel_width <= 0) return 0;
+  return (int64_t)kDwMaxSplits * out_feat * in_feat_per_group * kernel_height * kernel_width * (int64_t)sizeof(float);
+}
+
+int at_conv2d_bwd_weight(const void* output_grad, const void* input, void* weight_grad, void* workspace,
+                         int64_t workspace_bytes, int64_t batch, int64_t in_feat, int64_t in_height,
+                         int64_t in_width, int64_t out_feat, int64_t out_height, int64_t out_width,
+                         int64_t kernel_height, int64_t kernel_width, int64_t stride_height, int64_t stride_width,
+                         int64_t padding_height, int64_t padding_width, int64_t groups, int dtype,
+                         at_stream_t stream) {
+  if (!output_grad || !input || !weight_grad) return AT_ERR_NULL;
+  if (!dtype_valid(dtype)) return AT_ERR_DTYPE;
+  const ConvShape s{batch, in_feat, in_height, in_width, out_feat, kernel_height, kernel_width, stride_height,
+                    stride_width, padding_height, padding_width, groups, out_height, out_width};
+  int rc = check_shape(s);
+  if (rc) return rc;
+  ConvArgs g = base_args(s);
+  const int splits = dw_splits(s);
+  const int64_t total = s.O * g.Cg * s.KH * s.KW;
+  if (!workspace || workspace_bytes < (int64_t)splits * total * (int64_t)sizeof(float)) return AT_ERR_WORKSPACE;
+  g.a = output_grad; g.b = input; g.out = workspace;
+  g.M = g.Og; g.K = s.N * s.OH * s.OW; g.cols = g.Cg * g.KH * g.KW;
+  g.k_per_split = cdiv64(cdiv64(g.K, splits), TK) * TK;
+  const dim3 grid((unsigned)(cdiv64(g.M, TM) * cdiv64(g.cols, TN)), (unsigned)splits, (unsigned)g.groups);
+  return dispatch_dtype(dtype, [&](auto* tp) -> int {
+    typedef std::remove_pointer_t<decltype(tp)> T;
+    hipLaunchKernelGGL((conv_gemm_kernel<kConvDw, T, float>), grid, dim3(256), 0, (hipStream_t)stream, g);
+    int rc2 = launch_status();
+    if (rc2) return rc2;
+    hipLaunchKernelGGL((conv_dw_reduce_kernel<T>), dim3((unsigned)cdiv64(total, 256)), dim3(256), 0,
+                       (hipStream_t)stream, (const float*)workspace, (T*)weight_grad, splits, total);
+    return launch_status();
+  });
+}
+
+int at_channel_sum(const void* x, void* out, int64_t batch, int64_t feat, int64_t spatial, int x_dtype,
+                   int out_dtype, at_stream_t stream) {
+  if (!x || !out) return AT_ERR_NULL;
+  if (!dtype_valid(x_dtype) || !dtype_valid(out_dtype)) return AT_ERR_DTYPE;
+  if (batch <= 0 || feat <= 0 || spatial <= 0 || feat > INT32_MAX) return AT_ERR_DIM;
+  return dispatch_dtype(x_dtype, [&](auto* tp) -> int {
+    typedef std::remove_pointer_t<decltype(tp)> T;
+    hipLaunchKernelGGL((channel_sum_kernel<T>), dim3((unsigned)feat), dim3(256), 0, (hipStream_t)stream,
+                       (const T*)x, out, out_dtype, batch, (int)feat, spatial);
+    return launch_status();
+  });
+}
+
+}  // extern "C"

@@ -210,6 +210,83 @@ int64_t at_colsum_workspace_bytes(int64_t rows, int64_t cols);
 int at_colsum(const void* x, void* out, void* workspace, int64_t workspace_bytes, int64_t rows,
               int64_t cols, int64_t x_stride, int x_dtype, int out_dtype, at_stream_t stream);
 
+/* ------------------------------------------------------------------------------------------
+ * BatchNorm with fused affine, residual, pre-activation store and activation — replaces
+ * batch_norm_forward_kernel / batch_norm_backward_kernel, attorch/batch_norm_kernels.py:44-236
+ * and :246-381 (launched from attorch/batch_norm_layer.py:142-157 and :227-233) and the
+ * act_func_backward_kernel launch at batch_norm_layer.py:204-206.
+ * Tensors are contiguous [batch, feat, spatial] (NC, NCL or NCHW flattened; spatial = 1 for 2D
+ * inputs) — no transposed view is needed.  All tensors of one call share `dtype`; weight/bias
+ * share param_dtype; running statistics share running_dtype.
+ *   fwd: batch statistics when is_train or !track_running_stats (biased variance normalises,
+ *        running statistics are updated in place with the unbiased variance when is_train and
+ *        track_running_stats), running statistics otherwise;
+ *        output = act(weight*(input-mean)*inv_std + bias + pre_act_add); affine only when both
+ *        weight and bias are non-null; pre_act_add nullable (add_pre_act False); pre_act
+ *        non-null (and != output) stores the value before the activation (save_pre_act);
+ *        mean / inv_std nullable (save_stats False).
+ *   bwd: g = output_grad * act'(pre_act) is written to pre_act_grad (required when
+ *        act != AT_ACT_NONE; it is also the residual gradient, batch_norm_layer.py:244);
+ *        input_grad = inv_std*(weight*g - (sum(x_hat*g)*weight/n * x_hat + sum(g)*weight/n));
+ *        weight_grad = sum(x_hat*g), bias_grad = sum(g) (fp32 [feat], nullable).
+ * workspace: at_batch_norm_workspace_bytes(feat) bytes for either direction.
+ * ------------------------------------------------------------------------------------------ */
+int64_t at_batch_norm_workspace_bytes(int64_t feat);
+
+int at_batch_norm_fwd(const void* input, const void* weight, const void* bias, float* mean,
+                      float* inv_std, const void* pre_act_add, void* pre_act, void* output,
+                      void* running_mean, void* running_var, void* workspace,
+                      int64_t workspace_bytes, int64_t batch, int64_t feat, int64_t spatial,
+                      float momentum, float eps, int act, float param, int track_running_stats,
+                      int is_train, int dtype, int param_dtype, int running_dtype,
+                      at_stream_t stream);
+
+int at_batch_norm_bwd(const void* output_grad, const void* pre_act, const void* input,
+                      const float* mean, const float* inv_std, const void* weight,
+                      void* input_grad, void* pre_act_grad, float* weight_grad, float* bias_grad,
+                      void* workspace, int64_t workspace_bytes, int64_t batch, int64_t feat,
+                      int64_t spatial, int act, float param, int dtype, int param_dtype,
+                      at_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Conv2d (NCHW, zero padding, stride, groups, no dilation) — replaces conv2d_forward_kernel,
+ * attorch/conv_kernels.py:68-207 (launched from attorch/conv_layer.py:102-112), the bias add
+ * at conv_layer.py:114-116, and the torch calls of the backward pass at conv_layer.py:153-162
+ * (torch.nn.grad.conv2d_input, conv2d_weight and the bias sum).
+ * Tensors are contiguous: input [batch, in_feat, in_height, in_width], weight
+ * [out_feat, in_feat / groups, kernel_height, kernel_width], output
+ * [batch, out_feat, out_height, out_width] with out = (in + 2*padding - kernel) / stride + 1
+ * (conv_layer.py:18-36), which the call checks.  bias nullable.
+ *   bwd_weight needs at_conv2d_bwd_weight_workspace_bytes(...) bytes (split-K partials).
+ *   at_channel_sum: out[feat] = sum over batch and space of a [batch, feat, spatial] tensor.
+ * ------------------------------------------------------------------------------------------ */
+int at_conv2d_fwd(const void* input, const void* weight, const void* bias, void* output,
+                  int64_t batch, int64_t in_feat, int64_t in_height, int64_t in_width,
+                  int64_t out_feat, int64_t out_height, int64_t out_width, int64_t kernel_height,
+                  int64_t kernel_width, int64_t stride_height, int64_t stride_width,
+                  int64_t padding_height, int64_t padding_width, int64_t groups, int in_dtype,
+                  int bias_dtype, int out_dtype, at_stream_t stream);
+
+int at_conv2d_bwd_input(const void* output_grad, const void* weight, void* input_grad,
+                        int64_t batch, int64_t in_feat, int64_t in_height, int64_t in_width,
+                        int64_t out_feat, int64_t out_height, int64_t out_width,
+                        int64_t kernel_height, int64_t kernel_width, int64_t stride_height,
+                        int64_t stride_width, int64_t padding_height, int64_t padding_width,
+                        int64_t groups, int dtype, at_stream_t stream);
+
+int64_t at_conv2d_bwd_weight_workspace_bytes(int64_t out_feat, int64_t in_feat_per_group,
+                                             int64_t kernel_height, int64_t kernel_width);
+
+int at_conv2d_bwd_weight(const void* output_grad, const void* input, void* weight_grad,
+                         void* workspace, int64_t workspace_bytes, int64_t batch, int64_t in_feat,
+                         int64_t in_height, int64_t in_width, int64_t out_feat, int64_t out_height,
+                         int64_t out_width, int64_t kernel_height, int64_t kernel_width,
+                         int64_t stride_height, int64_t stride_width, int64_t padding_height,
+                         int64_t padding_width, int64_t groups, int dtype, at_stream_t stream);
+
+int at_channel_sum(const void* x, void* out, int64_t batch, int64_t feat, int64_t spatial,
+                   int x_dtype, int out_dtype, at_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
