@@ -1,0 +1,64 @@
+"""
+Shared helpers of the parity tests: seeded inputs, tolerances and comparison.
+
+Tolerances are the ones the build targets: rtol 1e-4 / atol 1e-5 for float32 and
+rtol 2e-2 / atol 2e-2 for float16 / bfloat16 outputs and gradients.  Reduction outputs whose
+magnitude grows with the number of summed rows (parameter gradients) are compared after
+dividing both sides by max(1, max|expected|).
+"""
+
+from typing import Optional, Sequence, Tuple
+
+import torch
+from torch import Tensor
+
+TOLERANCES = {torch.float32: (1e-4, 1e-5), torch.float16: (2e-2, 2e-2), torch.bfloat16: (2e-2, 2e-2)}
+DTYPES = (torch.float32, torch.float16, torch.bfloat16)
+ACT_FUNCS = (None, 'sigmoid', 'logsigmoid', 'tanh', 'relu', 'gelu', 'geluapprox', 'silu', 'relu6',
+             'hardsigmoid', 'hardtanh', 'hardswish', 'selu', 'mish', 'softplus', 'softsign',
+             'tanhshrink', 'leaky_relu_0.01', 'elu_1', 'celu_1', 'hardshrink_0.5', 'softshrink_0.5')
+
+
+def compute_dtype(dtype: torch.dtype) -> torch.dtype:
+    """
+    Precision the oracle computes in for a storage dtype (float64 pins float32 kernels).
+    """
+    return torch.float64 if dtype is torch.float32 else torch.float32
+
+
+def randn(shape: Sequence[int], seed: int, dtype: torch.dtype = torch.float32,
+          scale: float = 1.0, shift: float = 0.0) -> Tensor:
+    """
+    Seeded CPU normal tensor, generated in float32 and rounded to dtype.
+    """
+    gen = torch.Generator().manual_seed(seed)
+    return (shift + scale * torch.randn(tuple(shape), generator=gen)).to(dtype)
+
+
+def assert_close(actual: Optional[Tensor], expected: Optional[Tensor], dtype: torch.dtype,
+                 what: str, normalize: bool = False, atol_scale: float = 1.0,
+                 reference_tolerance: bool = False) -> None:
+    """
+    Compares a device result with the CPU oracle at the tolerance of `dtype`.
+    reference_tolerance=True widens the float32 tolerance to the rtol = atol = 1e-3 of the
+    reference's own tests, for ill-conditioned cases only (see the callers).
+    """
+    if expected is None:
+        assert actual is None, f'{what}: expected None'
+        return
+    assert actual is not None, f'{what}: got None'
+    rtol, atol = TOLERANCES[dtype]
+    if reference_tolerance and dtype is torch.float32:
+        rtol, atol = 1e-3, 1e-3
+    a = actual.detach().double().cpu()
+    e = expected.detach().double().cpu()
+    assert a.shape == e.shape, f'{what}: shape {tuple(a.shape)} != {tuple(e.shape)}'
+    if normalize:
+        scale = max(1.0, e.abs().max().item()) if e.numel() else 1.0
+        a, e = a / scale, e / scale
+    torch.testing.assert_close(a, e, rtol=rtol, atol=atol * atol_scale, equal_nan=True,
+                               msg=lambda m: f'{what}: {m}')
+
+
+def grads(*tensors: Optional[Tensor]) -> Tuple[Optional[Tensor], ...]:
+    return tuple(None if t is None else t.grad for t in tensors)

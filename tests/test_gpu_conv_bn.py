@@ -1,0 +1,139 @@
+"""
+GPU parity tests of Conv2d / Conv1d (forward and the three gradients) and BatchNorm1d/2d
+(training statistics, running statistics, residual, fused activation, eval mode) against the
+CPU oracle; grids follow the reference's tests/test_conv_layer.py and
+tests/test_batch_norm_layer.py.
+"""
+
+import pytest
+import torch
+
+import attorch_amd
+import oracle
+from .helpers import DTYPES, assert_close, compute_dtype, randn
+
+pytestmark = pytest.mark.gpu
+
+CONV_CASES = [
+    # input shape, out channels, kernel, stride, padding, groups
+    ((2, 8, 11, 9), 12, (3, 3), (1, 1), (1, 1), 1),
+    ((2, 8, 11, 9), 12, (5, 3), (2, 1), (3, 0), 2),
+    ((2, 8, 11, 9), 8, (2, 4), (1, 2), (1, 3), 8),
+    ((2, 6, 12, 12), 6, (1, 1), (1, 1), (0, 0), 1),
+    ((1, 3, 64, 64), 16, (7, 7), (2, 2), (3, 3), 1),
+    ((2, 16, 9, 9), 32, (4, 4), (2, 2), (2, 2), 4),
+    ((4, 64, 28, 28), 64, (3, 3), (1, 1), (1, 1), 1),
+    ((2, 32, 14, 14), 48, (3, 5), (2, 1), (1, 2), 1),
+]
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape, out_dim, kernel, stride, padding, groups', CONV_CASES)
+@pytest.mark.parametrize('bias', [False, True])
+def test_conv2d(shape, out_dim, kernel, stride, padding, groups, bias, dtype) -> None:
+    fan_in = shape[1] // groups * kernel[0] * kernel[1]
+    x = randn(shape, 1, dtype)
+    w = randn((out_dim, shape[1] // groups, *kernel), 2, dtype, fan_in ** -0.5)
+    b = randn((out_dim,), 3, dtype) if bias else None
+    cd = compute_dtype(dtype)
+    y_ref = oracle.conv2d_forward(x, w, b, stride, padding, groups, dtype, compute=cd)
+    dy = randn(y_ref.shape, 4, dtype)
+    dx_ref, dw_ref, db_ref = oracle.conv2d_backward(dy, x, w, stride, padding, groups, dtype, compute=cd)
+
+    xd, wd = x.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
+    bd = b.cuda().requires_grad_(True) if bias else None
+    y = attorch_amd.Conv2dAutoGrad.apply(xd, wd, bd, *stride, *padding, groups)
+    y.backward(dy.cuda())
+    assert y.dtype is dtype
+    assert_close(y, y_ref, dtype, 'output', normalize=True)
+    assert_close(xd.grad, dx_ref, dtype, 'input_grad', normalize=True)
+    assert_close(wd.grad, dw_ref, dtype, 'weight_grad', normalize=True)
+    if bias:
+        assert_close(bd.grad, db_ref, dtype, 'bias_grad', normalize=True)
+
+
+def test_conv_modules_match_torch() -> None:
+    torch.manual_seed(0)
+    ours = attorch_amd.Conv2d(8, 16, 3, stride=2, padding=1, groups=2)
+    torch.manual_seed(0)
+    theirs = torch.nn.Conv2d(8, 16, 3, stride=2, padding=1, groups=2, device='cuda')
+    x = randn((3, 8, 17, 13), 1).cuda()
+    torch.testing.assert_close(ours(x), theirs(x), rtol=1e-4, atol=1e-5)
+    torch.manual_seed(0)
+    ours1d = attorch_amd.Conv1d(6, 4, 5, stride=2, padding=2)
+    torch.manual_seed(0)
+    theirs1d = torch.nn.Conv1d(6, 4, 5, stride=2, padding=2, device='cuda')
+    x1 = randn((3, 6, 50), 2).cuda()
+    torch.testing.assert_close(ours1d(x1), theirs1d(x1), rtol=1e-4, atol=1e-5)
+    with torch.autocast('cuda', dtype=torch.float16):
+        assert ours(x).dtype is torch.float16
+
+
+BN_SHAPES = [(6, 5), (128, 1024), (2048, 768), (8, 960, 196), (2048, 64, 16), (2, 3, 224, 224),
+             (16, 64, 56, 56), (32, 128, 7, 7), (3, 7, 3, 5)]
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', BN_SHAPES)
+@pytest.mark.parametrize('affine', [False, True])
+@pytest.mark.parametrize('residual', [False, True])
+@pytest.mark.parametrize('act_func', [None, 'relu', 'silu', 'leaky_relu_0.01'])
+def test_batch_norm_training(shape, dtype, affine, residual, act_func) -> None:
+    feat = shape[1]
+    x = randn(shape, 1, dtype)
+    w = randn((feat,), 2, dtype) if affine else None
+    b = randn((feat,), 3, dtype) if affine else None
+    res = randn(shape, 4, dtype) if residual else None
+    dy = randn(shape, 5, dtype)
+    running_mean = randn((feat,), 6)
+    running_var = randn((feat,), 7).abs() + 0.5
+    cd = compute_dtype(dtype)
+    name, param = oracle.parse_act_func(act_func)
+    y_ref, pre_act_ref, mean, inv_std, rm_ref, rv_ref = oracle.batch_norm_forward(
+        x, True, w, b, running_mean, running_var, 0.2, 1e-5, True, res, name, param, compute=cd)
+
+    xd = x.cuda().requires_grad_(True)
+    wd = w.cuda().requires_grad_(True) if affine else None
+    bd = b.cuda().requires_grad_(True) if affine else None
+    rd = res.cuda().requires_grad_(True) if residual else None
+    rm, rv = running_mean.cuda(), running_var.cuda()
+    y = attorch_amd.BatchNormAutoGrad.apply(xd, True, wd, bd, rm, rv, 0.2, 1e-5, True, rd, act_func)
+    saved = [None if t is None else t.detach().cpu() for t in y.grad_fn.saved_tensors]
+    y.backward(dy.cuda())
+    assert y.dtype is dtype and y.shape == x.shape
+    assert_close(y, y_ref, dtype, 'output')
+    assert_close(rm, rm_ref, torch.float32, 'running_mean')
+    assert_close(rv, rv_ref, torch.float32, 'running_var')     # unbiased variance in the running stat
+
+    pre_act = saved[4] if name is not None else None            # device's own pre-activation, see Linear test
+    if name is not None:
+        assert_close(pre_act, pre_act_ref, dtype, 'pre_act')
+    dx_ref, dw_ref, db_ref, dres_ref = oracle.batch_norm_backward(
+        dy, x, saved[1], saved[2], w, affine, pre_act, name, param, compute=cd)
+    assert_close(xd.grad, dx_ref, dtype, 'input_grad', normalize=True)
+    if affine:
+        assert_close(wd.grad, dw_ref.to(dtype), dtype, 'weight_grad', normalize=True)
+        assert_close(bd.grad, db_ref.to(dtype), dtype, 'bias_grad', normalize=True)
+    if residual:
+        assert_close(rd.grad, dres_ref, dtype, 'residual_grad')
+
+
+@pytest.mark.parametrize('track_running_stats', [False, True])
+def test_batch_norm_modules_train_then_eval(track_running_stats) -> None:
+    torch.manual_seed(0)
+    ours = attorch_amd.BatchNorm2d(12, momentum=0.2, act_func='relu', track_running_stats=track_running_stats)
+    theirs = torch.nn.BatchNorm2d(12, momentum=0.2, track_running_stats=track_running_stats, device='cuda')
+    with torch.no_grad():
+        ours.weight.normal_(), ours.bias.normal_()
+        theirs.weight.copy_(ours.weight), theirs.bias.copy_(ours.bias)
+    x, res = randn((8, 12, 9, 7), 1).cuda(), randn((8, 12, 9, 7), 2).cuda()
+    for _ in range(2):
+        torch.testing.assert_close(ours(x, res), torch.relu(theirs(x) + res), rtol=1e-4, atol=1e-5)
+    if track_running_stats:
+        torch.testing.assert_close(ours.running_mean, theirs.running_mean, rtol=1e-4, atol=1e-5)
+        torch.testing.assert_close(ours.running_var, theirs.running_var, rtol=1e-4, atol=1e-5)
+    ours.eval(), theirs.eval()
+    torch.testing.assert_close(ours(x, res), torch.relu(theirs(x) + res), rtol=1e-4, atol=1e-5)
+    ours1d = attorch_amd.BatchNorm1d(12)
+    torch.testing.assert_close(ours1d(x.flatten(2)), torch.nn.BatchNorm1d(12, device='cuda')(x.flatten(2)),
+                               rtol=1e-4, atol=1e-5)

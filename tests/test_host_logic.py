@@ -1,0 +1,149 @@
+"""
+CPU-only tests of the host side: the C-ABI library loads and exports every symbol the header
+declares, argument errors come back as negative codes without touching a GPU, the Python
+wrappers raise the reference's exception types, and nothing falls back to a CPU path.
+"""
+
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+import attorch_amd
+from attorch_amd import _lib
+from attorch_amd.act import ACT_IDS, act_id, parse_act_func
+from attorch_amd.utils import get_output_dtype
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = (ROOT / 'include' / 'attorch_hip.h').read_text()
+
+
+def declared_symbols():
+    return sorted(set(re.findall(r'^\s*(?:int|int64_t|const char\*)\s+(at_\w+)\s*\(', HEADER, flags=re.M)))
+
+
+def test_library_exports_every_declared_symbol() -> None:
+    lib = ctypes.CDLL(str(_lib.LIB_PATH))
+    names = declared_symbols()
+    assert len(names) >= 25
+    for name in names:
+        assert hasattr(lib, name), f'{name} declared in include/attorch_hip.h but not exported'
+    assert set(names) == set(_lib.PROTOTYPES), 'ctypes prototypes out of sync with the header'
+
+
+def test_header_activation_ids_match_python_table() -> None:
+    ids = dict(re.findall(r'#define AT_ACT_(\w+) (\d+)', HEADER))
+    for name, value in ACT_IDS.items():
+        key = 'NONE' if name is None else name.upper()
+        assert int(ids[key]) == value
+    assert int(ids['COUNT']) == len(ACT_IDS)
+
+
+def test_version_and_error_strings() -> None:
+    lib = _lib.load()
+    assert lib.at_version() >= 100
+    assert b'null' in lib.at_error_string(-1)
+    assert b'success' in lib.at_error_string(0)
+    with pytest.raises(RuntimeError, match='workspace'):
+        _lib.check(-5, 'demo')
+
+
+def test_argument_errors_without_gpu() -> None:
+    lib = _lib.load()
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.addressof(buf)
+    # null pointers
+    assert lib.at_rms_norm_fwd(None, None, None, p, 4, 8, 8, 8, 1e-5, 0, 0, 0, None) == -1
+    assert lib.at_softmax_fwd(p, None, 4, 8, 8, 8, 0, 0, 0, 0, None) == -1
+    assert lib.at_linear_fwd(None, p, None, None, p, 4, 8, 8, 8, 8, 8, 8, 0, 0.0, 0, 0, 0, None) == -1
+    # bad dtype / dims / strides / activation
+    assert lib.at_layer_norm_fwd(p, None, None, None, None, p, 4, 8, 8, 8, 1e-5, 7, 0, 0, None) == -3
+    assert lib.at_layer_norm_fwd(p, None, None, None, None, p, 4, 0, 8, 8, 1e-5, 0, 0, 0, None) == -2
+    assert lib.at_softmax_fwd(p, p, 4, 8, 4, 8, 0, 0, 0, 0, None) == -2
+    assert lib.at_linear_fwd(p, p, None, None, p, 4, 8, 8, 8, 8, 8, 8, 99, 0.0, 0, 0, 0, None) == -4
+    assert lib.at_act_bwd(p, p, p, 4, 8, 8, 8, 8, 0, 0.0, 0, 0, None) == -4
+    # missing / short workspace
+    assert lib.at_cross_entropy_fwd_bwd(p, p, None, p, None, None, 0, 4, 8, 8, 8, -100, 0, 0, 0, None) == -5
+    assert lib.at_layer_norm_bwd(p, p, p, p, p, p, p, None, p, 16, 4, 8, 8, 8, 8, 0, 0, 0, 0, None) == -5
+    assert lib.at_batch_norm_fwd(p, None, None, None, None, None, None, p, None, None, None, 0,
+                                 4, 8, 1, 0.1, 1e-5, 0, 0.0, 0, 1, 0, 0, 0, None) == -5
+    # inconsistent convolution geometry
+    dims = [1, 4, 8, 8, 4, 9, 9, 3, 3, 1, 1, 1, 1, 1]
+    assert lib.at_conv2d_fwd(p, p, None, p, *dims, 0, 0, 0, None) == -2
+    assert lib.at_norm_bwd_workspace_bytes(16, 8, 2) == 16 * 8 * 4 * 2
+    assert lib.at_cross_entropy_workspace_bytes(10) == 56
+
+
+def test_get_output_dtype_policy(monkeypatch) -> None:
+    for dtype in (torch.float32, torch.float16, torch.bfloat16):
+        for mode in (None, 'fp16', 'fp32'):
+            assert get_output_dtype(dtype, mode) is dtype       # autocast disabled: flows through
+    # torch refuses to enable 'cuda' autocast on a host without a GPU, so the state is faked here;
+    # the GPU suite exercises the real context manager.
+    monkeypatch.setattr(torch, 'is_autocast_enabled', lambda *a: True)
+    monkeypatch.setattr(torch, 'get_autocast_dtype', lambda *a: torch.float16)
+    assert get_output_dtype(torch.float32, None) is torch.float32
+    assert get_output_dtype(torch.float32, 'fp16') is torch.float16
+    assert get_output_dtype(torch.float16, 'fp32') is torch.float32
+    with pytest.raises(RuntimeError):
+        get_output_dtype(torch.float32, 'bf16')
+    monkeypatch.setattr(torch, 'get_autocast_dtype', lambda *a: torch.bfloat16)
+    assert get_output_dtype(torch.float32, 'fp16') is torch.bfloat16
+
+
+def test_activation_strings() -> None:
+    assert parse_act_func('leaky_relu_0.01') == ('leaky_relu', 0.01)
+    assert act_id(*parse_act_func('geluapprox')) == 6
+    assert act_id(None, None) == 0
+    with pytest.raises(RuntimeError):
+        act_id('swish', None)
+    with pytest.raises(RuntimeError):
+        act_id('elu', None)
+
+
+def test_module_errors_match_reference() -> None:
+    with pytest.raises(RuntimeError, match='integer'):
+        attorch_amd.LayerNorm((8,), device='cpu')
+    with pytest.raises(RuntimeError, match='integer'):
+        attorch_amd.RMSNorm((8,), device='cpu')
+    with pytest.raises(RuntimeError, match='averaging'):
+        attorch_amd.CrossEntropyLoss(reduction='sum')
+    with pytest.raises(RuntimeError, match='label smoothing'):
+        attorch_amd.CrossEntropyLoss(label_smoothing=0.1)
+    with pytest.raises(RuntimeError, match='dilation'):
+        attorch_amd.Conv2d(4, 4, 3, dilation=2, device='cpu')
+    with pytest.raises(RuntimeError, match='padding mode'):
+        attorch_amd.Conv2d(4, 4, 3, padding_mode='reflect', device='cpu')
+    with pytest.raises(RuntimeError, match='last dimension'):
+        attorch_amd.Softmax(dim=0)(torch.zeros(2, 3))
+    with pytest.raises(AssertionError):
+        attorch_amd.LinearAutoGrad.apply(torch.zeros(2, 3), torch.zeros(4, 5), None, None)
+    with pytest.raises(AssertionError):
+        attorch_amd.CrossEntropyLossAutoGrad.apply(torch.zeros(2, 3, 4), torch.zeros(2, dtype=torch.long))
+
+
+def test_linear_weight_layout_and_state_dict() -> None:
+    layer = attorch_amd.Linear(6, 4, act_func='relu', device='cpu')
+    assert tuple(layer.weight.shape) == (6, 4)          # [in, out], unlike torch
+    assert tuple(layer.state_dict()['weight'].shape) == (6, 4)
+
+
+def test_no_cpu_fallback() -> None:
+    x = torch.zeros(2, 8)
+    for call in (lambda: attorch_amd.LayerNorm(8, device='cpu')(x),
+                 lambda: attorch_amd.RMSNorm(8, device='cpu')(x),
+                 lambda: attorch_amd.Softmax(dim=-1)(x),
+                 lambda: attorch_amd.Linear(8, 4, device='cpu')(x),
+                 lambda: attorch_amd.CrossEntropyLoss()(x, torch.zeros(2, dtype=torch.long)),
+                 lambda: attorch_amd.BatchNorm1d(8, device='cpu')(x),
+                 lambda: attorch_amd.Conv2d(2, 2, 1, device='cpu')(torch.zeros(1, 2, 2, 2))):
+        with pytest.raises(RuntimeError, match='no CPU path'):
+            call()
+
+
+def test_product_never_imports_the_oracle() -> None:
+    for path in (ROOT / 'attorch_amd').rglob('*.py'):
+        text = path.read_text()
+        assert 'import oracle' not in text and 'from oracle' not in text, path
