@@ -1,0 +1,559 @@
+"""
+Benchmark of the attorch layer-kernel hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs c4,c2,...] [--no-cpu]
+
+A "step" is one forward + backward pass of the headline workload over one batch of synthetic
+input that is already resident in HBM: attorch_amd.Linear with fused GELU(tanh), bf16,
+X[16384, 4096] x W[4096, 16384] (BASELINE config 4, the configuration the 70 %-of-MFMA-peak
+target is quoted on).  One JSON line is printed; besides the contract fields it carries
+  roofline      the dominant kernel (the forward MFMA GEMM with its fused epilogue) against
+                the MI355X dense bf16 MFMA peak, timed with HIP events on the launch stream
+  cpu_baseline  the CPU oracle of the same workload on a bounded sample of rows, timed on
+                this host's cores (a reported baseline, not a target)
+  configs       the other BASELINE configs (c1 Linear fp32, c2 LayerNorm / RMSNorm / Softmax
+                / LogSoftmax, c3 CrossEntropy, c5 Conv2d + BatchNorm2d), each as absolute
+                throughput, fraction of its roofline and CPU baseline.
+Buffers of the bandwidth-bound configs are rotated over several sets so the 256 MB Infinity
+Cache cannot serve them.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+from typing import Callable, Dict, List, Tuple
+
+import torch
+
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E, GB/s
+PEAK_MFMA_16BIT_TFLOPS = 2500.0  # dense bf16 / fp16 MFMA
+PEAK_MFMA_FP32_TFLOPS = 157.3    # dense fp32 MFMA
+
+
+def parse_args() -> argparse.Namespace:
+    parser = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawTextHelpFormatter)
+    parser.add_argument('--gpus', type=int, default=1)
+    parser.add_argument('--steps', type=int, default=20)
+    parser.add_argument('--warmup', type=int, default=5)
+    parser.add_argument('--configs', type=str, default='c1,c2,c3,c5',
+                        help='secondary configs to measure besides the headline (c4); "none" skips them')
+    parser.add_argument('--no-cpu', action='store_true', help='skip the CPU baselines')
+    return parser.parse_args()
+
+
+def gpu_time_ms(fn: Callable[[], None], iters: int, warmup: int = 2) -> float:
+    """
+    Average duration of fn's GPU work in ms, from HIP events recorded on the stream the
+    kernels are launched on (PyTorch's current stream).
+    """
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def wall_time_ms(fn: Callable[[], None], steps: int, warmup: int) -> float:
+    """
+    Wall-clock ms per step: warm-up, then exactly `steps` calls bracketed by device syncs.
+    """
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def cpu_time_s(fn: Callable[[], None], reps: int = 3) -> float:
+    fn()
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return sorted(times)[len(times) // 2]
+
+
+def gen(shape, seed, dtype, scale=1.0, shift=0.0):
+    g = torch.Generator().manual_seed(seed)
+    return (shift + scale * torch.randn(shape, generator=g)).to(dtype)
+
+
+class Raw:
+    """
+    Direct calls into the C ABI with preallocated tensors (kernel-level timing).
+    """
+    def __init__(self):
+        from attorch_amd import _lib
+        self.lib = _lib.load()
+        self._lib = _lib
+
+    def stream(self):
+        return torch.cuda.current_stream().cuda_stream
+
+    def check(self, rc, what):
+        self._lib.check(rc, what)
+
+
+# ------------------------------------------------------------------------------------------
+# c4 / c1: Linear
+# ------------------------------------------------------------------------------------------
+def linear_workload(cfg: str):
+    if cfg == 'c4':
+        m, k, n, dtype, act = 16384, 4096, 16384, torch.bfloat16, 'geluapprox'
+        x = gen((m, k), 4001, dtype)
+        w = gen((k, n), 4002, dtype, 0.02)
+        b = torch.zeros(n, dtype=dtype)
+    else:
+        m, k, n, dtype, act = 512, 784, 256, torch.float32, 'relu'
+        x = gen((m, k), 1001, dtype)
+        torch.manual_seed(1002)
+        lin = torch.nn.Linear(k, n)
+        w = lin.weight.detach().T.contiguous()
+        b = lin.bias.detach().clone()
+    dy = gen((m, n), 1000 * int(cfg[1]) + 3, dtype)
+    return m, k, n, dtype, act, x, w, b, dy
+
+
+def bench_linear(cfg: str, steps: int, warmup: int, with_cpu: bool) -> Dict:
+    import attorch_amd
+    from attorch_amd.act import act_id, parse_act_func
+    raw = Raw()
+    lib = raw.lib
+    m, k, n, dtype, act, x, w, b, dy = linear_workload(cfg)
+    dt = raw._lib.dtype_id(dtype)
+    xd, dyd = x.cuda(), dy.cuda()
+    layer = attorch_amd.Linear(k, n, bias=True, act_func=act, dtype=dtype)
+    with torch.no_grad():
+        layer.weight.copy_(w.cuda())
+        layer.bias.copy_(b.cuda())
+    xin = xd.clone().requires_grad_(True)
+
+    def step():
+        xin.grad = None
+        layer.weight.grad = None
+        layer.bias.grad = None
+        layer(xin).backward(dyd)
+
+    ms_step = wall_time_ms(step, steps, warmup)
+    flop = 6.0 * m * k * n
+    peak = PEAK_MFMA_16BIT_TFLOPS if dtype is not torch.float32 else PEAK_MFMA_FP32_TFLOPS
+
+    # kernel-level timing through the C ABI
+    wd, bd = layer.weight.detach(), layer.bias.detach()
+    y = torch.empty((m, n), dtype=dtype, device='cuda')
+    pre = torch.empty_like(y)
+    dz = torch.empty_like(y)
+    dx = torch.empty((m, k), dtype=dtype, device='cuda')
+    dw = torch.empty((k, n), dtype=dtype, device='cuda')
+    db = torch.empty(n, dtype=dtype, device='cuda')
+    wsb = lib.at_colsum_workspace_bytes(m, n)
+    ws = torch.empty(wsb, dtype=torch.uint8, device='cuda')
+    name, param = parse_act_func(act)
+    aid = act_id(name, param)
+    st = raw.stream
+
+    def k_fwd():
+        raw.check(lib.at_linear_fwd(xd.data_ptr(), wd.data_ptr(), bd.data_ptr(), pre.data_ptr(), y.data_ptr(),
+                                    m, k, n, k, n, n, n, aid, 0.0, dt, dt, dt, st()), 'fwd')
+
+    def k_act():
+        raw.check(lib.at_act_bwd(dyd.data_ptr(), pre.data_ptr(), dz.data_ptr(), m, n, n, n, n, aid, 0.0, dt, dt,
+                                 st()), 'act_bwd')
+
+    def k_dx():
+        raw.check(lib.at_linear_bwd_input(dz.data_ptr(), wd.data_ptr(), dx.data_ptr(), m, k, n, n, n, k, dt, dt,
+                                          st()), 'dx')
+
+    def k_dw():
+        raw.check(lib.at_linear_bwd_weight(xd.data_ptr(), dz.data_ptr(), dw.data_ptr(), m, k, n, k, n, n, dt, dt,
+                                           st()), 'dw')
+
+    def k_db():
+        raw.check(lib.at_colsum(dz.data_ptr(), db.data_ptr(), ws.data_ptr(), wsb, m, n, n, dt, dt, st()), 'colsum')
+
+    iters = max(3, min(steps, 10))
+    kernels = {}
+    for kname, fn in (('linear_fwd', k_fwd), ('act_bwd', k_act), ('linear_bwd_input', k_dx),
+                      ('linear_bwd_weight', k_dw), ('colsum', k_db)):
+        kernels[kname] = gpu_time_ms(fn, iters)
+    gemm_flop = 2.0 * m * k * n
+    fwd_tflops = gemm_flop / kernels['linear_fwd'] / 1e9
+    out = {
+        'workload': f'{cfg}: Linear {str(dtype)[6:]} fwd+bwd X[{m},{k}] W[{k},{n}] act={act}',
+        'metric': 'Linear fwd+bwd TFLOP/s', 'value': flop / ms_step / 1e9, 'unit': 'TFLOP/s',
+        'ms_per_step': ms_step,
+        'kernel_ms': kernels,
+        'kernel_tflops': {kk: gemm_flop / kernels[kk] / 1e9
+                          for kk in ('linear_fwd', 'linear_bwd_input', 'linear_bwd_weight')},
+        'roofline': {'bound': 'mfma', 'kernel': 'linear_fwd (GEMM + bias + activation epilogue)',
+                     'achieved': fwd_tflops, 'peak': peak, 'unit': 'TFLOP/s', 'frac': fwd_tflops / peak,
+                     'traffic': None},
+        'frac_of_peak_step': flop / ms_step / 1e9 / peak,
+    }
+    if with_cpu:
+        import oracle
+        rows = min(m, 2048)
+        xs, dys = x[:rows], dy[:rows]
+        name, param = parse_act_func(act)
+        torch.set_num_threads(os.cpu_count())
+
+        def cpu_step():
+            yy, pre_act = oracle.linear_forward(xs, w, b, name, param, dtype)
+            oracle.linear_backward(dys, xs, w, pre_act, name, param, dtype)
+
+        sec = cpu_time_s(cpu_step)
+        out['cpu_baseline'] = {'value': 6.0 * rows * k * n / sec / 1e12, 'unit': 'TFLOP/s',
+                               'cores': torch.get_num_threads(), 'kind': 'port',
+                               'sample': f'first {rows} of {m} rows, full K and N, oracle fwd+bwd in fp32 compute'}
+    return out
+
+
+# ------------------------------------------------------------------------------------------
+# c2: LayerNorm / RMSNorm / Softmax / LogSoftmax, bf16 [8192, 4096]
+# ------------------------------------------------------------------------------------------
+def bench_rows(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
+    raw = Raw()
+    lib = raw.lib
+    rows_, feat, dtype = 8192, 4096, torch.bfloat16
+    dt = raw._lib.dtype_id(dtype)
+    nsets = 6
+    xs = [gen((rows_, feat), 2001 + i, dtype).cuda() for i in range(nsets)]
+    dys = [gen((rows_, feat), 2101 + i, dtype).cuda() for i in range(nsets)]
+    ys = [torch.empty_like(xs[0]) for _ in range(nsets)]
+    dxs = [torch.empty_like(xs[0]) for _ in range(nsets)]
+    w = gen((feat,), 2201, dtype, 0.1, 1.0).cuda()
+    b = gen((feat,), 2202, dtype, 0.1).cuda()
+    mean = torch.empty(rows_, device='cuda')
+    rstd = torch.empty(rows_, device='cuda')
+    dwg = torch.empty(feat, device='cuda')
+    dbg = torch.empty(feat, device='cuda')
+    wsb = lib.at_norm_bwd_workspace_bytes(rows_, feat, 2)
+    ws = torch.empty(wsb, dtype=torch.uint8, device='cuda')
+    tbytes = rows_ * feat * 2
+    st = raw.stream
+    counter = [0]
+
+    def nxt():
+        counter[0] = (counter[0] + 1) % nsets
+        return counter[0]
+
+    def ln_f():
+        i = nxt()
+        raw.check(lib.at_layer_norm_fwd(xs[i].data_ptr(), w.data_ptr(), b.data_ptr(), mean.data_ptr(),
+                                        rstd.data_ptr(), ys[i].data_ptr(), rows_, feat, feat, feat, 1e-5, dt, dt,
+                                        dt, st()), 'ln_fwd')
+
+    def ln_b():
+        i = nxt()
+        raw.check(lib.at_layer_norm_bwd(dys[i].data_ptr(), xs[i].data_ptr(), mean.data_ptr(), rstd.data_ptr(),
+                                        w.data_ptr(), dxs[i].data_ptr(), dwg.data_ptr(), dbg.data_ptr(),
+                                        ws.data_ptr(), wsb, rows_, feat, feat, feat, feat, dt, dt, dt, dt, st()),
+                  'ln_bwd')
+
+    def rms_f():
+        i = nxt()
+        raw.check(lib.at_rms_norm_fwd(xs[i].data_ptr(), w.data_ptr(), rstd.data_ptr(), ys[i].data_ptr(), rows_,
+                                      feat, feat, feat, 1e-5, dt, dt, dt, st()), 'rms_fwd')
+
+    def rms_b():
+        i = nxt()
+        raw.check(lib.at_rms_norm_bwd(dys[i].data_ptr(), xs[i].data_ptr(), rstd.data_ptr(), w.data_ptr(),
+                                      dxs[i].data_ptr(), dwg.data_ptr(), ws.data_ptr(), wsb, rows_, feat, feat,
+                                      feat, feat, dt, dt, dt, dt, st()), 'rms_bwd')
+
+    def sm(log):
+        def f():
+            i = nxt()
+            raw.check(lib.at_softmax_fwd(xs[i].data_ptr(), ys[i].data_ptr(), rows_, feat, feat, feat, 0, log, dt,
+                                         dt, st()), 'softmax_fwd')
+
+        def bwd():
+            i = nxt()
+            raw.check(lib.at_softmax_bwd(dys[i].data_ptr(), ys[i].data_ptr(), dxs[i].data_ptr(), rows_, feat,
+                                         feat, feat, feat, 0, log, dt, dt, dt, st()), 'softmax_bwd')
+        return f, bwd
+
+    import oracle
+    results = []
+    iters = max(10, steps)
+    sm_f, sm_b = sm(0)
+    lsm_f, lsm_b = sm(1)
+    xc, dyc, wc, bc = xs[0].cpu(), dys[0].cpu(), w.cpu(), b.cpu()
+    crow = 2048  # CPU sample rows
+
+    def cpu_ln():
+        y, m_, r_ = oracle.layer_norm_forward(xc[:crow], wc, bc, 1e-5, dtype)
+        oracle.layer_norm_backward(dyc[:crow], xc[:crow], m_, r_, wc, dtype)
+
+    def cpu_rms():
+        y, r_ = oracle.rms_norm_forward(xc[:crow], wc, 1e-5)
+        oracle.rms_norm_backward(dyc[:crow], xc[:crow], r_, wc)
+
+    def cpu_sm(log):
+        def f():
+            y = oracle.softmax_forward(xc[:crow], False, log, dtype)
+            oracle.softmax_backward(dyc[:crow], y, False, log)
+        return f
+
+    for name, f, bwd, cpu in (('LayerNorm', ln_f, ln_b, cpu_ln), ('RMSNorm', rms_f, rms_b, cpu_rms),
+                              ('Softmax', sm_f, sm_b, cpu_sm(False)), ('LogSoftmax', lsm_f, lsm_b, cpu_sm(True))):
+        ms_f = gpu_time_ms(f, iters, warmup)
+        ms_b = gpu_time_ms(bwd, iters, warmup)
+        gbs = 5 * tbytes / (ms_f + ms_b) / 1e6
+        entry = {
+            'workload': f'c2: {name} bf16 fwd+bwd X[{rows_},{feat}]', 'metric': 'HBM GB/s', 'value': gbs,
+            'unit': 'GB/s', 'ms_fwd': ms_f, 'ms_bwd': ms_b,
+            'fwd_gbs': 2 * tbytes / ms_f / 1e6, 'bwd_gbs': 3 * tbytes / ms_b / 1e6,
+            'roofline': {'bound': 'hbm', 'achieved': gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                         'frac': gbs / PEAK_HBM_GBS, 'traffic': None},
+            'buffer_rotation': f'{nsets} sets of X/dY/Y/dX (64 MiB each)',
+        }
+        if with_cpu:
+            sec = cpu_time_s(cpu)
+            entry['cpu_baseline'] = {'value': 5 * crow * feat * 2 / sec / 1e9, 'unit': 'GB/s',
+                                     'cores': torch.get_num_threads(), 'kind': 'port',
+                                     'sample': f'first {crow} of {rows_} rows, oracle fwd+bwd'}
+        results.append(entry)
+    return results
+
+
+# ------------------------------------------------------------------------------------------
+# c3: CrossEntropy fp16 [8192, 50257]
+# ------------------------------------------------------------------------------------------
+def bench_cross_entropy(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
+    raw = Raw()
+    lib = raw.lib
+    rows_, feat, dtype = 8192, 50257, torch.float16
+    dt = raw._lib.dtype_id(dtype)
+    logits = gen((rows_, feat), 3001, dtype, 2.0).cuda()
+    g = torch.Generator().manual_seed(3002)
+    target = torch.randint(0, feat, (rows_,), generator=g)
+    target[torch.rand(rows_, generator=g) < 0.05] = -100
+    weight = (0.5 + torch.rand(feat, generator=g)).cuda()
+    tgt = target.cuda()
+    dlogits = torch.empty_like(logits)
+    loss = torch.empty((), dtype=dtype, device='cuda')
+    wsb = lib.at_cross_entropy_workspace_bytes(rows_)
+    ws = torch.empty(wsb, dtype=torch.uint8, device='cuda')
+    one = torch.ones((), dtype=dtype, device='cuda')
+    tbytes = rows_ * feat * 2
+    st = raw.stream
+    results = []
+    import oracle
+    for label, wt in (('unweighted', None), ('class-weighted', weight)):
+        def f():
+            raw.check(lib.at_cross_entropy_fwd_bwd(logits.data_ptr(), tgt.data_ptr(),
+                                                   None if wt is None else wt.data_ptr(), loss.data_ptr(),
+                                                   dlogits.data_ptr(), ws.data_ptr(), wsb, rows_, feat, feat, feat,
+                                                   -100, dt, 0, dt, st()), 'ce')
+            raw.check(lib.at_cross_entropy_scale_grad(dlogits.data_ptr(), one.data_ptr(), rows_, feat, feat, dt, dt,
+                                                      st()), 'ce_scale')
+        ms = gpu_time_ms(f, max(5, steps // 2), warmup)
+        gbs = 2 * tbytes / ms / 1e6
+        entry = {
+            'workload': f'c3: CrossEntropyLoss fp16 fwd+bwd logits[{rows_},{feat}], 5% ignore_index, {label}',
+            'metric': 'HBM GB/s', 'value': gbs, 'unit': 'GB/s', 'ms_fwd_bwd': ms,
+            'roofline': {'bound': 'hbm', 'achieved': gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                         'frac': gbs / PEAK_HBM_GBS, 'traffic': None},
+        }
+        if with_cpu and wt is None:
+            crow = 512
+            lc, tc = logits[:crow].cpu(), target[:crow]
+
+            def cpu():
+                oracle.cross_entropy_forward(lc, tc, None, -100, dtype)
+                oracle.cross_entropy_backward(torch.tensor(1.0), lc, tc, None, -100, dtype)
+            sec = cpu_time_s(cpu)
+            entry['cpu_baseline'] = {'value': 2 * crow * feat * 2 / sec / 1e9, 'unit': 'GB/s',
+                                     'cores': torch.get_num_threads(), 'kind': 'port',
+                                     'sample': f'first {crow} of {rows_} rows, oracle loss + gradient'}
+        results.append(entry)
+    return results
+
+
+# ------------------------------------------------------------------------------------------
+# c5: Conv2d 3x3 + BatchNorm2d(train) + residual + ReLU, bf16 [128, 64, 56, 56]
+# ------------------------------------------------------------------------------------------
+def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
+    import attorch_amd
+    raw = Raw()
+    lib = raw.lib
+    n, c, h, w_ = 128, 64, 56, 56
+    dtype = torch.bfloat16
+    dt = raw._lib.dtype_id(dtype)
+    nsets = 3
+    xs = [gen((n, c, h, w_), 5001 + i, dtype).cuda() for i in range(nsets)]
+    ress = [gen((n, c, h, w_), 5011 + i, dtype).cuda() for i in range(nsets)]
+    dys = [gen((n, c, h, w_), 5021 + i, dtype).cuda() for i in range(nsets)]
+    torch.manual_seed(5031)
+    wt = torch.nn.init.kaiming_normal_(torch.empty(c, c, 3, 3)).to(dtype).cuda()
+    ys = [torch.empty_like(xs[0]) for _ in range(nsets)]
+    pres = [torch.empty_like(xs[0]) for _ in range(nsets)]
+    dzs = [torch.empty_like(xs[0]) for _ in range(nsets)]
+    dxs = [torch.empty_like(xs[0]) for _ in range(nsets)]
+    dwt = torch.empty_like(wt)
+    bn_w = torch.ones(c, dtype=dtype, device='cuda')
+    bn_b = torch.zeros(c, dtype=dtype, device='cuda')
+    rm, rv = torch.zeros(c, device='cuda'), torch.ones(c, device='cuda')
+    mean, rstd = torch.empty(c, device='cuda'), torch.empty(c, device='cuda')
+    wg, bg = torch.empty(c, device='cuda'), torch.empty(c, device='cuda')
+    bn_wsb = lib.at_batch_norm_workspace_bytes(c)
+    bn_ws = torch.empty(bn_wsb, dtype=torch.uint8, device='cuda')
+    cw_wsb = lib.at_conv2d_bwd_weight_workspace_bytes(c, c, 3, 3)
+    cw_ws = torch.empty(cw_wsb, dtype=torch.uint8, device='cuda')
+    dims = (n, c, h, w_, c, h, w_, 3, 3, 1, 1, 1, 1, 1)
+    st = raw.stream
+    counter = [0]
+
+    def nxt():
+        counter[0] = (counter[0] + 1) % nsets
+        return counter[0]
+
+    def conv_f():
+        i = nxt()
+        raw.check(lib.at_conv2d_fwd(xs[i].data_ptr(), wt.data_ptr(), None, ys[i].data_ptr(), *dims, dt, dt, dt,
+                                    st()), 'conv_fwd')
+
+    def conv_dx():
+        i = nxt()
+        raw.check(lib.at_conv2d_bwd_input(dys[i].data_ptr(), wt.data_ptr(), dxs[i].data_ptr(), *dims, dt, st()),
+                  'conv_dx')
+
+    def conv_dw():
+        i = nxt()
+        raw.check(lib.at_conv2d_bwd_weight(dys[i].data_ptr(), xs[i].data_ptr(), dwt.data_ptr(), cw_ws.data_ptr(),
+                                           cw_wsb, *dims, dt, st()), 'conv_dw')
+
+    def bn_f():
+        i = nxt()
+        raw.check(lib.at_batch_norm_fwd(xs[i].data_ptr(), bn_w.data_ptr(), bn_b.data_ptr(), mean.data_ptr(),
+                                        rstd.data_ptr(), ress[i].data_ptr(), pres[i].data_ptr(), ys[i].data_ptr(),
+                                        rm.data_ptr(), rv.data_ptr(), bn_ws.data_ptr(), bn_wsb, n, c, h * w_, 0.1,
+                                        1e-5, 4, 0.0, 1, 1, dt, dt, 0, st()), 'bn_fwd')
+
+    def bn_b_():
+        i = nxt()
+        raw.check(lib.at_batch_norm_bwd(dys[i].data_ptr(), pres[i].data_ptr(), xs[i].data_ptr(), mean.data_ptr(),
+                                        rstd.data_ptr(), bn_w.data_ptr(), dxs[i].data_ptr(), dzs[i].data_ptr(),
+                                        wg.data_ptr(), bg.data_ptr(), bn_ws.data_ptr(), bn_wsb, n, c, h * w_, 4, 0.0,
+                                        dt, dt, st()), 'bn_bwd')
+
+    iters = max(5, steps // 2)
+    for i in range(nsets):   # pre-activations must exist before the backward timing
+        counter[0] = i - 1
+        bn_f()
+    t = {k_: gpu_time_ms(f, iters, warmup) for k_, f in (('conv_fwd', conv_f), ('conv_bwd_input', conv_dx),
+                                                        ('conv_bwd_weight', conv_dw), ('bn_fwd', bn_f),
+                                                        ('bn_bwd', bn_b_))}
+    gflop = 2.0 * n * c * h * w_ * c * 9 / 1e9
+    conv_ms = t['conv_fwd'] + t['conv_bwd_input'] + t['conv_bwd_weight']
+    conv_tf = 3 * gflop / conv_ms
+    tbytes = n * c * h * w_ * 2
+    bn_gbs = 9 * tbytes / (t['bn_fwd'] + t['bn_bwd']) / 1e6
+    conv_entry = {
+        'workload': f'c5: Conv2d 3x3 s1 p1 bf16 fwd+bwd X[{n},{c},{h},{w_}] W[{c},{c},3,3]',
+        'metric': 'conv TFLOP/s', 'value': conv_tf, 'unit': 'TFLOP/s', 'kernel_ms': {k_: t[k_] for k_ in t if 'conv' in k_},
+        'roofline': {'bound': 'mfma', 'achieved': conv_tf, 'peak': PEAK_MFMA_16BIT_TFLOPS, 'unit': 'TFLOP/s',
+                     'frac': conv_tf / PEAK_MFMA_16BIT_TFLOPS, 'traffic': None},
+    }
+    bn_entry = {
+        'workload': f'c5: BatchNorm2d(train)+residual+ReLU bf16 fwd+bwd X[{n},{c},{h},{w_}]',
+        'metric': 'HBM GB/s', 'value': bn_gbs, 'unit': 'GB/s', 'ms_fwd': t['bn_fwd'], 'ms_bwd': t['bn_bwd'],
+        'roofline': {'bound': 'hbm', 'achieved': bn_gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                     'frac': bn_gbs / PEAK_HBM_GBS, 'traffic': None},
+        'buffer_rotation': f'{nsets} sets of 7 tensors (49 MiB each)',
+    }
+    # the block end to end through the modules (conv -> bn + residual + relu, fwd + bwd)
+    conv = attorch_amd.Conv2d(c, c, 3, padding=1, bias=False, dtype=dtype)
+    bn = attorch_amd.BatchNorm2d(c, act_func='relu', dtype=dtype)
+    with torch.no_grad():
+        conv.weight.copy_(wt)
+    xin = xs[0].clone().requires_grad_(True)
+    rin = ress[0].clone().requires_grad_(True)
+
+    def block():
+        xin.grad = None
+        rin.grad = None
+        conv.weight.grad = None
+        bn.weight.grad = None
+        bn.bias.grad = None
+        bn(conv(xin), rin).backward(dys[0])
+
+    conv_entry['block_ms_fwd_bwd_modules'] = wall_time_ms(block, max(3, steps // 4), 2)
+    if with_cpu:
+        import oracle
+        cn = 8
+        xc, rc, dyc, wc = xs[0][:cn].cpu(), ress[0][:cn].cpu(), dys[0][:cn].cpu(), wt.cpu()
+
+        def cpu_conv():
+            oracle.conv2d_forward(xc, wc, None, (1, 1), (1, 1), 1, dtype)
+            oracle.conv2d_backward(dyc, xc, wc, (1, 1), (1, 1), 1, dtype)
+
+        def cpu_bn():
+            out, pre_act, m_, r_, _, _ = oracle.batch_norm_forward(xc, True, bn_w.cpu(), bn_b.cpu(), rm.cpu(), rv.cpu(),
+                                                                   0.1, 1e-5, True, rc, 'relu', None)
+            oracle.batch_norm_backward(dyc, xc, m_, r_, bn_w.cpu(), True, pre_act, 'relu', None)
+        sec = cpu_time_s(cpu_conv)
+        conv_entry['cpu_baseline'] = {'value': 3 * gflop * cn / n / sec / 1e3, 'unit': 'TFLOP/s',
+                                      'cores': torch.get_num_threads(), 'kind': 'port',
+                                      'sample': f'first {cn} of {n} images, oracle fwd+bwd'}
+        sec = cpu_time_s(cpu_bn)
+        bn_entry['cpu_baseline'] = {'value': 9 * tbytes * cn / n / sec / 1e9, 'unit': 'GB/s',
+                                    'cores': torch.get_num_threads(), 'kind': 'port',
+                                    'sample': f'first {cn} of {n} images, oracle fwd+bwd'}
+    return [conv_entry, bn_entry]
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print(f'bench.py: this build targets one GPU; --gpus {args.gpus} is not supported (every BASELINE '
+              'config is a single-GPU workload). Run with --gpus 1.', file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print('bench.py: no HIP device visible; the kernels have no CPU path.', file=sys.stderr)
+        return 2
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    torch.set_num_threads(os.cpu_count())
+    with_cpu = not args.no_cpu
+    head = bench_linear('c4', args.steps, args.warmup, with_cpu)
+    extra: List[Dict] = []
+    wanted = [] if args.configs == 'none' else args.configs.split(',')
+    if 'c1' in wanted:
+        extra.append(bench_linear('c1', max(args.steps, 50), args.warmup, with_cpu))
+    if 'c2' in wanted:
+        extra.extend(bench_rows(args.steps, args.warmup, with_cpu))
+    if 'c3' in wanted:
+        extra.extend(bench_cross_entropy(args.steps, args.warmup, with_cpu))
+    if 'c5' in wanted:
+        extra.extend(bench_conv_bn(args.steps, args.warmup, with_cpu))
+    line = {
+        'metric': 'Linear fwd+bwd TFLOP/s; norm/softmax/CE HBM GB/s; % of MI355X roofline',
+        'value': head['value'], 'unit': 'TFLOP/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'ms_per_step': head['ms_per_step'], 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+        'dtype': 'bf16', 'data': 'synthetic',
+        'config': {'workload': head['workload'], 'step': 'attorch_amd.Linear forward + backward (dX, dW, db)',
+                   'algorithmic_flop_per_step': 6 * 16384 * 4096 * 16384},
+        'roofline': head['roofline'],
+        'cpu_baseline': head.get('cpu_baseline'),
+        'frac_of_peak_step': head['frac_of_peak_step'],
+        'kernel_ms': head['kernel_ms'], 'kernel_tflops': head['kernel_tflops'],
+        'configs': extra,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == '__main__':
+    sys.exit(main())
