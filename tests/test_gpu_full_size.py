@@ -1,0 +1,174 @@
+"""
+Full-size checks at the BASELINE configurations (c1-c5).  Where the CPU oracle finishes in
+seconds the whole result is compared; otherwise a slice is compared against the oracle and
+size-independent properties cover the rest (rows of a softmax gradient sum to zero, ignored
+rows are exactly zero, a weight gradient over the batch is the sum of the gradients of its
+halves, column sums match).
+"""
+
+import pytest
+import torch
+
+import attorch_amd
+import oracle
+from .helpers import assert_close, randn
+
+pytestmark = pytest.mark.gpu
+BF16, F16, F32 = torch.bfloat16, torch.float16, torch.float32
+
+
+def test_c1_linear_fp32_relu() -> None:
+    x = randn((512, 784), 1001)
+    torch.manual_seed(1002)
+    lin = torch.nn.Linear(784, 256)
+    w, b = lin.weight.detach().T.contiguous(), lin.bias.detach()
+    dy = randn((512, 256), 1003)
+    xd, wd, bd = (t.cuda().requires_grad_(True) for t in (x, w, b))
+    y = attorch_amd.LinearAutoGrad.apply(xd, wd, bd, 'relu')
+    pre_act = y.grad_fn.saved_tensors[1].detach().cpu()
+    y.backward(dy.cuda())
+    y_ref, _ = oracle.linear_forward(x, w, b, 'relu', None, F32, compute=torch.float64)
+    dx_ref, dw_ref, db_ref = oracle.linear_backward(dy, x, w, pre_act, 'relu', None, F32, compute=torch.float64)
+    assert_close(y, y_ref, F32, 'output')
+    assert_close(xd.grad, dx_ref, F32, 'input_grad', normalize=True)
+    assert_close(wd.grad, dw_ref, F32, 'weight_grad', normalize=True)
+    assert_close(bd.grad, db_ref, F32, 'bias_grad', normalize=True)
+
+
+def test_c2_norms_and_softmax_bf16() -> None:
+    shape = (8192, 4096)
+    x, dy = randn(shape, 2001, BF16), randn(shape, 2002, BF16)
+    w, b = randn((4096,), 2003, BF16, 0.1, 1.0), randn((4096,), 2004, BF16, 0.1)
+    xd, wd, bd = (t.cuda().requires_grad_(True) for t in (x, w, b))
+    y = attorch_amd.LayerNormAutoGrad.apply(xd, wd, bd, 1e-5, True)
+    y.backward(dy.cuda())
+    y_ref, mean, inv_std = oracle.layer_norm_forward(x, w, b, 1e-5, BF16)
+    dx_ref, dw_ref, db_ref = oracle.layer_norm_backward(dy, x, mean, inv_std, w, BF16)
+    assert_close(y, y_ref, BF16, 'layer_norm output')
+    assert_close(xd.grad, dx_ref, BF16, 'layer_norm input_grad')
+    assert_close(wd.grad, dw_ref.to(BF16), BF16, 'layer_norm weight_grad', normalize=True)
+    assert_close(bd.grad, db_ref.to(BF16), BF16, 'layer_norm bias_grad', normalize=True)
+
+    xd, wd = x.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
+    y = attorch_amd.RMSNormAutoGrad.apply(xd, wd, 1e-5)
+    y.backward(dy.cuda())
+    y_ref, inv_rms = oracle.rms_norm_forward(x, w, 1e-5)
+    dx_ref, dw_ref = oracle.rms_norm_backward(dy, x, inv_rms, w)
+    assert_close(y, y_ref, BF16, 'rms_norm output')
+    assert_close(xd.grad, dx_ref, BF16, 'rms_norm input_grad')
+    assert_close(wd.grad, dw_ref.to(BF16), BF16, 'rms_norm weight_grad', normalize=True)
+
+    for log in (False, True):
+        xd = x.cuda().requires_grad_(True)
+        y = attorch_amd.SoftmaxAutoGrad.apply(xd, False, log)
+        y.backward(dy.cuda())
+        assert_close(y, oracle.softmax_forward(x, False, log, BF16), BF16, f'softmax(log={log}) output')
+        assert_close(xd.grad, oracle.softmax_backward(dy, y.detach().cpu(), False, log), BF16,
+                     f'softmax(log={log}) input_grad')
+
+
+@pytest.mark.parametrize('weighted', [False, True])
+def test_c3_cross_entropy_fp16(weighted) -> None:
+    rows, vocab = 8192, 50257
+    logits = randn((rows, vocab), 3001, F16, 2.0)
+    gen = torch.Generator().manual_seed(3002)
+    target = torch.randint(0, vocab, (rows,), generator=gen)
+    target[torch.rand(rows, generator=gen) < 0.05] = -100
+    weight = 0.5 + torch.rand(vocab, generator=gen) if weighted else None
+    xd = logits.cuda().requires_grad_(True)
+    loss = attorch_amd.CrossEntropyLossAutoGrad.apply(xd, target.cuda(), None if weight is None else weight.cuda(),
+                                                      -100)
+    loss.backward()
+    grad = xd.grad
+
+    # loss: the oracle row by row in slices, combined with the global divisor
+    keep = target != -100
+    row_w = (weight[target.clamp(min=0)] if weighted else torch.ones(rows)) * keep
+    denom = row_w.sum().double()
+    total = torch.zeros((), dtype=torch.float64)
+    for start in range(0, rows, 1024):
+        sl = slice(start, start + 1024)
+        part, part_denom = oracle.cross_entropy_forward(logits[sl], target[sl], weight, -100, torch.float64)
+        total += part * part_denom.double()
+    assert_close(loss, (total / denom).float(), F16, 'loss')
+
+    # gradient: a slice against the oracle (rescaled from the slice's divisor to the global one)
+    sl = slice(4096, 4096 + 256)
+    local = row_w[sl].sum().double()
+    ref = oracle.cross_entropy_backward((local / denom).float(), logits[sl], target[sl], weight, -100, F32)
+    kept = float(keep.sum())
+    assert_close(grad[sl].float() * kept, ref * kept, F16, 'input_grad slice')
+    # properties over the full gradient
+    assert torch.all(grad[(~keep).cuda()] == 0), 'ignored rows must be exactly zero'
+    row_sums = grad.float().sum(dim=1) * kept
+    assert row_sums.abs().max().item() < 0.25, 'rows of softmax - onehot sum to zero (fp16 rounding aside)'
+    picked = grad[torch.arange(rows)[keep].cuda(), target[keep].cuda()]
+    assert torch.all(picked < 0), 'the target column of every kept row has a negative gradient'
+
+
+def test_c4_linear_bf16_gelu() -> None:
+    m, k, n = 16384, 4096, 16384
+    x, w, b = randn((m, k), 4001, BF16), randn((k, n), 4002, BF16, 0.02), torch.zeros(n, dtype=BF16)
+    dy = randn((m, n), 4003, BF16)
+    xd, wd, bd = (t.cuda().requires_grad_(True) for t in (x, w, b))
+    y = attorch_amd.LinearAutoGrad.apply(xd, wd, bd, 'geluapprox')
+    pre_act = y.grad_fn.saved_tensors[1].detach()
+    y.backward(dy.cuda())
+
+    rows = torch.cat([torch.arange(0, 48), torch.arange(8000, 8032), torch.arange(m - 48, m)])
+    y_ref, pre_ref = oracle.linear_forward(x[rows], w, b, 'geluapprox', None, BF16)
+    assert_close(y[rows.cuda()], y_ref, BF16, 'output rows')
+    assert_close(pre_act[rows.cuda()], pre_ref, BF16, 'pre_act rows')
+    # backward of the sampled rows from the device's own pre-activation
+    dx_ref, _, _ = oracle.linear_backward(dy[rows], x[rows], w, pre_act[rows.cuda()].cpu(), 'geluapprox', None, BF16)
+    assert_close(xd.grad[rows.cuda()], dx_ref, BF16, 'input_grad rows', normalize=True)
+    # weight gradient: a band of input features over the whole batch, and the bias gradient
+    dz = (dy.float() * oracle.act_grad(pre_act.cpu().float(), 'geluapprox')).to(BF16)
+    cols = torch.cat([torch.arange(0, 8), torch.arange(2048, 2056), torch.arange(k - 8, k)])
+    dw_ref = (x[:, cols].float().T @ dz.float()).to(BF16)
+    assert_close(wd.grad[cols.cuda()], dw_ref, BF16, 'weight_grad rows', normalize=True)
+    assert_close(bd.grad, dz.float().sum(dim=0).to(BF16), BF16, 'bias_grad', normalize=True)
+
+
+def test_c5_conv_bn_residual_relu_bf16() -> None:
+    n, c, h, w_ = 128, 64, 56, 56
+    x, res, dy = randn((n, c, h, w_), 5001, BF16), randn((n, c, h, w_), 5002, BF16), randn((n, c, h, w_), 5003, BF16)
+    torch.manual_seed(5004)
+    wt = torch.nn.init.kaiming_normal_(torch.empty(c, c, 3, 3)).to(BF16)
+    xd, wd = x.cuda().requires_grad_(True), wt.cuda().requires_grad_(True)
+    conv_out = attorch_amd.Conv2dAutoGrad.apply(xd, wd, None, 1, 1, 1, 1, 1)
+    conv_out.backward(dy.cuda())
+    sub = slice(60, 64)
+    assert_close(conv_out[sub], oracle.conv2d_forward(x[sub], wt, None, (1, 1), (1, 1), 1, BF16), BF16,
+                 'conv output slice', normalize=True)
+    dx_ref, dw_sub_ref, _ = oracle.conv2d_backward(dy[sub], x[sub], wt, (1, 1), (1, 1), 1, BF16)
+    assert_close(xd.grad[sub], dx_ref, BF16, 'conv input_grad slice', normalize=True)
+    # weight gradient: the slice alone against the oracle, the full batch as the sum of its halves
+    halves = []
+    for part in (slice(0, 64), slice(64, 128), sub):
+        xp, wp = x[part].cuda().requires_grad_(True), wt.cuda().requires_grad_(True)
+        attorch_amd.Conv2dAutoGrad.apply(xp, wp, None, 1, 1, 1, 1, 1).backward(dy[part].cuda())
+        halves.append(wp.grad.float())
+    assert_close(halves[2], dw_sub_ref, BF16, 'conv weight_grad slice', normalize=True)
+    assert_close(wd.grad.float(), halves[0] + halves[1], BF16, 'conv weight_grad additivity', normalize=True)
+
+    bn_w, bn_b = randn((c,), 5005, BF16, 0.1, 1.0), randn((c,), 5006, BF16, 0.1)
+    rm, rv = torch.zeros(c), torch.ones(c)
+    conv_cpu = conv_out.detach().cpu()
+    cd, rd = conv_out.detach().requires_grad_(True), res.cuda().requires_grad_(True)
+    wdv, bdv = bn_w.cuda().requires_grad_(True), bn_b.cuda().requires_grad_(True)
+    rmd, rvd = rm.cuda(), rv.cuda()
+    out = attorch_amd.BatchNormAutoGrad.apply(cd, True, wdv, bdv, rmd, rvd, 0.1, 1e-5, True, rd, 'relu')
+    saved = [t.detach().cpu() for t in out.grad_fn.saved_tensors]
+    out.backward(dy.cuda())
+    out_ref, _, _, _, rm_ref, rv_ref = oracle.batch_norm_forward(conv_cpu, True, bn_w, bn_b, rm, rv, 0.1, 1e-5, True,
+                                                                 res, 'relu', None)
+    assert_close(out, out_ref, BF16, 'batch_norm output')
+    assert_close(rmd, rm_ref, F32, 'running_mean')
+    assert_close(rvd, rv_ref, F32, 'running_var')
+    dx_ref, dw_ref, db_ref, dres_ref = oracle.batch_norm_backward(dy, conv_cpu, saved[1], saved[2], bn_w, True, saved[4],
+                                                                  'relu', None)
+    assert_close(cd.grad, dx_ref, BF16, 'batch_norm input_grad', normalize=True)
+    assert_close(wdv.grad, dw_ref.to(BF16), BF16, 'batch_norm weight_grad', normalize=True)
+    assert_close(bdv.grad, db_ref.to(BF16), BF16, 'batch_norm bias_grad', normalize=True)
+    assert_close(rd.grad, dres_ref, BF16, 'batch_norm residual_grad')
