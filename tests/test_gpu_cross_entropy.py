@@ -52,6 +52,9 @@ def test_cross_entropy(shape, dtype, weighted, ignore_fraction, upstream) -> Non
     assert_close(xd.grad * kept, grad_ref.to(cd) * kept, dtype, 'input_grad')
     ignored = (target == -100).cuda()
     assert torch.all(xd.grad[ignored] == 0), 'ignored rows must get exactly zero gradient'
+    if dtype is torch.float32:
+        # rows of softmax - onehot sum to zero
+        assert (xd.grad.sum(dim=1) * kept).abs().max().item() < 1e-3
 
 
 def test_special_cases() -> None:
