@@ -36,7 +36,8 @@ PROTOTYPES = {
     'at_linear_fwd': (I, [P, P, P, P, P, L, L, L, L, L, L, L, I, F, I, I, I, P]),
     'at_linear_bwd_input': (I, [P, P, P, L, L, L, L, L, L, I, I, P]),
     'at_linear_bwd_weight': (I, [P, P, P, L, L, L, L, L, L, I, I, P]),
-    'at_act_bwd': (I, [P, P, P, L, L, L, L, L, I, F, I, I, P]),
+    'at_act_bwd_workspace_bytes': (L, [L, L]),
+    'at_act_bwd': (I, [P, P, P, P, P, L, L, L, L, L, L, I, F, I, I, I, P]),
     'at_colsum_workspace_bytes': (L, [L, L]),
     'at_colsum': (I, [P, P, P, L, L, L, L, I, I, P]),
     'at_batch_norm_workspace_bytes': (L, [L]),

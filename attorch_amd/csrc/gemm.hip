@@ -55,87 +55,150 @@ template <> struct Mfma16<f16_t> {
 constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int kGemmThreads = 256;
 constexpr int kTileBytes = BM * BK * 2;  // one operand tile, 32 KiB
+constexpr int kEpiPitch = BN * 2 + 16;   // bytes per row of the epilogue tile in LDS (padded against bank conflicts)
+constexpr int kEpiBytes = BM * kEpiPitch;
+
+__device__ __forceinline__ bool aligned16_dev(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // Byte offset of 16-byte chunk `chunk` (0..7) of row `row` inside a [256][64] 16-bit tile.
 __device__ __forceinline__ int lds_chunk_offset(int row, int chunk) {
   return row * (BK * 2) + ((chunk ^ ((row ^ (row >> 3)) & 7)) << 4);
 }
 
-// 8x8 transpose of 16-bit elements held as 8 rows of 128 bits: out[c] = column c.
-__device__ __forceinline__ void transpose8x8(const uint4 (&in)[8], uint4 (&out)[8]) {
-  const uint32_t w[8][4] = {{in[0].x, in[0].y, in[0].z, in[0].w}, {in[1].x, in[1].y, in[1].z, in[1].w},
-                            {in[2].x, in[2].y, in[2].z, in[2].w}, {in[3].x, in[3].y, in[3].z, in[3].w},
-                            {in[4].x, in[4].y, in[4].z, in[4].w}, {in[5].x, in[5].y, in[5].z, in[5].w},
-                            {in[6].x, in[6].y, in[6].z, in[6].w}, {in[7].x, in[7].y, in[7].z, in[7].w}};
-#pragma unroll
-  for (int c = 0; c < 8; ++c) {
-    uint32_t o[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      // rows 2j (low half) and 2j+1 (high half), column c lives in word c/2, half c%2
-      o[j] = (c & 1) ? __builtin_amdgcn_perm(w[2 * j + 1][c >> 1], w[2 * j][c >> 1], 0x07060302u)
-                     : __builtin_amdgcn_perm(w[2 * j + 1][c >> 1], w[2 * j][c >> 1], 0x05040100u);
-    }
-    out[c] = make_uint4(o[0], o[1], o[2], o[3]);
-  }
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void lds_void_t;
+constexpr int kOobOffset = (int)0x80000000u;  // beyond any buffer this kernel accepts (< 2 GiB)
+
+// LDS image of one operand tile of a k-tile.
+//  * CONTRACT_CONTIG (memory [outer][k]): 256 rows x 128 bytes, 16-byte chunks XOR-swizzled by
+//    the row (lds_chunk_offset); fragments are plain 128-bit reads.
+//  * otherwise (memory [k][outer]): 64 k-rows x 512 bytes kept as loaded; every pair of rows
+//    is one contiguous KiB (one wave-wide load) followed by 64 bytes of padding, which
+//    spreads the 8 rows a transposing fragment read touches evenly over the banks.
+constexpr int kPairPitch = 1024 + 64;
+template <bool CONTRACT_CONTIG> constexpr int operand_tile_bytes() { return CONTRACT_CONTIG ? kTileBytes : 32 * kPairPitch; }
+
+// Global -> LDS without passing through registers (buffer_load ... lds): each wave-wide load
+// moves 64 lanes x 16 bytes into one contiguous KiB of LDS, each lane choosing its own global
+// address.  Buffer addressing gives zero fill for rows past the end of the tensor.
+// The loads are issued as inline assembly on purpose: the compiler cannot tell that a load into
+// one LDS stage does not alias the fragment reads of the other stage and would otherwise wait
+// for every outstanding load (vmcnt(0)) before the next LDS read.  The kernel waits for them
+// itself, once, before the barrier that publishes the stage.
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void lds_dma_16(const i32x4& rsrc, int byte_offset, const char* lds_dst) {
+  // LDS byte address of lane 0's 16 bytes; wave-uniform by construction, made so for the compiler
+  const unsigned m0 = (unsigned)__builtin_amdgcn_readfirstlane((int)(uintptr_t)lds_dst);
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(m0), "v"(byte_offset), "s"(rsrc)
+               : "m0");
 }
 
-// Operand staging.  CONTRACT_CONTIG: memory is [outer][k] (k contiguous); otherwise [k][outer].
-template <typename T, bool CONTRACT_CONTIG>
-struct OperandStage {
-  uint4 r[8];
+__device__ __forceinline__ void lds_dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
-  __device__ __forceinline__ void load(const T* __restrict__ base, int64_t ld, int outer0, int outer_total,
-                                       int k0, int K) {
-    const int t = threadIdx.x;
+template <typename T, bool CONTRACT_CONTIG>
+struct OperandLoader {
+  i32x4 rsrc;
+  int lane_off;   // byte offset of this lane's first load at k-tile 0
+  int blk_step;   // bytes between the 8 loads of a lane
+  int k_step;     // bytes per k-tile
+  int k_lane;     // k of this lane inside a k-tile (contract-contiguous layout only)
+  int K;
+
+  static __device__ __forceinline__ i32x4 make_rsrc(const void* base, int64_t bytes) {
+    const uint64_t addr = reinterpret_cast<uint64_t>(base);
+    i32x4 r;
+    r.x = (int)(uint32_t)addr;
+    r.y = (int)(uint32_t)((addr >> 32) & 0xffffu);   // stride 0: raw buffer
+    r.z = (int)bytes;                                  // num_records in bytes
+    r.w = 0x00020000;                                  // 32-bit untyped data format
+    return r;
+  }
+
+  __device__ __forceinline__ void init(const T* base, int64_t ld, int outer0, int outer_total, int K_) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    K = K_;
     if (CONTRACT_CONTIG) {
-      const int c = t & 7;
-      const int k = k0 + c * 8;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int o = outer0 + (t >> 3) + 32 * i;
-        r[i] = (o < outer_total && k < K) ? *reinterpret_cast<const uint4*>(base + (int64_t)o * ld + k)
-                                          : make_uint4(0, 0, 0, 0);
-      }
+      rsrc = make_rsrc(base, outer_total * ld * 2);
+      // load i of wave w fills rows 8q .. 8q+7 (q = 8w + i); lane -> (row, position), and the
+      // position holds chunk (position ^ swizzle(row)) so that the reads find chunk c at c ^ swizzle
+      const int row = wave * 64 + (lane >> 3);            // + 8 i
+      k_lane = 0;
+      lane_off = (int)(((int64_t)(outer0 + row) * ld) * 2);
+      blk_step = (int)(8 * ld * 2);
+      k_step = BK * 2;
     } else {
-      const int o = outer0 + (t & 31) * 8;
-      const int kb = k0 + (t >> 5) * 8;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int k = kb + i;
-        r[i] = (o < outer_total && k < K) ? *reinterpret_cast<const uint4*>(base + (int64_t)k * ld + o)
-                                          : make_uint4(0, 0, 0, 0);
-      }
+      rsrc = make_rsrc(base, K_ * ld * 2);
+      // load i of wave w fills k-rows 2q, 2q+1 (q = 8w + i); lane -> k-row 2q + lane/32, 8 columns at (lane%32)*8
+      const int krow = wave * 16 + (lane >> 5);            // + 2 i
+      k_lane = 0;
+      lane_off = (int)(((int64_t)krow * ld + outer0 + (lane & 31) * 8) * 2);
+      blk_step = (int)(2 * ld * 2);
+      k_step = (int)(BK * ld * 2);
     }
   }
 
-  __device__ __forceinline__ void store(char* tile) const {
-    const int t = threadIdx.x;
-    if (CONTRACT_CONTIG) {
-      const int c = t & 7;
+  // Issues the 8 loads of this lane for k-tile `kt` into `tile` (LDS).
+  __device__ __forceinline__ void issue(int kt, char* tile) const {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int row = (t >> 3) + 32 * i;
-        *reinterpret_cast<uint4*>(tile + lds_chunk_offset(row, c)) = r[i];
+    for (int i = 0; i < 8; ++i) issue_one(kt, tile, i);
+  }
+
+  // Load i (0..7) of this lane for k-tile `kt`.
+  __device__ __forceinline__ void issue_one(int kt, char* tile, int i) const {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    {
+      const int q = wave * 8 + i;
+      int off;
+      char* dst;
+      if (CONTRACT_CONTIG) {
+        const int row = q * 8 + (lane >> 3);
+        const int chunk = (lane & 7) ^ ((row ^ (row >> 3)) & 7);
+        const int k = kt * BK + chunk * 8;
+        off = k < K ? lane_off + i * blk_step + k * 2 : kOobOffset;   // K tail reads as zeros
+        dst = tile + q * 1024;
+      } else {
+        off = lane_off + i * blk_step + kt * k_step;                  // k-rows past K fall out of range
+        dst = tile + q * kPairPitch;
       }
-    } else {
-      uint4 tr[8];
-      transpose8x8(r, tr);
-      const int chunk = t >> 5;
-#pragma unroll
-      for (int c = 0; c < 8; ++c) {
-        const int row = (t & 31) * 8 + c;
-        *reinterpret_cast<uint4*>(tile + lds_chunk_offset(row, chunk)) = tr[c];
-      }
+      lds_dma_16(rsrc, off, dst);
     }
   }
 };
+
+// Fragment of 32 rows (outer index) x 16 k for one MFMA operand: 8 consecutive k per lane.
+template <bool CONTRACT_CONTIG>
+__device__ __forceinline__ uint4 read_frag(const char* tile, int outer_base, int ks) {
+  const int lane = threadIdx.x & 63;
+  if (CONTRACT_CONTIG) {
+    return *reinterpret_cast<const uint4*>(tile + lds_chunk_offset(outer_base + (lane & 31), ks * 2 + (lane >> 5)));
+  } else {
+    // ds_read_b64_tr_b16: within 16 lanes, result[l][e] = source[4e + l/4][l%4]; the source lane
+    // 4e + q therefore points at k-row (k0 + e), columns 4q .. 4q+3, and lane l receives
+    // k0 .. k0+3 of column l.  Two reads give the 8 k of this lane's half.
+    const int i = lane & 15, g = lane >> 4;
+    const int col = outer_base + (g & 1) * 16 + (i & 3) * 4;
+    const int krow = ks * 16 + (g >> 1) * 8 + (i >> 2);
+    const char* p0 = tile + (krow >> 1) * kPairPitch + (krow & 1) * 512 + col * 2;
+    const int krow1 = krow + 4;
+    const char* p1 = tile + (krow1 >> 1) * kPairPitch + (krow1 & 1) * 512 + col * 2;
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p0);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p1);
+    const uint2 a = __builtin_bit_cast(uint2, lo), b = __builtin_bit_cast(uint2, hi);
+    return make_uint4(a.x, a.y, b.x, b.y);
+  }
+}
 
 // ACT is the compile-time activation id of the epilogue (the act switch must fold away: the
 // epilogue is fully unrolled over 256 accumulator registers).
 template <typename T, bool A_MC, bool B_KC, int ACT>
 __global__ __launch_bounds__(kGemmThreads) void gemm_mfma16_kernel(GemmArgs g) {
-  __shared__ __attribute__((aligned(16))) char lds[4 * kTileBytes];  // [stage][A|B]
+  constexpr bool A_KC = !A_MC;
+  constexpr int kATile = operand_tile_bytes<A_KC>(), kBTile = operand_tile_bytes<B_KC>();
+  constexpr int kStage = kATile + kBTile;
+  constexpr int kLds = 2 * kStage > kEpiBytes ? 2 * kStage : kEpiBytes;
+  __shared__ __attribute__((aligned(1024))) char lds[kLds];  // main loop: [stage][A|B]; epilogue: output tile
   const T* __restrict__ A = reinterpret_cast<const T*>(g.a);
   const T* __restrict__ B = reinterpret_cast<const T*>(g.b);
 
@@ -158,6 +221,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_mfma16_kernel(GemmArgs g) {
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave >> 1, wn = wave & 1;
+  const int frag_row = lane & 31, frag_half = lane >> 5;
 
   f32x16 acc[4][4];
 #pragma unroll
@@ -167,93 +231,126 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_mfma16_kernel(GemmArgs g) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  OperandStage<T, !A_MC> sa;
-  OperandStage<T, B_KC> sb;
+  OperandLoader<T, A_KC> la;
+  OperandLoader<T, B_KC> lb;
+  la.init(A, g.lda, m0, g.M, g.K);
+  lb.init(B, g.ldb, n0, g.N, g.K);
   const int KT = (g.K + BK - 1) / BK;
 
-  sa.load(A, g.lda, m0, g.M, 0, g.K);
-  sb.load(B, g.ldb, n0, g.N, 0, g.K);
-  sa.store(lds);
-  sb.store(lds + kTileBytes);
+  la.issue(0, lds);
+  lb.issue(0, lds + kATile);
+  lds_dma_wait_all();
   __syncthreads();
 
-  const int frag_row = lane & 31, frag_half = lane >> 5;
-  for (int kt = 0; kt < KT; ++kt) {
-    char* cur = lds + (kt & 1) * 2 * kTileBytes;
-    char* nxt = lds + ((kt & 1) ^ 1) * 2 * kTileBytes;
-    const bool more = kt + 1 < KT;
-    if (more) {
-      sa.load(A, g.lda, m0, g.M, (kt + 1) * BK, g.K);
-      sb.load(B, g.ldb, n0, g.N, (kt + 1) * BK, g.K);
+  auto load_frags = [&](const char* stage, int ks, uint4 (&af)[4], uint4 (&bf)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      af[i] = read_frag<A_KC>(stage, wm * 128 + i * 32, ks);
+      bf[i] = read_frag<B_KC>(stage + kATile, wn * 128 + i * 32, ks);
     }
+  };
+
+  // One k-tile = four k-steps of 16 MFMAs (512 matrix-pipe cycles each).  With a single wave
+  // per SIMD nothing else hides latency, so the other instructions of the iteration are
+  // slotted between MFMAs: the 16 global->LDS loads of the next tile during k-step 0, the
+  // fragment reads of k-step s+1 during k-step s.  The loads of tile kt+1 stay in flight for
+  // the whole iteration and are only waited for at the barrier that ends it.
+  // (sched_group_barrier masks: 0x8 MFMA, 0x2 VALU, 0x20 VMEM read, 0x100 LDS read.)
+  for (int kt = 0; kt < KT; ++kt) {
+    char* cur = lds + (kt & 1) * kStage;
+    char* nxt = lds + ((kt & 1) ^ 1) * kStage;
+    uint4 af[2][4], bf[2][4];
+    load_frags(cur, 0, af[0], bf[0]);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
-      uint4 af[4], bf[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        af[i] = *reinterpret_cast<const uint4*>(cur + lds_chunk_offset(wm * 128 + i * 32 + frag_row, ks * 2 + frag_half));
-        bf[i] = *reinterpret_cast<const uint4*>(cur + kTileBytes +
-                                                lds_chunk_offset(wn * 128 + i * 32 + frag_row, ks * 2 + frag_half));
-      }
+      if (ks + 1 < BK / 16) load_frags(cur, ks + 1, af[(ks + 1) & 1], bf[(ks + 1) & 1]);
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < 4; ++j) {
+          // One global->LDS load of the next tile behind each MFMA of k-step 0.  Unconditional:
+          // past the last k-tile every offset is out of range and the loads write zeros into
+          // a stage nobody reads, so the loop body has no branches.
+          if (ks == 0) {
+            if (i < 2) la.issue_one(kt + 1, nxt, i * 4 + j);
+            else lb.issue_one(kt + 1, nxt + kATile, (i - 2) * 4 + j);
+          }
           // operands swapped: the accumulator holds C^T, i.e. 4 consecutive n per lane
-          acc[i][j] = Mfma16<T>::run(bf[j], af[i], acc[i][j]);
+          acc[i][j] = Mfma16<T>::run(bf[ks & 1][j], af[ks & 1][i], acc[i][j]);
+        }
+      if (ks < BK / 16 - 1) {
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
-    if (more) {
-      sa.store(nxt);
-      sb.store(nxt + kTileBytes);
-    }
-    __syncthreads();
+    lds_dma_wait_all();   // this wave's part of the next stage has landed
+    __syncthreads();      // ... and so has everybody else's; the current stage may be overwritten
   }
 
-  // ---- epilogue: lane holds, for tile (i, j) and register group rg, C[m][n .. n+3] with
-  //      m = m0 + wm*128 + i*32 + lane%32, n = n0 + wn*128 + j*32 + rg*8 + (lane/32)*4 ----
+  // ---- epilogue ----
+  // A lane holds, for tile (i, j) and register group rg, C[m][n .. n+3] with
+  //   m = wm*128 + i*32 + lane%32,  n = wn*128 + j*32 + rg*8 + (lane/32)*4   (tile-local).
+  // Storing that straight to memory touches 32 rows per instruction with 16 bytes each; instead
+  // the finished tile goes through LDS (free after the main loop) and leaves as whole rows:
+  // 32 lanes x 16 bytes = one 512-byte row segment per half-wave.
   T* __restrict__ C = reinterpret_cast<T*>(g.c);
   T* __restrict__ P = reinterpret_cast<T*>(g.pre_act);
-  const bool vec_ok = ((g.ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(C) & 7u) == 0) &&
-                      (!P || (((g.ldp & 3) == 0) && ((reinterpret_cast<uintptr_t>(P) & 7u) == 0)));
+  const bool rows16 = ((g.ldc & 7) == 0) && aligned16_dev(C) && (n0 + BN <= g.N) &&
+                      (!P || (((g.ldp & 7) == 0) && aligned16_dev(P)));
+  constexpr int n_out = ACT != AT_ACT_NONE ? 2 : 1;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int pass = 0; pass < n_out; ++pass) {
+    const bool is_pre = (n_out == 2 && pass == 0);
+    T* __restrict__ dst = is_pre ? P : C;
+    const int64_t ldd = is_pre ? g.ldp : g.ldc;
+    if (is_pre && !P) continue;   // uniform
+    __syncthreads();              // previous readers of LDS (main loop or previous pass) are done
 #pragma unroll
-    for (int rg = 0; rg < 4; ++rg) {
-      const int n = n0 + wn * 128 + j * 32 + rg * 8 + frag_half * 4;
-      float bv[4] = {0.f, 0.f, 0.f, 0.f};
-      if (g.bias) {
+    for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (n + e < g.N) bv[e] = load_scalar_f32(g.bias, g.bias_dt, n + e);
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int m = m0 + wm * 128 + i * 32 + frag_row;
-        if (m >= g.M || n >= g.N) continue;
-        float v[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][rg * 4 + e] + bv[e];
-        const bool full = vec_ok && n + 3 < g.N;
-        if (ACT != AT_ACT_NONE) {
-          if (P) {
-            T* pp = P + (int64_t)m * g.ldp + n;
-            if (full) store_f32<T, 4>(pp, v);
-            else {
-#pragma unroll
-              for (int e = 0; e < 4; ++e)
-                if (n + e < g.N) pp[e] = from_f32<T>(v[e]);
-            }
-          }
-#pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = act_forward(ACT, v[e], g.param);
-        }
-        T* cp = C + (int64_t)m * g.ldc + n;
-        if (full) store_f32<T, 4>(cp, v);
-        else {
+      for (int rg = 0; rg < 4; ++rg) {
+        const int nl = wn * 128 + j * 32 + rg * 8 + frag_half * 4;
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (g.bias) {
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            if (n + e < g.N) cp[e] = from_f32<T>(v[e]);
+            if (n0 + nl + e < g.N) bv[e] = load_scalar_f32(g.bias, g.bias_dt, n0 + nl + e);
         }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            v[e] = acc[i][j][rg * 4 + e] + bv[e];
+            if (ACT != AT_ACT_NONE && !is_pre) v[e] = act_forward(ACT, v[e], g.param);
+          }
+          const int ml = wm * 128 + i * 32 + frag_row;
+          store_f32<T, 4>(reinterpret_cast<T*>(lds + ml * kEpiPitch) + nl, v);
+        }
+      }
+    __syncthreads();
+    // 256 lanes: 8 rows per sweep, 32 lanes x 16 bytes per row
+    const int rsub = threadIdx.x >> 5, cseg = (threadIdx.x & 31) * 8;
+#pragma unroll 4
+    for (int r0 = 0; r0 < BM; r0 += 8) {
+      const int ml = r0 + rsub;
+      const int m = m0 + ml;
+      if (m >= g.M) continue;
+      const uint4 v = *reinterpret_cast<const uint4*>(lds + ml * kEpiPitch + cseg * 2);
+      T* out = dst + (int64_t)m * ldd + n0 + cseg;
+      if (rows16) {
+        *reinterpret_cast<uint4*>(out) = v;
+      } else {
+        union { uint4 raw; T e[8]; } u;
+        u.raw = v;
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (n0 + cseg + e < g.N) out[e] = u.e[e];
       }
     }
   }
@@ -333,32 +430,65 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(SimpleArgs g) {
 }
 
 // ------------------------------------------------------------------------------------------
-// Elementwise activation backward with fused column sum (bias gradient).
-//   dz = dy * act'(z);  bias partials: one fp32 row per workgroup row-slice.
+// Elementwise activation backward, optionally with the bias gradient fused in:
+//   dz = dy * act'(z);  part[slice, n] = sum over the rows of the slice of dz (rounded as stored).
+// grid = (column groups of 256 * 8, row slices); each lane owns 8 consecutive columns and walks
+// the rows of its slice, so the column sums need no cross-lane traffic.
 // ------------------------------------------------------------------------------------------
-template <typename TDY, typename TZ>
+template <typename TDY, typename TZ, bool VEC_OK>
 __global__ __launch_bounds__(256) void act_bwd_kernel(
-    const TDY* __restrict__ dy, const TZ* __restrict__ z, TZ* __restrict__ dz, int64_t M, int N,
-    int64_t dys, int64_t zs, int64_t dzs, int act, float param, int vec_ok) {
+    const TDY* __restrict__ dy, const TZ* __restrict__ z, TZ* __restrict__ dz, float* __restrict__ part,
+    int64_t M, int N, int64_t dys, int64_t zs, int64_t dzs, int act, float param, int64_t rows_per_slice) {
   constexpr int VEC = 8;
-  const int64_t chunks_per_row = (N + VEC - 1) / VEC;
-  const int64_t total = M * chunks_per_row;
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-    const int64_t r = i / chunks_per_row;
-    const int c = (int)(i - r * chunks_per_row) * VEC;
-    if (vec_ok) {
-      float d[VEC], zz[VEC];
-      load_f32<TDY, VEC>(dy + r * dys + c, d);
-      load_f32<TZ, VEC>(z + r * zs + c, zz);
+  const int c = (blockIdx.x * 256 + threadIdx.x) * VEC;
+  if (c >= N) return;
+  const int64_t r0 = (int64_t)blockIdx.y * rows_per_slice;
+  const int64_t r1 = r0 + rows_per_slice < M ? r0 + rows_per_slice : M;
+  float sum[VEC];
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) d[j] *= act_derivative(act, zz[j], param);
-      store_f32<TZ, VEC>(dz + r * dzs + c, d);
-    } else {
-      for (int j = 0; j < VEC && c + j < N; ++j)
-        dz[r * dzs + c + j] =
-            from_f32<TZ>(to_f32(dy[r * dys + c + j]) * act_derivative(act, to_f32(z[r * zs + c + j]), param));
+  for (int j = 0; j < VEC; ++j) sum[j] = 0.f;
+  constexpr int ROWS = 4;  // rows in flight per lane
+  for (int64_t rb = r0; rb < r1; rb += ROWS) {
+    float d[ROWS][VEC], zz[ROWS][VEC];
+#pragma unroll
+    for (int u = 0; u < ROWS; ++u) {
+      const int64_t r = rb + u;
+      if (r < r1) {
+        if (VEC_OK) {
+          load_f32<TDY, VEC>(dy + r * dys + c, d[u]);
+          load_f32<TZ, VEC>(z + r * zs + c, zz[u]);
+        } else {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) {
+            const bool ok = c + j < N;
+            d[u][j] = ok ? to_f32(dy[r * dys + c + j]) : 0.f;
+            zz[u][j] = ok ? to_f32(z[r * zs + c + j]) : 0.f;
+          }
+        }
+      }
     }
+#pragma unroll
+    for (int u = 0; u < ROWS; ++u) {
+      const int64_t r = rb + u;
+      if (r < r1) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          d[u][j] = to_f32(from_f32<TZ>(d[u][j] * act_derivative(act, zz[u][j], param)));  // summed as stored
+          sum[j] += d[u][j];
+        }
+        if (VEC_OK) store_f32<TZ, VEC>(dz + r * dzs + c, d[u]);
+        else {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j)
+            if (c + j < N) dz[r * dzs + c + j] = from_f32<TZ>(d[u][j]);
+        }
+      }
+    }
+  }
+  if (part) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+      if (c + j < N) part[(int64_t)blockIdx.y * N + c + j] = sum[j];
   }
 }
 
@@ -416,6 +546,9 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
               (ldb % 8) == 0 && (K % 8) == 0;
   if (!a_contig_k) fast = fast && (M % 8) == 0;
   if (!b_contig_k) fast = fast && (N % 8) == 0;
+  // buffer descriptors address each operand with 32-bit byte offsets below 2 GiB
+  const int64_t a_bytes = (a_contig_k ? M : K) * lda * 2, b_bytes = (b_contig_k ? N : K) * ldb * 2;
+  if (a_bytes >= ((int64_t)1 << 31) || b_bytes >= ((int64_t)1 << 31)) fast = false;
   // Small problems do not fill 256x256 tiles; the generic kernel has finer tiles.
   if (M * N < (int64_t)BM * BN / 2 || M < 64 || N < 64) fast = false;
 
@@ -434,14 +567,17 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
         } else {
           switch (act) {
 #define AT_FWD_CASE(ID) case ID: hipLaunchKernelGGL((gemm_mfma16_kernel<T, false, false, ID>), dim3(grid), dim3(kGemmThreads), 0, stream, g); break;
-            AT_FWD_CASE(AT_ACT_NONE) AT_FWD_CASE(AT_ACT_SIGMOID) AT_FWD_CASE(AT_ACT_LOGSIGMOID)
-            AT_FWD_CASE(AT_ACT_TANH) AT_FWD_CASE(AT_ACT_RELU) AT_FWD_CASE(AT_ACT_GELU)
-            AT_FWD_CASE(AT_ACT_GELUAPPROX) AT_FWD_CASE(AT_ACT_SILU) AT_FWD_CASE(AT_ACT_RELU6)
+            AT_FWD_CASE(AT_ACT_NONE) AT_FWD_CASE(AT_ACT_RELU) AT_FWD_CASE(AT_ACT_GELUAPPROX)
+#ifndef AT_QUICK_BUILD  // development builds instantiate three epilogues only
+            AT_FWD_CASE(AT_ACT_SIGMOID) AT_FWD_CASE(AT_ACT_LOGSIGMOID)
+            AT_FWD_CASE(AT_ACT_TANH) AT_FWD_CASE(AT_ACT_GELU)
+            AT_FWD_CASE(AT_ACT_SILU) AT_FWD_CASE(AT_ACT_RELU6)
             AT_FWD_CASE(AT_ACT_HARDSIGMOID) AT_FWD_CASE(AT_ACT_HARDTANH) AT_FWD_CASE(AT_ACT_HARDSWISH)
             AT_FWD_CASE(AT_ACT_SELU) AT_FWD_CASE(AT_ACT_MISH) AT_FWD_CASE(AT_ACT_SOFTPLUS)
             AT_FWD_CASE(AT_ACT_SOFTSIGN) AT_FWD_CASE(AT_ACT_TANHSHRINK) AT_FWD_CASE(AT_ACT_LEAKY_RELU)
             AT_FWD_CASE(AT_ACT_ELU) AT_FWD_CASE(AT_ACT_CELU) AT_FWD_CASE(AT_ACT_HARDSHRINK)
             AT_FWD_CASE(AT_ACT_SOFTSHRINK)
+#endif
 #undef AT_FWD_CASE
             default: return AT_ERR_ACT;
           }
@@ -466,6 +602,7 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
 }
 
 constexpr int kColsumSlices = 64;
+constexpr int kActBwdMaxSlices = 512;
 
 }  // namespace
 }  // namespace at_hip
@@ -501,33 +638,54 @@ int at_linear_bwd_weight(const void* input, const void* pre_act_grad, void* weig
                   (hipStream_t)stream);
 }
 
-int at_act_bwd(const void* output_grad, const void* input, void* input_grad, int64_t rows, int64_t cols,
-               int64_t output_grad_stride, int64_t input_stride, int64_t input_grad_stride, int act,
-               float param, int grad_dtype, int input_dtype, at_stream_t stream) {
+int64_t at_act_bwd_workspace_bytes(int64_t rows, int64_t cols) {
+  if (rows <= 0 || cols <= 0) return 0;
+  return (int64_t)kActBwdMaxSlices * cols * (int64_t)sizeof(float);
+}
+
+int at_act_bwd(const void* output_grad, const void* input, void* input_grad, void* bias_grad, void* workspace,
+               int64_t workspace_bytes, int64_t rows, int64_t cols, int64_t output_grad_stride,
+               int64_t input_stride, int64_t input_grad_stride, int act, float param, int grad_dtype,
+               int input_dtype, int bias_grad_dtype, at_stream_t stream) {
   if (!output_grad || !input || !input_grad) return AT_ERR_NULL;
-  if (!dtype_valid(grad_dtype) || !dtype_valid(input_dtype)) return AT_ERR_DTYPE;
+  if (!dtype_valid(grad_dtype) || !dtype_valid(input_dtype) || (bias_grad && !dtype_valid(bias_grad_dtype)))
+    return AT_ERR_DTYPE;
   if (!act_valid(act) || act == AT_ACT_NONE) return AT_ERR_ACT;
   if (rows < 0 || cols <= 0 || cols > INT32_MAX) return AT_ERR_DIM;
   if (output_grad_stride < cols || input_stride < cols || input_grad_stride < cols) return AT_ERR_DIM;
-  if (rows == 0) return AT_OK;
+  if (bias_grad && (!workspace || workspace_bytes < at_act_bwd_workspace_bytes(rows, cols))) return AT_ERR_WORKSPACE;
+  if (rows == 0) return bias_grad ? AT_ERR_DIM : AT_OK;
   const int gs = dtype_size(grad_dtype), is = dtype_size(input_dtype);
-  const int vec_ok = cols % 8 == 0 && aligned16(output_grad) && aligned16(input) && aligned16(input_grad) &&
-                     (output_grad_stride * gs) % 16 == 0 && (input_stride * is) % 16 == 0 &&
-                     (input_grad_stride * is) % 16 == 0;
-  const int64_t chunks = rows * cdiv64(cols, 8);
-  int64_t blocks = cdiv64(chunks, 256);
-  const int64_t cap = (int64_t)device_cu_count() * 16;
-  if (blocks > cap) blocks = cap;
-  return dispatch_dtype(grad_dtype, [&](auto* tg) -> int {
+  const bool vec_ok = cols % 8 == 0 && aligned16(output_grad) && aligned16(input) && aligned16(input_grad) &&
+                      (output_grad_stride * gs) % 16 == 0 && (input_stride * is) % 16 == 0 &&
+                      (input_grad_stride * is) % 16 == 0;
+  // enough workgroups to fill the chip, few enough row slices to keep the partial buffer small
+  const unsigned gx = (unsigned)cdiv64(cols, 256 * 8);
+  int64_t slices = cdiv64((int64_t)device_cu_count() * 16, gx);
+  if (slices > kActBwdMaxSlices) slices = kActBwdMaxSlices;
+  if (slices > rows) slices = rows;
+  const int64_t rows_per_slice = cdiv64(rows, slices);
+  slices = cdiv64(rows, rows_per_slice);
+  float* part = bias_grad ? (float*)workspace : nullptr;
+  int rc = dispatch_dtype(grad_dtype, [&](auto* tg) -> int {
     typedef std::remove_pointer_t<decltype(tg)> TG;
     return dispatch_dtype(input_dtype, [&](auto* tz) -> int {
       typedef std::remove_pointer_t<decltype(tz)> TZ;
-      hipLaunchKernelGGL((act_bwd_kernel<TG, TZ>), dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                         (const TG*)output_grad, (const TZ*)input, (TZ*)input_grad, rows, (int)cols,
-                         output_grad_stride, input_stride, input_grad_stride, act, param, vec_ok);
+      if (vec_ok)
+        hipLaunchKernelGGL((act_bwd_kernel<TG, TZ, true>), dim3(gx, (unsigned)slices), dim3(256), 0,
+                           (hipStream_t)stream, (const TG*)output_grad, (const TZ*)input, (TZ*)input_grad, part, rows,
+                           (int)cols, output_grad_stride, input_stride, input_grad_stride, act, param, rows_per_slice);
+      else
+        hipLaunchKernelGGL((act_bwd_kernel<TG, TZ, false>), dim3(gx, (unsigned)slices), dim3(256), 0,
+                           (hipStream_t)stream, (const TG*)output_grad, (const TZ*)input, (TZ*)input_grad, part, rows,
+                           (int)cols, output_grad_stride, input_stride, input_grad_stride, act, param, rows_per_slice);
       return launch_status();
     });
   });
+  if (rc || !bias_grad) return rc;
+  hipLaunchKernelGGL(colsum_final_kernel, dim3((unsigned)cdiv64(cols, 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const float*)workspace, bias_grad, bias_grad_dtype, (int)slices, (int)cols);
+  return launch_status();
 }
 
 int64_t at_colsum_workspace_bytes(int64_t rows, int64_t cols) {

@@ -134,22 +134,31 @@ class LinearAutoGrad(torch.autograd.Function):
         stream = _lib.stream_of(input)
 
         with torch.cuda.device_of(input):
+            bias_grad = None
             if ctx.act_func is None:
                 pre_act_grad = output_grad
             else:
                 pre_act_grad = torch.empty((batch_dim, out_feat_dim), dtype=pre_act.dtype,
                                            device=device)
+                # the bias gradient (column sums of pre_act_grad) comes out of the same pass
+                fuse_bias = ctx.bias_requires_grad and batch_dim > 0
+                workspace = workspace_bytes = None
+                if fuse_bias:
+                    bias_grad = torch.empty(out_feat_dim, dtype=pre_act.dtype, device=device)
+                    workspace_bytes = lib.at_act_bwd_workspace_bytes(batch_dim, out_feat_dim)
+                    workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=device)
                 _lib.check(lib.at_act_bwd(
                     _lib.ptr(output_grad), _lib.ptr(pre_act), _lib.ptr(pre_act_grad),
+                    _lib.ptr(bias_grad), _lib.ptr(workspace), workspace_bytes or 0,
                     batch_dim, out_feat_dim, output_grad.stride(0), pre_act.stride(0),
                     pre_act_grad.stride(0), ctx.act, 0.0 if ctx.param is None else ctx.param,
-                    _lib.dtype_id(output_grad.dtype), _lib.dtype_id(pre_act.dtype), stream),
-                    'at_act_bwd')
+                    _lib.dtype_id(output_grad.dtype), _lib.dtype_id(pre_act.dtype),
+                    _lib.dtype_id(pre_act.dtype), stream), 'at_act_bwd')
 
             # The products run in the output dtype, as under the reference's
             # torch.autocast(dtype=output_dtype) block (linear_layer.py:152-155).
             grad_mm = _matrix(pre_act_grad.to(output_dtype))
-            input_grad = weight_grad = bias_grad = None
+            input_grad = weight_grad = None
             if input.requires_grad:
                 weight_mm = _matrix(weight.to(output_dtype))
                 input_grad = torch.empty((batch_dim, in_feat_dim), dtype=output_dtype, device=device)
@@ -171,7 +180,7 @@ class LinearAutoGrad(torch.autograd.Function):
                         in_feat_dim, out_feat_dim, input_mm.stride(0), grad_mm.stride(0),
                         weight_grad.stride(0), _lib.dtype_id(output_dtype),
                         _lib.dtype_id(output_dtype), stream), 'at_linear_bwd_weight')
-            if ctx.bias_requires_grad:
+            if ctx.bias_requires_grad and bias_grad is None:
                 bias_grad = torch.empty(out_feat_dim, dtype=pre_act_grad.dtype, device=device)
                 if batch_dim == 0:
                     bias_grad.zero_()

@@ -167,9 +167,12 @@ def bench_linear(cfg: str, steps: int, warmup: int, with_cpu: bool) -> Dict:
         raw.check(lib.at_linear_fwd(xd.data_ptr(), wd.data_ptr(), bd.data_ptr(), pre.data_ptr(), y.data_ptr(),
                                     m, k, n, k, n, n, n, aid, 0.0, dt, dt, dt, st()), 'fwd')
 
+    awsb = lib.at_act_bwd_workspace_bytes(m, n)
+    aws = torch.empty(awsb, dtype=torch.uint8, device='cuda')
+
     def k_act():
-        raw.check(lib.at_act_bwd(dyd.data_ptr(), pre.data_ptr(), dz.data_ptr(), m, n, n, n, n, aid, 0.0, dt, dt,
-                                 st()), 'act_bwd')
+        raw.check(lib.at_act_bwd(dyd.data_ptr(), pre.data_ptr(), dz.data_ptr(), db.data_ptr(), aws.data_ptr(), awsb,
+                                 m, n, n, n, n, aid, 0.0, dt, dt, dt, st()), 'act_bwd')
 
     def k_dx():
         raw.check(lib.at_linear_bwd_input(dz.data_ptr(), wd.data_ptr(), dx.data_ptr(), m, k, n, n, n, k, dt, dt,
@@ -184,8 +187,8 @@ def bench_linear(cfg: str, steps: int, warmup: int, with_cpu: bool) -> Dict:
 
     iters = max(3, min(steps, 10))
     kernels = {}
-    for kname, fn in (('linear_fwd', k_fwd), ('act_bwd', k_act), ('linear_bwd_input', k_dx),
-                      ('linear_bwd_weight', k_dw), ('colsum', k_db)):
+    for kname, fn in (('linear_fwd', k_fwd), ('act_bwd_with_bias_grad', k_act), ('linear_bwd_input', k_dx),
+                      ('linear_bwd_weight', k_dw), ('colsum_unfused', k_db)):
         kernels[kname] = gpu_time_ms(fn, iters)
     gemm_flop = 2.0 * m * k * n
     fwd_tflops = gemm_flop / kernels['linear_fwd'] / 1e9

@@ -177,7 +177,9 @@ int at_cross_entropy_scale_grad(void* dlogits, const void* output_grad, int64_t 
  *   bwd_input:  input_grad[batch, in_feat]   = pre_act_grad[batch, out_feat] @ weight^T
  *   bwd_weight: weight_grad[in_feat, out_feat] = input^T @ pre_act_grad
  *   act_bwd:    input_grad = output_grad * act'(input) over a [rows, cols] matrix (a flat
- *               tensor is rows = 1); input_grad has input's dtype (linear_layer.py:138).
+ *               tensor is rows = 1); input_grad has input's dtype (linear_layer.py:138).  When
+ *               bias_grad is non-null the column sums of input_grad (linear_layer.py:156) come
+ *               out of the same pass; that needs at_act_bwd_workspace_bytes(rows, cols) bytes.
  *   colsum:     out[cols] = sum over rows (bias gradient, linear_layer.py:156); workspace of
  *               at_colsum_workspace_bytes(rows, cols) bytes; fixed summation order.
  * 16-bit operands whose pointers and strides are 16-byte aligned (and K, plus the contiguous
@@ -200,9 +202,12 @@ int at_linear_bwd_weight(const void* input, const void* pre_act_grad, void* weig
                          int64_t grad_stride, int64_t weight_grad_stride, int in_dtype,
                          int out_dtype, at_stream_t stream);
 
-int at_act_bwd(const void* output_grad, const void* input, void* input_grad, int64_t rows,
-               int64_t cols, int64_t output_grad_stride, int64_t input_stride,
-               int64_t input_grad_stride, int act, float param, int grad_dtype, int input_dtype,
+int64_t at_act_bwd_workspace_bytes(int64_t rows, int64_t cols);
+
+int at_act_bwd(const void* output_grad, const void* input, void* input_grad, void* bias_grad,
+               void* workspace, int64_t workspace_bytes, int64_t rows, int64_t cols,
+               int64_t output_grad_stride, int64_t input_stride, int64_t input_grad_stride, int act,
+               float param, int grad_dtype, int input_dtype, int bias_grad_dtype,
                at_stream_t stream);
 
 int64_t at_colsum_workspace_bytes(int64_t rows, int64_t cols);

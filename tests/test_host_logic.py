@@ -63,7 +63,8 @@ def test_argument_errors_without_gpu() -> None:
     assert lib.at_layer_norm_fwd(p, None, None, None, None, p, 4, 0, 8, 8, 1e-5, 0, 0, 0, None) == -2
     assert lib.at_softmax_fwd(p, p, 4, 8, 4, 8, 0, 0, 0, 0, None) == -2
     assert lib.at_linear_fwd(p, p, None, None, p, 4, 8, 8, 8, 8, 8, 8, 99, 0.0, 0, 0, 0, None) == -4
-    assert lib.at_act_bwd(p, p, p, 4, 8, 8, 8, 8, 0, 0.0, 0, 0, None) == -4
+    assert lib.at_act_bwd(p, p, p, None, None, 0, 4, 8, 8, 8, 8, 0, 0.0, 0, 0, 0, None) == -4
+    assert lib.at_act_bwd(p, p, p, p, None, 0, 4, 8, 8, 8, 8, 4, 0.0, 0, 0, 0, None) == -5
     # missing / short workspace
     assert lib.at_cross_entropy_fwd_bwd(p, p, None, p, None, None, 0, 4, 8, 8, 8, -100, 0, 0, 0, None) == -5
     assert lib.at_layer_norm_bwd(p, p, p, p, p, p, p, None, p, 16, 4, 8, 8, 8, 8, 0, 0, 0, 0, None) == -5
