@@ -84,6 +84,11 @@ __global__ __launch_bounds__(kCeBlock, 4) void ce_row_kernel(
     return;
   }
 
+  // Vectors per lane that this row really uses; uniform, so the unrolled sweeps below skip the
+  // rest of the cache with scalar branches.
+  const int n_iter = (n_int + kCeBlock - 1) / kCeBlock;
+  constexpr float kLog2e = 1.4426950408889634f;
+
   uint4 cache[CACHE_VECS];
 #pragma unroll
   for (int i = 0; i < CACHE_VECS; ++i) {
@@ -96,10 +101,12 @@ __global__ __launch_bounds__(kCeBlock, 4) void ce_row_kernel(
   float m = edge_x;
 #pragma unroll
   for (int i = 0; i < CACHE_VECS; ++i) {
-    float f[VEC];
-    unpack16<T>(cache[i], f);
+    if (i < n_iter) {
+      float f[VEC];
+      unpack16<T>(cache[i], f);
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) m = fmaxf(m, f[j]);
+      for (int j = 0; j < VEC; ++j) m = fmaxf(m, f[j]);
+    }
   }
   m = group_reduce(m, kCeBlock, scratch, MaxOp(), -INFINITY);
   // Keep the row cached as raw data: without this the compiler may keep widened fp32 copies
@@ -107,44 +114,52 @@ __global__ __launch_bounds__(kCeBlock, 4) void ce_row_kernel(
 #pragma unroll
   for (int i = 0; i < CACHE_VECS; ++i) keep_raw(cache[i]);
 
-  float s = __expf(edge_x - m);
+  // Second sweep: e = exp(x - max) replaces x in the cache (in the storage format: the gradient
+  // is rounded to it anyway), so the third sweep is a multiplication.
+  const float m2 = m * kLog2e;
+  const float edge_e = exp2f(fmaf(edge_x, kLog2e, -m2));   // exp2(-inf) = 0 without an edge
+  float s = edge_e;
 #pragma unroll
   for (int i = 0; i < CACHE_VECS; ++i) {
-    float f[VEC];
-    unpack16<T>(cache[i], f);
+    if (i < n_iter) {
+      float f[VEC];
+      unpack16<T>(cache[i], f);
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) s += __expf(f[j] - m);   // exp(-inf) = 0 for the padding
+      for (int j = 0; j < VEC; ++j) {
+        f[j] = __builtin_amdgcn_exp2f(fmaf(f[j], kLog2e, -m2));   // 0 for the -inf padding
+        s += f[j];
+      }
+      cache[i] = pack16<T>(f);
+    }
   }
   s = group_reduce(s, kCeBlock, scratch, SumOp(), 0.f);
 #pragma unroll
   for (int i = 0; i < CACHE_VECS; ++i) keep_raw(cache[i]);
 
   const float wt = weight ? load_scalar_f32(weight, wdt, t) : 1.f;
-  if (tid == 0) row_loss[row] = (__logf(s) - to_f32(xr[t]) + m) * wt;
+  const float x_t = to_f32(xr[t]);
+  if (tid == 0) row_loss[row] = (__logf(s) - x_t + m) * wt;
   if (!dr) return;
 
   const float scale = wt / denom[0];
   const float k = scale / s;
-  const int tv = (int)t - head_n;  // target position relative to the first interior element
 #pragma unroll
   for (int i = 0; i < CACHE_VECS; ++i) {
     const int v = tid + i * kCeBlock;
-    if (v < n_int) {
+    if (i < n_iter && v < n_int) {
       float f[VEC];
       unpack16<T>(cache[i], f);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        f[j] = __expf(f[j] - m) * k;
-        if (v * VEC + j == tv) f[j] -= scale;
-      }
+      for (int j = 0; j < VEC; ++j) f[j] *= k;
       dv[v] = pack16<T>(f);
     }
   }
-  if (edge >= 0) {
-    float g = __expf(edge_x - m) * k;
-    if (edge == (int)t) g -= scale;
-    dr[edge] = from_f32<T>(g);
-  }
+  if (edge >= 0) dr[edge] = from_f32<T>(edge_e * k);
+  // The target column gets softmax - 1: the lane that stored the column overwrites it (stores of
+  // one lane to one address stay in order).
+  const int tv = (int)t - head_n;   // target position relative to the first interior element
+  const bool owner = (tv >= 0 && tv < n_int * VEC) ? ((tv / VEC) % kCeBlock == tid) : (edge == (int)t);
+  if (owner) dr[t] = from_f32<T>(fmaf(__builtin_amdgcn_exp2f(fmaf(x_t, kLog2e, -m2)), k, -scale));
 }
 
 // Streaming kernel: any dtypes, any alignment, any width; the row is read twice (online

@@ -5,10 +5,13 @@
 // several waves of one workgroup for wide rows).  Each lane keeps its chunks of the row in
 // registers (ITERS chunks of VEC elements, 128-bit accesses on the vector path), so the row is
 // read from memory exactly once even though the math needs two or three sweeps.  Rows wider
-// than the register budget use the streaming instantiation (ITERS == 0), which re-reads the
-// row from cache.  Parameter gradients of the norms are accumulated per lane across a
+// than the register budget use the streaming kernels, which give a row to one workgroup and
+// re-read it from cache for every sweep.  Parameter gradients of the norms are accumulated per lane across a
 // persistent grid, reduced across the workgroup through LDS, written as one partial row per
 // workgroup and summed by a second launch in fixed order (deterministic, no atomics).
+#include <map>
+#include <mutex>
+#include <tuple>
 #include <type_traits>
 
 #include "at_common.h"
@@ -17,6 +20,50 @@ namespace at_hip {
 namespace {
 
 template <int ITERS> constexpr int cache_len() { return ITERS > 0 ? ITERS : 1; }
+
+// Makes an index opaque to the optimiser.  Parameter vectors do not depend on the row, so inside
+// a row loop the compiler would hoist their loads out of the loop and keep them (widened to
+// fp32) in registers for the whole kernel; an opaque index ties each load to its iteration.
+__device__ __forceinline__ int64_t opaque_index(int64_t i) {
+  int lo = (int)i;
+  asm volatile("" : "+v"(lo));
+  return (int64_t)lo;
+}
+
+// One chunk of a row as a lane keeps it between the sweeps of a kernel.  When the chunk is
+// exactly 128 bits of storage it stays packed (4 registers for 8 bf16 / fp16 values) and is
+// widened on use; otherwise it is kept as fp32.
+template <typename T, int VEC, bool PACKED = (sizeof(T) * VEC == 16)>
+struct Chunk;
+
+template <typename T, int VEC>
+struct Chunk<T, VEC, true> {
+  uint4 raw;
+  __device__ __forceinline__ void load(const T* p) { raw = *reinterpret_cast<const uint4*>(p); }
+  __device__ __forceinline__ void fill(float v) {
+    float f[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) f[j] = v;
+    raw = pack16<T>(f);
+  }
+  __device__ __forceinline__ void get(float (&f)[VEC]) const { unpack16<T>(raw, f); }
+  __device__ __forceinline__ void pin() { keep_raw(raw); }
+};
+
+template <typename T, int VEC>
+struct Chunk<T, VEC, false> {
+  float v[VEC];
+  __device__ __forceinline__ void load(const T* p) { load_f32<T, VEC>(p, v); }
+  __device__ __forceinline__ void fill(float x) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) v[j] = x;
+  }
+  __device__ __forceinline__ void get(float (&f)[VEC]) const {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) f[j] = v[j];
+  }
+  __device__ __forceinline__ void pin() {}
+};
 
 struct RowPlan {
   int vec;         // elements per chunk: 8 / 4 on the vector path, 1 on the scalar path
@@ -46,110 +93,262 @@ inline RowPlan plan_rows(int64_t feat, int vec, int min_block, int wave_rows_ite
   return p;
 }
 
+// group_reduce at the cost of one workgroup barrier instead of two: the slot row alternates with
+// `parity`, which the caller flips after every call.  A wave writes a slot row again only after
+// the barrier of the call in between, which every wave reaches after its reads of that row.
+template <typename Op>
+__device__ __forceinline__ float group_reduce_alt(float v, int group, float (*slots)[16], int& parity,
+                                                  Op op, float identity) {
+  if (group <= kWave) return wave_reduce(v, group, op);
+  v = wave_reduce(v, kWave, op);
+  const int wave = threadIdx.x / kWave;
+  const int waves_per_group = group / kWave;
+  if ((threadIdx.x & (kWave - 1)) == 0) slots[parity][wave] = v;
+  __syncthreads();
+  const int first = (wave / waves_per_group) * waves_per_group;
+  float r = identity;
+  for (int i = 0; i < waves_per_group; ++i) r = op(r, slots[parity][first + i]);
+  parity ^= 1;
+  return r;
+}
+
+// Sums two values over the group at the cost of one workgroup barrier.  `slots` alternates with
+// `parity` from call to call: a wave can only write a slot again after passing the barrier of
+// the call in between, which every wave reaches only after its reads of that slot.
+__device__ __forceinline__ void group_sum2(float& a, float& b, int group, float (*slots)[16][2],
+                                           int parity) {
+  a = wave_reduce(a, group < kWave ? group : kWave, SumOp());
+  b = wave_reduce(b, group < kWave ? group : kWave, SumOp());
+  if (group <= kWave) return;
+  const int wave = threadIdx.x / kWave;
+  const int waves_per_group = group / kWave;
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+    slots[parity][wave][0] = a;
+    slots[parity][wave][1] = b;
+  }
+  __syncthreads();
+  const int first = (wave / waves_per_group) * waves_per_group;
+  a = 0.f;
+  b = 0.f;
+  for (int i = 0; i < waves_per_group; ++i) {
+    a += slots[parity][first + i][0];
+    b += slots[parity][first + i][1];
+  }
+}
+
+// The chunks one lane holds of one row of one tensor: ITERS chunks, `group` lanes apart.
+template <typename T, int VEC, int ITERS>
+struct RowCache {
+  Chunk<T, VEC> ch[ITERS];
+  // Issues the loads of this lane's chunks of `row`.  Nothing is read for an invalid row or past
+  // the end of the row; those chunks hold `pad`.
+  __device__ __forceinline__ void load(const T* __restrict__ base, int64_t row, int64_t stride,
+                                       bool valid, int lane, int group, int chunks, float pad) {
+    const T* r = base + (valid ? row : 0) * stride;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int c = lane + it * group;
+      if (valid && c < chunks) ch[it].load(r + (int64_t)c * VEC);
+      else ch[it].fill(pad);
+    }
+  }
+  __device__ __forceinline__ void pin() {
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) ch[it].pin();
+  }
+};
+
+// The register-cached kernels below are persistent: the grid is sized to what the machine keeps
+// resident and every workgroup walks its row-blocks with a grid stride.  A row must be complete
+// before any of its output can be written, so a wave that handled one row at a time would
+// alternate between waiting on reads and issuing writes; instead the loads of the next row-block
+// are issued before the current one is reduced and written, which keeps reads and writes of
+// different rows in flight together.  Memory operations retire in order per wave, so nothing
+// that the current row waits on may be issued after the prefetch: parameters are held in
+// registers (packed) and per-row statistics travel with the prefetch.
+
 // ------------------------------------------------------------------------------------------
 // Norm forward.  LAYER = true: LayerNorm (mean subtracted, optional bias); false: RMSNorm.
 // ------------------------------------------------------------------------------------------
-template <bool LAYER, typename TX, typename TY, int VEC, int ITERS>
-__global__ __launch_bounds__(1024) void norm_fwd_kernel(
-    const TX* __restrict__ x, const void* __restrict__ w, const void* __restrict__ b,
+template <bool LAYER, typename TX, typename TY, typename TW, int VEC, int ITERS>
+__global__ __launch_bounds__(512) void norm_fwd_kernel(
+    const TX* __restrict__ x, const TW* __restrict__ w, const TW* __restrict__ b,
     float* __restrict__ mean_out, float* __restrict__ rstd_out, TY* __restrict__ y,
-    int64_t batch, int feat, int64_t xs, int64_t ys, float eps, int wdt, int group_log2) {
-  __shared__ float scratch[16];
+    int64_t batch, int feat, int64_t xs, int64_t ys, float eps, int group_log2) {
+  static_assert(ITERS > 0, "rows are cached in registers");
+  // parameters stay in registers when a chunk of them is one 128-bit word
+  constexpr bool HOIST = sizeof(TW) * VEC == 16;
+  __shared__ float slots[2][16];
+  int parity = 0;
   const int group = 1 << group_log2;
   const int lane = threadIdx.x & (group - 1);
-  const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> group_log2) + (threadIdx.x >> group_log2);
-  const bool valid = row < batch;
+  const int rpb = blockDim.x >> group_log2;
+  const int rib = threadIdx.x >> group_log2;
   const int chunks = feat / VEC;
-  const int n_it = ITERS > 0 ? ITERS : (chunks + group - 1) / group;
-  const TX* xr = x + (valid ? row : 0) * xs;
-  float cache[cache_len<ITERS>()][VEC];
   const float inv_feat = 1.0f / (float)feat;
+  const int64_t row_blocks = (batch + rpb - 1) / rpb;
+  const int64_t row_step = (int64_t)gridDim.x * rpb;
 
-  float mean = 0.f;
-  if (LAYER) {
-    float s = 0.f;
+  Chunk<TW, VEC> pw[HOIST ? ITERS : 1], pb[(HOIST && LAYER) ? ITERS : 1];
+  if (HOIST) {
 #pragma unroll
-    for (int it = 0; it < n_it; ++it) {
+    for (int it = 0; it < ITERS; ++it) {
       const int c = lane + it * group;
-      float v[VEC];
-      if (valid && c < chunks) load_f32<TX, VEC>(xr + (int64_t)c * VEC, v);
-      else {
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) v[j] = 0.f;
-      }
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        s += v[j];
-        if (ITERS > 0) cache[ITERS > 0 ? it : 0][j] = v[j];
+      if (w && c < chunks) pw[HOIST ? it : 0].load(w + (int64_t)c * VEC);
+      else pw[HOIST ? it : 0].fill(1.f);
+      if (LAYER) {
+        if (w && b && c < chunks) pb[(HOIST && LAYER) ? it : 0].load(b + (int64_t)c * VEC);
+        else pb[(HOIST && LAYER) ? it : 0].fill(0.f);
       }
     }
-    mean = group_reduce(s, group, scratch, SumOp(), 0.f) * inv_feat;
   }
 
-  float ss = 0.f;
+  RowCache<TX, VEC, ITERS> cur, nxt;
+  {
+    const int64_t row0 = (int64_t)blockIdx.x * rpb + rib;
+    cur.load(x, row0, xs, row0 < batch, lane, group, chunks, 0.f);
+  }
+#pragma unroll 1
+  for (int64_t rb = blockIdx.x; rb < row_blocks; rb += gridDim.x) {
+    const int64_t row = rb * rpb + rib;
+    const bool valid = row < batch;
+    nxt.load(x, row + row_step, xs, row + row_step < batch, lane, group, chunks, 0.f);
+    if (HOIST) {   // opaque per iteration: otherwise their widening to fp32 is hoisted out of the loop
 #pragma unroll
-  for (int it = 0; it < n_it; ++it) {
-    const int c = lane + it * group;
-    float v[VEC];
-    if (ITERS > 0 && LAYER) {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) v[j] = cache[ITERS > 0 ? it : 0][j];
-    } else {
-      if (valid && c < chunks) load_f32<TX, VEC>(xr + (int64_t)c * VEC, v);
-      else {
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) v[j] = 0.f;
-      }
-      if (ITERS > 0) {
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) cache[ITERS > 0 ? it : 0][j] = v[j];
+      for (int it = 0; it < ITERS; ++it) {
+        pw[HOIST ? it : 0].pin();
+        if (LAYER) pb[(HOIST && LAYER) ? it : 0].pin();
       }
     }
-    if (c < chunks) {
+    __builtin_amdgcn_sched_barrier(0);
+
+    float s = 0.f;
+    if (LAYER) {
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        const float d = v[j] - mean;
-        ss += d * d;
+      for (int it = 0; it < ITERS; ++it) {
+        float v[VEC];
+        cur.ch[it].get(v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) s += v[j];
       }
+    }
+    const float mean = LAYER ? group_reduce_alt(s, group, slots, parity, SumOp(), 0.f) * inv_feat : 0.f;
+    if (LAYER) cur.pin();   // re-widen per sweep instead of keeping the row as fp32
+
+    float ss = 0.f;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int c = lane + it * group;
+      if (!LAYER || c < chunks) {   // padding is zero: harmless without a mean
+        float v[VEC];
+        cur.ch[it].get(v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float d = v[j] - mean;
+          ss += d * d;
+        }
+      }
+    }
+    ss = group_reduce_alt(ss, group, slots, parity, SumOp(), 0.f);
+    const float rstd = rsqrtf(ss * inv_feat + eps);
+    cur.pin();
+
+    if (valid && lane == 0) {
+      if (LAYER && mean_out) mean_out[row] = mean;
+      if (rstd_out) rstd_out[row] = rstd;
+    }
+    if (valid) {
+      TY* yr = y + row * ys;
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const int c = lane + it * group;
+        if (c < chunks) {
+          float v[VEC];
+          cur.ch[it].get(v);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) v[j] = (v[j] - mean) * rstd;
+          if (w) {
+            float wv[VEC];
+            if (HOIST) pw[HOIST ? it : 0].get(wv);
+            else load_f32<TW, VEC>(w + opaque_index((int64_t)c * VEC), wv);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] *= wv[j];
+            if (LAYER && b) {
+              float bv[VEC];
+              if (HOIST) pb[(HOIST && LAYER) ? it : 0].get(bv);
+              else load_f32<TW, VEC>(b + opaque_index((int64_t)c * VEC), bv);
+#pragma unroll
+              for (int j = 0; j < VEC; ++j) v[j] += bv[j];
+            }
+          }
+          store_f32<TY, VEC>(yr + (int64_t)c * VEC, v);
+        }
+      }
+    }
+    cur = nxt;
+    cur.pin();
+  }
+}
+
+// Streaming forward for rows too wide for the register cache: one row per workgroup, the row is
+// re-read (from cache) for each sweep.
+template <bool LAYER, typename TX, typename TY, int VEC>
+__global__ __launch_bounds__(1024) void norm_fwd_stream_kernel(
+    const TX* __restrict__ x, const void* __restrict__ w, const void* __restrict__ b,
+    float* __restrict__ mean_out, float* __restrict__ rstd_out, TY* __restrict__ y, int feat,
+    int64_t xs, int64_t ys, float eps, int wdt) {
+  __shared__ float scratch[16];
+  const int group = blockDim.x;
+  const int lane = threadIdx.x;
+  const int64_t row = blockIdx.x;
+  const int chunks = feat / VEC;
+  const float inv_feat = 1.0f / (float)feat;
+  const TX* xr = x + row * xs;
+  TY* yr = y + row * ys;
+  float s = 0.f;
+  if (LAYER) {
+    for (int c = lane; c < chunks; c += group) {
+      float v[VEC];
+      load_f32<TX, VEC>(xr + (int64_t)c * VEC, v);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) s += v[j];
+    }
+  }
+  const float mean = LAYER ? group_reduce(s, group, scratch, SumOp(), 0.f) * inv_feat : 0.f;
+  float ss = 0.f;
+  for (int c = lane; c < chunks; c += group) {
+    float v[VEC];
+    load_f32<TX, VEC>(xr + (int64_t)c * VEC, v);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const float d = v[j] - mean;
+      ss += d * d;
     }
   }
   ss = group_reduce(ss, group, scratch, SumOp(), 0.f);
   const float rstd = rsqrtf(ss * inv_feat + eps);
-
-  if (valid && lane == 0) {
+  if (lane == 0) {
     if (LAYER && mean_out) mean_out[row] = mean;
     if (rstd_out) rstd_out[row] = rstd;
   }
-  if (!valid) return;
-
-  TY* yr = y + row * ys;
+  for (int c = lane; c < chunks; c += group) {
+    float v[VEC];
+    load_f32<TX, VEC>(xr + (int64_t)c * VEC, v);
 #pragma unroll
-  for (int it = 0; it < n_it; ++it) {
-    const int c = lane + it * group;
-    if (c < chunks) {
-      float v[VEC];
-      if (ITERS > 0) {
+    for (int j = 0; j < VEC; ++j) v[j] = (v[j] - mean) * rstd;
+    if (w) {
+      float wv[VEC];
+      load_param_f32<VEC>(w, wdt, (int64_t)c * VEC, wv);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) v[j] = cache[ITERS > 0 ? it : 0][j];
-      } else {
-        load_f32<TX, VEC>(xr + (int64_t)c * VEC, v);
+      for (int j = 0; j < VEC; ++j) v[j] *= wv[j];
+      if (LAYER && b) {
+        float bv[VEC];
+        load_param_f32<VEC>(b, wdt, (int64_t)c * VEC, bv);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] += bv[j];
       }
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) v[j] = (v[j] - mean) * rstd;
-      if (w) {
-        float wv[VEC];
-        load_param_f32<VEC>(w, wdt, (int64_t)c * VEC, wv);
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) v[j] *= wv[j];
-        if (LAYER && b) {
-          float bv[VEC];
-          load_param_f32<VEC>(b, wdt, (int64_t)c * VEC, bv);
-#pragma unroll
-          for (int j = 0; j < VEC; ++j) v[j] += bv[j];
-        }
-      }
-      store_f32<TY, VEC>(yr + (int64_t)c * VEC, v);
     }
+    store_f32<TY, VEC>(yr + (int64_t)c * VEC, v);
   }
 }
 
@@ -159,14 +358,18 @@ __global__ __launch_bounds__(1024) void norm_fwd_kernel(
 //   part_w / part_b: [gridDim.x, feat] fp32 partial rows (null when not wanted).
 // Dynamic LDS: blockDim.x * VEC floats (only used when a workgroup holds several rows).
 // ------------------------------------------------------------------------------------------
-template <bool LAYER, typename TDY, typename TX, typename TDX, int VEC, int ITERS>
+template <bool LAYER, typename TDY, typename TX, typename TDX, typename TW, int VEC, int ITERS>
 __global__ __launch_bounds__(512) void norm_bwd_kernel(
     const TDY* __restrict__ dy, const TX* __restrict__ x, const float* __restrict__ mean_in,
-    const float* __restrict__ rstd_in, const void* __restrict__ w, TDX* __restrict__ dx,
+    const float* __restrict__ rstd_in, const TW* __restrict__ w, TDX* __restrict__ dx,
     float* __restrict__ part_w, float* __restrict__ part_b, int64_t batch, int feat,
-    int64_t dys, int64_t xs, int64_t dxs, int wdt, int group_log2) {
-  static_assert(ITERS > 0, "the persistent backward kernel caches the row in registers");
-  __shared__ float scratch[16];
+    int64_t dys, int64_t xs, int64_t dxs, int group_log2) {
+  static_assert(ITERS > 0, "rows are cached in registers");
+  constexpr bool HOIST = sizeof(TW) * VEC == 16;
+  // With few chunks per lane the normalised input and the scaled gradient of the first sweep stay
+  // in registers as fp32 for the second; otherwise the second sweep recomputes them.
+  constexpr bool KEEP = ITERS * VEC <= 16;
+  __shared__ float slots[2][16][2];
   extern __shared__ float red[];
   const int group = 1 << group_log2;
   const int lane = threadIdx.x & (group - 1);
@@ -175,61 +378,105 @@ __global__ __launch_bounds__(512) void norm_bwd_kernel(
   const int chunks = feat / VEC;
   const float inv_feat = 1.0f / (float)feat;
   const int64_t row_blocks = (batch + rpb - 1) / rpb;
+  const int64_t row_step = (int64_t)gridDim.x * rpb;
 
-  float acc_w[ITERS][VEC], acc_b[ITERS][VEC];
-#pragma unroll
-  for (int it = 0; it < ITERS; ++it)
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) { acc_w[it][j] = 0.f; acc_b[it][j] = 0.f; }
-
-  float wv[ITERS][VEC];
+  float acc_w[ITERS][VEC], acc_b[LAYER ? ITERS : 1][VEC];
+  Chunk<TW, VEC> pw[HOIST ? ITERS : 1];
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
-    const int c = lane + it * group;
-    if (w && c < chunks) load_param_f32<VEC>(w, wdt, (int64_t)c * VEC, wv[it]);
-    else {
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) wv[it][j] = 1.f;
+    for (int j = 0; j < VEC; ++j) {
+      acc_w[it][j] = 0.f;
+      if (LAYER) acc_b[LAYER ? it : 0][j] = 0.f;
+    }
+    if (HOIST) {
+      const int c = lane + it * group;
+      if (w && c < chunks) pw[HOIST ? it : 0].load(w + (int64_t)c * VEC);
+      else pw[HOIST ? it : 0].fill(1.f);
     }
   }
 
+  // the row stays in registers in its storage format between the two sweeps
+  RowCache<TDY, VEC, ITERS> cdy, ndy;
+  RowCache<TX, VEC, ITERS> cx, nx;
+  float mean = 0.f, rstd = 0.f, nmean = 0.f, nrstd = 0.f;
+  int parity = 0;
+  {
+    const int64_t row0 = (int64_t)blockIdx.x * rpb + rib;
+    const bool v0 = row0 < batch;
+    if (v0) {
+      if (LAYER) mean = mean_in[row0];
+      rstd = rstd_in[row0];
+    }
+    cdy.load(dy, row0, dys, v0, lane, group, chunks, 0.f);
+    cx.load(x, row0, xs, v0, lane, group, chunks, 0.f);
+  }
+#pragma unroll 1
   for (int64_t rb = blockIdx.x; rb < row_blocks; rb += gridDim.x) {
     const int64_t row = rb * rpb + rib;
     const bool valid = row < batch;
-    const int64_t rr = valid ? row : 0;
-    const TDY* dyr = dy + rr * dys;
-    const TX* xr = x + rr * xs;
-    const float mean = (LAYER && valid) ? mean_in[rr] : 0.f;
-    const float rstd = valid ? rstd_in[rr] : 0.f;
+    {
+      const int64_t nrow = row + row_step;
+      const bool nv = nrow < batch;
+      nmean = 0.f;
+      nrstd = 0.f;
+      if (nv) {
+        if (LAYER) nmean = mean_in[nrow];
+        nrstd = rstd_in[nrow];
+      }
+      ndy.load(dy, nrow, dys, nv, lane, group, chunks, 0.f);
+      nx.load(x, nrow, xs, nv, lane, group, chunks, 0.f);
+    }
+    if (HOIST) {   // opaque per iteration: otherwise their widening to fp32 is hoisted out of the loop
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) pw[HOIST ? it : 0].pin();
+    }
+    __builtin_amdgcn_sched_barrier(0);
 
-    float xh[ITERS][VEC], g[ITERS][VEC];
+    // padding chunks and invalid rows hold dy = 0, so every product below vanishes for them
     float s1 = 0.f, s2 = 0.f;
+    float keep_h[KEEP ? ITERS : 1][VEC], keep_g[KEEP ? ITERS : 1][VEC];
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int c = lane + it * group;
-      float dv[VEC], xv[VEC];
-      if (valid && c < chunks) {
-        load_f32<TDY, VEC>(dyr + (int64_t)c * VEC, dv);
-        load_f32<TX, VEC>(xr + (int64_t)c * VEC, xv);
+      float dv[VEC], xv[VEC], wv[VEC];
+      cdy.ch[it].get(dv);
+      cx.ch[it].get(xv);
+      if (HOIST) pw[HOIST ? it : 0].get(wv);
+      else if (w && c < chunks) load_f32<TW, VEC>(w + opaque_index((int64_t)c * VEC), wv);
+      else {
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          const float h = (xv[j] - mean) * rstd;
-          const float gg = dv[j] * wv[it][j];
-          xh[it][j] = h;
-          g[it][j] = gg;
-          s1 += h * gg;
-          s2 += gg;
-          acc_w[it][j] += dv[j] * h;
-          acc_b[it][j] += dv[j];
-        }
-      } else {
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) { xh[it][j] = 0.f; g[it][j] = 0.f; }
+        for (int j = 0; j < VEC; ++j) wv[j] = 1.f;
       }
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float h = (xv[j] - mean) * rstd;
+        const float gg = dv[j] * wv[j];
+        s1 += h * gg;
+        s2 += gg;
+        acc_w[it][j] += dv[j] * h;
+        if (LAYER) acc_b[LAYER ? it : 0][j] += dv[j];
+        // Accumulate here and now: left alone, the compiler sinks these updates to the end of
+        // the iteration and keeps every widened operand alive until then.
+        asm volatile("" : "+v"(acc_w[it][j]));
+        if (LAYER) asm volatile("" : "+v"(acc_b[LAYER ? it : 0][j]));
+        if (KEEP) {
+          keep_h[KEEP ? it : 0][j] = h;
+          keep_g[KEEP ? it : 0][j] = gg;
+        }
+      }
+      // one chunk at a time: keeps the widened temporaries of a single chunk live, not of all
+      __builtin_amdgcn_sched_barrier(0);
     }
-    s1 = group_reduce(s1, group, scratch, SumOp(), 0.f) * inv_feat;
-    if (LAYER) s2 = group_reduce(s2, group, scratch, SumOp(), 0.f) * inv_feat;
-    else s2 = 0.f;
+    group_sum2(s1, s2, group, slots, parity);
+    parity ^= 1;
+    // the input gradient is rstd * (g - (h * s1 + s2) / feat); rstd / feat folded into the sums
+    s1 *= inv_feat * rstd;
+    s2 = LAYER ? s2 * inv_feat * rstd : 0.f;
+    if (!KEEP) {
+      cdy.pin();
+      cx.pin();
+    }
 
     if (valid) {
       TDX* dxr = dx + row * dxs;
@@ -238,12 +485,37 @@ __global__ __launch_bounds__(512) void norm_bwd_kernel(
         const int c = lane + it * group;
         if (c < chunks) {
           float o[VEC];
+          if (KEEP) {
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) o[j] = rstd * (g[it][j] - (xh[it][j] * s1 + s2));
+            for (int j = 0; j < VEC; ++j)
+              o[j] = fmaf(keep_g[KEEP ? it : 0][j], rstd, -fmaf(keep_h[KEEP ? it : 0][j], s1, s2));
+          } else {
+            float dv[VEC], xv[VEC], wv[VEC];
+            cdy.ch[it].get(dv);
+            cx.ch[it].get(xv);
+            if (HOIST) pw[HOIST ? it : 0].get(wv);
+            else if (w) load_f32<TW, VEC>(w + opaque_index((int64_t)c * VEC), wv);
+            else {
+#pragma unroll
+              for (int j = 0; j < VEC; ++j) wv[j] = 1.f;
+            }
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+              const float h = (xv[j] - mean) * rstd;
+              o[j] = fmaf(dv[j] * wv[j], rstd, -fmaf(h, s1, s2));
+            }
+          }
           store_f32<TDX, VEC>(dxr + (int64_t)c * VEC, o);
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
+    cdy = ndy;
+    cx = nx;
+    mean = nmean;
+    rstd = nrstd;
+    cdy.pin();
+    cx.pin();
   }
 
   if (!part_w && !part_b) return;
@@ -257,7 +529,7 @@ __global__ __launch_bounds__(512) void norm_bwd_kernel(
       const int c = lane + it * group;
       float v[VEC];
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) v[j] = is_w ? acc_w[it][j] : acc_b[it][j];
+      for (int j = 0; j < VEC; ++j) v[j] = (is_w || !LAYER) ? acc_w[it][j] : acc_b[LAYER ? it : 0][j];
       if (rpb > 1) {
         __syncthreads();
 #pragma unroll
@@ -303,7 +575,7 @@ __global__ __launch_bounds__(1024) void norm_bwd_stream_kernel(
     float dv[VEC], xv[VEC], wv[VEC];
     load_f32<TDY, VEC>(dyr + (int64_t)c * VEC, dv);
     load_f32<TX, VEC>(xr + (int64_t)c * VEC, xv);
-    if (w) load_param_f32<VEC>(w, wdt, (int64_t)c * VEC, wv);
+    if (w) load_param_f32<VEC>(w, wdt, opaque_index((int64_t)c * VEC), wv);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
       const float gg = w ? dv[j] * wv[j] : dv[j];
@@ -317,7 +589,7 @@ __global__ __launch_bounds__(1024) void norm_bwd_stream_kernel(
     float dv[VEC], xv[VEC], wv[VEC], o[VEC];
     load_f32<TDY, VEC>(dyr + (int64_t)c * VEC, dv);
     load_f32<TX, VEC>(xr + (int64_t)c * VEC, xv);
-    if (w) load_param_f32<VEC>(w, wdt, (int64_t)c * VEC, wv);
+    if (w) load_param_f32<VEC>(w, wdt, opaque_index((int64_t)c * VEC), wv);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
       const float gg = w ? dv[j] * wv[j] : dv[j];
@@ -349,32 +621,41 @@ __global__ void norm_param_grad_cols_kernel(
   if (LAYER && part_b) part_b[(int64_t)blockIdx.y * feat + col] = ab;
 }
 
-// out[f] = sum over p of part[p, f], fixed order.  Block = 256 threads = 16 column quads x 16
-// row slices; grid.x covers the columns in steps of 64, grid.y selects the gradient.
+// out[f] = sum over p of part[p, f], in a fixed order.  A workgroup owns 16 columns: 4 column
+// quads x 64 row slices; grid.x covers the columns in steps of 16, grid.y selects the gradient.
+constexpr int kReduceCols = 16;
 __global__ __launch_bounds__(256) void reduce_partials_kernel(
     const float* __restrict__ part0, float* __restrict__ out0, const float* __restrict__ part1,
     float* __restrict__ out1, int parts, int feat) {
-  __shared__ float sm[16][65];
+  __shared__ float sm[64][kReduceCols + 1];
   const float* part = blockIdx.y == 0 ? part0 : part1;
   float* out = blockIdx.y == 0 ? out0 : out1;
   if (!part || !out) return;
-  const int cq = threadIdx.x & 15, slice = threadIdx.x >> 4;
-  const int col = blockIdx.x * 64 + cq * 4;
+  const int cq = threadIdx.x & 3, slice = threadIdx.x >> 2;
+  const int col = blockIdx.x * kReduceCols + cq * 4;
   float a[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int p = slice; p < parts; p += 16) {
-    const float* src = part + (int64_t)p * feat + col;
+  if (col + 3 < feat && (feat & 3) == 0 && (reinterpret_cast<uintptr_t>(part) & 15) == 0) {
+#pragma unroll 4
+    for (int p = slice; p < parts; p += 64) {
+      const float4 v = *reinterpret_cast<const float4*>(part + (int64_t)p * feat + col);
+      a[0] += v.x; a[1] += v.y; a[2] += v.z; a[3] += v.w;
+    }
+  } else {
+    for (int p = slice; p < parts; p += 64) {
+      const float* src = part + (int64_t)p * feat + col;
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      if (col + j < feat) a[j] += src[j];
+      for (int j = 0; j < 4; ++j)
+        if (col + j < feat) a[j] += src[j];
+    }
   }
 #pragma unroll
   for (int j = 0; j < 4; ++j) sm[slice][cq * 4 + j] = a[j];
   __syncthreads();
-  if (threadIdx.x < 64) {
+  if (threadIdx.x < kReduceCols) {
     float s = 0.f;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) s += sm[r][threadIdx.x];
-    const int c = blockIdx.x * 64 + threadIdx.x;
+    for (int r = 0; r < 64; ++r) s += sm[r][threadIdx.x];
+    const int c = blockIdx.x * kReduceCols + threadIdx.x;
     if (c < feat) out[c] = s;
   }
 }
@@ -386,82 +667,116 @@ template <typename TX, typename TY, int VEC, int ITERS>
 __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
     const TX* __restrict__ x, TY* __restrict__ y, int64_t batch, int feat, int64_t xs, int64_t ys,
     int neg, int log, int group_log2) {
-  __shared__ float scratch[16];
+  static_assert(ITERS > 0, "rows are cached in registers");
+  __shared__ float slots[2][16];
+  int parity = 0;
   const int group = 1 << group_log2;
   const int lane = threadIdx.x & (group - 1);
-  const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> group_log2) + (threadIdx.x >> group_log2);
-  const bool valid = row < batch;
+  const int rpb = blockDim.x >> group_log2;
+  const int rib = threadIdx.x >> group_log2;
   const int chunks = feat / VEC;
-  const int n_it = ITERS > 0 ? ITERS : (chunks + group - 1) / group;
-  const TX* xr = x + (valid ? row : 0) * xs;
   const float sign = neg ? -1.f : 1.f;
-  float cache[cache_len<ITERS>()][VEC];
+  const float pad = -sign * INFINITY;   // padding never wins the max and adds exp(-inf) = 0
+  const int64_t row_blocks = (batch + rpb - 1) / rpb;
+  const int64_t row_step = (int64_t)gridDim.x * rpb;
 
-  float m = -INFINITY;
-#pragma unroll
-  for (int it = 0; it < n_it; ++it) {
-    const int c = lane + it * group;
-    float v[VEC];
-    if (valid && c < chunks) {
-      load_f32<TX, VEC>(xr + (int64_t)c * VEC, v);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) v[j] *= sign;
-    } else {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) v[j] = -INFINITY;
-    }
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      m = fmaxf(m, v[j]);
-      if (ITERS > 0) cache[ITERS > 0 ? it : 0][j] = v[j];
-    }
+  RowCache<TX, VEC, ITERS> cur, nxt;
+  {
+    const int64_t row0 = (int64_t)blockIdx.x * rpb + rib;
+    cur.load(x, row0, xs, row0 < batch, lane, group, chunks, pad);
   }
-  m = group_reduce(m, group, scratch, MaxOp(), -INFINITY);
+#pragma unroll 1
+  for (int64_t rb = blockIdx.x; rb < row_blocks; rb += gridDim.x) {
+    const int64_t row = rb * rpb + rib;
+    const bool valid = row < batch;
+    nxt.load(x, row + row_step, xs, row + row_step < batch, lane, group, chunks, pad);
+    __builtin_amdgcn_sched_barrier(0);
 
-  float s = 0.f;
+    float m = -INFINITY;
 #pragma unroll
-  for (int it = 0; it < n_it; ++it) {
-    const int c = lane + it * group;
-    if (ITERS > 0) {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        const float d = cache[ITERS > 0 ? it : 0][j] - m;
-        const float e = __expf(d);
-        s += e;
-        cache[ITERS > 0 ? it : 0][j] = log ? d : e;
-      }
-    } else if (valid && c < chunks) {
+    for (int it = 0; it < ITERS; ++it) {
       float v[VEC];
-      load_f32<TX, VEC>(xr + (int64_t)c * VEC, v);
+      cur.ch[it].get(v);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) m = fmaxf(m, v[j] * sign);
+    }
+    m = group_reduce_alt(m, group, slots, parity, MaxOp(), -INFINITY);
+    if (!valid) m = 0.f;   // an invalid row is all padding: keep its arithmetic finite
+    cur.pin();
+
+    float s = 0.f;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      float v[VEC];
+      cur.ch[it].get(v);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) s += __expf(v[j] * sign - m);
     }
-  }
-  s = group_reduce(s, group, scratch, SumOp(), 0.f);
-  if (!valid) return;
-  const float inv = 1.0f / s;
-  const float lg = __logf(s);
+    s = group_reduce_alt(s, group, slots, parity, SumOp(), 0.f);
+    cur.pin();
 
-  TY* yr = y + row * ys;
+    if (valid) {
+      const float inv = 1.0f / s;
+      const float lg = __logf(s);
+      TY* yr = y + row * ys;
 #pragma unroll
-  for (int it = 0; it < n_it; ++it) {
-    const int c = lane + it * group;
-    if (c < chunks) {
-      float v[VEC];
-      if (ITERS > 0) {
+      for (int it = 0; it < ITERS; ++it) {
+        const int c = lane + it * group;
+        if (c < chunks) {
+          float v[VEC];
+          cur.ch[it].get(v);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j)
-          v[j] = log ? cache[ITERS > 0 ? it : 0][j] - lg : cache[ITERS > 0 ? it : 0][j] * inv;
-      } else {
-        load_f32<TX, VEC>(xr + (int64_t)c * VEC, v);
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          const float d = v[j] * sign - m;
-          v[j] = log ? d - lg : __expf(d) * inv;
+          for (int j = 0; j < VEC; ++j) {
+            const float d = v[j] * sign - m;
+            v[j] = log ? d - lg : __expf(d) * inv;
+          }
+          store_f32<TY, VEC>(yr + (int64_t)c * VEC, v);
         }
       }
-      store_f32<TY, VEC>(yr + (int64_t)c * VEC, v);
     }
+    cur = nxt;
+    cur.pin();
+  }
+}
+
+// Streaming forward for rows too wide for the register cache: one row per workgroup.
+template <typename TX, typename TY, int VEC>
+__global__ __launch_bounds__(1024) void softmax_fwd_stream_kernel(
+    const TX* __restrict__ x, TY* __restrict__ y, int feat, int64_t xs, int64_t ys, int neg, int log) {
+  __shared__ float scratch[16];
+  const int group = blockDim.x;
+  const int lane = threadIdx.x;
+  const int chunks = feat / VEC;
+  const float sign = neg ? -1.f : 1.f;
+  const TX* xr = x + (int64_t)blockIdx.x * xs;
+  TY* yr = y + (int64_t)blockIdx.x * ys;
+  float m = -INFINITY;
+  for (int c = lane; c < chunks; c += group) {
+    float v[VEC];
+    load_f32<TX, VEC>(xr + (int64_t)c * VEC, v);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) m = fmaxf(m, v[j] * sign);
+  }
+  m = group_reduce(m, group, scratch, MaxOp(), -INFINITY);
+  float s = 0.f;
+  for (int c = lane; c < chunks; c += group) {
+    float v[VEC];
+    load_f32<TX, VEC>(xr + (int64_t)c * VEC, v);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) s += __expf(v[j] * sign - m);
+  }
+  s = group_reduce(s, group, scratch, SumOp(), 0.f);
+  const float inv = 1.0f / s;
+  const float lg = __logf(s);
+  for (int c = lane; c < chunks; c += group) {
+    float v[VEC];
+    load_f32<TX, VEC>(xr + (int64_t)c * VEC, v);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const float d = v[j] * sign - m;
+      v[j] = log ? d - lg : __expf(d) * inv;
+    }
+    store_f32<TY, VEC>(yr + (int64_t)c * VEC, v);
   }
 }
 
@@ -469,58 +784,99 @@ template <typename TDY, typename TY, typename TDX, int VEC, int ITERS>
 __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
     const TDY* __restrict__ dy, const TY* __restrict__ y, TDX* __restrict__ dx, int64_t batch,
     int feat, int64_t dys, int64_t ys, int64_t dxs, int neg, int log, int group_log2) {
-  __shared__ float scratch[16];
+  static_assert(ITERS > 0, "rows are cached in registers");
+  __shared__ float slots[2][16];
+  int parity = 0;
   const int group = 1 << group_log2;
   const int lane = threadIdx.x & (group - 1);
-  const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> group_log2) + (threadIdx.x >> group_log2);
-  const bool valid = row < batch;
+  const int rpb = blockDim.x >> group_log2;
+  const int rib = threadIdx.x >> group_log2;
   const int chunks = feat / VEC;
-  const int n_it = ITERS > 0 ? ITERS : (chunks + group - 1) / group;
-  const int64_t rr = valid ? row : 0;
-  const TDY* dyr = dy + rr * dys;
-  const TY* yr = y + rr * ys;
-  float cdy[cache_len<ITERS>()][VEC], cy[cache_len<ITERS>()][VEC];
+  const float sign = neg ? -1.f : 1.f;
+  const int64_t row_blocks = (batch + rpb - 1) / rpb;
+  const int64_t row_step = (int64_t)gridDim.x * rpb;
 
+  RowCache<TDY, VEC, ITERS> cdy, ndy;
+  RowCache<TY, VEC, ITERS> cy, ny;
+  {
+    const int64_t row0 = (int64_t)blockIdx.x * rpb + rib;
+    cdy.load(dy, row0, dys, row0 < batch, lane, group, chunks, 0.f);
+    cy.load(y, row0, ys, row0 < batch, lane, group, chunks, 0.f);
+  }
+#pragma unroll 1
+  for (int64_t rb = blockIdx.x; rb < row_blocks; rb += gridDim.x) {
+    const int64_t row = rb * rpb + rib;
+    const bool valid = row < batch;
+    ndy.load(dy, row + row_step, dys, row + row_step < batch, lane, group, chunks, 0.f);
+    ny.load(y, row + row_step, ys, row + row_step < batch, lane, group, chunks, 0.f);
+    __builtin_amdgcn_sched_barrier(0);
+
+    float s = 0.f;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      float dv[VEC], yv[VEC];
+      cdy.ch[it].get(dv);
+      cy.ch[it].get(yv);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) s += log ? dv[j] : dv[j] * yv[j];
+    }
+    s = group_reduce_alt(s, group, slots, parity, SumOp(), 0.f);
+    cdy.pin();
+    cy.pin();
+
+    if (valid) {
+      TDX* dxr = dx + row * dxs;
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const int c = lane + it * group;
+        if (c < chunks) {
+          float dv[VEC], yv[VEC], o[VEC];
+          cdy.ch[it].get(dv);
+          cy.ch[it].get(yv);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j)
+            o[j] = sign * (log ? dv[j] - __expf(yv[j]) * s : yv[j] * (dv[j] - s));
+          store_f32<TDX, VEC>(dxr + (int64_t)c * VEC, o);
+        }
+      }
+    }
+    cdy = ndy;
+    cy = ny;
+    cdy.pin();
+    cy.pin();
+  }
+}
+
+// Streaming backward for rows too wide for the register cache: one row per workgroup.
+template <typename TDY, typename TY, typename TDX, int VEC>
+__global__ __launch_bounds__(1024) void softmax_bwd_stream_kernel(
+    const TDY* __restrict__ dy, const TY* __restrict__ y, TDX* __restrict__ dx, int feat,
+    int64_t dys, int64_t ys, int64_t dxs, int neg, int log) {
+  __shared__ float scratch[16];
+  const int group = blockDim.x;
+  const int lane = threadIdx.x;
+  const int chunks = feat / VEC;
+  const float sign = neg ? -1.f : 1.f;
+  const TDY* dyr = dy + (int64_t)blockIdx.x * dys;
+  const TY* yr = y + (int64_t)blockIdx.x * ys;
+  TDX* dxr = dx + (int64_t)blockIdx.x * dxs;
   float s = 0.f;
-#pragma unroll
-  for (int it = 0; it < n_it; ++it) {
-    const int c = lane + it * group;
+  for (int c = lane; c < chunks; c += group) {
     float dv[VEC], yv[VEC];
-    if (valid && c < chunks) {
-      load_f32<TDY, VEC>(dyr + (int64_t)c * VEC, dv);
-      load_f32<TY, VEC>(yr + (int64_t)c * VEC, yv);
-    } else {
+    load_f32<TDY, VEC>(dyr + (int64_t)c * VEC, dv);
+    load_f32<TY, VEC>(yr + (int64_t)c * VEC, yv);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) { dv[j] = 0.f; yv[j] = 0.f; }
-    }
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      s += log ? dv[j] : dv[j] * yv[j];
-      if (ITERS > 0) { cdy[ITERS > 0 ? it : 0][j] = dv[j]; cy[ITERS > 0 ? it : 0][j] = yv[j]; }
-    }
+    for (int j = 0; j < VEC; ++j) s += log ? dv[j] : dv[j] * yv[j];
   }
   s = group_reduce(s, group, scratch, SumOp(), 0.f);
-  if (!valid) return;
-  const float sign = neg ? -1.f : 1.f;
-
-  TDX* dxr = dx + row * dxs;
+  for (int c = lane; c < chunks; c += group) {
+    float dv[VEC], yv[VEC], o[VEC];
+    load_f32<TDY, VEC>(dyr + (int64_t)c * VEC, dv);
+    load_f32<TY, VEC>(yr + (int64_t)c * VEC, yv);
 #pragma unroll
-  for (int it = 0; it < n_it; ++it) {
-    const int c = lane + it * group;
-    if (c < chunks) {
-      float dv[VEC], yv[VEC], o[VEC];
-      if (ITERS > 0) {
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) { dv[j] = cdy[ITERS > 0 ? it : 0][j]; yv[j] = cy[ITERS > 0 ? it : 0][j]; }
-      } else {
-        load_f32<TDY, VEC>(dyr + (int64_t)c * VEC, dv);
-        load_f32<TY, VEC>(yr + (int64_t)c * VEC, yv);
-      }
-#pragma unroll
-      for (int j = 0; j < VEC; ++j)
-        o[j] = sign * (log ? dv[j] - __expf(yv[j]) * s : yv[j] * (dv[j] - s));
-      store_f32<TDX, VEC>(dxr + (int64_t)c * VEC, o);
-    }
+    for (int j = 0; j < VEC; ++j)
+      o[j] = sign * (log ? dv[j] - __expf(yv[j]) * s : yv[j] * (dv[j] - s));
+    store_f32<TDX, VEC>(dxr + (int64_t)c * VEC, o);
   }
 }
 
@@ -541,16 +897,14 @@ inline int narrow_vec(int dt_a, int dt_b, int dt_c) {
     case 1: { constexpr int ITERS = 1; __VA_ARGS__; break; }       \
     case 2: { constexpr int ITERS = 2; __VA_ARGS__; break; }       \
     case 4: { constexpr int ITERS = 4; __VA_ARGS__; break; }       \
-    case 8: { constexpr int ITERS = 8; __VA_ARGS__; break; }       \
-    default: { constexpr int ITERS = 0; __VA_ARGS__; break; }      \
+    default: { constexpr int ITERS = 8; __VA_ARGS__; break; }      \
   }
 
-#define AT_DISPATCH_ITERS_CACHED(ITERS_VALUE, ...)                 \
+#define AT_DISPATCH_ITERS4(ITERS_VALUE, ...)                      \
   switch (ITERS_VALUE) {                                           \
     case 1: { constexpr int ITERS = 1; __VA_ARGS__; break; }       \
     case 2: { constexpr int ITERS = 2; __VA_ARGS__; break; }       \
-    case 4: { constexpr int ITERS = 4; __VA_ARGS__; break; }       \
-    default: { constexpr int ITERS = 8; __VA_ARGS__; break; }      \
+    default: { constexpr int ITERS = 4; __VA_ARGS__; break; }      \
   }
 
 // Allowed (in, out) storage pairs: out == in, or out == fp32 (autocast-to-fp32 policy).
@@ -566,8 +920,37 @@ inline int dispatch_pair(int in_dt, int out_dt, F&& f) {
 
 inline int check_rows(int64_t batch, int64_t feat, int64_t s0, int64_t s1, int64_t s2) {
   if (batch < 0 || feat <= 0 || feat > (int64_t)1 << 30) return AT_ERR_DIM;
+  if (batch > (int64_t)0x7fffffff) return AT_ERR_DIM;  // one workgroup per row on the streaming path
   if (s0 < feat || s1 < feat || s2 < feat) return AT_ERR_DIM;
   return AT_OK;
+}
+
+// Workgroups of `fn` one CU keeps resident at this block size (asked once per kernel).
+inline int resident_blocks(const void* fn, int block, size_t lds) {
+  static std::mutex mu;
+  static std::map<std::tuple<const void*, int, size_t>, int> known;
+  std::lock_guard<std::mutex> lock(mu);
+  const auto key = std::make_tuple(fn, block, lds);
+  auto it = known.find(key);
+  if (it != known.end()) return it->second;
+  int n = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, fn, block, lds) != hipSuccess || n <= 0) {
+    (void)hipGetLastError();
+    n = 1;
+  }
+  known.emplace(key, n);
+  return n;
+}
+
+// Grid of a persistent row kernel: no more workgroups than stay resident at once, and as even a
+// number of row-blocks per workgroup as that allows.  max_blocks > 0 caps the grid further.
+inline unsigned persistent_grid(const void* fn, int block, size_t lds, int64_t row_blocks,
+                                int64_t max_blocks) {
+  int64_t cap = (int64_t)device_cu_count() * resident_blocks(fn, block, lds);
+  if (max_blocks > 0 && cap > max_blocks) cap = max_blocks;
+  if (row_blocks <= cap) return (unsigned)row_blocks;
+  const int64_t rounds = cdiv64(row_blocks, cap);
+  return (unsigned)cdiv64(row_blocks, rounds);
 }
 
 template <bool LAYER>
@@ -580,42 +963,52 @@ int norm_fwd(const void* x, const void* weight, const void* bias, float* mean, f
   if (rc) return rc;
   if (batch == 0) return AT_OK;
   if (!weight) bias = nullptr;
+  if (weight && wdt != xdt && wdt != AT_DTYPE_F32) return AT_ERR_DTYPE;  // parameters: input dtype or fp32
   int vec = narrow_vec(xdt, ydt, AT_DTYPE_F32);
   const bool vector_ok = feat % vec == 0 && rows_vectorizable(x, xs, xdt) &&
                          rows_vectorizable(y, ys, ydt) && (!weight || aligned16(weight)) &&
                          (!bias || aligned16(bias));
   if (!vector_ok) vec = 1;
-  const RowPlan p = plan_rows(feat, vec, 256, 8, 1024);
-  const int rpb = p.block >> p.group_log2;
-  const dim3 grid((unsigned)cdiv64(batch, rpb));
+  // few chunks per lane: many resident waves hide the latency of the row reductions
+  const RowPlan p = plan_rows(feat, vec, 256, 2, 512);
   return dispatch_pair(xdt, ydt, [&](auto* tx, auto* ty) -> int {
     typedef std::remove_pointer_t<decltype(tx)> TX;
     typedef std::remove_pointer_t<decltype(ty)> TY;
     constexpr int VECW = sizeof(TX) == 4 && sizeof(TY) == 4 ? 4 : 8;
-    if (vec != 1) {
-      AT_DISPATCH_ITERS(p.iters, hipLaunchKernelGGL((norm_fwd_kernel<LAYER, TX, TY, VECW, ITERS>), grid,
-                                                    dim3(p.block), 0, stream, (const TX*)x, weight, bias,
-                                                    mean, rstd, (TY*)y, batch, (int)feat, xs, ys, eps,
-                                                    wdt, p.group_log2));
-    } else {
-      AT_DISPATCH_ITERS(p.iters, hipLaunchKernelGGL((norm_fwd_kernel<LAYER, TX, TY, 1, ITERS>), grid,
-                                                    dim3(p.block), 0, stream, (const TX*)x, weight, bias,
-                                                    mean, rstd, (TY*)y, batch, (int)feat, xs, ys, eps,
-                                                    wdt, p.group_log2));
+    if (p.iters == 0) {
+      if (vec != 1)
+        hipLaunchKernelGGL((norm_fwd_stream_kernel<LAYER, TX, TY, VECW>), dim3((unsigned)batch), dim3(1024),
+                           0, stream, (const TX*)x, weight, bias, mean, rstd, (TY*)y, (int)feat, xs, ys,
+                           eps, wdt);
+      else
+        hipLaunchKernelGGL((norm_fwd_stream_kernel<LAYER, TX, TY, 1>), dim3((unsigned)batch), dim3(1024), 0,
+                           stream, (const TX*)x, weight, bias, mean, rstd, (TY*)y, (int)feat, xs, ys, eps,
+                           wdt);
+      return launch_status();
     }
+    const int64_t row_blocks = cdiv64(batch, p.block >> p.group_log2);
+#define AT_NORM_FWD_LAUNCH(TW, VV)                                                                       \
+  AT_DISPATCH_ITERS(p.iters, {                                                                           \
+    auto kernel = norm_fwd_kernel<LAYER, TX, TY, TW, VV, ITERS>;                                         \
+    const unsigned grid = persistent_grid((const void*)kernel, p.block, 0, row_blocks, 0);               \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(p.block), 0, stream, (const TX*)x, (const TW*)weight,    \
+                       (const TW*)bias, mean, rstd, (TY*)y, batch, (int)feat, xs, ys, eps,               \
+                       p.group_log2);                                                                    \
+  })
+    // parameters are stored either like the input or in fp32
+    if (weight && wdt == AT_DTYPE_F32 && xdt != AT_DTYPE_F32) {
+      if (vec != 1) { AT_NORM_FWD_LAUNCH(float, VECW); } else { AT_NORM_FWD_LAUNCH(float, 1); }
+    } else {
+      if (vec != 1) { AT_NORM_FWD_LAUNCH(TX, VECW); } else { AT_NORM_FWD_LAUNCH(TX, 1); }
+    }
+#undef AT_NORM_FWD_LAUNCH
     return launch_status();
   });
 }
 
 constexpr int kBwdBlock = 512;        // 8 waves: room for 256 VGPRs per lane
 constexpr int kStreamSlices = 256;    // row slices of the column kernel in the streaming fallback
-constexpr int kMaxPartialRows = 1024; // upper bound on partial rows (CU count or kStreamSlices)
-
-inline int bwd_grid_blocks(int64_t row_blocks) {
-  int64_t cap = (int64_t)device_cu_count();
-  if (cap > kMaxPartialRows) cap = kMaxPartialRows;
-  return (int)(row_blocks < cap ? row_blocks : cap);
-}
+constexpr int kMaxPartialRows = 1024; // upper bound on partial rows (grid size or kStreamSlices)
 
 template <bool LAYER>
 int norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd, const void* weight,
@@ -626,6 +1019,7 @@ int norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd
   if (!dtype_valid(dydt) || !dtype_valid(xdt) || !dtype_valid(dxdt) || (weight && !dtype_valid(wdt)))
     return AT_ERR_DTYPE;
   if (dxdt != dydt) return AT_ERR_DTYPE;  // the input gradient is produced in the output dtype
+  if (weight && wdt != xdt && wdt != AT_DTYPE_F32) return AT_ERR_DTYPE;  // parameters: input dtype or fp32
   int rc = check_rows(batch, feat, dys, xs, dxs);
   if (rc) return rc;
   if (!LAYER) bias_grad = nullptr;
@@ -637,7 +1031,7 @@ int norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd
   }
   if (batch == 0) {
     if (n_grads)  // zero partial rows: the reduction writes exact zeros
-      hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)cdiv64(feat, 64), bias_grad ? 2 : 1),
+      hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)cdiv64(feat, kReduceCols), bias_grad ? 2 : 1),
                          dim3(256), 0, stream, (const float*)workspace, weight_grad,
                          (const float*)workspace, bias_grad, 0, (int)feat);
     return launch_status();
@@ -647,7 +1041,11 @@ int norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd
                          rows_vectorizable(x, xs, xdt) && rows_vectorizable(dx, dxs, dxdt) &&
                          (!weight || aligned16(weight));
   if (!vector_ok) vec = 1;
-  const RowPlan p = plan_rows(feat, vec, kBwdBlock, vec == 4 ? 8 : 4, kBwdBlock);
+  // The backward kernel keeps ITERS * VEC fp32 column accumulators per parameter gradient next
+  // to two rows of both cached tensors: it prefers two chunks per lane (rows spread over more
+  // waves) and stops at four; wider rows stream.
+  RowPlan p = plan_rows(feat, vec, kBwdBlock, 2, kBwdBlock);
+  if (p.iters > 4) p.iters = 0;
   float* part_w = weight_grad ? (float*)workspace : nullptr;
   int parts = 0;
 
@@ -657,21 +1055,25 @@ int norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd
     constexpr int VECW = sizeof(TX) == 4 && sizeof(TDY) == 4 ? 4 : 8;
     if (p.iters != 0) {
       const int rpb = p.block >> p.group_log2;
-      parts = bwd_grid_blocks(cdiv64(batch, rpb));
-      float* part_b = bias_grad ? part_w + (int64_t)parts * feat : nullptr;
-      if (vec != 1) {
-        const size_t lds = rpb > 1 ? (size_t)p.block * VECW * sizeof(float) : 0;
-        AT_DISPATCH_ITERS_CACHED(p.iters, hipLaunchKernelGGL(
-            (norm_bwd_kernel<LAYER, TDY, TX, TDY, VECW, ITERS>), dim3(parts), dim3(p.block), lds, stream,
-            (const TDY*)dy, (const TX*)x, mean, rstd, weight, (TDY*)dx, part_w, part_b, batch, (int)feat,
-            dys, xs, dxs, wdt, p.group_log2));
+      const int64_t row_blocks = cdiv64(batch, rpb);
+#define AT_NORM_BWD_LAUNCH(TW, VV)                                                                       \
+  {                                                                                                      \
+    const size_t lds = rpb > 1 ? (size_t)p.block * VV * sizeof(float) : 0;                              \
+    AT_DISPATCH_ITERS4(p.iters, {                                                                        \
+      auto kernel = norm_bwd_kernel<LAYER, TDY, TX, TDY, TW, VV, ITERS>;                                 \
+      parts = (int)persistent_grid((const void*)kernel, p.block, lds, row_blocks, kMaxPartialRows);      \
+      float* part_b = bias_grad ? part_w + (int64_t)parts * feat : nullptr;                              \
+      hipLaunchKernelGGL(kernel, dim3(parts), dim3(p.block), lds, stream, (const TDY*)dy, (const TX*)x,  \
+                         mean, rstd, (const TW*)weight, (TDY*)dx, part_w, part_b, batch, (int)feat, dys, \
+                         xs, dxs, p.group_log2);                                                         \
+    });                                                                                                  \
+  }
+      if (weight && wdt == AT_DTYPE_F32 && xdt != AT_DTYPE_F32) {
+        if (vec != 1) AT_NORM_BWD_LAUNCH(float, VECW) else AT_NORM_BWD_LAUNCH(float, 1)
       } else {
-        const size_t lds = rpb > 1 ? (size_t)p.block * sizeof(float) : 0;
-        AT_DISPATCH_ITERS_CACHED(p.iters, hipLaunchKernelGGL(
-            (norm_bwd_kernel<LAYER, TDY, TX, TDY, 1, ITERS>), dim3(parts), dim3(p.block), lds, stream,
-            (const TDY*)dy, (const TX*)x, mean, rstd, weight, (TDY*)dx, part_w, part_b, batch, (int)feat,
-            dys, xs, dxs, wdt, p.group_log2));
+        if (vec != 1) AT_NORM_BWD_LAUNCH(TX, VECW) else AT_NORM_BWD_LAUNCH(TX, 1)
       }
+#undef AT_NORM_BWD_LAUNCH
     } else {
       if (vec != 1)
         hipLaunchKernelGGL((norm_bwd_stream_kernel<LAYER, TDY, TX, TDY, VECW>), dim3((unsigned)batch),
@@ -697,7 +1099,7 @@ int norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd
   if (rc) return rc;
   if (n_grads) {
     float* part_b = bias_grad ? part_w + (int64_t)parts * feat : nullptr;
-    hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)cdiv64(feat, 64), bias_grad ? 2 : 1),
+    hipLaunchKernelGGL(reduce_partials_kernel, dim3((unsigned)cdiv64(feat, kReduceCols), bias_grad ? 2 : 1),
                        dim3(256), 0, stream, part_w, weight_grad, part_b, bias_grad, parts, (int)feat);
     rc = launch_status();
   }
@@ -751,7 +1153,8 @@ int at_layer_norm_bwd(const void* dy, const void* x, const float* mean, const fl
 }
 
 int at_softmax_fwd(const void* x, void* y, int64_t batch, int64_t feat, int64_t x_stride,
-                   int64_t y_stride, int neg, int log, int x_dtype, int y_dtype, at_stream_t stream) {
+                   int64_t y_stride, int neg, int log, int x_dtype, int y_dtype, at_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
   if (!x || !y) return AT_ERR_NULL;
   if (!dtype_valid(x_dtype) || !dtype_valid(y_dtype)) return AT_ERR_DTYPE;
   int rc = check_rows(batch, feat, x_stride, y_stride, feat);
@@ -760,30 +1163,38 @@ int at_softmax_fwd(const void* x, void* y, int64_t batch, int64_t feat, int64_t 
   int vec = narrow_vec(x_dtype, y_dtype, AT_DTYPE_F32);
   if (!(feat % vec == 0 && rows_vectorizable(x, x_stride, x_dtype) && rows_vectorizable(y, y_stride, y_dtype)))
     vec = 1;
-  const RowPlan p = plan_rows(feat, vec, 256, 8, 1024);
-  const dim3 grid((unsigned)cdiv64(batch, p.block >> p.group_log2));
+  const RowPlan p = plan_rows(feat, vec, 256, 4, 1024);
   return dispatch_pair(x_dtype, y_dtype, [&](auto* tx, auto* ty) -> int {
     typedef std::remove_pointer_t<decltype(tx)> TX;
     typedef std::remove_pointer_t<decltype(ty)> TY;
     constexpr int VECW = sizeof(TX) == 4 && sizeof(TY) == 4 ? 4 : 8;
-    if (vec != 1) {
-      AT_DISPATCH_ITERS(p.iters, hipLaunchKernelGGL((softmax_fwd_kernel<TX, TY, VECW, ITERS>), grid,
-                                                    dim3(p.block), 0, (hipStream_t)stream, (const TX*)x,
-                                                    (TY*)y, batch, (int)feat, x_stride, y_stride, neg,
-                                                    log, p.group_log2));
-    } else {
-      AT_DISPATCH_ITERS(p.iters, hipLaunchKernelGGL((softmax_fwd_kernel<TX, TY, 1, ITERS>), grid,
-                                                    dim3(p.block), 0, (hipStream_t)stream, (const TX*)x,
-                                                    (TY*)y, batch, (int)feat, x_stride, y_stride, neg,
-                                                    log, p.group_log2));
+    if (p.iters == 0) {
+      if (vec != 1)
+        hipLaunchKernelGGL((softmax_fwd_stream_kernel<TX, TY, VECW>), dim3((unsigned)batch), dim3(1024), 0,
+                           stream, (const TX*)x, (TY*)y, (int)feat, x_stride, y_stride, neg, log);
+      else
+        hipLaunchKernelGGL((softmax_fwd_stream_kernel<TX, TY, 1>), dim3((unsigned)batch), dim3(1024), 0,
+                           stream, (const TX*)x, (TY*)y, (int)feat, x_stride, y_stride, neg, log);
+      return launch_status();
     }
+    const int64_t row_blocks = cdiv64(batch, p.block >> p.group_log2);
+#define AT_SOFTMAX_FWD_LAUNCH(VV)                                                                        \
+  AT_DISPATCH_ITERS(p.iters, {                                                                           \
+    auto kernel = softmax_fwd_kernel<TX, TY, VV, ITERS>;                                                 \
+    const unsigned grid = persistent_grid((const void*)kernel, p.block, 0, row_blocks, 0);               \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(p.block), 0, stream, (const TX*)x, (TY*)y, batch,        \
+                       (int)feat, x_stride, y_stride, neg, log, p.group_log2);                           \
+  })
+    if (vec != 1) { AT_SOFTMAX_FWD_LAUNCH(VECW); } else { AT_SOFTMAX_FWD_LAUNCH(1); }
+#undef AT_SOFTMAX_FWD_LAUNCH
     return launch_status();
   });
 }
 
 int at_softmax_bwd(const void* dy, const void* y, void* dx, int64_t batch, int64_t feat,
                    int64_t dy_stride, int64_t y_stride, int64_t dx_stride, int neg, int log,
-                   int dy_dtype, int y_dtype, int dx_dtype, at_stream_t stream) {
+                   int dy_dtype, int y_dtype, int dx_dtype, at_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
   if (!dy || !y || !dx) return AT_ERR_NULL;
   if (!dtype_valid(dy_dtype) || !dtype_valid(y_dtype) || !dtype_valid(dx_dtype)) return AT_ERR_DTYPE;
   if (dx_dtype != y_dtype) return AT_ERR_DTYPE;  // input_grad = empty_like(output), softmax_layers.py:78
@@ -794,23 +1205,35 @@ int at_softmax_bwd(const void* dy, const void* y, void* dx, int64_t batch, int64
   if (!(feat % vec == 0 && rows_vectorizable(dy, dy_stride, dy_dtype) &&
         rows_vectorizable(y, y_stride, y_dtype) && rows_vectorizable(dx, dx_stride, dx_dtype)))
     vec = 1;
-  const RowPlan p = plan_rows(feat, vec, 256, vec == 4 ? 8 : 4, 1024);
-  const dim3 grid((unsigned)cdiv64(batch, p.block >> p.group_log2));
+  // two rows of two tensors are held at once: four chunks per lane and tensor at most
+  RowPlan p = plan_rows(feat, vec, 256, 2, 1024);
+  if (p.iters > 4) p.iters = 0;
   return dispatch_pair(dy_dtype, y_dtype, [&](auto* tdy, auto* ty) -> int {
     typedef std::remove_pointer_t<decltype(tdy)> TDY;
     typedef std::remove_pointer_t<decltype(ty)> TY;
     constexpr int VECW = sizeof(TDY) == 4 && sizeof(TY) == 4 ? 4 : 8;
-    if (vec != 1) {
-      AT_DISPATCH_ITERS(p.iters, hipLaunchKernelGGL((softmax_bwd_kernel<TDY, TY, TY, VECW, ITERS>), grid,
-                                                    dim3(p.block), 0, (hipStream_t)stream, (const TDY*)dy,
-                                                    (const TY*)y, (TY*)dx, batch, (int)feat, dy_stride,
-                                                    y_stride, dx_stride, neg, log, p.group_log2));
-    } else {
-      AT_DISPATCH_ITERS(p.iters, hipLaunchKernelGGL((softmax_bwd_kernel<TDY, TY, TY, 1, ITERS>), grid,
-                                                    dim3(p.block), 0, (hipStream_t)stream, (const TDY*)dy,
-                                                    (const TY*)y, (TY*)dx, batch, (int)feat, dy_stride,
-                                                    y_stride, dx_stride, neg, log, p.group_log2));
+    if (p.iters == 0) {
+      if (vec != 1)
+        hipLaunchKernelGGL((softmax_bwd_stream_kernel<TDY, TY, TY, VECW>), dim3((unsigned)batch), dim3(1024),
+                           0, stream, (const TDY*)dy, (const TY*)y, (TY*)dx, (int)feat, dy_stride, y_stride,
+                           dx_stride, neg, log);
+      else
+        hipLaunchKernelGGL((softmax_bwd_stream_kernel<TDY, TY, TY, 1>), dim3((unsigned)batch), dim3(1024), 0,
+                           stream, (const TDY*)dy, (const TY*)y, (TY*)dx, (int)feat, dy_stride, y_stride,
+                           dx_stride, neg, log);
+      return launch_status();
     }
+    const int64_t row_blocks = cdiv64(batch, p.block >> p.group_log2);
+#define AT_SOFTMAX_BWD_LAUNCH(VV)                                                                        \
+  AT_DISPATCH_ITERS4(p.iters, {                                                                          \
+    auto kernel = softmax_bwd_kernel<TDY, TY, TY, VV, ITERS>;                                            \
+    const unsigned grid = persistent_grid((const void*)kernel, p.block, 0, row_blocks, 0);               \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(p.block), 0, stream, (const TDY*)dy, (const TY*)y,       \
+                       (TY*)dx, batch, (int)feat, dy_stride, y_stride, dx_stride, neg, log,              \
+                       p.group_log2);                                                                    \
+  })
+    if (vec != 1) { AT_SOFTMAX_BWD_LAUNCH(VECW); } else { AT_SOFTMAX_BWD_LAUNCH(1); }
+#undef AT_SOFTMAX_BWD_LAUNCH
     return launch_status();
   });
 }

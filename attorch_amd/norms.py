@@ -17,8 +17,16 @@ from . import _lib
 from .utils import get_output_dtype
 
 
-def _param_for_kernel(param: Optional[Tensor]) -> Optional[Tensor]:
-    return None if param is None else param.contiguous()
+def _param_for_kernel(param: Optional[Tensor], input: Tensor) -> Optional[Tensor]:
+    """
+    Parameters reach the kernels stored like the input or in fp32; any other pairing
+    (e.g. a 16-bit parameter beside an fp32 input) is widened to fp32 first.
+    """
+    if param is None:
+        return None
+    if param.dtype not in (input.dtype, torch.float32):
+        param = param.float()
+    return param.contiguous()
 
 
 class LayerNormAutoGrad(torch.autograd.Function):
@@ -67,8 +75,8 @@ class LayerNormAutoGrad(torch.autograd.Function):
         else:
             mean = inv_std = None
 
-        weight_k = _param_for_kernel(weight) if scale_by_weight else None
-        bias_k = _param_for_kernel(bias) if add_bias else None
+        weight_k = _param_for_kernel(weight, flattened_input) if scale_by_weight else None
+        bias_k = _param_for_kernel(bias, flattened_input) if add_bias else None
         if add_bias and bias_k.dtype != weight_k.dtype:
             bias_k = bias_k.to(weight_k.dtype)
 
@@ -117,7 +125,7 @@ class LayerNormAutoGrad(torch.autograd.Function):
             workspace_bytes = lib.at_norm_bwd_workspace_bytes(batch_dim, feat_dim,
                                                               2 if add_bias else 1)
             workspace = torch.empty(workspace_bytes, device=device, dtype=torch.uint8)
-        weight_k = _param_for_kernel(weight) if scale_by_weight else None
+        weight_k = _param_for_kernel(weight, flattened_input) if scale_by_weight else None
 
         with torch.cuda.device_of(flattened_input):
             _lib.check(lib.at_layer_norm_bwd(
@@ -207,7 +215,7 @@ class RMSNormAutoGrad(torch.autograd.Function):
                          (scale_by_weight and weight.requires_grad))
         inv_rms = (torch.empty(batch_dim, device=input.device, dtype=torch.float32)
                    if requires_grad else None)
-        weight_k = _param_for_kernel(weight)
+        weight_k = _param_for_kernel(weight, flattened_input)
 
         with torch.cuda.device_of(input):
             _lib.check(lib.at_rms_norm_fwd(
@@ -248,7 +256,7 @@ class RMSNormAutoGrad(torch.autograd.Function):
             weight_grad = torch.empty(feat_dim, device=device, dtype=torch.float32)
             workspace_bytes = lib.at_norm_bwd_workspace_bytes(batch_dim, feat_dim, 1)
             workspace = torch.empty(workspace_bytes, device=device, dtype=torch.uint8)
-        weight_k = _param_for_kernel(weight)
+        weight_k = _param_for_kernel(weight, flattened_input)
 
         with torch.cuda.device_of(flattened_input):
             _lib.check(lib.at_rms_norm_bwd(

@@ -15,7 +15,9 @@ pytestmark = pytest.mark.gpu
 
 SHAPES = [(96,), (768,), (8000,), (1, 8000), (4, 2000), (8, 1024), (32, 1024), (2048, 768), (6144, 256),
           (8096, 32), (12288, 1), (2049, 2), (4097, 4), (8, 960, 196), (2048, 64, 16), (33, 4096),
-          (7, 8200), (5, 12345), (3, 40000), (2, 70001)]
+          (7, 8200), (5, 12345), (3, 40000), (2, 70001),
+          # more row-blocks than the persistent grids hold at once: several rows per workgroup
+          (100001, 40), (20000, 520), (600000, 8)]
 
 
 @pytest.mark.parametrize('dtype', DTYPES)
