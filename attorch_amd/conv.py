@@ -39,6 +39,15 @@ def conv2d_output_size(
     return (in_size + 2 * padding - kernel_size) // stride + 1
 
 
+def _workspace(n_bytes: int, device: torch.device) -> Tuple[Optional[Tensor], int]:
+    """
+    Scratch buffer of the size a kernel asked for (None when it asked for nothing).
+    """
+    if n_bytes <= 0:
+        return None, 0
+    return torch.empty(n_bytes, dtype=torch.uint8, device=device), n_bytes
+
+
 class Conv2dAutoGrad(torch.autograd.Function):
     """
     Autodiff for 2D convolutional layer (attorch/conv_layer.py:39-164).
@@ -102,11 +111,14 @@ class Conv2dAutoGrad(torch.autograd.Function):
                 kernel_height, kernel_width, stride_height, stride_width,
                 padding_height, padding_width, groups)
 
+        dtype = _lib.dtype_id(output_dtype)
         with torch.cuda.device_of(input):
+            workspace, workspace_bytes = _workspace(
+                lib.at_conv2d_fwd_workspace_bytes(*dims, dtype, dtype), input.device)
             _lib.check(lib.at_conv2d_fwd(
-                _lib.ptr(input_k), _lib.ptr(weight_k), _lib.ptr(bias_k), _lib.ptr(output), *dims,
-                _lib.dtype_id(output_dtype), _lib.dtype_id(output_dtype),
-                _lib.dtype_id(output_dtype), _lib.stream_of(input)), 'at_conv2d_fwd')
+                _lib.ptr(input_k), _lib.ptr(weight_k), _lib.ptr(bias_k), _lib.ptr(output),
+                _lib.ptr(workspace), workspace_bytes, *dims, dtype, dtype, dtype,
+                _lib.stream_of(input)), 'at_conv2d_fwd')
 
         requires_grad = (input.requires_grad or
                          weight.requires_grad or
@@ -144,15 +156,17 @@ class Conv2dAutoGrad(torch.autograd.Function):
             if input.requires_grad:
                 weight_k = weight.to(output_dtype).contiguous()
                 input_grad = torch.empty(input.shape, dtype=output_dtype, device=device)
+                workspace, workspace_bytes = _workspace(
+                    lib.at_conv2d_bwd_input_workspace_bytes(*dims, dtype), device)
                 _lib.check(lib.at_conv2d_bwd_input(
-                    _lib.ptr(output_grad), _lib.ptr(weight_k), _lib.ptr(input_grad), *dims,
-                    dtype, stream), 'at_conv2d_bwd_input')
+                    _lib.ptr(output_grad), _lib.ptr(weight_k), _lib.ptr(input_grad),
+                    _lib.ptr(workspace), workspace_bytes, *dims, dtype, stream),
+                    'at_conv2d_bwd_input')
             if weight.requires_grad:
                 input_k = input.to(output_dtype).contiguous()
                 weight_grad = torch.empty(weight.shape, dtype=output_dtype, device=device)
-                workspace_bytes = lib.at_conv2d_bwd_weight_workspace_bytes(
-                    out_feat_dim, in_feat_dim // groups, kernel_height, kernel_width)
-                workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=device)
+                workspace, workspace_bytes = _workspace(
+                    lib.at_conv2d_bwd_weight_workspace_bytes(*dims, dtype), device)
                 _lib.check(lib.at_conv2d_bwd_weight(
                     _lib.ptr(output_grad), _lib.ptr(input_k), _lib.ptr(weight_grad),
                     _lib.ptr(workspace), workspace_bytes, *dims, dtype, stream),

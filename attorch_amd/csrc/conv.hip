@@ -12,6 +12,7 @@
 #include <type_traits>
 
 #include "at_common.h"
+#include "conv_igemm.h"
 
 namespace at_hip {
 namespace {
@@ -272,17 +273,49 @@ using namespace at_hip;
 
 extern "C" {
 
-int at_conv2d_fwd(const void* input, const void* weight, const void* bias, void* output, int64_t batch,
-                  int64_t in_feat, int64_t in_height, int64_t in_width, int64_t out_feat, int64_t out_height,
-                  int64_t out_width, int64_t kernel_height, int64_t kernel_width, int64_t stride_height,
-                  int64_t stride_width, int64_t padding_height, int64_t padding_width, int64_t groups,
-                  int in_dtype, int bias_dtype, int out_dtype, at_stream_t stream) {
+namespace {
+inline ConvProblem problem_of(const ConvShape& s, int dtype) {
+  return ConvProblem{s.N, s.C, s.H, s.W, s.O, s.KH, s.KW, s.sh, s.sw, s.ph, s.pw, s.groups, s.OH, s.OW, dtype};
+}
+inline ConvShape shape_of(int64_t batch, int64_t in_feat, int64_t in_height, int64_t in_width, int64_t out_feat,
+                          int64_t out_height, int64_t out_width, int64_t kernel_height, int64_t kernel_width,
+                          int64_t stride_height, int64_t stride_width, int64_t padding_height,
+                          int64_t padding_width, int64_t groups) {
+  return ConvShape{batch, in_feat, in_height, in_width, out_feat, kernel_height, kernel_width, stride_height,
+                   stride_width, padding_height, padding_width, groups, out_height, out_width};
+}
+}  // namespace
+
+int64_t at_conv2d_fwd_workspace_bytes(int64_t batch, int64_t in_feat, int64_t in_height, int64_t in_width,
+                                      int64_t out_feat, int64_t out_height, int64_t out_width,
+                                      int64_t kernel_height, int64_t kernel_width, int64_t stride_height,
+                                      int64_t stride_width, int64_t padding_height, int64_t padding_width,
+                                      int64_t groups, int in_dtype, int out_dtype) {
+  const ConvShape s = shape_of(batch, in_feat, in_height, in_width, out_feat, out_height, out_width, kernel_height,
+                               kernel_width, stride_height, stride_width, padding_height, padding_width, groups);
+  if (check_shape(s) || in_dtype != out_dtype) return 0;
+  return conv_igemm_fwd_workspace(problem_of(s, in_dtype));
+}
+
+int at_conv2d_fwd(const void* input, const void* weight, const void* bias, void* output, void* workspace,
+                  int64_t workspace_bytes, int64_t batch, int64_t in_feat, int64_t in_height, int64_t in_width,
+                  int64_t out_feat, int64_t out_height, int64_t out_width, int64_t kernel_height,
+                  int64_t kernel_width, int64_t stride_height, int64_t stride_width, int64_t padding_height,
+                  int64_t padding_width, int64_t groups, int in_dtype, int bias_dtype, int out_dtype,
+                  at_stream_t stream) {
   if (!input || !weight || !output) return AT_ERR_NULL;
   if (!dtype_valid(in_dtype) || !dtype_valid(out_dtype) || (bias && !dtype_valid(bias_dtype))) return AT_ERR_DTYPE;
-  const ConvShape s{batch, in_feat, in_height, in_width, out_feat, kernel_height, kernel_width, stride_height,
-                    stride_width, padding_height, padding_width, groups, out_height, out_width};
+  const ConvShape s = shape_of(batch, in_feat, in_height, in_width, out_feat, out_height, out_width, kernel_height,
+                               kernel_width, stride_height, stride_width, padding_height, padding_width, groups);
   int rc = check_shape(s);
   if (rc) return rc;
+  if (in_dtype == out_dtype) {
+    // 16-bit matrix-core path when the shape allows and the caller brought the workspace for it
+    const ConvProblem p = problem_of(s, in_dtype);
+    const int64_t need = conv_igemm_fwd_workspace(p);
+    if (need > 0 && workspace && workspace_bytes >= need && aligned16(workspace))
+      return conv_igemm_fwd(p, input, weight, bias, bias_dtype, output, workspace, (hipStream_t)stream);
+  }
   ConvArgs g = base_args(s);
   g.a = input; g.b = weight; g.out = output; g.bias = bias; g.bias_dt = bias_dtype;
   g.M = s.N * s.OH * s.OW; g.K = (int64_t)g.Cg * g.KH * g.KW; g.cols = g.Og;
@@ -297,17 +330,35 @@ int at_conv2d_fwd(const void* input, const void* weight, const void* bias, void*
   });
 }
 
-int at_conv2d_bwd_input(const void* output_grad, const void* weight, void* input_grad, int64_t batch,
-                        int64_t in_feat, int64_t in_height, int64_t in_width, int64_t out_feat,
-                        int64_t out_height, int64_t out_width, int64_t kernel_height, int64_t kernel_width,
-                        int64_t stride_height, int64_t stride_width, int64_t padding_height,
-                        int64_t padding_width, int64_t groups, int dtype, at_stream_t stream) {
+int64_t at_conv2d_bwd_input_workspace_bytes(int64_t batch, int64_t in_feat, int64_t in_height, int64_t in_width,
+                                            int64_t out_feat, int64_t out_height, int64_t out_width,
+                                            int64_t kernel_height, int64_t kernel_width, int64_t stride_height,
+                                            int64_t stride_width, int64_t padding_height, int64_t padding_width,
+                                            int64_t groups, int dtype) {
+  const ConvShape s = shape_of(batch, in_feat, in_height, in_width, out_feat, out_height, out_width, kernel_height,
+                               kernel_width, stride_height, stride_width, padding_height, padding_width, groups);
+  if (check_shape(s)) return 0;
+  return conv_igemm_dx_workspace(problem_of(s, dtype));
+}
+
+int at_conv2d_bwd_input(const void* output_grad, const void* weight, void* input_grad, void* workspace,
+                        int64_t workspace_bytes, int64_t batch, int64_t in_feat, int64_t in_height,
+                        int64_t in_width, int64_t out_feat, int64_t out_height, int64_t out_width,
+                        int64_t kernel_height, int64_t kernel_width, int64_t stride_height, int64_t stride_width,
+                        int64_t padding_height, int64_t padding_width, int64_t groups, int dtype,
+                        at_stream_t stream) {
   if (!output_grad || !weight || !input_grad) return AT_ERR_NULL;
   if (!dtype_valid(dtype)) return AT_ERR_DTYPE;
-  const ConvShape s{batch, in_feat, in_height, in_width, out_feat, kernel_height, kernel_width, stride_height,
-                    stride_width, padding_height, padding_width, groups, out_height, out_width};
+  const ConvShape s = shape_of(batch, in_feat, in_height, in_width, out_feat, out_height, out_width, kernel_height,
+                               kernel_width, stride_height, stride_width, padding_height, padding_width, groups);
   int rc = check_shape(s);
   if (rc) return rc;
+  {
+    const ConvProblem p = problem_of(s, dtype);
+    const int64_t need = conv_igemm_dx_workspace(p);
+    if (need > 0 && workspace && workspace_bytes >= need && aligned16(workspace))
+      return conv_igemm_dx(p, output_grad, weight, input_grad, workspace, (hipStream_t)stream);
+  }
   ConvArgs g = base_args(s);
   g.a = output_grad; g.b = weight; g.out = input_grad;
   g.M = s.N * s.H * s.W; g.K = (int64_t)g.Og * g.KH * g.KW; g.cols = g.Cg;
@@ -319,10 +370,18 @@ int at_conv2d_bwd_input(const void* output_grad, const void* weight, void* input
   });
 }
 
-int64_t at_conv2d_bwd_weight_workspace_bytes(int64_t out_feat, int64_t in_feat_per_group, int64_t kernel_height,
-                                             int64_t kernel_width) {
-  if (out_feat <= 0 || in_feat_per_group <= 0 || kernel_height <= 0 || kernel_width <= 0) return 0;
-  return (int64_t)kDwMaxSplits * out_feat * in_feat_per_group * kernel_height * kernel_width * (int64_t)sizeof(float);
+int64_t at_conv2d_bwd_weight_workspace_bytes(int64_t batch, int64_t in_feat, int64_t in_height, int64_t in_width,
+                                             int64_t out_feat, int64_t out_height, int64_t out_width,
+                                             int64_t kernel_height, int64_t kernel_width, int64_t stride_height,
+                                             int64_t stride_width, int64_t padding_height, int64_t padding_width,
+                                             int64_t groups, int dtype) {
+  const ConvShape s = shape_of(batch, in_feat, in_height, in_width, out_feat, out_height, out_width, kernel_height,
+                               kernel_width, stride_height, stride_width, padding_height, padding_width, groups);
+  if (check_shape(s)) return 0;
+  const int64_t generic = (int64_t)kDwMaxSplits * out_feat * (in_feat / groups) * kernel_height * kernel_width *
+                          (int64_t)sizeof(float);
+  const int64_t fast = conv_igemm_dw_workspace(problem_of(s, dtype));
+  return fast > generic ? fast : generic;
 }
 
 int at_conv2d_bwd_weight(const void* output_grad, const void* input, void* weight_grad, void* workspace,
@@ -333,10 +392,16 @@ int at_conv2d_bwd_weight(const void* output_grad, const void* input, void* weigh
                          at_stream_t stream) {
   if (!output_grad || !input || !weight_grad) return AT_ERR_NULL;
   if (!dtype_valid(dtype)) return AT_ERR_DTYPE;
-  const ConvShape s{batch, in_feat, in_height, in_width, out_feat, kernel_height, kernel_width, stride_height,
-                    stride_width, padding_height, padding_width, groups, out_height, out_width};
+  const ConvShape s = shape_of(batch, in_feat, in_height, in_width, out_feat, out_height, out_width, kernel_height,
+                               kernel_width, stride_height, stride_width, padding_height, padding_width, groups);
   int rc = check_shape(s);
   if (rc) return rc;
+  {
+    const ConvProblem p = problem_of(s, dtype);
+    const int64_t need = conv_igemm_dw_workspace(p);
+    if (need > 0 && workspace && workspace_bytes >= need && aligned16(workspace))
+      return conv_igemm_dw(p, output_grad, input, weight_grad, workspace, (hipStream_t)stream);
+  }
   ConvArgs g = base_args(s);
   const int splits = dw_splits(s);
   const int64_t total = s.O * g.Cg * s.KH * s.KW;

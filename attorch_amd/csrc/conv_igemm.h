@@ -1,0 +1,40 @@
+// Implicit-GEMM convolution on the 16-bit matrix cores (bf16 / fp16, fp32 accumulate).
+//
+// The kernels work on channels-last copies of the activations: with the channel index
+// contiguous, one 16-byte access holds 8 consecutive values of the contraction index, which is
+// what a matrix-core operand wants, and a filter tap outside the image is a whole row of zeros.
+// The tensors of the C ABI stay NCHW; the copies live in caller-provided workspace.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace at_hip {
+
+struct ConvProblem {
+  int64_t N, C, H, W, O, KH, KW, sh, sw, ph, pw, groups, OH, OW;
+  int dtype;   // AT_DTYPE_F16 or AT_DTYPE_BF16 for every tensor
+};
+
+// True when the 16-bit implicit-GEMM kernels cover the problem (channel counts per group in
+// multiples of 64, 32-bit addressable tensors; the input gradient additionally needs stride 1).
+bool conv_igemm_supports_fwd(const ConvProblem& p);
+bool conv_igemm_supports_dx(const ConvProblem& p);
+bool conv_igemm_supports_dw(const ConvProblem& p);
+
+int64_t conv_igemm_fwd_workspace(const ConvProblem& p);
+int64_t conv_igemm_dx_workspace(const ConvProblem& p);
+int64_t conv_igemm_dw_workspace(const ConvProblem& p);
+
+// Y = conv(X, W) + bias, all NCHW.
+int conv_igemm_fwd(const ConvProblem& p, const void* x, const void* w, const void* bias, int bias_dt,
+                   void* y, void* workspace, hipStream_t stream);
+// dX = conv_transpose(dY, W), all NCHW (stride 1 only).
+int conv_igemm_dx(const ConvProblem& p, const void* dy, const void* w, void* dx, void* workspace,
+                  hipStream_t stream);
+// dW[O][C/groups][KH][KW] = correlation of dY with X, all NCHW.
+int conv_igemm_dw(const ConvProblem& p, const void* dy, const void* x, void* dw, void* workspace,
+                  hipStream_t stream);
+
+}  // namespace at_hip

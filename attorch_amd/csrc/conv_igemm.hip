@@ -1,0 +1,645 @@
+// Implicit-GEMM convolution kernels for 16-bit tensors on v_mfma_f32_32x32x16 (see conv_igemm.h).
+//
+//   forward / input gradient (conv_igemm_kernel):
+//     out[(n,oh,ow), co] = sum over taps (kh,kw) and channels c of
+//                          act[n, oh*s+kh-p, ow*s+kw-p, c] * wt[co, (kh,kw), c]
+//     GEMM rows are output pixels, columns output channels, the contraction runs tap-major and
+//     channel-minor; a k-tile of 64 is 64 channels of one tap, so an operand row of the
+//     activations is 128 contiguous bytes of a channels-last pixel (or zeros outside the image).
+//     128 x 64 x 64 tiles, 4 waves, operand tiles straight from global memory into LDS, double
+//     buffered; the finished tile is transposed through LDS and leaves as NCHW rows.
+//     The input gradient is the same product over dY with the taps mirrored and the roles of
+//     the channel counts exchanged (stride 1).
+//   weight gradient (conv_dw_kernel):
+//     dW[co, (kh,kw), c] = sum over pixels of dY[pixel, co] * X[pixel shifted by the tap, c]
+//     Both operands have the contraction index (the pixel) as their row index: they are kept
+//     in LDS as loaded and transposed by the fragment reads (ds_read_b64_tr_b16).  The pixel
+//     range is split over workgroups; fp32 partial tiles are summed in fixed order afterwards.
+#include "conv_igemm.h"
+
+#include <type_traits>
+
+#include "at_mfma.h"
+
+namespace at_hip {
+namespace {
+
+// q = n / d for 0 <= n < 2^31 with one multiply-high and a shift.
+struct FastDiv {
+  uint32_t mul;
+  int shift;   // < 0: d == 1
+  uint32_t d;
+};
+
+inline FastDiv make_fastdiv(int64_t d) {
+  FastDiv f;
+  f.d = (uint32_t)d;
+  if (d <= 1) {
+    f.mul = 0;
+    f.shift = -1;
+    return f;
+  }
+  int l = 0;
+  while (((int64_t)1 << l) < d) ++l;
+  const unsigned __int128 num = (unsigned __int128)1 << (31 + l);
+  f.mul = (uint32_t)((num + (unsigned __int128)d - 1) / (unsigned __int128)d);
+  f.shift = l - 1;
+  return f;
+}
+
+__device__ __forceinline__ int fast_div(int n, const FastDiv& f) {
+  return f.shift < 0 ? n : (int)(__umulhi((uint32_t)n, f.mul) >> f.shift);
+}
+
+// ------------------------------------------------------------------------------------------
+// Layout changes.
+// ------------------------------------------------------------------------------------------
+// [N][C][HW] -> [N][HW][C] through a 64 x 64 LDS tile; 128-bit accesses on both sides when the
+// shapes allow (vec_in: HW % 8 == 0 and aligned source; vec_out: C % 8 == 0 and aligned target).
+template <typename T>
+__global__ __launch_bounds__(256) void nchw_to_nhwc_kernel(const T* __restrict__ src, T* __restrict__ dst,
+                                                            int C, int HW, int vec_in, int vec_out) {
+  __shared__ uint32_t tile[64][33];   // [channel][pixel pair], padded
+  const int n = blockIdx.z;
+  const int c0 = blockIdx.y * 64, p0 = blockIdx.x * 64;
+  const T* s = src + (int64_t)n * C * HW;
+  T* d = dst + (int64_t)n * HW * C;
+  const int t = threadIdx.x;
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int cl = pass * 32 + (t >> 3), pv = (t & 7) * 8;
+    const int c = c0 + cl, p = p0 + pv;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (c < C) {
+      const T* q = s + (int64_t)c * HW + p;
+      if (vec_in && p + 8 <= HW) {
+        v = *reinterpret_cast<const uint4*>(q);
+      } else {
+        union { uint4 raw; T e[8]; } u;
+        u.raw = v;
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (p + e < HW) u.e[e] = q[e];
+        v = u.raw;
+      }
+    }
+    tile[cl][pv / 2 + 0] = v.x;
+    tile[cl][pv / 2 + 1] = v.y;
+    tile[cl][pv / 2 + 2] = v.z;
+    tile[cl][pv / 2 + 3] = v.w;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int pl = pass * 32 + (t >> 3), cv = (t & 7) * 8;
+    const int p = p0 + pl, c = c0 + cv;
+    if (p >= HW || c >= C) continue;
+    uint32_t w[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t lo = tile[cv + 2 * e][pl >> 1], hi = tile[cv + 2 * e + 1][pl >> 1];
+      const int sh = (pl & 1) * 16;
+      w[e] = ((lo >> sh) & 0xffffu) | (((hi >> sh) & 0xffffu) << 16);
+    }
+    T* q = d + (int64_t)p * C + c;
+    if (vec_out && c + 8 <= C) {
+      *reinterpret_cast<uint4*>(q) = make_uint4(w[0], w[1], w[2], w[3]);
+    } else {
+      union { uint32_t raw[4]; T e[8]; } u;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) u.raw[e] = w[e];
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (c + e < C) q[e] = u.e[e];
+    }
+  }
+}
+
+// W[O][Cg][KH][KW] -> wt[rows][taps * cols]:
+//   forward  (flip = 0): wt[o][tap][c]              = W[o][c][tap]               (rows O,  cols Cg)
+//   dX       (flip = 1): wt[g*Cg + c][tap'][o in g] = W[g*Og + o][c][taps-1-tap'] (rows C, cols Og)
+template <typename T>
+__global__ void conv_weight_taps_kernel(const T* __restrict__ w, T* __restrict__ wt, int O, int Cg, int Og,
+                                        int taps, int flip, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  if (!flip) {
+    const int c = (int)(i % Cg);
+    const int tap = (int)((i / Cg) % taps);
+    const int o = (int)(i / ((int64_t)Cg * taps));
+    wt[i] = w[((int64_t)o * Cg + c) * taps + tap];
+  } else {
+    const int ol = (int)(i % Og);
+    const int tap = (int)((i / Og) % taps);
+    const int row = (int)(i / ((int64_t)Og * taps));   // g * Cg + c
+    const int g = row / Cg, c = row - g * Cg;
+    wt[i] = w[(((int64_t)g * Og + ol) * Cg + c) * taps + (taps - 1 - tap)];
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Forward / input-gradient kernel.
+// ------------------------------------------------------------------------------------------
+constexpr int CBM = 128, CBN = 64, CBK = 64;
+constexpr int kCATile = CBM * 128, kCBTile = CBN * 128, kCStage = kCATile + kCBTile;
+constexpr int kCEpiPitch = CBM * 2 + 16;   // bytes per output-channel row of the epilogue tile
+
+struct IgemmArgs {
+  const void* act;    // [N][IH][IW][Ctot]
+  const void* wt;     // [groups * Og][taps * Cg]
+  void* out;          // [N][groups * Og][OH][OW]
+  const void* bias;   // [groups * Og] or null
+  int bias_dt;
+  int IH, IW, Ctot, Cg, Og, KW, OW, OHW, sh, sw, ph, pw;
+  int M;              // N * OH * OW
+  int K;              // taps * Cg
+  int KT;             // K / 64
+  int tiles_per_tap;  // Cg / 64
+  int nbn;            // column tiles per group
+  int vec_store;      // OHW % 8 == 0 and 16-byte aligned output
+  int64_t act_bytes, wt_bytes;
+  FastDiv div_ohw, div_ow;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void conv_igemm_kernel(IgemmArgs g) {
+  __shared__ __attribute__((aligned(1024))) char lds[2 * kCStage];
+  const int grp = blockIdx.z;
+  const int tile_m = blockIdx.x / g.nbn, tile_n = blockIdx.x - tile_m * g.nbn;
+  const int m0 = tile_m * CBM, n0 = tile_n * CBN;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // ---- operand loaders: a wave-wide load fills 8 tile rows of 128 bytes ----
+  const i32x4 ra = make_buffer_rsrc(g.act, g.act_bytes);
+  const i32x4 rb = make_buffer_rsrc(g.wt, g.wt_bytes);
+  int a_ih0[4], a_iw0[4], a_base[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = (wave * 4 + i) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row ^ (row >> 3)) & 7);   // the chunk that belongs at this lane's LDS position
+    const int m = m0 + row;
+    if (m < g.M) {
+      const int n = fast_div(m, g.div_ohw);
+      const int p = m - n * g.OHW;
+      const int oh = fast_div(p, g.div_ow);
+      const int ow = p - oh * g.OW;
+      a_ih0[i] = oh * g.sh - g.ph;
+      a_iw0[i] = ow * g.sw - g.pw;
+      // element offset of the lane's chunk at input pixel (0, 0) of image n
+      a_base[i] = n * g.IH * g.IW * g.Ctot + grp * g.Cg + chunk * 8;
+    } else {
+      a_ih0[i] = -(1 << 24);   // never inside the image
+      a_iw0[i] = 0;
+      a_base[i] = 0;
+    }
+  }
+  int b_off[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = (wave * 2 + i) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row ^ (row >> 3)) & 7);
+    const int co = n0 + row;
+    b_off[i] = co < g.Og ? ((grp * g.Og + co) * g.K + chunk * 8) * 2 : kOobOffset;
+  }
+
+  // k-tile to issue next: tap (kh, kw) and first channel
+  int nk_kh = 0, nk_kw = 0, nk_ct = 0, nk = 0;
+  auto issue = [&](char* stage) {
+    const int cb = nk_ct * 64;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int ih = a_ih0[i] + nk_kh, iw = a_iw0[i] + nk_kw;
+      const bool ok = (unsigned)ih < (unsigned)g.IH && (unsigned)iw < (unsigned)g.IW;
+      const int off = (a_base[i] + (ih * g.IW + iw) * g.Ctot + cb) * 2;
+      lds_dma_16(ra, ok ? off : kOobOffset, stage + (wave * 4 + i) * 1024);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      lds_dma_16(rb, b_off[i] == kOobOffset ? kOobOffset : b_off[i] + nk * (CBK * 2),
+                 stage + kCATile + (wave * 2 + i) * 1024);
+    ++nk;
+    if (++nk_ct == g.tiles_per_tap) {
+      nk_ct = 0;
+      if (++nk_kw == g.KW) {
+        nk_kw = 0;
+        ++nk_kh;
+      }
+    }
+  };
+
+  f32x16 acc[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[t][e] = 0.f;
+
+  issue(lds);
+  lds_dma_wait_all();
+  __syncthreads();
+  for (int kt = 0; kt < g.KT; ++kt) {
+    const char* cur = lds + (kt & 1) * kCStage;
+    char* nxt = lds + ((kt & 1) ^ 1) * kCStage;
+    if (kt + 1 < g.KT) issue(nxt);
+#pragma unroll
+    for (int ks = 0; ks < CBK / 16; ++ks) {
+      const uint4 a0 = read_frag_kc(cur, wm * 64, ks);
+      const uint4 a1 = read_frag_kc(cur, wm * 64 + 32, ks);
+      const uint4 b = read_frag_kc(cur + kCATile, wn * 32, ks);
+      acc[0] = Mfma16<T>::run(a0, b, acc[0]);
+      acc[1] = Mfma16<T>::run(a1, b, acc[1]);
+    }
+    lds_dma_wait_all();   // this wave's part of the next stage has landed
+    __syncthreads();      // ... and everybody else's; the current stage may be overwritten
+  }
+
+  // ---- epilogue: lane holds, for tile t and register r, pixel wm*64 + t*32 + (r/4)*8 +
+  // (lane/32)*4 + r%4 of output channel wn*32 + lane%32; the tile goes through LDS as
+  // [channel][pixel] and leaves as runs of 8 pixels of one channel (NCHW rows) ----
+  T* __restrict__ out = reinterpret_cast<T*>(g.out);
+  {
+    const int col = wn * 32 + (lane & 31);
+    float bv = 0.f;
+    if (g.bias && n0 + col < g.Og) bv = load_scalar_f32(g.bias, g.bias_dt, grp * g.Og + n0 + col);
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = acc[t][rg * 4 + e] + bv;
+        const int pix = wm * 64 + t * 32 + rg * 8 + (lane >> 5) * 4;
+        store_f32<T, 4>(reinterpret_cast<T*>(lds + col * kCEpiPitch) + pix, v);
+      }
+  }
+  __syncthreads();
+  const int Otot = g.Og * (int)gridDim.z;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    const int id = threadIdx.x + 256 * s;
+    const int col = id >> 4, pc = id & 15;
+    const int co = n0 + col, m = m0 + pc * 8;
+    if (co >= g.Og || m >= g.M) continue;
+    const uint4 v = *reinterpret_cast<const uint4*>(lds + col * kCEpiPitch + pc * 16);
+    if (g.vec_store) {
+      const int n = fast_div(m, g.div_ohw);
+      const int p = m - n * g.OHW;
+      *reinterpret_cast<uint4*>(out + ((int64_t)n * Otot + grp * g.Og + co) * g.OHW + p) = v;
+    } else {
+      union { uint4 raw; T e[8]; } u;
+      u.raw = v;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int mm = m + e;
+        if (mm < g.M) {
+          const int n = fast_div(mm, g.div_ohw);
+          const int p = mm - n * g.OHW;
+          out[((int64_t)n * Otot + grp * g.Og + co) * g.OHW + p] = u.e[e];
+        }
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Weight-gradient kernel.
+// ------------------------------------------------------------------------------------------
+// Operand tile in LDS: 64 pixel rows x 128 bytes (64 channels) as loaded, the 16-byte chunk
+// index XORed with 2 * (row % 4): the four consecutive rows a transposing read touches then
+// sit in four different 32-byte bank groups.
+__device__ __forceinline__ int dw_chunk_swizzle(int row) { return (row & 3) << 1; }
+
+// Fragment of 32 channels x 16 pixels for one MFMA operand: 8 consecutive pixels per lane.
+// ds_read_b64_tr_b16: within 16 lanes, result[l][e] = source[4e + l/4][l%4]; source lane 4e + q
+// points at pixel row (k0 + e), channels 4q .. 4q+3, and lane l receives k0 .. k0+3 of channel l.
+__device__ __forceinline__ uint4 read_frag_tr(const char* tile, int ch_base, int ks) {
+  const int lane = threadIdx.x & 63;
+  const int i = lane & 15, gq = lane >> 4;
+  const int byte = (ch_base + (gq & 1) * 16 + (i & 3) * 4) * 2;
+  const int krow = ks * 16 + (gq >> 1) * 8 + (i >> 2);
+  const int krow1 = krow + 4;   // same row % 4: same swizzle
+  const int inrow = (((byte >> 4) ^ dw_chunk_swizzle(krow)) << 4) + (byte & 15);
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(tile + krow * 128 + inrow));
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(tile + krow1 * 128 + inrow));
+  const uint2 a = __builtin_bit_cast(uint2, lo), b = __builtin_bit_cast(uint2, hi);
+  return make_uint4(a.x, a.y, b.x, b.y);
+}
+
+constexpr int kDwTile = 64 * 128;        // one operand tile: 64 pixels x 64 channels
+constexpr int kDwStage = 2 * kDwTile;
+
+struct DwArgs {
+  const void* dy;     // [N*OH*OW][Otot]
+  const void* x;      // [N][H][W][Ctot]
+  float* part;        // [splits][Otot][taps * Cg]
+  int H, W, Ctot, Otot, Cg, Og, KW, OW, OHW, sh, sw, ph, pw;
+  int P;              // N * OH * OW
+  int K;              // taps * Cg
+  int tiles_per_tap;  // Cg / 64
+  int nbn;            // column tiles (taps * Cg / 64)
+  int p_per_split;    // pixels per split, a multiple of 64
+  int64_t dy_bytes, x_bytes;
+  FastDiv div_ohw, div_ow;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void conv_dw_kernel(DwArgs g) {
+  __shared__ __attribute__((aligned(1024))) char lds[2 * kDwStage];
+  const int grp = blockIdx.z, split = blockIdx.y;
+  const int tile_m = blockIdx.x / g.nbn, tile_n = blockIdx.x - tile_m * g.nbn;
+  const int co0 = tile_m * 64;                               // within the group
+  const int tap = tile_n / g.tiles_per_tap;
+  const int c0 = (tile_n - tap * g.tiles_per_tap) * 64;      // within the group
+  const int kh = tap / g.KW, kw = tap - kh * g.KW;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  const int p_begin = split * g.p_per_split;
+  const int p_end = p_begin + g.p_per_split < g.P ? p_begin + g.p_per_split : g.P;
+  const int KT = (p_end - p_begin + 63) / 64;
+
+  const i32x4 ra = make_buffer_rsrc(g.dy, g.dy_bytes);
+  const i32x4 rb = make_buffer_rsrc(g.x, g.x_bytes);
+  // a wave-wide load fills 8 pixel rows; lane -> (row, position), fetching the chunk that belongs there
+  int row_l[2], a_col[2], b_col[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = (wave * 2 + i) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ dw_chunk_swizzle(row);
+    row_l[i] = row;
+    // channels past the end of the group read as zeros (their products are never stored)
+    a_col[i] = co0 + chunk * 8 < g.Og ? grp * g.Og + co0 + chunk * 8 : -1;
+    b_col[i] = c0 + chunk * 8 < g.Cg ? grp * g.Cg + c0 + chunk * 8 : -1;
+  }
+
+  auto issue = [&](int kt, char* stage) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int p = p_begin + kt * 64 + row_l[i];
+      const bool live = p < p_end;
+      int offa = kOobOffset, offb = kOobOffset;
+      if (live) {
+        if (a_col[i] >= 0) offa = (p * g.Otot + a_col[i]) * 2;
+        const int n = fast_div(p, g.div_ohw);
+        const int q = p - n * g.OHW;
+        const int oh = fast_div(q, g.div_ow);
+        const int ow = q - oh * g.OW;
+        const int ih = oh * g.sh - g.ph + kh, iw = ow * g.sw - g.pw + kw;
+        if (b_col[i] >= 0 && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W)
+          offb = (((n * g.H + ih) * g.W + iw) * g.Ctot + b_col[i]) * 2;
+      }
+      lds_dma_16(ra, offa, stage + (wave * 2 + i) * 1024);
+      lds_dma_16(rb, offb, stage + kDwTile + (wave * 2 + i) * 1024);
+    }
+  };
+
+  f32x16 acc;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+
+  if (KT > 0) {
+    issue(0, lds);
+    lds_dma_wait_all();
+  }
+  __syncthreads();
+  for (int kt = 0; kt < KT; ++kt) {
+    const char* cur = lds + (kt & 1) * kDwStage;
+    char* nxt = lds + ((kt & 1) ^ 1) * kDwStage;
+    if (kt + 1 < KT) issue(kt + 1, nxt);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const uint4 a = read_frag_tr(cur, wm * 32, ks);
+      const uint4 b = read_frag_tr(cur + kDwTile, wn * 32, ks);
+      acc = Mfma16<T>::run(a, b, acc);
+    }
+    lds_dma_wait_all();
+    __syncthreads();
+  }
+
+  // lane holds, in register r, output channel wm*32 + (r/4)*8 + (lane/32)*4 + r%4 and column
+  // wn*32 + lane%32: 32 lanes write 32 consecutive floats of one partial row
+  float* part = g.part + (int64_t)split * g.Otot * g.K;
+  const int c = c0 + wn * 32 + (lane & 31);
+  if (c < g.Cg) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int co = co0 + wm * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+      if (co < g.Og) part[(int64_t)(grp * g.Og + co) * g.K + tap * g.Cg + c] = acc[r];
+    }
+  }
+}
+
+// dW[o][c][tap] = sum over splits of part[split][o][tap * Cg + c], fixed order.  A workgroup
+// owns 64 consecutive partial columns; its four waves each sum every fourth split.
+template <typename T>
+__global__ __launch_bounds__(256) void conv_dw_finish_kernel(const float* __restrict__ part, T* __restrict__ dw,
+                                                              int splits, int Cg, int taps, int64_t total) {
+  __shared__ float sm[4][64];
+  const int col = threadIdx.x & 63, slice = threadIdx.x >> 6;
+  const int64_t i = (int64_t)blockIdx.x * 64 + col;   // index into a partial: (o, tap, c)
+  float s = 0.f;
+  if (i < total) {
+#pragma unroll 4
+    for (int sp = slice; sp < splits; sp += 4) s += part[(int64_t)sp * total + i];
+  }
+  sm[slice][col] = s;
+  __syncthreads();
+  if (slice == 0 && i < total) {
+    s = (sm[0][col] + sm[1][col]) + (sm[2][col] + sm[3][col]);
+    const int c = (int)(i % Cg);
+    const int tap = (int)((i / Cg) % taps);
+    const int64_t o = i / ((int64_t)Cg * taps);
+    dw[(o * Cg + c) * taps + tap] = from_f32<T>(s);
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Host side.
+// ------------------------------------------------------------------------------------------
+constexpr int64_t kMaxBytes = (int64_t)1 << 31;   // 32-bit buffer offsets
+constexpr int kDwMaxSplits = 256;
+
+inline int64_t round256(int64_t v) { return (v + 255) & ~(int64_t)255; }
+inline bool is16(int dt) { return dt == AT_DTYPE_F16 || dt == AT_DTYPE_BF16; }
+
+template <typename F>
+inline int dispatch16(int dt, F&& f) {
+  if (dt == AT_DTYPE_F16) return f((f16_t*)0);
+  if (dt == AT_DTYPE_BF16) return f((bf16_t*)0);
+  return AT_ERR_DTYPE;
+}
+
+inline bool sizes_ok(const ConvProblem& p) {
+  const int64_t x_bytes = p.N * p.C * p.H * p.W * 2, y_bytes = p.N * p.O * p.OH * p.OW * 2;
+  const int64_t w_bytes = p.O * (p.C / p.groups) * p.KH * p.KW * 2;
+  return x_bytes < kMaxBytes && y_bytes < kMaxBytes && w_bytes < kMaxBytes && p.groups <= 65535 &&
+         p.N <= 65535;
+}
+
+int to_nhwc(const void* src, void* dst, int64_t N, int64_t C, int64_t HW, int dt, hipStream_t stream) {
+  const int vec_in = (HW % 8 == 0) && aligned16(src);
+  const int vec_out = (C % 8 == 0) && aligned16(dst);
+  const dim3 grid((unsigned)cdiv64(HW, 64), (unsigned)cdiv64(C, 64), (unsigned)N);
+  return dispatch16(dt, [&](auto* tp) -> int {
+    typedef std::remove_pointer_t<decltype(tp)> T;
+    hipLaunchKernelGGL((nchw_to_nhwc_kernel<T>), grid, dim3(256), 0, stream, (const T*)src, (T*)dst, (int)C,
+                       (int)HW, vec_in, vec_out);
+    return launch_status();
+  });
+}
+
+int weight_taps(const void* w, void* wt, const ConvProblem& p, int flip, hipStream_t stream) {
+  const int64_t total = p.O * (p.C / p.groups) * p.KH * p.KW;
+  return dispatch16(p.dtype, [&](auto* tp) -> int {
+    typedef std::remove_pointer_t<decltype(tp)> T;
+    hipLaunchKernelGGL((conv_weight_taps_kernel<T>), dim3((unsigned)cdiv64(total, 256)), dim3(256), 0, stream,
+                       (const T*)w, (T*)wt, (int)p.O, (int)(p.C / p.groups), (int)(p.O / p.groups),
+                       (int)(p.KH * p.KW), flip, total);
+    return launch_status();
+  });
+}
+
+// One product out[(n,oh,ow), co] over channels-last `act`; see IgemmArgs for the meaning of the fields.
+int run_igemm(IgemmArgs g, int64_t n_img, int64_t OH, int groups, int dt, hipStream_t stream) {
+  g.OHW = (int)(OH * g.OW);
+  g.M = (int)(n_img * g.OHW);
+  g.K = g.KT * 64;
+  g.tiles_per_tap = g.Cg / 64;
+  g.nbn = (int)cdiv64(g.Og, CBN);
+  g.vec_store = (g.OHW % 8 == 0) && aligned16(g.out);
+  g.div_ohw = make_fastdiv(g.OHW);
+  g.div_ow = make_fastdiv(g.OW);
+  const dim3 grid((unsigned)(cdiv64(g.M, CBM) * g.nbn), 1, (unsigned)groups);
+  return dispatch16(dt, [&](auto* tp) -> int {
+    typedef std::remove_pointer_t<decltype(tp)> T;
+    hipLaunchKernelGGL((conv_igemm_kernel<T>), grid, dim3(256), 0, stream, g);
+    return launch_status();
+  });
+}
+
+}  // namespace
+
+bool conv_igemm_supports_fwd(const ConvProblem& p) {
+  return is16(p.dtype) && (p.C / p.groups) % 64 == 0 && sizes_ok(p) && p.N * p.OH * p.OW < kMaxBytes;
+}
+
+bool conv_igemm_supports_dx(const ConvProblem& p) {
+  return is16(p.dtype) && (p.O / p.groups) % 64 == 0 && sizes_ok(p) && p.sh == 1 && p.sw == 1 &&
+         p.ph <= p.KH - 1 && p.pw <= p.KW - 1 && p.N * p.H * p.W < kMaxBytes;
+}
+
+bool conv_igemm_supports_dw(const ConvProblem& p) {
+  return is16(p.dtype) && (p.C / p.groups) % 8 == 0 && (p.O / p.groups) % 8 == 0 && sizes_ok(p) &&
+         p.N * p.OH * p.OW < kMaxBytes - 64 * kDwMaxSplits;
+}
+
+int64_t conv_igemm_fwd_workspace(const ConvProblem& p) {
+  if (!conv_igemm_supports_fwd(p)) return 0;
+  return round256(p.N * p.C * p.H * p.W * 2) + round256(p.O * (p.C / p.groups) * p.KH * p.KW * 2);
+}
+
+int64_t conv_igemm_dx_workspace(const ConvProblem& p) {
+  if (!conv_igemm_supports_dx(p)) return 0;
+  return round256(p.N * p.O * p.OH * p.OW * 2) + round256(p.O * (p.C / p.groups) * p.KH * p.KW * 2);
+}
+
+namespace {
+inline int dw_split_count(const ConvProblem& p) {
+  const int64_t P = p.N * p.OH * p.OW;
+  const int64_t tiles = cdiv64(p.O / p.groups, 64) * (p.KH * p.KW * cdiv64(p.C / p.groups, 64)) * p.groups;
+  int64_t want = cdiv64((int64_t)device_cu_count() * 4, tiles);
+  const int64_t by_len = cdiv64(P, 256);   // at least four k-tiles per split
+  if (want > by_len) want = by_len;
+  if (want > kDwMaxSplits) want = kDwMaxSplits;
+  return (int)(want < 1 ? 1 : want);
+}
+inline int64_t dw_padded_k(const ConvProblem& p) { return p.KH * p.KW * (p.C / p.groups); }
+}  // namespace
+
+int64_t conv_igemm_dw_workspace(const ConvProblem& p) {
+  if (!conv_igemm_supports_dw(p)) return 0;
+  return round256(p.N * p.O * p.OH * p.OW * 2) + round256(p.N * p.C * p.H * p.W * 2) +
+         round256((int64_t)kDwMaxSplits * p.O * dw_padded_k(p) * 4);
+}
+
+int conv_igemm_fwd(const ConvProblem& p, const void* x, const void* w, const void* bias, int bias_dt,
+                   void* y, void* workspace, hipStream_t stream) {
+  char* ws = static_cast<char*>(workspace);
+  void* xh = ws;
+  void* wt = ws + round256(p.N * p.C * p.H * p.W * 2);
+  int rc = to_nhwc(x, xh, p.N, p.C, p.H * p.W, p.dtype, stream);
+  if (rc) return rc;
+  rc = weight_taps(w, wt, p, 0, stream);
+  if (rc) return rc;
+  IgemmArgs g{};
+  g.act = xh; g.wt = wt; g.out = y; g.bias = bias; g.bias_dt = bias_dt;
+  g.IH = (int)p.H; g.IW = (int)p.W; g.Ctot = (int)p.C; g.Cg = (int)(p.C / p.groups); g.Og = (int)(p.O / p.groups);
+  g.KW = (int)p.KW; g.OW = (int)p.OW; g.sh = (int)p.sh; g.sw = (int)p.sw; g.ph = (int)p.ph; g.pw = (int)p.pw;
+  g.KT = (int)(p.KH * p.KW * (g.Cg / 64));
+  g.act_bytes = p.N * p.C * p.H * p.W * 2;
+  g.wt_bytes = p.O * g.Cg * p.KH * p.KW * 2;
+  return run_igemm(g, p.N, p.OH, (int)p.groups, p.dtype, stream);
+}
+
+int conv_igemm_dx(const ConvProblem& p, const void* dy, const void* w, void* dx, void* workspace,
+                  hipStream_t stream) {
+  char* ws = static_cast<char*>(workspace);
+  void* dyh = ws;
+  void* wt = ws + round256(p.N * p.O * p.OH * p.OW * 2);
+  int rc = to_nhwc(dy, dyh, p.N, p.O, p.OH * p.OW, p.dtype, stream);
+  if (rc) return rc;
+  rc = weight_taps(w, wt, p, 1, stream);
+  if (rc) return rc;
+  // dX[n, c, ih, iw] = sum_{taps', o} dY[n, ih + kh' - (KH-1-ph), iw + kw' - (KW-1-pw), o] * W[o, c, mirrored tap]
+  IgemmArgs g{};
+  g.act = dyh; g.wt = wt; g.out = dx; g.bias = nullptr; g.bias_dt = 0;
+  g.IH = (int)p.OH; g.IW = (int)p.OW; g.Ctot = (int)p.O; g.Cg = (int)(p.O / p.groups); g.Og = (int)(p.C / p.groups);
+  g.KW = (int)p.KW; g.OW = (int)p.W; g.sh = 1; g.sw = 1; g.ph = (int)(p.KH - 1 - p.ph); g.pw = (int)(p.KW - 1 - p.pw);
+  g.KT = (int)(p.KH * p.KW * (g.Cg / 64));
+  g.act_bytes = p.N * p.O * p.OH * p.OW * 2;
+  g.wt_bytes = p.O * (p.C / p.groups) * p.KH * p.KW * 2;
+  return run_igemm(g, p.N, p.H, (int)p.groups, p.dtype, stream);
+}
+
+int conv_igemm_dw(const ConvProblem& p, const void* dy, const void* x, void* dw, void* workspace,
+                  hipStream_t stream) {
+  char* ws = static_cast<char*>(workspace);
+  void* dyh = ws;
+  void* xh = ws + round256(p.N * p.O * p.OH * p.OW * 2);
+  float* part = reinterpret_cast<float*>(ws + round256(p.N * p.O * p.OH * p.OW * 2) +
+                                         round256(p.N * p.C * p.H * p.W * 2));
+  int rc = to_nhwc(dy, dyh, p.N, p.O, p.OH * p.OW, p.dtype, stream);
+  if (rc) return rc;
+  rc = to_nhwc(x, xh, p.N, p.C, p.H * p.W, p.dtype, stream);
+  if (rc) return rc;
+  DwArgs g{};
+  g.dy = dyh; g.x = xh; g.part = part;
+  g.H = (int)p.H; g.W = (int)p.W; g.Ctot = (int)p.C; g.Otot = (int)p.O; g.Cg = (int)(p.C / p.groups);
+  g.Og = (int)(p.O / p.groups); g.KW = (int)p.KW; g.OW = (int)p.OW; g.OHW = (int)(p.OH * p.OW);
+  g.sh = (int)p.sh; g.sw = (int)p.sw; g.ph = (int)p.ph; g.pw = (int)p.pw;
+  g.P = (int)(p.N * p.OH * p.OW);
+  g.K = (int)dw_padded_k(p);
+  g.tiles_per_tap = (int)cdiv64(g.Cg, 64);
+  g.nbn = (int)(p.KH * p.KW) * g.tiles_per_tap;
+  const int splits = dw_split_count(p);
+  g.p_per_split = (int)(cdiv64(cdiv64(g.P, splits), 64) * 64);
+  g.dy_bytes = p.N * p.O * p.OH * p.OW * 2;
+  g.x_bytes = p.N * p.C * p.H * p.W * 2;
+  g.div_ohw = make_fastdiv(g.OHW);
+  g.div_ow = make_fastdiv(g.OW);
+  const int real_splits = (int)cdiv64(g.P, g.p_per_split);
+  const dim3 grid((unsigned)(cdiv64(g.Og, 64) * g.nbn), (unsigned)real_splits, (unsigned)p.groups);
+  const int64_t total = p.O * (int64_t)g.K;
+  return dispatch16(p.dtype, [&](auto* tp) -> int {
+    typedef std::remove_pointer_t<decltype(tp)> T;
+    hipLaunchKernelGGL((conv_dw_kernel<T>), grid, dim3(256), 0, stream, g);
+    int rc2 = launch_status();
+    if (rc2) return rc2;
+    hipLaunchKernelGGL((conv_dw_finish_kernel<T>), dim3((unsigned)cdiv64(total, 64)), dim3(256), 0, stream,
+                       (const float*)part, (T*)dw, real_splits, g.Cg, (int)(p.KH * p.KW), total);
+    return launch_status();
+  });
+}
+
+}  // namespace at_hip

@@ -3,12 +3,14 @@
 // Two kernels:
 //  * gemm_mfma16_kernel — bf16/fp16 operands on v_mfma_f32_32x32x16 (MFMA-bound).  256x256x64
 //    macro-tile per 256-lane workgroup (4 waves, 128x128 each, 256 accumulator registers per
-//    lane), LDS double-buffered (2 x 64 KiB), one barrier per k-tile, global loads of tile
-//    k+1 in flight while tile k is multiplied.  LDS tiles are [row][k] with the 16-byte chunk
-//    index XOR-swizzled by the row, so both the 128-bit fragment reads and the tile writes are
-//    bank-conflict free.  Operands whose contraction index is not the contiguous one in
-//    memory (W in the forward product, X and dZ in the weight gradient) are transposed 8x8 in
-//    registers (byte permutes) between the global load and the LDS write.  Workgroup ids are
+//    lane), LDS double-buffered, one barrier per k-tile.  Tiles go from global memory straight
+//    into LDS (buffer_load ... lds), the loads of tile k+1 in flight while tile k is
+//    multiplied.  An operand whose contraction index is contiguous in memory is kept as
+//    [row][k] with the 16-byte chunk index XOR-swizzled by the row (bank-conflict-free 128-bit
+//    fragment reads); an operand stored the other way round (W in the forward product, X and
+//    dZ in the weight gradient) is kept as loaded and transposed by the fragment reads
+//    themselves (ds_read_b64_tr_b16).  Fragments are double-buffered in registers, and the
+//    finished tile leaves through LDS as whole 512-byte row segments.  Workgroup ids are
 //    remapped so that each XCD (own L2) works on a compact block of output tiles.
 //  * gemm_simple_kernel — any dtype, any strides, fp32 MFMA (32x32x2), 64x64 tile; used for
 //    fp32 tensors and for 16-bit shapes the fast kernel cannot address with 128-bit accesses.
@@ -16,14 +18,10 @@
 #include <type_traits>
 
 #include "at_act.h"
-#include "at_common.h"
+#include "at_mfma.h"
 
 namespace at_hip {
 namespace {
-
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
 struct GemmArgs {
   const void* a;      // A(m, k)
@@ -38,36 +36,13 @@ struct GemmArgs {
   int bias_dt;
 };
 
-template <typename T> struct Mfma16;
-template <> struct Mfma16<bf16_t> {
-  static __device__ __forceinline__ f32x16 run(const uint4& a, const uint4& b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
-                                                   c, 0, 0, 0);
-  }
-};
-template <> struct Mfma16<f16_t> {
-  static __device__ __forceinline__ f32x16 run(const uint4& a, const uint4& b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b),
-                                                  c, 0, 0, 0);
-  }
-};
-
 constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int kGemmThreads = 256;
 constexpr int kTileBytes = BM * BK * 2;  // one operand tile, 32 KiB
 constexpr int kEpiPitch = BN * 2 + 16;   // bytes per row of the epilogue tile in LDS (padded against bank conflicts)
 constexpr int kEpiBytes = BM * kEpiPitch;
 
-__device__ __forceinline__ bool aligned16_dev(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
-
-// Byte offset of 16-byte chunk `chunk` (0..7) of row `row` inside a [256][64] 16-bit tile.
-__device__ __forceinline__ int lds_chunk_offset(int row, int chunk) {
-  return row * (BK * 2) + ((chunk ^ ((row ^ (row >> 3)) & 7)) << 4);
-}
-
-typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void lds_void_t;
-constexpr int kOobOffset = (int)0x80000000u;  // beyond any buffer this kernel accepts (< 2 GiB)
 
 // LDS image of one operand tile of a k-tile.
 //  * CONTRACT_CONTIG (memory [outer][k]): 256 rows x 128 bytes, 16-byte chunks XOR-swizzled by
@@ -78,24 +53,6 @@ constexpr int kOobOffset = (int)0x80000000u;  // beyond any buffer this kernel a
 constexpr int kPairPitch = 1024 + 64;
 template <bool CONTRACT_CONTIG> constexpr int operand_tile_bytes() { return CONTRACT_CONTIG ? kTileBytes : 32 * kPairPitch; }
 
-// Global -> LDS without passing through registers (buffer_load ... lds): each wave-wide load
-// moves 64 lanes x 16 bytes into one contiguous KiB of LDS, each lane choosing its own global
-// address.  Buffer addressing gives zero fill for rows past the end of the tensor.
-// The loads are issued as inline assembly on purpose: the compiler cannot tell that a load into
-// one LDS stage does not alias the fragment reads of the other stage and would otherwise wait
-// for every outstanding load (vmcnt(0)) before the next LDS read.  The kernel waits for them
-// itself, once, before the barrier that publishes the stage.
-typedef int i32x4 __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ void lds_dma_16(const i32x4& rsrc, int byte_offset, const char* lds_dst) {
-  // LDS byte address of lane 0's 16 bytes; wave-uniform by construction, made so for the compiler
-  const unsigned m0 = (unsigned)__builtin_amdgcn_readfirstlane((int)(uintptr_t)lds_dst);
-  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(m0), "v"(byte_offset), "s"(rsrc)
-               : "m0");
-}
-
-__device__ __forceinline__ void lds_dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-
 template <typename T, bool CONTRACT_CONTIG>
 struct OperandLoader {
   i32x4 rsrc;
@@ -105,21 +62,11 @@ struct OperandLoader {
   int k_lane;     // k of this lane inside a k-tile (contract-contiguous layout only)
   int K;
 
-  static __device__ __forceinline__ i32x4 make_rsrc(const void* base, int64_t bytes) {
-    const uint64_t addr = reinterpret_cast<uint64_t>(base);
-    i32x4 r;
-    r.x = (int)(uint32_t)addr;
-    r.y = (int)(uint32_t)((addr >> 32) & 0xffffu);   // stride 0: raw buffer
-    r.z = (int)bytes;                                  // num_records in bytes
-    r.w = 0x00020000;                                  // 32-bit untyped data format
-    return r;
-  }
-
   __device__ __forceinline__ void init(const T* base, int64_t ld, int outer0, int outer_total, int K_) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     K = K_;
     if (CONTRACT_CONTIG) {
-      rsrc = make_rsrc(base, outer_total * ld * 2);
+      rsrc = make_buffer_rsrc(base, outer_total * ld * 2);
       // load i of wave w fills rows 8q .. 8q+7 (q = 8w + i); lane -> (row, position), and the
       // position holds chunk (position ^ swizzle(row)) so that the reads find chunk c at c ^ swizzle
       const int row = wave * 64 + (lane >> 3);            // + 8 i
@@ -128,7 +75,7 @@ struct OperandLoader {
       blk_step = (int)(8 * ld * 2);
       k_step = BK * 2;
     } else {
-      rsrc = make_rsrc(base, K_ * ld * 2);
+      rsrc = make_buffer_rsrc(base, K_ * ld * 2);
       // load i of wave w fills k-rows 2q, 2q+1 (q = 8w + i); lane -> k-row 2q + lane/32, 8 columns at (lane%32)*8
       const int krow = wave * 16 + (lane >> 5);            // + 2 i
       k_lane = 0;
@@ -171,7 +118,7 @@ template <bool CONTRACT_CONTIG>
 __device__ __forceinline__ uint4 read_frag(const char* tile, int outer_base, int ks) {
   const int lane = threadIdx.x & 63;
   if (CONTRACT_CONTIG) {
-    return *reinterpret_cast<const uint4*>(tile + lds_chunk_offset(outer_base + (lane & 31), ks * 2 + (lane >> 5)));
+    return read_frag_kc(tile, outer_base, ks);
   } else {
     // ds_read_b64_tr_b16: within 16 lanes, result[l][e] = source[4e + l/4][l%4]; the source lane
     // 4e + q therefore points at k-row (k0 + e), columns 4q .. 4q+3, and lane l receives

@@ -413,9 +413,12 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
     wg, bg = torch.empty(c, device='cuda'), torch.empty(c, device='cuda')
     bn_wsb = lib.at_batch_norm_workspace_bytes(c)
     bn_ws = torch.empty(bn_wsb, dtype=torch.uint8, device='cuda')
-    cw_wsb = lib.at_conv2d_bwd_weight_workspace_bytes(c, c, 3, 3)
-    cw_ws = torch.empty(cw_wsb, dtype=torch.uint8, device='cuda')
     dims = (n, c, h, w_, c, h, w_, 3, 3, 1, 1, 1, 1, 1)
+    cf_wsb = lib.at_conv2d_fwd_workspace_bytes(*dims, dt, dt)
+    cx_wsb = lib.at_conv2d_bwd_input_workspace_bytes(*dims, dt)
+    cw_wsb = lib.at_conv2d_bwd_weight_workspace_bytes(*dims, dt)
+    conv_wsb = max(cf_wsb, cx_wsb, cw_wsb, 16)
+    conv_ws = torch.empty(conv_wsb, dtype=torch.uint8, device='cuda')
     st = raw.stream
     counter = [0]
 
@@ -425,18 +428,18 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
 
     def conv_f():
         i = nxt()
-        raw.check(lib.at_conv2d_fwd(xs[i].data_ptr(), wt.data_ptr(), None, ys[i].data_ptr(), *dims, dt, dt, dt,
-                                    st()), 'conv_fwd')
+        raw.check(lib.at_conv2d_fwd(xs[i].data_ptr(), wt.data_ptr(), None, ys[i].data_ptr(), conv_ws.data_ptr(),
+                                    conv_wsb, *dims, dt, dt, dt, st()), 'conv_fwd')
 
     def conv_dx():
         i = nxt()
-        raw.check(lib.at_conv2d_bwd_input(dys[i].data_ptr(), wt.data_ptr(), dxs[i].data_ptr(), *dims, dt, st()),
-                  'conv_dx')
+        raw.check(lib.at_conv2d_bwd_input(dys[i].data_ptr(), wt.data_ptr(), dxs[i].data_ptr(), conv_ws.data_ptr(),
+                                          conv_wsb, *dims, dt, st()), 'conv_dx')
 
     def conv_dw():
         i = nxt()
-        raw.check(lib.at_conv2d_bwd_weight(dys[i].data_ptr(), xs[i].data_ptr(), dwt.data_ptr(), cw_ws.data_ptr(),
-                                           cw_wsb, *dims, dt, st()), 'conv_dw')
+        raw.check(lib.at_conv2d_bwd_weight(dys[i].data_ptr(), xs[i].data_ptr(), dwt.data_ptr(), conv_ws.data_ptr(),
+                                           conv_wsb, *dims, dt, st()), 'conv_dw')
 
     def bn_f():
         i = nxt()

@@ -262,25 +262,52 @@ int at_batch_norm_bwd(const void* output_grad, const void* pre_act, const void* 
  * [out_feat, in_feat / groups, kernel_height, kernel_width], output
  * [batch, out_feat, out_height, out_width] with out = (in + 2*padding - kernel) / stride + 1
  * (conv_layer.py:18-36), which the call checks.  bias nullable.
- *   bwd_weight needs at_conv2d_bwd_weight_workspace_bytes(...) bytes (split-K partials).
+ *   Workspace: 16-bit tensors with channel counts per group in multiples of 64 run on the
+ *   matrix cores from channels-last copies kept in caller-provided workspace; each
+ *   at_conv2d_*_workspace_bytes(...) returns the bytes that path wants for the given shape
+ *   (0: no such path).  forward and bwd_input fall back to the generic kernel when the
+ *   workspace is null or smaller; bwd_weight always needs its workspace (split-K partials).
  *   at_channel_sum: out[feat] = sum over batch and space of a [batch, feat, spatial] tensor.
  * ------------------------------------------------------------------------------------------ */
+int64_t at_conv2d_fwd_workspace_bytes(int64_t batch, int64_t in_feat, int64_t in_height,
+                                      int64_t in_width, int64_t out_feat, int64_t out_height,
+                                      int64_t out_width, int64_t kernel_height,
+                                      int64_t kernel_width, int64_t stride_height,
+                                      int64_t stride_width, int64_t padding_height,
+                                      int64_t padding_width, int64_t groups, int in_dtype,
+                                      int out_dtype);
+
 int at_conv2d_fwd(const void* input, const void* weight, const void* bias, void* output,
-                  int64_t batch, int64_t in_feat, int64_t in_height, int64_t in_width,
-                  int64_t out_feat, int64_t out_height, int64_t out_width, int64_t kernel_height,
-                  int64_t kernel_width, int64_t stride_height, int64_t stride_width,
-                  int64_t padding_height, int64_t padding_width, int64_t groups, int in_dtype,
-                  int bias_dtype, int out_dtype, at_stream_t stream);
+                  void* workspace, int64_t workspace_bytes, int64_t batch, int64_t in_feat,
+                  int64_t in_height, int64_t in_width, int64_t out_feat, int64_t out_height,
+                  int64_t out_width, int64_t kernel_height, int64_t kernel_width,
+                  int64_t stride_height, int64_t stride_width, int64_t padding_height,
+                  int64_t padding_width, int64_t groups, int in_dtype, int bias_dtype,
+                  int out_dtype, at_stream_t stream);
+
+int64_t at_conv2d_bwd_input_workspace_bytes(int64_t batch, int64_t in_feat, int64_t in_height,
+                                            int64_t in_width, int64_t out_feat,
+                                            int64_t out_height, int64_t out_width,
+                                            int64_t kernel_height, int64_t kernel_width,
+                                            int64_t stride_height, int64_t stride_width,
+                                            int64_t padding_height, int64_t padding_width,
+                                            int64_t groups, int dtype);
 
 int at_conv2d_bwd_input(const void* output_grad, const void* weight, void* input_grad,
-                        int64_t batch, int64_t in_feat, int64_t in_height, int64_t in_width,
-                        int64_t out_feat, int64_t out_height, int64_t out_width,
-                        int64_t kernel_height, int64_t kernel_width, int64_t stride_height,
-                        int64_t stride_width, int64_t padding_height, int64_t padding_width,
-                        int64_t groups, int dtype, at_stream_t stream);
+                        void* workspace, int64_t workspace_bytes, int64_t batch, int64_t in_feat,
+                        int64_t in_height, int64_t in_width, int64_t out_feat,
+                        int64_t out_height, int64_t out_width, int64_t kernel_height,
+                        int64_t kernel_width, int64_t stride_height, int64_t stride_width,
+                        int64_t padding_height, int64_t padding_width, int64_t groups, int dtype,
+                        at_stream_t stream);
 
-int64_t at_conv2d_bwd_weight_workspace_bytes(int64_t out_feat, int64_t in_feat_per_group,
-                                             int64_t kernel_height, int64_t kernel_width);
+int64_t at_conv2d_bwd_weight_workspace_bytes(int64_t batch, int64_t in_feat, int64_t in_height,
+                                             int64_t in_width, int64_t out_feat,
+                                             int64_t out_height, int64_t out_width,
+                                             int64_t kernel_height, int64_t kernel_width,
+                                             int64_t stride_height, int64_t stride_width,
+                                             int64_t padding_height, int64_t padding_width,
+                                             int64_t groups, int dtype);
 
 int at_conv2d_bwd_weight(const void* output_grad, const void* input, void* weight_grad,
                          void* workspace, int64_t workspace_bytes, int64_t batch, int64_t in_feat,

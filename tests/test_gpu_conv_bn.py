@@ -24,6 +24,13 @@ CONV_CASES = [
     ((2, 16, 9, 9), 32, (4, 4), (2, 2), (2, 2), 4),
     ((4, 64, 28, 28), 64, (3, 3), (1, 1), (1, 1), 1),
     ((2, 32, 14, 14), 48, (3, 5), (2, 1), (1, 2), 1),
+    # channel counts per group in multiples of 64: the 16-bit dtypes take the matrix-core path;
+    # odd spatial sizes, partial tiles, groups, strides and asymmetric kernels on purpose
+    ((3, 64, 7, 7), 96, (3, 3), (1, 1), (1, 1), 1),
+    ((2, 128, 10, 12), 128, (3, 3), (2, 2), (1, 1), 2),
+    ((2, 128, 9, 8), 64, (1, 1), (1, 1), (0, 0), 1),
+    ((1, 64, 12, 10), 64, (5, 3), (1, 1), (2, 0), 1),
+    ((5, 64, 20, 24), 64, (3, 3), (1, 1), (1, 1), 1),
 ]
 
 

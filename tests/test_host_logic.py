@@ -72,7 +72,17 @@ def test_argument_errors_without_gpu() -> None:
                                  4, 8, 1, 0.1, 1e-5, 0, 0.0, 0, 1, 0, 0, 0, None) == -5
     # inconsistent convolution geometry
     dims = [1, 4, 8, 8, 4, 9, 9, 3, 3, 1, 1, 1, 1, 1]
-    assert lib.at_conv2d_fwd(p, p, None, p, *dims, 0, 0, 0, None) == -2
+    assert lib.at_conv2d_fwd(p, p, None, p, None, 0, *dims, 0, 0, 0, None) == -2
+    # workspace queries: the matrix-core convolution path wants 16-bit tensors and channel
+    # counts per group in multiples of 64; anything else asks for no forward workspace
+    good = [2, 64, 8, 8, 128, 8, 8, 3, 3, 1, 1, 1, 1, 1]
+    assert lib.at_conv2d_fwd_workspace_bytes(*good, 2, 2) >= 2 * 64 * 8 * 8 * 2 + 128 * 64 * 9 * 2
+    assert lib.at_conv2d_fwd_workspace_bytes(*good, 0, 0) == 0
+    assert lib.at_conv2d_fwd_workspace_bytes(*dims, 2, 2) == 0
+    assert lib.at_conv2d_bwd_input_workspace_bytes(*good, 1) > 0
+    strided = list(good); strided[5] = strided[6] = 4; strided[9] = strided[10] = 2
+    assert lib.at_conv2d_bwd_input_workspace_bytes(*strided, 1) == 0
+    assert lib.at_conv2d_bwd_weight_workspace_bytes(*good, 0) > 0
     assert lib.at_norm_bwd_workspace_bytes(16, 8, 2) == 16 * 8 * 4 * 2
     assert lib.at_cross_entropy_workspace_bytes(10) == 56
 
