@@ -11,14 +11,18 @@ namespace at_hip {
 inline bool act_valid(int act) { return act >= AT_ACT_NONE && act < AT_ACT_COUNT; }
 inline bool act_needs_param(int act) { return act >= AT_ACT_LEAKY_RELU && act <= AT_ACT_SOFTSHRINK; }
 
-__device__ __forceinline__ float act_sigmoid(float x) { return 1.f / (1.f + __expf(-x)); }
+// 1 / x by the hardware reciprocal (1 ulp) instead of the correctly rounded division sequence,
+// which is an order of magnitude longer; every use below feeds a result that is rounded again.
+__device__ __forceinline__ float act_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+__device__ __forceinline__ float act_sigmoid(float x) { return act_rcp(1.f + __expf(-x)); }
 __device__ __forceinline__ float act_tanh(float x) { return 2.f * act_sigmoid(2.f * x) - 1.f; }
 
 // erf by Abramowitz & Stegun 7.1.26 (absolute error < 1.5e-7): small enough to inline into the
 // fully unrolled GEMM epilogue, which the libm erff is not.
 __device__ __forceinline__ float act_erf(float x) {
   const float ax = fabsf(x);
-  const float t = 1.f / (1.f + 0.3275911f * ax);
+  const float t = act_rcp(1.f + 0.3275911f * ax);
   const float poly = ((((1.061405429f * t - 1.453152027f) * t + 1.421413741f) * t - 0.284496736f) * t +
                       0.254829592f) * t;
   return copysignf(1.f - poly * __expf(-ax * ax), x);
@@ -34,7 +38,8 @@ __device__ __forceinline__ float act_forward(int act, float x, float p) {
     case AT_ACT_TANH: return act_tanh(x);
     case AT_ACT_RELU: return fmaxf(0.f, x);
     case AT_ACT_GELU: return 0.5f * (1.f + act_erf(0.707106781f * x)) * x;
-    case AT_ACT_GELUAPPROX: return 0.5f * (1.f + act_tanh(0.7978845608f * x * (1.f + 0.044715f * x * x))) * x;
+    // 0.5 * (1 + tanh(u)) = sigmoid(2u)
+    case AT_ACT_GELUAPPROX: return x * act_sigmoid(1.5957691216f * x * (1.f + 0.044715f * x * x));
     case AT_ACT_SILU: return x * act_sigmoid(x);
     case AT_ACT_RELU6: return fminf(fmaxf(0.f, x), 6.f);
     case AT_ACT_HARDSIGMOID: return fmaxf(0.f, fminf(1.f, x / 6.f + 0.5f));
@@ -57,7 +62,7 @@ __device__ __forceinline__ float act_forward(int act, float x, float p) {
 __device__ __forceinline__ float act_derivative(int act, float x, float p) {
   switch (act) {
     case AT_ACT_SIGMOID: { const float s = act_sigmoid(x); return s * (1.f - s); }
-    case AT_ACT_LOGSIGMOID: return 1.f / (1.f + __expf(x));
+    case AT_ACT_LOGSIGMOID: return act_rcp(1.f + __expf(x));
     case AT_ACT_TANH: { const float t = act_tanh(x); return 1.f - t * t; }
     case AT_ACT_RELU: return x <= 0.f ? 0.f : 1.f;
     case AT_ACT_GELU: {
@@ -65,8 +70,9 @@ __device__ __forceinline__ float act_derivative(int act, float x, float p) {
       return 0.39894228f * __expf(-0.5f * x * x) * x + cdf;
     }
     case AT_ACT_GELUAPPROX: {
-      const float t = act_tanh(0.7978845608f * x * (1.f + 0.044715f * x * x));
-      return 0.5f * (1.f + t + x * (1.f - t * t) * 0.7978845608f * (1.f + 3.f * 0.044715f * x * x));
+      // with s = sigmoid(2u): 0.5 * (1 + tanh u) = s and 0.5 * (1 - tanh^2 u) = 2 s (1 - s)
+      const float sg = act_sigmoid(1.5957691216f * x * (1.f + 0.044715f * x * x));
+      return sg + x * 2.f * sg * (1.f - sg) * 0.7978845608f * (1.f + 3.f * 0.044715f * x * x);
     }
     case AT_ACT_SILU: { const float s = act_sigmoid(x); return s * (x * (1.f - s) + 1.f); }
     case AT_ACT_RELU6: return (0.f < x && x < 6.f) ? 1.f : 0.f;

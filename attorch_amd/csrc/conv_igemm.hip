@@ -338,6 +338,8 @@ struct DwArgs {
   int K;              // taps * Cg
   int tiles_per_tap;  // Cg / 64
   int nbn;            // column tiles (taps * Cg / 64)
+  int mtiles;         // row tiles (Og / 64)
+  int splits;         // pixel ranges
   int p_per_split;    // pixels per split, a multiple of 64
   int64_t dy_bytes, x_bytes;
   FastDiv div_ohw, div_ow;
@@ -346,8 +348,16 @@ struct DwArgs {
 template <typename T>
 __global__ __launch_bounds__(256) void conv_dw_kernel(DwArgs g) {
   __shared__ __attribute__((aligned(1024))) char lds[2 * kDwStage];
-  const int grp = blockIdx.z, split = blockIdx.y;
-  const int tile_m = blockIdx.x / g.nbn, tile_n = blockIdx.x - tile_m * g.nbn;
+  // Consecutive workgroup ids go to different XCDs (each with its own L2).  The tiles of one
+  // pixel range all read the same rows of dY and X, so they are given to one XCD: id -> (XCD,
+  // position on it) -> split = XCD + 8 * (position / tiles), tile = position % tiles.
+  const int grp = blockIdx.z;
+  const int tiles = g.mtiles * g.nbn;
+  const int xcd = blockIdx.x & 7, pos = blockIdx.x >> 3;
+  const int split = xcd + 8 * (pos / tiles);
+  if (split >= g.splits) return;   // padding of the grid, uniform for the workgroup
+  const int tile = pos % tiles;
+  const int tile_m = tile / g.nbn, tile_n = tile - tile_m * g.nbn;
   const int co0 = tile_m * 64;                               // within the group
   const int tap = tile_n / g.tiles_per_tap;
   const int c0 = (tile_n - tap * g.tiles_per_tap) * 64;      // within the group
@@ -629,7 +639,9 @@ int conv_igemm_dw(const ConvProblem& p, const void* dy, const void* x, void* dw,
   g.div_ohw = make_fastdiv(g.OHW);
   g.div_ow = make_fastdiv(g.OW);
   const int real_splits = (int)cdiv64(g.P, g.p_per_split);
-  const dim3 grid((unsigned)(cdiv64(g.Og, 64) * g.nbn), (unsigned)real_splits, (unsigned)p.groups);
+  g.mtiles = (int)cdiv64(g.Og, 64);
+  g.splits = real_splits;
+  const dim3 grid((unsigned)(g.mtiles * g.nbn * (cdiv64(real_splits, 8) * 8)), 1, (unsigned)p.groups);
   const int64_t total = p.O * (int64_t)g.K;
   return dispatch16(p.dtype, [&](auto* tp) -> int {
     typedef std::remove_pointer_t<decltype(tp)> T;

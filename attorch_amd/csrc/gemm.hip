@@ -454,13 +454,37 @@ __global__ __launch_bounds__(256) void colsum_partial_kernel(const T* __restrict
   part[(int64_t)blockIdx.y * N + n] = s;
 }
 
+// out[n] = sum over slices of part[slice][n], fixed order.  A workgroup owns 16 columns: 4 column
+// quads x 64 slice lanes, folded through LDS.
+constexpr int kColsumFinalCols = 16;
 __global__ __launch_bounds__(256) void colsum_final_kernel(const float* __restrict__ part, void* __restrict__ out,
                                                           int out_dt, int slices, int N) {
-  const int n = blockIdx.x * 256 + threadIdx.x;
-  if (n >= N) return;
-  float s = 0.f;
-  for (int p = 0; p < slices; ++p) s += part[(int64_t)p * N + n];
-  store_scalar_f32(out, out_dt, n, s);
+  __shared__ float sm[64][kColsumFinalCols + 1];
+  const int cq = threadIdx.x & 3, lane_slice = threadIdx.x >> 2;
+  const int col = blockIdx.x * kColsumFinalCols + cq * 4;
+  float a[4] = {0.f, 0.f, 0.f, 0.f};
+  if (col + 3 < N && (N & 3) == 0 && aligned16_dev(part)) {
+#pragma unroll 4
+    for (int p = lane_slice; p < slices; p += 64) {
+      const float4 v = *reinterpret_cast<const float4*>(part + (int64_t)p * N + col);
+      a[0] += v.x; a[1] += v.y; a[2] += v.z; a[3] += v.w;
+    }
+  } else {
+    for (int p = lane_slice; p < slices; p += 64)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (col + j < N) a[j] += part[(int64_t)p * N + col + j];
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) sm[lane_slice][cq * 4 + j] = a[j];
+  __syncthreads();
+  if (threadIdx.x < kColsumFinalCols) {
+    float s = 0.f;
+#pragma unroll
+    for (int r = 0; r < 64; ++r) s += sm[r][threadIdx.x];
+    const int n = blockIdx.x * kColsumFinalCols + threadIdx.x;
+    if (n < N) store_scalar_f32(out, out_dt, n, s);
+  }
 }
 
 template <typename F>
@@ -630,7 +654,7 @@ int at_act_bwd(const void* output_grad, const void* input, void* input_grad, voi
     });
   });
   if (rc || !bias_grad) return rc;
-  hipLaunchKernelGGL(colsum_final_kernel, dim3((unsigned)cdiv64(cols, 256)), dim3(256), 0, (hipStream_t)stream,
+  hipLaunchKernelGGL(colsum_final_kernel, dim3((unsigned)cdiv64(cols, kColsumFinalCols)), dim3(256), 0, (hipStream_t)stream,
                      (const float*)workspace, bias_grad, bias_grad_dtype, (int)slices, (int)cols);
   return launch_status();
 }
@@ -657,8 +681,8 @@ int at_colsum(const void* x, void* out, void* workspace, int64_t workspace_bytes
     return launch_status();
   });
   if (rc) return rc;
-  hipLaunchKernelGGL(colsum_final_kernel, dim3(gx), dim3(256), 0, (hipStream_t)stream,
-                     (const float*)workspace, out, out_dtype, slices, (int)cols);
+  hipLaunchKernelGGL(colsum_final_kernel, dim3((unsigned)cdiv64(cols, kColsumFinalCols)), dim3(256), 0,
+                     (hipStream_t)stream, (const float*)workspace, out, out_dtype, slices, (int)cols);
   return launch_status();
 }
 

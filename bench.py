@@ -40,6 +40,9 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument('--configs', type=str, default='c1,c2,c3,c5',
                         help='secondary configs to measure besides the headline (c4); "none" skips them')
     parser.add_argument('--no-cpu', action='store_true', help='skip the CPU baselines')
+    parser.add_argument('--calibrate-copy', action='store_true',
+                        help='also run a plain 256 MiB -> 256 MiB device copy, the known-size kernel that '
+                             'hardware byte counters of a profiling run are scaled by')
     return parser.parse_args()
 
 
@@ -533,6 +536,13 @@ def main() -> int:
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
     torch.set_num_threads(os.cpu_count())
     with_cpu = not args.no_cpu
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device='cuda').fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     head = bench_linear('c4', args.steps, args.warmup, with_cpu)
     extra: List[Dict] = []
     wanted = [] if args.configs == 'none' else args.configs.split(',')
