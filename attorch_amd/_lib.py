@@ -45,9 +45,10 @@ PROTOTYPES = {
     'at_conv2d_fwd_workspace_bytes': (L, [L] * 14 + [I, I]),
     'at_conv2d_fwd': (I, [P, P, P, P, P, L] + [L] * 14 + [I, I, I, P]),
     'at_conv2d_bwd_input_workspace_bytes': (L, [L] * 14 + [I]),
-    'at_conv2d_bwd_input': (I, [P, P, P, P, L] + [L] * 14 + [I, P]),
+    'at_conv2d_bwd_input': (I, [P, P, P, P, P, L] + [L] * 14 + [I, P]),
     'at_conv2d_bwd_weight_workspace_bytes': (L, [L] * 14 + [I]),
-    'at_conv2d_bwd_weight': (I, [P, P, P, P, L] + [L] * 14 + [I, P]),
+    'at_conv2d_bwd_weight': (I, [P, P, P, P, P, P, L] + [L] * 14 + [I, P]),
+    'at_nchw_to_nhwc': (I, [P, P, L, L, L, I, P]),
     'at_channel_sum': (I, [P, P, L, L, L, I, I, P]),
     'at_batch_norm_bwd': (I, [P, P, P, P, P, P, P, P, P, P, P, L, L, L, L, I, F, I, I, P]),
 }

@@ -126,6 +126,9 @@ class Conv2dAutoGrad(torch.autograd.Function):
         ctx.dims = dims
         ctx.bias_requires_grad = False if bias is None else bias.requires_grad
         ctx.output_dtype = output_dtype
+        # The matrix-core path leaves a channels-last copy of the input at the start of its
+        # workspace; the weight gradient reuses it instead of transposing the input again.
+        ctx.input_nhwc = workspace if requires_grad and weight.requires_grad else None
         if requires_grad:
             ctx.save_for_backward(input, weight)
 
@@ -153,22 +156,31 @@ class Conv2dAutoGrad(torch.autograd.Function):
 
         input_grad = weight_grad = bias_grad = None
         with torch.cuda.device_of(input):
+            input_workspace_bytes = (lib.at_conv2d_bwd_input_workspace_bytes(*dims, dtype)
+                                     if input.requires_grad else 0)
+            # one channels-last copy of the output gradient serves both products
+            output_grad_nhwc = None
+            if input_workspace_bytes > 0 and weight.requires_grad:
+                output_grad_nhwc = torch.empty_like(output_grad)
+                _lib.check(lib.at_nchw_to_nhwc(
+                    _lib.ptr(output_grad), _lib.ptr(output_grad_nhwc), batch_dim, out_feat_dim,
+                    out_height * out_width, dtype, stream), 'at_nchw_to_nhwc')
             if input.requires_grad:
                 weight_k = weight.to(output_dtype).contiguous()
                 input_grad = torch.empty(input.shape, dtype=output_dtype, device=device)
-                workspace, workspace_bytes = _workspace(
-                    lib.at_conv2d_bwd_input_workspace_bytes(*dims, dtype), device)
+                workspace, workspace_bytes = _workspace(input_workspace_bytes, device)
                 _lib.check(lib.at_conv2d_bwd_input(
-                    _lib.ptr(output_grad), _lib.ptr(weight_k), _lib.ptr(input_grad),
-                    _lib.ptr(workspace), workspace_bytes, *dims, dtype, stream),
-                    'at_conv2d_bwd_input')
+                    _lib.ptr(output_grad), _lib.ptr(output_grad_nhwc), _lib.ptr(weight_k),
+                    _lib.ptr(input_grad), _lib.ptr(workspace), workspace_bytes, *dims, dtype,
+                    stream), 'at_conv2d_bwd_input')
             if weight.requires_grad:
                 input_k = input.to(output_dtype).contiguous()
                 weight_grad = torch.empty(weight.shape, dtype=output_dtype, device=device)
                 workspace, workspace_bytes = _workspace(
                     lib.at_conv2d_bwd_weight_workspace_bytes(*dims, dtype), device)
                 _lib.check(lib.at_conv2d_bwd_weight(
-                    _lib.ptr(output_grad), _lib.ptr(input_k), _lib.ptr(weight_grad),
+                    _lib.ptr(output_grad), _lib.ptr(output_grad_nhwc), _lib.ptr(input_k),
+                    _lib.ptr(ctx.input_nhwc), _lib.ptr(weight_grad),
                     _lib.ptr(workspace), workspace_bytes, *dims, dtype, stream),
                     'at_conv2d_bwd_weight')
             if ctx.bias_requires_grad:

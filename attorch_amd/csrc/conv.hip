@@ -341,8 +341,8 @@ int64_t at_conv2d_bwd_input_workspace_bytes(int64_t batch, int64_t in_feat, int6
   return conv_igemm_dx_workspace(problem_of(s, dtype));
 }
 
-int at_conv2d_bwd_input(const void* output_grad, const void* weight, void* input_grad, void* workspace,
-                        int64_t workspace_bytes, int64_t batch, int64_t in_feat, int64_t in_height,
+int at_conv2d_bwd_input(const void* output_grad, const void* output_grad_nhwc, const void* weight,
+                        void* input_grad, void* workspace, int64_t workspace_bytes, int64_t batch, int64_t in_feat, int64_t in_height,
                         int64_t in_width, int64_t out_feat, int64_t out_height, int64_t out_width,
                         int64_t kernel_height, int64_t kernel_width, int64_t stride_height, int64_t stride_width,
                         int64_t padding_height, int64_t padding_width, int64_t groups, int dtype,
@@ -357,7 +357,7 @@ int at_conv2d_bwd_input(const void* output_grad, const void* weight, void* input
     const ConvProblem p = problem_of(s, dtype);
     const int64_t need = conv_igemm_dx_workspace(p);
     if (need > 0 && workspace && workspace_bytes >= need && aligned16(workspace))
-      return conv_igemm_dx(p, output_grad, weight, input_grad, workspace, (hipStream_t)stream);
+      return conv_igemm_dx(p, output_grad, output_grad_nhwc, weight, input_grad, workspace, (hipStream_t)stream);
   }
   ConvArgs g = base_args(s);
   g.a = output_grad; g.b = weight; g.out = input_grad;
@@ -384,8 +384,8 @@ int64_t at_conv2d_bwd_weight_workspace_bytes(int64_t batch, int64_t in_feat, int
   return fast > generic ? fast : generic;
 }
 
-int at_conv2d_bwd_weight(const void* output_grad, const void* input, void* weight_grad, void* workspace,
-                         int64_t workspace_bytes, int64_t batch, int64_t in_feat, int64_t in_height,
+int at_conv2d_bwd_weight(const void* output_grad, const void* output_grad_nhwc, const void* input,
+                         const void* input_nhwc, void* weight_grad, void* workspace, int64_t workspace_bytes, int64_t batch, int64_t in_feat, int64_t in_height,
                          int64_t in_width, int64_t out_feat, int64_t out_height, int64_t out_width,
                          int64_t kernel_height, int64_t kernel_width, int64_t stride_height, int64_t stride_width,
                          int64_t padding_height, int64_t padding_width, int64_t groups, int dtype,
@@ -400,7 +400,8 @@ int at_conv2d_bwd_weight(const void* output_grad, const void* input, void* weigh
     const ConvProblem p = problem_of(s, dtype);
     const int64_t need = conv_igemm_dw_workspace(p);
     if (need > 0 && workspace && workspace_bytes >= need && aligned16(workspace))
-      return conv_igemm_dw(p, output_grad, input, weight_grad, workspace, (hipStream_t)stream);
+      return conv_igemm_dw(p, output_grad, output_grad_nhwc, input, input_nhwc, weight_grad, workspace,
+                           (hipStream_t)stream);
   }
   ConvArgs g = base_args(s);
   const int splits = dw_splits(s);
@@ -419,6 +420,12 @@ int at_conv2d_bwd_weight(const void* output_grad, const void* input, void* weigh
                        (hipStream_t)stream, (const float*)workspace, (T*)weight_grad, splits, total);
     return launch_status();
   });
+}
+
+int at_nchw_to_nhwc(const void* src, void* dst, int64_t batch, int64_t feat, int64_t spatial, int dtype,
+                    at_stream_t stream) {
+  if (!src || !dst) return AT_ERR_NULL;
+  return conv_nchw_to_nhwc(src, dst, batch, feat, spatial, dtype, (hipStream_t)stream);
 }
 
 int at_channel_sum(const void* x, void* out, int64_t batch, int64_t feat, int64_t spatial, int x_dtype,

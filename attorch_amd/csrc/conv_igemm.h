@@ -30,11 +30,16 @@ int64_t conv_igemm_dw_workspace(const ConvProblem& p);
 // Y = conv(X, W) + bias, all NCHW.
 int conv_igemm_fwd(const ConvProblem& p, const void* x, const void* w, const void* bias, int bias_dt,
                    void* y, void* workspace, hipStream_t stream);
-// dX = conv_transpose(dY, W), all NCHW (stride 1 only).
-int conv_igemm_dx(const ConvProblem& p, const void* dy, const void* w, void* dx, void* workspace,
-                  hipStream_t stream);
-// dW[O][C/groups][KH][KW] = correlation of dY with X, all NCHW.
-int conv_igemm_dw(const ConvProblem& p, const void* dy, const void* x, void* dw, void* workspace,
-                  hipStream_t stream);
+// dX = conv_transpose(dY, W), all NCHW (stride 1 only).  dy_nhwc: optional channels-last copy of
+// dY the caller already holds (saves the copy made here).
+int conv_igemm_dx(const ConvProblem& p, const void* dy, const void* dy_nhwc, const void* w, void* dx,
+                  void* workspace, hipStream_t stream);
+// dW[O][C/groups][KH][KW] = correlation of dY with X, all NCHW.  dy_nhwc / x_nhwc: optional
+// channels-last copies the caller already holds.
+int conv_igemm_dw(const ConvProblem& p, const void* dy, const void* dy_nhwc, const void* x, const void* x_nhwc,
+                  void* dw, void* workspace, hipStream_t stream);
+// [N][C][HW] -> [N][HW][C] for a 16-bit dtype.
+int conv_nchw_to_nhwc(const void* src, void* dst, int64_t N, int64_t C, int64_t HW, int dtype,
+                      hipStream_t stream);
 
 }  // namespace at_hip

@@ -137,6 +137,26 @@ __global__ void conv_weight_taps_kernel(const T* __restrict__ w, T* __restrict__
   }
 }
 
+// wt[groups * Og][K] -> fragment-major copy for the kernel that reads the weights straight into
+// registers: the 64 lanes x 16 bytes of one operand fragment (32 output channels x 16 k) are
+// contiguous, ordered [group][channel tile of 32][k / 16][lane]; channels past Og are zeros.
+template <typename T>
+__global__ void conv_weight_frags_kernel(const T* __restrict__ wt, T* __restrict__ wf, int Og, int K, int ntiles,
+                                         int64_t total_chunks) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total_chunks) return;
+  const int lane = (int)(i & 63);
+  const int64_t frag = i >> 6;
+  const int ksteps = K / 16;
+  const int kstep = (int)(frag % ksteps);
+  const int tile = (int)((frag / ksteps) % ntiles);
+  const int grp = (int)(frag / ((int64_t)ksteps * ntiles));
+  const int co = tile * 32 + (lane & 31);
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (co < Og) v = *reinterpret_cast<const uint4*>(wt + (int64_t)(grp * Og + co) * K + kstep * 16 + (lane >> 5) * 8);
+  reinterpret_cast<uint4*>(wf)[i] = v;
+}
+
 // ------------------------------------------------------------------------------------------
 // Forward / input-gradient kernel.
 // ------------------------------------------------------------------------------------------
@@ -147,6 +167,7 @@ constexpr int kCEpiPitch = CBM * 2 + 16;   // bytes per output-channel row of th
 struct IgemmArgs {
   const void* act;    // [N][IH][IW][Ctot]
   const void* wt;     // [groups * Og][taps * Cg]
+  void* wf;           // fragment-major copy of wt (room for groups * ceil32(Og) * K elements)
   void* out;          // [N][groups * Og][OH][OW]
   const void* bias;   // [groups * Og] or null
   int bias_dt;
@@ -295,6 +316,189 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(IgemmArgs g) {
           const int n = fast_div(mm, g.div_ohw);
           const int p = mm - n * g.OHW;
           out[((int64_t)n * Otot + grp * g.Og + co) * g.OHW + p] = u.e[e];
+        }
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Forward / input-gradient kernel, input window resident in LDS.
+// ------------------------------------------------------------------------------------------
+// The 128 output pixels of a tile read, over all taps, a contiguous range of channels-last input
+// pixels (flattened over image, row, column): tap (kh, kw) of output pixel m sits at
+// q(m) + kh*IW + kw with q(m) growing with m.  When that range fits in LDS it is loaded once per
+// 64-channel chunk (instead of once per tap), the operand fragments of every tap are read from it
+// at shifted rows, and taps outside the image read a row of zeros.  The weights go from cache
+// straight into registers, so the main loop needs no barrier.
+constexpr int kHaloRows = 288;                       // input pixels a tile may span
+constexpr int kHaloBytes = (kHaloRows + 1) * 128;    // + the zero row
+
+template <typename T>
+__global__ __launch_bounds__(256) void conv_igemm_halo_kernel(IgemmArgs g) {
+  __shared__ __attribute__((aligned(1024))) char lds[kHaloBytes];
+  const int grp = blockIdx.z;
+  const int tile_m = blockIdx.x / g.nbn, tile_n = blockIdx.x - tile_m * g.nbn;
+  const int m0 = tile_m * CBM, n0 = tile_n * CBN;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int KH = g.KT / (g.tiles_per_tap * g.KW);
+
+  // q of (tap 0,0) for an output pixel, and whether the pixel exists
+  auto q_of = [&](int m, int& ih0, int& iw0) -> int {
+    const int n = fast_div(m, g.div_ohw);
+    const int p = m - n * g.OHW;
+    const int oh = fast_div(p, g.div_ow);
+    const int ow = p - oh * g.OW;
+    ih0 = oh * g.sh - g.ph;
+    iw0 = ow * g.sw - g.pw;
+    return (n * g.IH + ih0) * g.IW + iw0;
+  };
+  int dummy0, dummy1;
+  const int m_last = m0 + CBM - 1 < g.M ? m0 + CBM - 1 : g.M - 1;
+  const int q_lo = q_of(m0, dummy0, dummy1);
+  const int rows = q_of(m_last, dummy0, dummy1) + (KH - 1) * g.IW + g.KW - q_lo;   // <= kHaloRows (host check)
+
+  // this lane's two fragment rows (output pixels) and its weight row
+  int f_ih0[2], f_iw0[2], f_row[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int m = m0 + wm * 64 + t * 32 + (lane & 31);
+    if (m < g.M) {
+      f_row[t] = q_of(m, f_ih0[t], f_iw0[t]) - q_lo;
+    } else {
+      f_ih0[t] = -(1 << 24);
+      f_iw0[t] = 0;
+      f_row[t] = 0;
+    }
+  }
+  // byte offset of this lane inside the first fragment of its channel tile (fragment-major
+  // weights: one fragment = 64 lanes x 16 bytes, K / 16 fragments per tile)
+  const int ntiles32 = (g.Og + 31) >> 5;
+  const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(
+      g.wf, 0, (int)((int64_t)gridDim.z * ntiles32 * g.K * 64), 0x00020000);
+  const int wrow = ((grp * ntiles32 + (n0 >> 5) + wn) * (g.K >> 4)) * 1024 + lane * 16;
+
+  if (threadIdx.x < 32) reinterpret_cast<uint32_t*>(lds + kHaloRows * 128)[threadIdx.x] = 0u;   // the zero row
+
+  const i32x4 ra = make_buffer_rsrc(g.act, g.act_bytes);
+  f32x16 acc[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[t][e] = 0.f;
+
+  for (int cc = 0; cc < g.tiles_per_tap; ++cc) {
+    if (cc > 0) __syncthreads();   // everybody is done with the previous chunk's window
+    // Straight-line and unconditional on purpose (offsets first, then the loads back to back; a
+    // load past the window writes zeros into unused rows): any wait the compiler inserts for
+    // loads it tracks would also wait for the loads issued here, one after the other.
+    int doff[kHaloRows / 32];
+#pragma unroll
+    for (int i = 0; i < kHaloRows / 32; ++i) {
+      const int row = (wave + 4 * i) * 8 + (lane >> 3);
+      const int chunk = (lane & 7) ^ (row & 7);   // window rows are read at any offset: swizzle by row % 8 only
+      const int off = ((q_lo + row) * g.Ctot + grp * g.Cg + cc * 64 + chunk * 8) * 2;   // negative: out of range
+      doff[i] = row < rows ? off : kOobOffset;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < kHaloRows / 32; ++i) lds_dma_16(ra, doff[i], lds + (wave + 4 * i) * 1024);
+    lds_dma_wait_all();
+    __syncthreads();
+
+    const int wk = wrow + cc * 4096;   // 4 fragments per 64 channels
+    const int taps = KH * g.KW;
+    // weight fragments of a whole tap (4 k-steps) per buffer; the next tap's are fetched while
+    // this tap multiplies
+    uint4 b0[4], b1[4];
+    // Buffer loads without a branch around them (a missing channel reads zeros; one tap past
+    // the end reads values nobody uses): with conditional loads the compiler cannot count what is
+    // in flight and waits for the fragments it has just requested.
+    // The tap and k-step go into the scalar offset, so the vector offset is one register that
+    // never changes: no address arithmetic competes for the registers the loads land in.
+    auto fetch = [&](uint4 (&dst)[4], int tap) {
+      const int tap_bytes = tap < taps ? tap * g.tiles_per_tap * 4096 : 0;   // one past the end: any valid tap
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks)
+        dst[ks] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rw, wk, tap_bytes + ks * 1024, 0));
+    };
+    int kh = 0, kw = 0;
+    auto multiply = [&](const uint4 (&bw)[4]) {
+      int rowaddr[2], swz[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const int ih = f_ih0[t] + kh, iw = f_iw0[t] + kw;
+        const bool ok = (unsigned)ih < (unsigned)g.IH && (unsigned)iw < (unsigned)g.IW;
+        const int row = ok ? f_row[t] + kh * g.IW + kw : kHaloRows;
+        rowaddr[t] = row * 128;
+        swz[t] = row & 7;
+      }
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const int chunk = ks * 2 + (lane >> 5);
+        const uint4 a0 = *reinterpret_cast<const uint4*>(lds + rowaddr[0] + ((chunk ^ swz[0]) << 4));
+        const uint4 a1 = *reinterpret_cast<const uint4*>(lds + rowaddr[1] + ((chunk ^ swz[1]) << 4));
+        acc[0] = Mfma16<T>::run(a0, bw[ks], acc[0]);
+        acc[1] = Mfma16<T>::run(a1, bw[ks], acc[1]);
+      }
+      if (++kw == g.KW) {
+        kw = 0;
+        ++kh;
+      }
+    };
+    fetch(b0, 0);
+#pragma unroll 1
+    for (int tap = 0; tap < taps; tap += 2) {
+      fetch(b1, tap + 1);
+      multiply(b0);
+      if (tap + 1 < taps) {
+        fetch(b0, tap + 2);
+        multiply(b1);
+      }
+    }
+  }
+  __syncthreads();   // the window is dead: LDS becomes the output tile
+
+  T* __restrict__ out = reinterpret_cast<T*>(g.out);
+  {
+    const int col = wn * 32 + (lane & 31);
+    float bv = 0.f;
+    if (g.bias && n0 + col < g.Og) bv = load_scalar_f32(g.bias, g.bias_dt, grp * g.Og + n0 + col);
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = acc[t][rg * 4 + e] + bv;
+        const int pix = wm * 64 + t * 32 + rg * 8 + (lane >> 5) * 4;
+        store_f32<T, 4>(reinterpret_cast<T*>(lds + col * kCEpiPitch) + pix, v);
+      }
+  }
+  __syncthreads();
+  const int Otot = g.Og * (int)gridDim.z;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    const int id = threadIdx.x + 256 * s;
+    const int col = id >> 4, pc = id & 15;
+    const int oc = n0 + col, m = m0 + pc * 8;
+    if (oc >= g.Og || m >= g.M) continue;
+    const uint4 v = *reinterpret_cast<const uint4*>(lds + col * kCEpiPitch + pc * 16);
+    if (g.vec_store) {
+      const int n = fast_div(m, g.div_ohw);
+      const int p = m - n * g.OHW;
+      *reinterpret_cast<uint4*>(out + ((int64_t)n * Otot + grp * g.Og + oc) * g.OHW + p) = v;
+    } else {
+      union { uint4 raw; T e[8]; } u;
+      u.raw = v;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int mm = m + e;
+        if (mm < g.M) {
+          const int n = fast_div(mm, g.div_ohw);
+          const int p = mm - n * g.OHW;
+          out[((int64_t)n * Otot + grp * g.Og + oc) * g.OHW + p] = u.e[e];
         }
       }
     }
@@ -510,6 +714,35 @@ int weight_taps(const void* w, void* wt, const ConvProblem& p, int flip, hipStre
   });
 }
 
+// Largest number of input pixels (flattened over image, row, column) that the taps of one tile of
+// 128 consecutive output pixels span, or -1 when the position of tap (0, 0) does not grow with the
+// output pixel (very wide padding) or the answer would take too long to find.
+int64_t halo_rows_needed(const IgemmArgs& g, int64_t n_img, int64_t OH, int KH) {
+  const int64_t OW = g.OW, OHW = OH * OW, M = n_img * OHW;
+  if ((int64_t)g.sh * g.IW < (OW - 1) * g.sw) return -1;
+  if ((int64_t)g.IH * g.IW < (OH - 1) * g.sh * g.IW + (OW - 1) * g.sw) return -1;
+  auto q_of = [&](int64_t m) {
+    const int64_t n = m / OHW, p = m % OHW, oh = p / OW, ow = p % OW;
+    return (n * g.IH + oh * g.sh - g.ph) * g.IW + ow * g.sw - g.pw;
+  };
+  // The span depends only on where the tile starts inside its image, and that offset repeats
+  // with period OHW / gcd(OHW, 128) tiles.
+  int64_t a = OHW, b = CBM;
+  while (b) { const int64_t r = a % b; a = b; b = r; }
+  const int64_t period = OHW / a;
+  const int64_t tiles = cdiv64(M, CBM);
+  const int64_t walk = tiles < period ? tiles : period;
+  if (walk > 16384) return -1;
+  int64_t worst = 0;
+  for (int64_t t = 0; t < walk; ++t) {
+    const int64_t m0 = t * CBM;
+    const int64_t m_last = m0 + CBM - 1 < M ? m0 + CBM - 1 : M - 1;
+    const int64_t span = q_of(m_last) + (int64_t)(KH - 1) * g.IW + g.KW - q_of(m0);
+    if (span > worst) worst = span;
+  }
+  return worst;
+}
+
 // One product out[(n,oh,ow), co] over channels-last `act`; see IgemmArgs for the meaning of the fields.
 int run_igemm(IgemmArgs g, int64_t n_img, int64_t OH, int groups, int dt, hipStream_t stream) {
   g.OHW = (int)(OH * g.OW);
@@ -521,13 +754,31 @@ int run_igemm(IgemmArgs g, int64_t n_img, int64_t OH, int groups, int dt, hipStr
   g.div_ohw = make_fastdiv(g.OHW);
   g.div_ow = make_fastdiv(g.OW);
   const dim3 grid((unsigned)(cdiv64(g.M, CBM) * g.nbn), 1, (unsigned)groups);
+  const int KH = g.KT / (g.tiles_per_tap * g.KW);
+  const int64_t window = halo_rows_needed(g, n_img, OH, KH);
+  const bool resident = window > 0 && window <= kHaloRows;
   return dispatch16(dt, [&](auto* tp) -> int {
     typedef std::remove_pointer_t<decltype(tp)> T;
-    hipLaunchKernelGGL((conv_igemm_kernel<T>), grid, dim3(256), 0, stream, g);
+    if (resident) {
+      const int ntiles = (g.Og + 31) / 32;
+      const int64_t chunks = (int64_t)groups * ntiles * (g.K / 16) * 64;
+      hipLaunchKernelGGL((conv_weight_frags_kernel<T>), dim3((unsigned)cdiv64(chunks, 256)), dim3(256), 0, stream,
+                         (const T*)g.wt, (T*)g.wf, g.Og, g.K, ntiles, chunks);
+      hipLaunchKernelGGL((conv_igemm_halo_kernel<T>), grid, dim3(256), 0, stream, g);
+    } else {
+      hipLaunchKernelGGL((conv_igemm_kernel<T>), grid, dim3(256), 0, stream, g);
+    }
     return launch_status();
   });
 }
 
+}  // namespace
+
+namespace {
+// bytes of the fragment-major weight copy: output channels per group padded to 32
+inline int64_t frag_weight_bytes(int64_t groups, int64_t out_per_group, int64_t K) {
+  return groups * ((out_per_group + 31) / 32 * 32) * K * 2;
+}
 }  // namespace
 
 bool conv_igemm_supports_fwd(const ConvProblem& p) {
@@ -546,12 +797,14 @@ bool conv_igemm_supports_dw(const ConvProblem& p) {
 
 int64_t conv_igemm_fwd_workspace(const ConvProblem& p) {
   if (!conv_igemm_supports_fwd(p)) return 0;
-  return round256(p.N * p.C * p.H * p.W * 2) + round256(p.O * (p.C / p.groups) * p.KH * p.KW * 2);
+  return round256(p.N * p.C * p.H * p.W * 2) + round256(p.O * (p.C / p.groups) * p.KH * p.KW * 2) +
+         round256(frag_weight_bytes(p.groups, p.O / p.groups, (p.C / p.groups) * p.KH * p.KW));
 }
 
 int64_t conv_igemm_dx_workspace(const ConvProblem& p) {
   if (!conv_igemm_supports_dx(p)) return 0;
-  return round256(p.N * p.O * p.OH * p.OW * 2) + round256(p.O * (p.C / p.groups) * p.KH * p.KW * 2);
+  return round256(p.N * p.O * p.OH * p.OW * 2) + round256(p.O * (p.C / p.groups) * p.KH * p.KW * 2) +
+         round256(frag_weight_bytes(p.groups, p.C / p.groups, (p.O / p.groups) * p.KH * p.KW));
 }
 
 namespace {
@@ -584,6 +837,7 @@ int conv_igemm_fwd(const ConvProblem& p, const void* x, const void* w, const voi
   if (rc) return rc;
   IgemmArgs g{};
   g.act = xh; g.wt = wt; g.out = y; g.bias = bias; g.bias_dt = bias_dt;
+  g.wf = static_cast<char*>(wt) + round256(p.O * (p.C / p.groups) * p.KH * p.KW * 2);
   g.IH = (int)p.H; g.IW = (int)p.W; g.Ctot = (int)p.C; g.Cg = (int)(p.C / p.groups); g.Og = (int)(p.O / p.groups);
   g.KW = (int)p.KW; g.OW = (int)p.OW; g.sh = (int)p.sh; g.sw = (int)p.sw; g.ph = (int)p.ph; g.pw = (int)p.pw;
   g.KT = (int)(p.KH * p.KW * (g.Cg / 64));
@@ -592,18 +846,30 @@ int conv_igemm_fwd(const ConvProblem& p, const void* x, const void* w, const voi
   return run_igemm(g, p.N, p.OH, (int)p.groups, p.dtype, stream);
 }
 
-int conv_igemm_dx(const ConvProblem& p, const void* dy, const void* w, void* dx, void* workspace,
-                  hipStream_t stream) {
+int conv_nchw_to_nhwc(const void* src, void* dst, int64_t N, int64_t C, int64_t HW, int dtype,
+                      hipStream_t stream) {
+  if (!is16(dtype)) return AT_ERR_DTYPE;
+  if (N <= 0 || C <= 0 || HW <= 0 || N > 65535 || C > INT32_MAX || HW > INT32_MAX) return AT_ERR_DIM;
+  return to_nhwc(src, dst, N, C, HW, dtype, stream);
+}
+
+int conv_igemm_dx(const ConvProblem& p, const void* dy, const void* dy_nhwc, const void* w, void* dx,
+                  void* workspace, hipStream_t stream) {
   char* ws = static_cast<char*>(workspace);
-  void* dyh = ws;
+  const void* dyh = dy_nhwc;
   void* wt = ws + round256(p.N * p.O * p.OH * p.OW * 2);
-  int rc = to_nhwc(dy, dyh, p.N, p.O, p.OH * p.OW, p.dtype, stream);
+  int rc = AT_OK;
+  if (!dyh) {
+    rc = to_nhwc(dy, ws, p.N, p.O, p.OH * p.OW, p.dtype, stream);
+    dyh = ws;
+  }
   if (rc) return rc;
   rc = weight_taps(w, wt, p, 1, stream);
   if (rc) return rc;
   // dX[n, c, ih, iw] = sum_{taps', o} dY[n, ih + kh' - (KH-1-ph), iw + kw' - (KW-1-pw), o] * W[o, c, mirrored tap]
   IgemmArgs g{};
   g.act = dyh; g.wt = wt; g.out = dx; g.bias = nullptr; g.bias_dt = 0;
+  g.wf = static_cast<char*>(wt) + round256(p.O * (p.C / p.groups) * p.KH * p.KW * 2);
   g.IH = (int)p.OH; g.IW = (int)p.OW; g.Ctot = (int)p.O; g.Cg = (int)(p.O / p.groups); g.Og = (int)(p.C / p.groups);
   g.KW = (int)p.KW; g.OW = (int)p.W; g.sh = 1; g.sw = 1; g.ph = (int)(p.KH - 1 - p.ph); g.pw = (int)(p.KW - 1 - p.pw);
   g.KT = (int)(p.KH * p.KW * (g.Cg / 64));
@@ -612,16 +878,24 @@ int conv_igemm_dx(const ConvProblem& p, const void* dy, const void* w, void* dx,
   return run_igemm(g, p.N, p.H, (int)p.groups, p.dtype, stream);
 }
 
-int conv_igemm_dw(const ConvProblem& p, const void* dy, const void* x, void* dw, void* workspace,
-                  hipStream_t stream) {
+int conv_igemm_dw(const ConvProblem& p, const void* dy, const void* dy_nhwc, const void* x, const void* x_nhwc,
+                  void* dw, void* workspace, hipStream_t stream) {
   char* ws = static_cast<char*>(workspace);
-  void* dyh = ws;
-  void* xh = ws + round256(p.N * p.O * p.OH * p.OW * 2);
+  const void* dyh = dy_nhwc;
+  const void* xh = x_nhwc;
   float* part = reinterpret_cast<float*>(ws + round256(p.N * p.O * p.OH * p.OW * 2) +
                                          round256(p.N * p.C * p.H * p.W * 2));
-  int rc = to_nhwc(dy, dyh, p.N, p.O, p.OH * p.OW, p.dtype, stream);
+  int rc = AT_OK;
+  if (!dyh) {
+    rc = to_nhwc(dy, ws, p.N, p.O, p.OH * p.OW, p.dtype, stream);
+    dyh = ws;
+  }
   if (rc) return rc;
-  rc = to_nhwc(x, xh, p.N, p.C, p.H * p.W, p.dtype, stream);
+  if (!xh) {
+    void* dst = ws + round256(p.N * p.O * p.OH * p.OW * 2);
+    rc = to_nhwc(x, dst, p.N, p.C, p.H * p.W, p.dtype, stream);
+    xh = dst;
+  }
   if (rc) return rc;
   DwArgs g{};
   g.dy = dyh; g.x = xh; g.part = part;

@@ -422,6 +422,11 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
     cw_wsb = lib.at_conv2d_bwd_weight_workspace_bytes(*dims, dt)
     conv_wsb = max(cf_wsb, cx_wsb, cw_wsb, 16)
     conv_ws = torch.empty(conv_wsb, dtype=torch.uint8, device='cuda')
+    # as attorch_amd.Conv2d does it: the forward workspace (channels-last input at its start) is
+    # kept for the weight gradient, and one channels-last copy of dY serves both gradients
+    fwd_wss = [torch.empty(max(cf_wsb, 16), dtype=torch.uint8, device='cuda') for _ in range(nsets)]
+    dyhs = [torch.empty_like(dys[0]) for _ in range(nsets)]
+    share = cf_wsb > 0 and cx_wsb > 0
     st = raw.stream
     counter = [0]
 
@@ -431,17 +436,25 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
 
     def conv_f():
         i = nxt()
-        raw.check(lib.at_conv2d_fwd(xs[i].data_ptr(), wt.data_ptr(), None, ys[i].data_ptr(), conv_ws.data_ptr(),
-                                    conv_wsb, *dims, dt, dt, dt, st()), 'conv_fwd')
+        raw.check(lib.at_conv2d_fwd(xs[i].data_ptr(), wt.data_ptr(), None, ys[i].data_ptr(), fwd_wss[i].data_ptr(),
+                                    cf_wsb, *dims, dt, dt, dt, st()), 'conv_fwd')
+
+    def conv_dyh():
+        i = nxt()
+        if share:
+            raw.check(lib.at_nchw_to_nhwc(dys[i].data_ptr(), dyhs[i].data_ptr(), n, c, h * w_, dt, st()), 'nhwc')
 
     def conv_dx():
         i = nxt()
-        raw.check(lib.at_conv2d_bwd_input(dys[i].data_ptr(), wt.data_ptr(), dxs[i].data_ptr(), conv_ws.data_ptr(),
+        raw.check(lib.at_conv2d_bwd_input(dys[i].data_ptr(), dyhs[i].data_ptr() if share else None, wt.data_ptr(),
+                                          dxs[i].data_ptr(), conv_ws.data_ptr(),
                                           conv_wsb, *dims, dt, st()), 'conv_dx')
 
     def conv_dw():
         i = nxt()
-        raw.check(lib.at_conv2d_bwd_weight(dys[i].data_ptr(), xs[i].data_ptr(), dwt.data_ptr(), conv_ws.data_ptr(),
+        raw.check(lib.at_conv2d_bwd_weight(dys[i].data_ptr(), dyhs[i].data_ptr() if share else None,
+                                           xs[i].data_ptr(), fwd_wss[i].data_ptr() if share else None,
+                                           dwt.data_ptr(), conv_ws.data_ptr(),
                                            conv_wsb, *dims, dt, st()), 'conv_dw')
 
     def bn_f():
@@ -459,14 +472,19 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
                                         dt, dt, st()), 'bn_bwd')
 
     iters = max(5, steps // 2)
-    for i in range(nsets):   # pre-activations must exist before the backward timing
+    for i in range(nsets):   # pre-activations and channels-last copies must exist before the backward timing
         counter[0] = i - 1
         bn_f()
-    t = {k_: gpu_time_ms(f, iters, warmup) for k_, f in (('conv_fwd', conv_f), ('conv_bwd_input', conv_dx),
+        counter[0] = i - 1
+        conv_f()
+        counter[0] = i - 1
+        conv_dyh()
+    t = {k_: gpu_time_ms(f, iters, warmup) for k_, f in (('conv_fwd', conv_f), ('conv_grad_to_channels_last', conv_dyh),
+                                                        ('conv_bwd_input', conv_dx),
                                                         ('conv_bwd_weight', conv_dw), ('bn_fwd', bn_f),
                                                         ('bn_bwd', bn_b_))}
     gflop = 2.0 * n * c * h * w_ * c * 9 / 1e9
-    conv_ms = t['conv_fwd'] + t['conv_bwd_input'] + t['conv_bwd_weight']
+    conv_ms = t['conv_fwd'] + t['conv_grad_to_channels_last'] + t['conv_bwd_input'] + t['conv_bwd_weight']
     conv_tf = 3 * gflop / conv_ms
     tbytes = n * c * h * w_ * 2
     bn_gbs = 9 * tbytes / (t['bn_fwd'] + t['bn_bwd']) / 1e6

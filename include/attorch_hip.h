@@ -267,6 +267,10 @@ int at_batch_norm_bwd(const void* output_grad, const void* pre_act, const void* 
  *   at_conv2d_*_workspace_bytes(...) returns the bytes that path wants for the given shape
  *   (0: no such path).  forward and bwd_input fall back to the generic kernel when the
  *   workspace is null or smaller; bwd_weight always needs its workspace (split-K partials).
+ *   Channels-last copies can be shared between calls: at_conv2d_fwd leaves the copy of the
+ *   input ([batch, height, width, feat]) at the start of its workspace, at_nchw_to_nhwc makes
+ *   one of any 16-bit NCHW tensor, and the backward entry points take such copies through
+ *   their nullable *_nhwc arguments instead of making their own (matrix-core path only).
  *   at_channel_sum: out[feat] = sum over batch and space of a [batch, feat, spatial] tensor.
  * ------------------------------------------------------------------------------------------ */
 int64_t at_conv2d_fwd_workspace_bytes(int64_t batch, int64_t in_feat, int64_t in_height,
@@ -293,8 +297,8 @@ int64_t at_conv2d_bwd_input_workspace_bytes(int64_t batch, int64_t in_feat, int6
                                             int64_t padding_height, int64_t padding_width,
                                             int64_t groups, int dtype);
 
-int at_conv2d_bwd_input(const void* output_grad, const void* weight, void* input_grad,
-                        void* workspace, int64_t workspace_bytes, int64_t batch, int64_t in_feat,
+int at_conv2d_bwd_input(const void* output_grad, const void* output_grad_nhwc,
+                        const void* weight, void* input_grad, void* workspace, int64_t workspace_bytes, int64_t batch, int64_t in_feat,
                         int64_t in_height, int64_t in_width, int64_t out_feat,
                         int64_t out_height, int64_t out_width, int64_t kernel_height,
                         int64_t kernel_width, int64_t stride_height, int64_t stride_width,
@@ -309,12 +313,16 @@ int64_t at_conv2d_bwd_weight_workspace_bytes(int64_t batch, int64_t in_feat, int
                                              int64_t padding_height, int64_t padding_width,
                                              int64_t groups, int dtype);
 
-int at_conv2d_bwd_weight(const void* output_grad, const void* input, void* weight_grad,
+int at_conv2d_bwd_weight(const void* output_grad, const void* output_grad_nhwc,
+                         const void* input, const void* input_nhwc, void* weight_grad,
                          void* workspace, int64_t workspace_bytes, int64_t batch, int64_t in_feat,
                          int64_t in_height, int64_t in_width, int64_t out_feat, int64_t out_height,
                          int64_t out_width, int64_t kernel_height, int64_t kernel_width,
                          int64_t stride_height, int64_t stride_width, int64_t padding_height,
                          int64_t padding_width, int64_t groups, int dtype, at_stream_t stream);
+
+int at_nchw_to_nhwc(const void* src, void* dst, int64_t batch, int64_t feat, int64_t spatial,
+                    int dtype, at_stream_t stream);
 
 int at_channel_sum(const void* x, void* out, int64_t batch, int64_t feat, int64_t spatial,
                    int x_dtype, int out_dtype, at_stream_t stream);
