@@ -12,8 +12,9 @@
 //    themselves (ds_read_b64_tr_b16).  Fragments are double-buffered in registers, and the
 //    finished tile leaves through LDS as whole 512-byte row segments.  Workgroup ids are
 //    remapped so that each XCD (own L2) works on a compact block of output tiles.
-//  * gemm_simple_kernel — any dtype, any strides, fp32 MFMA (32x32x2), 64x64 tile; used for
-//    fp32 tensors and for 16-bit shapes the fast kernel cannot address with 128-bit accesses.
+//  * gemm_simple_kernel — any dtype, any strides, fp32 MFMA (32x32x2), 64x64x64 tile, next k-tile
+//    prefetched into registers; used for fp32 tensors and for 16-bit shapes the fast kernel cannot
+//    address with 128-bit accesses.
 // Both fuse bias, the optional pre-activation store and the activation into the epilogue.
 #include <type_traits>
 
@@ -315,7 +316,8 @@ struct SimpleArgs {
 
 template <typename TI, typename TO>
 __global__ __launch_bounds__(256) void gemm_simple_kernel(SimpleArgs g) {
-  constexpr int TM = 64, TN = 64, TK = 16;
+  constexpr int TM = 64, TN = 64, TK = 64;
+  constexpr int PER = TM * TK / 256;   // elements of each operand tile per lane
   __shared__ float sa[TK][TM + 1];
   __shared__ float sb[TK][TN + 1];
   const TI* __restrict__ A = reinterpret_cast<const TI*>(g.a);
@@ -328,23 +330,43 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(SimpleArgs g) {
 #pragma unroll
   for (int e = 0; e < 16; ++e) acc[e] = 0.f;
 
-  // Tile loads: pick the thread->element mapping that follows the unit stride of each operand.
+  // Tile loads: the thread->element mapping follows the unit stride of each operand.  The next
+  // k-tile is fetched into registers while the current one is multiplied (small problems are
+  // bound by the latency of these loads, not by their volume).
   const bool a_k_fast = g.sak == 1;
   const bool b_n_fast = g.sbn == 1;
-  for (int k0 = 0; k0 < g.K; k0 += TK) {
+  float ra[PER], rb[PER];
+  auto fetch = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int e = threadIdx.x + i * 256;  // 1024 elements per operand tile
+    for (int i = 0; i < PER; ++i) {
+      const int e = threadIdx.x + i * 256;
       int mm, kk;
-      if (a_k_fast) { kk = e & 15; mm = e >> 4; } else { mm = e & 63; kk = e >> 6; }
+      if (a_k_fast) { kk = e & (TK - 1); mm = e / TK; } else { mm = e & (TM - 1); kk = e / TM; }
       const int m = m0 + mm, k = k0 + kk;
-      sa[kk][mm] = (m < g.M && k < g.K) ? to_f32(A[(int64_t)m * g.sam + (int64_t)k * g.sak]) : 0.f;
+      ra[i] = (m < g.M && k < g.K) ? to_f32(A[(int64_t)m * g.sam + (int64_t)k * g.sak]) : 0.f;
       int nn, kb;
-      if (b_n_fast) { nn = e & 63; kb = e >> 6; } else { kb = e & 15; nn = e >> 4; }
+      if (b_n_fast) { nn = e & (TN - 1); kb = e / TN; } else { kb = e & (TK - 1); nn = e / TK; }
       const int n = n0 + nn, k2 = k0 + kb;
-      sb[kb][nn] = (n < g.N && k2 < g.K) ? to_f32(B[(int64_t)k2 * g.sbk + (int64_t)n * g.sbn]) : 0.f;
+      rb[i] = (n < g.N && k2 < g.K) ? to_f32(B[(int64_t)k2 * g.sbk + (int64_t)n * g.sbn]) : 0.f;
     }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int e = threadIdx.x + i * 256;
+      int mm, kk;
+      if (a_k_fast) { kk = e & (TK - 1); mm = e / TK; } else { mm = e & (TM - 1); kk = e / TM; }
+      sa[kk][mm] = ra[i];
+      int nn, kb;
+      if (b_n_fast) { nn = e & (TN - 1); kb = e / TN; } else { kb = e & (TK - 1); nn = e / TK; }
+      sb[kb][nn] = rb[i];
+    }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < g.K; k0 += TK) {
+    stage();
     __syncthreads();
+    if (k0 + TK < g.K) fetch(k0 + TK);
 #pragma unroll
     for (int ks = 0; ks < TK; ks += 2) {
       // operands swapped so that a lane ends up with 4 consecutive n of one m
