@@ -31,6 +31,21 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E, GB/s
 PEAK_MFMA_16BIT_TFLOPS = 2500.0  # dense bf16 / fp16 MFMA
 PEAK_MFMA_FP32_TFLOPS = 157.3    # dense fp32 MFMA
 
+# Bytes that cross between L2 and the memory fabric per launch (per forward + backward for the
+# multi-kernel workloads), from the rocprofv3 FETCH_SIZE / WRITE_SIZE passes summarised in
+# profiles/bench_all_configs.hbm_traffic.txt (scaled there by a copy of known size).  Counters are
+# taken in separate profiling runs, so these are recorded measurements, not live ones; reads that
+# the 256 MB Infinity Cache serves are included.
+MEASURED_TRAFFIC_BYTES = {
+    'c4_linear_fwd': 4331900620,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.09 GiB read, 1.0 GiB written
+    'c2_layer_norm': 387451410,       # norm_fwd + norm_bwd + reduce_partials
+    'c2_rms_norm': 378432107,
+    'c2_softmax': 335719684,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
+    'c3_cross_entropy': 1609265111,   # ce_row_kernel (ignored rows are not read)
+    'c5_conv': 644439252,             # 2 window kernels + weight gradient + 2 layout copies + weight reorders
+    'c5_batch_norm': 616866723,       # stats + apply + backward reduce + backward apply
+}
+
 
 def parse_args() -> argparse.Namespace:
     parser = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawTextHelpFormatter)
@@ -204,7 +219,7 @@ def bench_linear(cfg: str, steps: int, warmup: int, with_cpu: bool) -> Dict:
                           for kk in ('linear_fwd', 'linear_bwd_input', 'linear_bwd_weight')},
         'roofline': {'bound': 'mfma', 'kernel': 'linear_fwd (GEMM + bias + activation epilogue)',
                      'achieved': fwd_tflops, 'peak': peak, 'unit': 'TFLOP/s', 'frac': fwd_tflops / peak,
-                     'traffic': None},
+                     'traffic': MEASURED_TRAFFIC_BYTES['c4_linear_fwd'] if cfg == 'c4' else None},
         'frac_of_peak_step': flop / ms_step / 1e9 / peak,
     }
     if with_cpu:
@@ -312,6 +327,19 @@ def bench_rows(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
             oracle.softmax_backward(dyc[:crow], y, False, log)
         return f
 
+    # What a plain elementwise pass reaches on the same buffers, for scale: one read + one write of
+    # a tensor (torch.mul) and two reads + one write (torch.add), timed the same way.
+    def ew2():
+        i = nxt()
+        torch.mul(xs[i], 2.0, out=ys[i])
+
+    def ew3():
+        i = nxt()
+        torch.add(xs[i], dys[i], out=dxs[i])
+    stream_ref = {'read1_write1_gbs': 2 * tbytes / gpu_time_ms(ew2, iters, warmup) / 1e6,
+                  'read2_write1_gbs': 3 * tbytes / gpu_time_ms(ew3, iters, warmup) / 1e6}
+    traffic_key = {'LayerNorm': 'c2_layer_norm', 'RMSNorm': 'c2_rms_norm', 'Softmax': 'c2_softmax',
+                   'LogSoftmax': 'c2_softmax'}
     for name, f, bwd, cpu in (('LayerNorm', ln_f, ln_b, cpu_ln), ('RMSNorm', rms_f, rms_b, cpu_rms),
                               ('Softmax', sm_f, sm_b, cpu_sm(False)), ('LogSoftmax', lsm_f, lsm_b, cpu_sm(True))):
         ms_f = gpu_time_ms(f, iters, warmup)
@@ -322,8 +350,9 @@ def bench_rows(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
             'unit': 'GB/s', 'ms_fwd': ms_f, 'ms_bwd': ms_b,
             'fwd_gbs': 2 * tbytes / ms_f / 1e6, 'bwd_gbs': 3 * tbytes / ms_b / 1e6,
             'roofline': {'bound': 'hbm', 'achieved': gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
-                         'frac': gbs / PEAK_HBM_GBS, 'traffic': None},
+                         'frac': gbs / PEAK_HBM_GBS, 'traffic': MEASURED_TRAFFIC_BYTES[traffic_key[name]]},
             'buffer_rotation': f'{nsets} sets of X/dY/Y/dX (64 MiB each)',
+            'elementwise_reference': stream_ref,
         }
         if with_cpu:
             sec = cpu_time_s(cpu)
@@ -371,7 +400,7 @@ def bench_cross_entropy(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
             'workload': f'c3: CrossEntropyLoss fp16 fwd+bwd logits[{rows_},{feat}], 5% ignore_index, {label}',
             'metric': 'HBM GB/s', 'value': gbs, 'unit': 'GB/s', 'ms_fwd_bwd': ms,
             'roofline': {'bound': 'hbm', 'achieved': gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
-                         'frac': gbs / PEAK_HBM_GBS, 'traffic': None},
+                         'frac': gbs / PEAK_HBM_GBS, 'traffic': MEASURED_TRAFFIC_BYTES['c3_cross_entropy']},
         }
         if with_cpu and wt is None:
             crow = 512
@@ -492,13 +521,13 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
         'workload': f'c5: Conv2d 3x3 s1 p1 bf16 fwd+bwd X[{n},{c},{h},{w_}] W[{c},{c},3,3]',
         'metric': 'conv TFLOP/s', 'value': conv_tf, 'unit': 'TFLOP/s', 'kernel_ms': {k_: t[k_] for k_ in t if 'conv' in k_},
         'roofline': {'bound': 'mfma', 'achieved': conv_tf, 'peak': PEAK_MFMA_16BIT_TFLOPS, 'unit': 'TFLOP/s',
-                     'frac': conv_tf / PEAK_MFMA_16BIT_TFLOPS, 'traffic': None},
+                     'frac': conv_tf / PEAK_MFMA_16BIT_TFLOPS, 'traffic': MEASURED_TRAFFIC_BYTES['c5_conv']},
     }
     bn_entry = {
         'workload': f'c5: BatchNorm2d(train)+residual+ReLU bf16 fwd+bwd X[{n},{c},{h},{w_}]',
         'metric': 'HBM GB/s', 'value': bn_gbs, 'unit': 'GB/s', 'ms_fwd': t['bn_fwd'], 'ms_bwd': t['bn_bwd'],
         'roofline': {'bound': 'hbm', 'achieved': bn_gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
-                     'frac': bn_gbs / PEAK_HBM_GBS, 'traffic': None},
+                     'frac': bn_gbs / PEAK_HBM_GBS, 'traffic': MEASURED_TRAFFIC_BYTES['c5_batch_norm']},
         'buffer_rotation': f'{nsets} sets of 7 tensors (49 MiB each)',
     }
     # the block end to end through the modules (conv -> bn + residual + relu, fwd + bwd)
