@@ -76,6 +76,65 @@ def test_conv_modules_match_torch() -> None:
         assert ours(x).dtype is torch.float16
 
 
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_conv_matrix_core_path_agrees_with_generic_kernel(dtype) -> None:
+    """
+    Straight through the C ABI: with its workspace the 16-bit convolution runs on the matrix
+    cores from channels-last copies, without it on the generic gather kernel; both must agree
+    to 16-bit rounding, and the shared channels-last copies must not change a result.
+    """
+    from attorch_amd import _lib
+    lib = _lib.load()
+    n, c, h, w, o, k = 3, 64, 9, 10, 128, 3
+    dims = (n, c, h, w, o, h, w, k, k, 1, 1, 1, 1, 1)
+    dt = _lib.dtype_id(dtype)
+    x = randn((n, c, h, w), 1, dtype).cuda()
+    wt = randn((o, c, k, k), 2, dtype, (c * k * k) ** -0.5).cuda()
+    dy = randn((n, o, h, w), 3, dtype).cuda()
+    stream = _lib.stream_of(x)
+
+    def workspace(n_bytes):
+        assert n_bytes > 0
+        return torch.empty(n_bytes, dtype=torch.uint8, device='cuda'), n_bytes
+
+    ws_f, nb_f = workspace(lib.at_conv2d_fwd_workspace_bytes(*dims, dt, dt))
+    ws_x, nb_x = workspace(lib.at_conv2d_bwd_input_workspace_bytes(*dims, dt))
+    ws_w, nb_w = workspace(lib.at_conv2d_bwd_weight_workspace_bytes(*dims, dt))
+    y_fast, y_slow = torch.empty_like(dy), torch.empty_like(dy)
+    _lib.check(lib.at_conv2d_fwd(_lib.ptr(x), _lib.ptr(wt), None, _lib.ptr(y_fast), _lib.ptr(ws_f), nb_f,
+                                 *dims, dt, dt, dt, stream), 'fwd')
+    _lib.check(lib.at_conv2d_fwd(_lib.ptr(x), _lib.ptr(wt), None, _lib.ptr(y_slow), None, 0,
+                                 *dims, dt, dt, dt, stream), 'fwd')
+    assert_close(y_fast, y_slow.cpu(), dtype, 'output', normalize=True)
+    # the forward workspace starts with the channels-last input
+    x_nhwc = ws_f[:x.numel() * 2].view(dtype).view(n, h, w, c)
+    assert torch.equal(x_nhwc, x.permute(0, 2, 3, 1))
+
+    dy_nhwc = torch.empty_like(dy)
+    _lib.check(lib.at_nchw_to_nhwc(_lib.ptr(dy), _lib.ptr(dy_nhwc), n, o, h * w, dt, stream), 'nhwc')
+    assert torch.equal(dy_nhwc.view(n, h, w, o), dy.permute(0, 2, 3, 1))
+
+    dx_own, dx_shared, dx_slow = (torch.empty_like(x) for _ in range(3))
+    _lib.check(lib.at_conv2d_bwd_input(_lib.ptr(dy), None, _lib.ptr(wt), _lib.ptr(dx_own), _lib.ptr(ws_x), nb_x,
+                                       *dims, dt, stream), 'dx')
+    _lib.check(lib.at_conv2d_bwd_input(_lib.ptr(dy), _lib.ptr(dy_nhwc), _lib.ptr(wt), _lib.ptr(dx_shared),
+                                       _lib.ptr(ws_x), nb_x, *dims, dt, stream), 'dx')
+    _lib.check(lib.at_conv2d_bwd_input(_lib.ptr(dy), None, _lib.ptr(wt), _lib.ptr(dx_slow), None, 0,
+                                       *dims, dt, stream), 'dx')
+    assert torch.equal(dx_own, dx_shared)
+    assert_close(dx_own, dx_slow.cpu(), dtype, 'input_grad', normalize=True)
+
+    dw_own, dw_shared = torch.empty_like(wt), torch.empty_like(wt)
+    _lib.check(lib.at_conv2d_bwd_weight(_lib.ptr(dy), None, _lib.ptr(x), None, _lib.ptr(dw_own), _lib.ptr(ws_w),
+                                        nb_w, *dims, dt, stream), 'dw')
+    _lib.check(lib.at_conv2d_bwd_weight(_lib.ptr(dy), _lib.ptr(dy_nhwc), _lib.ptr(x), _lib.ptr(ws_f),
+                                        _lib.ptr(dw_shared), _lib.ptr(ws_w), nb_w, *dims, dt, stream), 'dw')
+    assert torch.equal(dw_own, dw_shared)
+    # a weight-gradient call without workspace is an error, not a silent fallback
+    assert lib.at_conv2d_bwd_weight(_lib.ptr(dy), None, _lib.ptr(x), None, _lib.ptr(dw_own), None, 0,
+                                    *dims, dt, stream) == -5
+
+
 BN_SHAPES = [(6, 5), (128, 1024), (2048, 768), (8, 960, 196), (2048, 64, 16), (2, 3, 224, 224),
              (16, 64, 56, 56), (32, 128, 7, 7), (3, 7, 3, 5)]
 
