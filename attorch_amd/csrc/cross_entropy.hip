@@ -53,7 +53,7 @@ __global__ __launch_bounds__(1024) void ce_finalize_kernel(
 // at most 7 + 7 "edge" elements before the first and after the last interior vector, each
 // owned by one of the first 16 lanes and moved with element accesses.
 template <typename T, int CACHE_VECS>
-__global__ __launch_bounds__(kCeBlock, 4) void ce_row_kernel(
+__global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_kernel(
     const T* __restrict__ logits, const int64_t* __restrict__ target, const void* __restrict__ weight,
     int wdt, const float* __restrict__ denom, float* __restrict__ row_loss, T* __restrict__ dlogits,
     int feat, int64_t xs, int64_t ds, int64_t ignore_index) {
@@ -296,6 +296,7 @@ int at_cross_entropy_fwd_bwd(const void* logits, const int64_t* target, const vo
       if (per_lane <= 2) AT_CE_LAUNCH(2);
       else if (per_lane <= 4) AT_CE_LAUNCH(4);
       else if (per_lane <= 8) AT_CE_LAUNCH(8);
+      else if (per_lane <= 13) AT_CE_LAUNCH(13);   // up to 13 vectors: registers for three workgroups per CU
       else AT_CE_LAUNCH(16);
 #undef AT_CE_LAUNCH
     } else if (out_dtype == logits_dtype) {
