@@ -2,11 +2,15 @@
 MI355X-native implementation of attorch's layer-kernel hot path.
 
 The public names match attorch's (Linear, LayerNorm, RMSNorm, Softmax, LogSoftmax, Softmin,
-CrossEntropyLoss, Conv2d, BatchNorm2d and their autograd Functions), so
+CrossEntropyLoss, Conv2d, BatchNorm2d, the activation layers with fused dropout, Dropout, and
+their autograd Functions), so
 `import attorch_amd as attorch` is a drop-in for that path.  All compute happens in
 hand-written gfx950 HIP kernels behind the C ABI declared in include/attorch_hip.h.
 """
 
+from .act_layers import (CELU, ELU, GELU, SELU, ActFuncAutoGrad, Dropout, DropoutAutoGrad, Hardshrink,
+                         Hardsigmoid, Hardswish, Hardtanh, LeakyReLU, LogSigmoid, Mish, ReLU, ReLU6,
+                         Sigmoid, SiLU, Softplus, Softshrink, Softsign, Tanh, Tanhshrink)
 from .batch_norm import BatchNorm1d, BatchNorm2d, BatchNormAutoGrad
 from .conv import Conv1d, Conv2d, Conv2dAutoGrad
 from .cross_entropy import CrossEntropyLoss, CrossEntropyLossAutoGrad

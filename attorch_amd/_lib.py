@@ -17,7 +17,7 @@ LIB_PATH = Path(__file__).resolve().parent / 'lib' / 'libattorch_hip.so'
 
 DTYPE_IDS = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
-P, I, L, F = c_void_p, c_int, c_int64, c_float
+P, I, L, F, U = c_void_p, c_int, c_int64, c_float, ctypes.c_uint32
 
 # name -> (restype, argtypes); the order is the order of include/attorch_hip.h
 PROTOTYPES = {
@@ -50,6 +50,8 @@ PROTOTYPES = {
     'at_conv2d_bwd_weight': (I, [P, P, P, P, P, P, L] + [L] * 14 + [I, P]),
     'at_nchw_to_nhwc': (I, [P, P, L, L, L, I, P]),
     'at_channel_sum': (I, [P, P, L, L, L, I, I, P]),
+    'at_act_dropout_fwd': (I, [P, P, L, I, F, F, U, I, P]),
+    'at_act_dropout_bwd': (I, [P, P, P, L, I, F, F, U, I, P]),
     'at_batch_norm_bwd': (I, [P, P, P, P, P, P, P, P, P, P, P, L, L, L, L, I, F, I, I, P]),
 }
 

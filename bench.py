@@ -338,10 +338,27 @@ def bench_rows(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
         torch.add(xs[i], dys[i], out=dxs[i])
     stream_ref = {'read1_write1_gbs': 2 * tbytes / gpu_time_ms(ew2, iters, warmup) / 1e6,
                   'read2_write1_gbs': 3 * tbytes / gpu_time_ms(ew3, iters, warmup) / 1e6}
+    # standalone activation layer with fused dropout on the same buffers (GELU-tanh, p = 0.1)
+    def act_f():
+        i = nxt()
+        raw.check(lib.at_act_dropout_fwd(xs[i].data_ptr(), ys[i].data_ptr(), rows_ * feat, 6, 0.0, 0.1, 4711, dt,
+                                         st()), 'act_fwd')
+
+    def act_b():
+        i = nxt()
+        raw.check(lib.at_act_dropout_bwd(dys[i].data_ptr(), xs[i].data_ptr(), dxs[i].data_ptr(), rows_ * feat, 6,
+                                         0.0, 0.1, 4711, dt, st()), 'act_bwd')
+
+    def cpu_act():
+        dropped = torch.rand(crow, feat) < 0.1
+        oracle.act_dropout_forward(xc[:crow], 'geluapprox', None, dropped, 0.1)
+        oracle.act_dropout_backward(dyc[:crow], xc[:crow], 'geluapprox', None, dropped, 0.1)
+
     traffic_key = {'LayerNorm': 'c2_layer_norm', 'RMSNorm': 'c2_rms_norm', 'Softmax': 'c2_softmax',
-                   'LogSoftmax': 'c2_softmax'}
+                   'LogSoftmax': 'c2_softmax', 'GELU(tanh)+Dropout(0.1) layer': None}
     for name, f, bwd, cpu in (('LayerNorm', ln_f, ln_b, cpu_ln), ('RMSNorm', rms_f, rms_b, cpu_rms),
-                              ('Softmax', sm_f, sm_b, cpu_sm(False)), ('LogSoftmax', lsm_f, lsm_b, cpu_sm(True))):
+                              ('Softmax', sm_f, sm_b, cpu_sm(False)), ('LogSoftmax', lsm_f, lsm_b, cpu_sm(True)),
+                              ('GELU(tanh)+Dropout(0.1) layer', act_f, act_b, cpu_act)):
         ms_f = gpu_time_ms(f, iters, warmup)
         ms_b = gpu_time_ms(bwd, iters, warmup)
         gbs = 5 * tbytes / (ms_f + ms_b) / 1e6
@@ -350,7 +367,7 @@ def bench_rows(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
             'unit': 'GB/s', 'ms_fwd': ms_f, 'ms_bwd': ms_b,
             'fwd_gbs': 2 * tbytes / ms_f / 1e6, 'bwd_gbs': 3 * tbytes / ms_b / 1e6,
             'roofline': {'bound': 'hbm', 'achieved': gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
-                         'frac': gbs / PEAK_HBM_GBS, 'traffic': MEASURED_TRAFFIC_BYTES[traffic_key[name]]},
+                         'frac': gbs / PEAK_HBM_GBS, 'traffic': MEASURED_TRAFFIC_BYTES.get(traffic_key[name])},
             'buffer_rotation': f'{nsets} sets of X/dY/Y/dX (64 MiB each)',
             'elementwise_reference': stream_ref,
         }

@@ -327,6 +327,27 @@ int at_nchw_to_nhwc(const void* src, void* dst, int64_t batch, int64_t feat, int
 int at_channel_sum(const void* x, void* out, int64_t batch, int64_t feat, int64_t spatial,
                    int x_dtype, int out_dtype, at_stream_t stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Standalone activation layers with fused dropout, and Dropout — replace
+ * act_func_forward_kernel / act_func_backward_kernel, attorch/act_kernels.py:845-927 (launched
+ * from attorch/act_layers.py:78-80,108-111), and dropout_forward_kernel /
+ * dropout_backward_kernel, attorch/dropout_kernels.py:54-112 (launched from
+ * attorch/dropout_layer.py:53-58,88-93).  Flat tensors of `size` elements, one dtype.
+ *   fwd: output     = dropout(act(input))                   (act_kernels.py:729-730)
+ *   bwd: input_grad = dropout'(output_grad) * act'(input)   (act_kernels.py:834-837)
+ * act = AT_ACT_NONE gives plain dropout (input may then be null in bwd).  drop_p = 0 disables
+ * dropout (pass 0 outside training).  A dropped element is exactly zero, kept ones are scaled
+ * by 1 / (1 - drop_p) (dropout_kernels.py:26-27).  The mask is a pure function of (seed,
+ * element index) — Philox4x32-10 (16 bits per element), not Triton's generator, so masks differ from the
+ * reference's for equal seeds; forward and backward of one call pair agree.
+ * ------------------------------------------------------------------------------------------ */
+int at_act_dropout_fwd(const void* input, void* output, int64_t size, int act, float param,
+                       float drop_p, uint32_t seed, int dtype, at_stream_t stream);
+
+int at_act_dropout_bwd(const void* output_grad, const void* input, void* input_grad,
+                       int64_t size, int act, float param, float drop_p, uint32_t seed,
+                       int dtype, at_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

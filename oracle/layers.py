@@ -437,3 +437,45 @@ def batch_norm_backward(
     dx = r * (w[None, :, None] * g - (t1 * pre_lin + t2))
     return (dx.to(input.dtype).view(input.shape), term1 if affine else None,
             term2 if affine else None, g_store.view(input.shape))
+
+
+# ---------------------------------------------------------------------------------------------
+# Activation layers with fused dropout, Dropout — attorch/act_kernels.py:631-927,
+# attorch/dropout_kernels.py:13-112, attorch/act_layers.py:20-117, attorch/dropout_layer.py:19-96
+# ---------------------------------------------------------------------------------------------
+def act_dropout_forward(
+    input: Tensor, act_func: Optional[str], param: Optional[float], dropped: Optional[Tensor],
+    drop_p: float, compute: torch.dtype = torch.float32,
+    ) -> Tensor:
+    """
+    output = dropout(act(input)) in the input's dtype: the activation is evaluated on the
+    widened input (act_kernels.py:654-727), then elements of the mask `dropped` become 0 and
+    the others are divided by 1 - drop_p (act_kernels.py:729-730, dropout_kernels.py:26-27).
+    The random mask itself is implementation defined (the reference draws it with tl.rand), so
+    it is an argument here: callers read it off the device result, as the reference's own
+    tests do (tests/test_act_layers.py:49-51, tests/test_dropout_layer.py:30).
+    `dropped` None means no dropout.
+    """
+    x = input.to(compute)
+    out = x if act_func is None else act_forward(x, act_func, param)
+    if dropped is not None:
+        out = torch.where(dropped, torch.zeros((), dtype=compute), out / (1 - drop_p))
+    return out.to(input.dtype)
+
+
+def act_dropout_backward(
+    output_grad: Tensor, input: Optional[Tensor], act_func: Optional[str], param: Optional[float],
+    dropped: Optional[Tensor], drop_p: float, compute: torch.dtype = torch.float32,
+    ) -> Tensor:
+    """
+    input_grad = dropout'(output_grad) * act'(input) (act_kernels.py:834-837): the upstream
+    gradient goes through the same mask and scale (dropout_kernels.py:45-46) and is multiplied
+    by the derivative of the activation at the forward input.
+    """
+    g = output_grad.to(compute)
+    if dropped is not None:
+        g = torch.where(dropped, torch.zeros((), dtype=compute), g / (1 - drop_p))
+    if act_func is not None:
+        g = g * act_grad(input.to(compute), act_func, param)
+    dtype = output_grad.dtype if input is None else input.dtype
+    return g.to(dtype)

@@ -70,6 +70,8 @@ def test_argument_errors_without_gpu() -> None:
     assert lib.at_layer_norm_bwd(p, p, p, p, p, p, p, None, p, 16, 4, 8, 8, 8, 8, 0, 0, 0, 0, None) == -5
     assert lib.at_batch_norm_fwd(p, None, None, None, None, None, None, p, None, None, None, 0,
                                  4, 8, 1, 0.1, 1e-5, 0, 0.0, 0, 1, 0, 0, 0, None) == -5
+    assert lib.at_act_dropout_fwd(p, p, 8, 0, 0.0, 1.5, 0, 0, None) == -2
+    assert lib.at_act_dropout_bwd(p, None, p, 8, 4, 0.0, 0.0, 0, 0, None) == -1
     # inconsistent convolution geometry
     dims = [1, 4, 8, 8, 4, 9, 9, 3, 3, 1, 1, 1, 1, 1]
     assert lib.at_conv2d_fwd(p, p, None, p, None, 0, *dims, 0, 0, 0, None) == -2

@@ -279,3 +279,29 @@ def test_batch_norm_eval_uses_running_stats() -> None:
     out2, _, _, _, _, _ = oracle.batch_norm_forward(x, False, w, b, None, None, 0.1, 1e-5, False, None, None,
                                                     None, compute=D)
     torch.testing.assert_close(out2, F.batch_norm(x, None, None, w, b, True, 0.1, 1e-5), **TOL)
+
+
+# ---------------------------------------------------------------------------------------------
+# activation layers with fused dropout
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize('act_func, param, torch_fn', [
+    ('relu', None, F.relu), ('geluapprox', None, lambda x: F.gelu(x, approximate='tanh')),
+    ('leaky_relu', 0.2, lambda x: F.leaky_relu(x, 0.2)), (None, None, lambda x: x)])
+@pytest.mark.parametrize('drop_p', [0.0, 0.3])
+def test_act_dropout_matches_torch_with_the_same_mask(act_func, param, torch_fn, drop_p) -> None:
+    # Independent statement: torch's activation + autograd, the mask applied as a constant
+    # multiplier mask / (1 - p) (what F.dropout does with its own mask).
+    torch.manual_seed(0)
+    x = torch.randn(64, 33, dtype=torch.float64, requires_grad=True)
+    dy = torch.randn(64, 33, dtype=torch.float64)
+    dropped = (torch.rand(64, 33) < drop_p) if drop_p > 0 else None
+    scale = torch.ones_like(x) if dropped is None else (~dropped).double() / (1 - drop_p)
+    expected = torch_fn(x) * scale
+    (expected_grad,) = torch.autograd.grad(expected, x, dy)
+    got = oracle.act_dropout_forward(x.detach(), act_func, param, dropped, drop_p, compute=torch.float64)
+    got_grad = oracle.act_dropout_backward(dy, x.detach(), act_func, param, dropped, drop_p,
+                                           compute=torch.float64)
+    torch.testing.assert_close(got, expected.detach(), rtol=1e-7, atol=1e-7)
+    torch.testing.assert_close(got_grad, expected_grad, rtol=1e-7, atol=1e-7)
+    if dropped is not None:
+        assert torch.count_nonzero(got[dropped]) == 0 and torch.count_nonzero(got_grad[dropped]) == 0
