@@ -18,3 +18,12 @@ from .linear import Linear, LinearAutoGrad
 from .norms import LayerNorm, LayerNormAutoGrad, RMSNorm, RMSNormAutoGrad
 from .softmax import LogSoftmax, Softmax, SoftmaxAutoGrad, Softmin
 from .utils import get_output_dtype
+
+__all__ = [
+    'ActFuncAutoGrad', 'BatchNorm1d', 'BatchNorm2d', 'BatchNormAutoGrad', 'CELU', 'Conv1d', 'Conv2d',
+    'Conv2dAutoGrad', 'CrossEntropyLoss', 'CrossEntropyLossAutoGrad', 'Dropout', 'DropoutAutoGrad', 'ELU',
+    'GELU', 'Hardshrink', 'Hardsigmoid', 'Hardswish', 'Hardtanh', 'LayerNorm', 'LayerNormAutoGrad',
+    'LeakyReLU', 'Linear', 'LinearAutoGrad', 'LogSigmoid', 'LogSoftmax', 'Mish', 'RMSNorm',
+    'RMSNormAutoGrad', 'ReLU', 'ReLU6', 'SELU', 'SiLU', 'Sigmoid', 'Softmax', 'SoftmaxAutoGrad', 'Softmin',
+    'Softplus', 'Softshrink', 'Softsign', 'Tanh', 'Tanhshrink', 'get_output_dtype',
+]
