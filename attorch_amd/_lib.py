@@ -35,7 +35,8 @@ PROTOTYPES = {
     'at_cross_entropy_scale_grad': (I, [P, P, L, L, L, I, I, P]),
     'at_linear_fwd': (I, [P, P, P, P, P, L, L, L, L, L, L, L, I, F, I, I, I, P]),
     'at_linear_bwd_input': (I, [P, P, P, L, L, L, L, L, L, I, I, P]),
-    'at_linear_bwd_weight': (I, [P, P, P, L, L, L, L, L, L, I, I, P]),
+    'at_linear_bwd_weight_workspace_bytes': (L, [L, L, L, I]),
+    'at_linear_bwd_weight': (I, [P, P, P, P, L, L, L, L, L, L, L, I, I, P]),
     'at_act_bwd_workspace_bytes': (L, [L, L]),
     'at_act_bwd': (I, [P, P, P, P, P, L, L, L, L, L, L, I, F, I, I, I, P]),
     'at_colsum_workspace_bytes': (L, [L, L]),

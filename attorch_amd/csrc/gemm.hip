@@ -1,6 +1,6 @@
 // Linear layer GEMMs: Y = act(X W + b) and the two backward products, fp32 accumulate.
 //
-// Two kernels:
+// Four kernels:
 //  * gemm_mfma16_kernel — bf16/fp16 operands on v_mfma_f32_32x32x16 (MFMA-bound).  256x256x64
 //    macro-tile per 256-lane workgroup (4 waves, 128x128 each, 256 accumulator registers per
 //    lane), LDS double-buffered, one barrier per k-tile.  Tiles go from global memory straight
@@ -12,10 +12,17 @@
 //    themselves (ds_read_b64_tr_b16).  Fragments are double-buffered in registers, and the
 //    finished tile leaves through LDS as whole 512-byte row segments.  Workgroup ids are
 //    remapped so that each XCD (own L2) works on a compact block of output tiles.
-//  * gemm_simple_kernel — any dtype, any strides, fp32 MFMA (32x32x2), 64x64x64 tile, next k-tile
-//    prefetched into registers; used for fp32 tensors and for 16-bit shapes the fast kernel cannot
-//    address with 128-bit accesses.
-// Both fuse bias, the optional pre-activation store and the activation into the epilogue.
+//  * gemm_mid16_kernel — the same operands in 128x128x64 tiles, two workgroups per CU, for
+//    problems with too few 256x256 tiles to fill the chip; for the weight gradient it can also
+//    split the contraction (the batch) over blockIdx.y into fp32 partial tiles that
+//    gemm_split_finish_kernel adds up in a fixed order.
+//  * gemm_small16_kernel — bf16/fp16 operands with any strides and extents (16-byte loads where
+//    an operand allows them, element loads otherwise), 64x64 or 128x32 tiles: skinny outputs,
+//    small problems, rows that are not 16-byte aligned.
+//  * gemm_simple_kernel — fp32 operands, any strides, fp32 MFMA (32x32x2), 64x64x64 tile, next
+//    k-tile prefetched into registers.
+// All fuse bias, the optional pre-activation store and the activation into the epilogue.
+#include <cstdlib>
 #include <type_traits>
 
 #include "at_act.h"
@@ -35,6 +42,12 @@ struct GemmArgs {
   int act;
   float param;
   int bias_dt;
+  // split of the contraction (128x128 kernel only): blockIdx.y takes k-tiles
+  // [y * kt_per_split, (y + 1) * kt_per_split) and stores its fp32 partial tile to
+  // partial[y][m][n] (row pitch ldw) instead of C
+  float* partial;
+  int kt_per_split;
+  int ldw;
 };
 
 constexpr int BM = 256, BN = 256, BK = 64;
@@ -67,7 +80,7 @@ struct OperandLoader {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     K = K_;
     if (CONTRACT_CONTIG) {
-      rsrc = make_buffer_rsrc(base, outer_total * ld * 2);
+      rsrc = make_buffer_rsrc(base, ((int64_t)(outer_total - 1) * ld + K_) * 2);   // the last row ends at its last element
       // load i of wave w fills rows 8q .. 8q+7 (q = 8w + i); lane -> (row, position), and the
       // position holds chunk (position ^ swizzle(row)) so that the reads find chunk c at c ^ swizzle
       const int row = wave * 64 + (lane >> 3);            // + 8 i
@@ -76,7 +89,9 @@ struct OperandLoader {
       blk_step = (int)(8 * ld * 2);
       k_step = BK * 2;
     } else {
-      rsrc = make_buffer_rsrc(base, K_ * ld * 2);
+      // up to the end of the 16-byte unit that holds the last element (rows start on such units,
+      // and the range check drops a dword that is only partly inside)
+      rsrc = make_buffer_rsrc(base, ((int64_t)(K_ - 1) * ld + ((outer_total + 7) & ~7)) * 2);
       // load i of wave w fills k-rows 2q, 2q+1 (q = 8w + i); lane -> k-row 2q + lane/32, 8 columns at (lane%32)*8
       const int krow = wave * 16 + (lane >> 5);            // + 2 i
       k_lane = 0;
@@ -305,7 +320,266 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_mfma16_kernel(GemmArgs g) {
 }
 
 // ------------------------------------------------------------------------------------------
-// Generic kernel: element strides for both operands, fp32 MFMA 32x32x2, 64x64x16 tiles.
+// Mid-size problems: 128x128x64 tiles, 2x2 waves of 64x64.  The same operands as the kernel above
+// for shapes whose 256x256 tiling would leave most of the CUs idle.  Two workgroups share a CU
+// (64 accumulator registers per lane, 66 KB of LDS) and cover each other's latencies, so the
+// loop is plain: issue the loads of tile kt+1, multiply tile kt, one barrier.  The activation
+// is applied after the accumulators have been staged in LDS as fp32, in a rolled loop, so one
+// kernel serves every activation.
+// ------------------------------------------------------------------------------------------
+constexpr int MT = 128;                          // tile edge
+constexpr int kMidTileBytes = MT * BK * 2;       // one operand tile, 16 KiB
+constexpr int kMidStage = 2 * kMidTileBytes;
+constexpr int kMidEpiPitch = MT + 4;             // floats per row of the staged output tile
+constexpr int kMidLds = 2 * kMidStage > MT * kMidEpiPitch * 4 ? 2 * kMidStage : MT * kMidEpiPitch * 4;
+
+// LDS image of an operand tile stored [k][outer] in memory: 64 k-rows x 256 bytes as loaded,
+// four rows per KiB (one wave-wide load), the 16-byte chunk index XORed with 4 * (k-row % 4) so
+// that the four rows a transposing fragment read touches fall on different banks.
+template <typename T, bool CONTRACT_CONTIG>
+struct MidLoader {
+  i32x4 rsrc;
+  int lane_off, blk_step, k_step, K;
+
+  __device__ __forceinline__ void init(const T* base, int64_t ld, int outer0, int outer_total, int K_) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    K = K_;
+    if (CONTRACT_CONTIG) {
+      rsrc = make_buffer_rsrc(base, ((int64_t)(outer_total - 1) * ld + K_) * 2);
+      lane_off = (int)(((int64_t)(outer0 + wave * 32 + (lane >> 3)) * ld) * 2);   // + 8 rows per load
+      blk_step = (int)(8 * ld * 2);
+      k_step = BK * 2;
+    } else {
+      rsrc = make_buffer_rsrc(base, ((int64_t)(K_ - 1) * ld + ((outer_total + 7) & ~7)) * 2);
+      const int krow = wave * 16 + (lane >> 4);                                    // + 4 k-rows per load
+      const int chunk = (lane & 15) ^ ((krow & 3) << 2);
+      lane_off = (int)(((int64_t)krow * ld + outer0 + chunk * 8) * 2);
+      blk_step = (int)(4 * ld * 2);
+      k_step = (int)(BK * ld * 2);
+    }
+  }
+  __device__ __forceinline__ void issue(int kt, char* tile) const {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int q = wave * 4 + i;
+      int off;
+      if (CONTRACT_CONTIG) {
+        const int row = q * 8 + (lane >> 3);
+        const int chunk = (lane & 7) ^ ((row ^ (row >> 3)) & 7);
+        const int k = kt * BK + chunk * 8;
+        off = k < K ? lane_off + i * blk_step + k * 2 : kOobOffset;
+      } else {
+        off = lane_off + i * blk_step + kt * k_step;
+      }
+      lds_dma_16(rsrc, off, tile + q * 1024);
+    }
+  }
+};
+
+template <bool CONTRACT_CONTIG>
+__device__ __forceinline__ uint4 read_frag_mid(const char* tile, int outer_base, int ks) {
+  const int lane = threadIdx.x & 63;
+  if (CONTRACT_CONTIG) {
+    return read_frag_kc(tile, outer_base, ks);
+  } else {
+    // see read_frag: source lane 4e + q of a 16-lane group points at k-row k0 + e, columns 4q .. 4q+3
+    const int i = lane & 15, g = lane >> 4;
+    const int col = outer_base + (g & 1) * 16 + (i & 3) * 4;
+    const int krow = ks * 16 + (g >> 1) * 8 + (i >> 2);
+    const char* p0 = tile + (krow >> 2) * 1024 + (krow & 3) * 256 + ((((col >> 3) ^ ((krow & 3) << 2)) & 15) << 4) +
+                     (col & 7) * 2;
+    const char* p1 = p0 + 1024;   // k-row + 4: the next KiB, same position
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p0);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p1);
+    const uint2 a = __builtin_bit_cast(uint2, lo), b = __builtin_bit_cast(uint2, hi);
+    return make_uint4(a.x, a.y, b.x, b.y);
+  }
+}
+
+template <typename T, bool A_MC, bool B_KC, bool SPLIT>
+__global__ __launch_bounds__(kGemmThreads, 2) void gemm_mid16_kernel(GemmArgs g) {
+  constexpr bool A_KC = !A_MC;
+  __shared__ __attribute__((aligned(1024))) char lds[kMidLds];
+  const T* __restrict__ A = reinterpret_cast<const T*>(g.a);
+  const T* __restrict__ B = reinterpret_cast<const T*>(g.b);
+
+  // workgroup -> output tile: consecutive ids go round the XCDs, so each XCD gets a contiguous
+  // run of tiles, walked in groups of 8 tile rows
+  const int nbm = (g.M + MT - 1) / MT, nbn = (g.N + MT - 1) / MT;
+  const int total = nbm * nbn;
+  int logical;
+  {
+    const int bid = blockIdx.x, xcd = bid & 7, idx = bid >> 3;
+    const int q = total >> 3, rem = total & 7;
+    logical = xcd * q + (xcd < rem ? xcd : rem) + idx;
+  }
+  constexpr int GROUP = 8;
+  const int per_group = GROUP * nbn;
+  const int first_m = (logical / per_group) * GROUP;
+  const int gsz = nbm - first_m < GROUP ? nbm - first_m : GROUP;
+  const int in_group = logical % per_group;
+  const int m0 = (first_m + in_group % gsz) * MT;
+  const int n0 = (in_group / gsz) * MT;
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  MidLoader<T, A_KC> la;
+  MidLoader<T, B_KC> lb;
+  la.init(A, g.lda, m0, g.M, g.K);
+  lb.init(B, g.ldb, n0, g.N, g.K);
+  int kt0 = 0, KT = (g.K + BK - 1) / BK;
+  if (SPLIT) {
+    kt0 = blockIdx.y * g.kt_per_split;
+    KT = kt0 + g.kt_per_split < KT ? kt0 + g.kt_per_split : KT;   // the host leaves no split empty
+  }
+  la.issue(kt0, lds);
+  lb.issue(kt0, lds + kMidTileBytes);
+  lds_dma_wait_all();
+  __syncthreads();
+
+  for (int kt = kt0; kt < KT; ++kt) {
+    const char* cur = lds + ((kt - kt0) & 1) * kMidStage;
+    char* nxt = lds + (((kt - kt0) & 1) ^ 1) * kMidStage;
+    if (kt + 1 < KT) {
+      la.issue(kt + 1, nxt);
+      lb.issue(kt + 1, nxt + kMidTileBytes);
+    }
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      uint4 af[2], bf[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        af[i] = read_frag_mid<A_KC>(cur, wm * 64 + i * 32, ks);
+        bf[i] = read_frag_mid<B_KC>(cur + kMidTileBytes, wn * 64 + i * 32, ks);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = Mfma16<T>::run(bf[j], af[i], acc[i][j]);   // C^T: 4 consecutive n per lane
+    }
+    lds_dma_wait_all();
+    __syncthreads();
+  }
+
+  // ---- epilogue: accumulators (+ bias) -> LDS as fp32 -> rows of 8 columns per lane ----
+  // A lane holds, for tile (i, j) and register group rg, C[m][n .. n+3] with
+  //   m = wm*64 + i*32 + lane%32,  n = wn*64 + j*32 + rg*8 + (lane/32)*4   (tile-local).
+  float* stage = reinterpret_cast<float*>(lds);
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {
+      const int nl = wn * 64 + j * 32 + rg * 8 + (lane >> 5) * 4;
+      float bv[4] = {0.f, 0.f, 0.f, 0.f};
+      if (g.bias) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (n0 + nl + e < g.N) bv[e] = load_scalar_f32(g.bias, g.bias_dt, n0 + nl + e);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int ml = wm * 64 + i * 32 + (lane & 31);
+        float4 v;
+        v.x = acc[i][j][rg * 4 + 0] + bv[0];
+        v.y = acc[i][j][rg * 4 + 1] + bv[1];
+        v.z = acc[i][j][rg * 4 + 2] + bv[2];
+        v.w = acc[i][j][rg * 4 + 3] + bv[3];
+        *reinterpret_cast<float4*>(stage + ml * kMidEpiPitch + nl) = v;
+      }
+    }
+  __syncthreads();
+  // 256 lanes: 16 rows per sweep, 16 lanes x 8 columns per row
+  const int rsub = threadIdx.x >> 4, cseg = (threadIdx.x & 15) * 8;
+  if (SPLIT) {
+    // partial tile as fp32; ldw is a multiple of 8, so whole segments stay inside the row
+    float* part = g.partial + (int64_t)blockIdx.y * g.M * g.ldw;
+    for (int r0 = 0; r0 < MT; r0 += 16) {
+      const int ml = r0 + rsub, m = m0 + ml;
+      if (m >= g.M || n0 + cseg >= g.N) continue;
+      float* out = part + (int64_t)m * g.ldw + n0 + cseg;
+      *reinterpret_cast<float4*>(out) = *reinterpret_cast<const float4*>(stage + ml * kMidEpiPitch + cseg);
+      *reinterpret_cast<float4*>(out + 4) = *reinterpret_cast<const float4*>(stage + ml * kMidEpiPitch + cseg + 4);
+    }
+    return;
+  }
+  T* __restrict__ C = reinterpret_cast<T*>(g.c);
+  T* __restrict__ P = g.act != AT_ACT_NONE ? reinterpret_cast<T*>(g.pre_act) : nullptr;
+  const bool rows16 = ((g.ldc & 7) == 0) && aligned16_dev(C) && (n0 + MT <= g.N) &&
+                      (!P || (((g.ldp & 7) == 0) && aligned16_dev(P)));
+  for (int r0 = 0; r0 < MT; r0 += 16) {
+    const int ml = r0 + rsub, m = m0 + ml;
+    if (m >= g.M) continue;
+    float v[8];
+    *reinterpret_cast<float4*>(v) = *reinterpret_cast<const float4*>(stage + ml * kMidEpiPitch + cseg);
+    *reinterpret_cast<float4*>(v + 4) = *reinterpret_cast<const float4*>(stage + ml * kMidEpiPitch + cseg + 4);
+    if (P) {
+      T* out = P + (int64_t)m * g.ldp + n0 + cseg;
+      if (rows16) {
+        store_f32<T, 8>(out, v);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (n0 + cseg + e < g.N) out[e] = from_f32<T>(v[e]);
+      }
+    }
+    if (g.act != AT_ACT_NONE) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = act_forward(g.act, v[e], g.param);
+    }
+    T* out = C + (int64_t)m * g.ldc + n0 + cseg;
+    if (rows16) {
+      store_f32<T, 8>(out, v);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (n0 + cseg + e < g.N) out[e] = from_f32<T>(v[e]);
+    }
+  }
+}
+
+// C[m][n] = sum over the splits of partial[s][m][n], rounded once.  One lane per 8 columns.
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_split_finish_kernel(const float* __restrict__ partial, T* __restrict__ C,
+                                                                int M, int N, int ldw, int64_t ldc, int splits) {
+  const int segs = ldw / 8;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)M * segs) return;
+  const int m = (int)(idx / segs), n = (int)(idx % segs) * 8;
+  if (n >= N) return;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  const float* src = partial + (int64_t)m * ldw + n;
+  for (int sidx = 0; sidx < splits; ++sidx) {
+    const float4 lo = *reinterpret_cast<const float4*>(src), hi = *reinterpret_cast<const float4*>(src + 4);
+    acc[0] += lo.x; acc[1] += lo.y; acc[2] += lo.z; acc[3] += lo.w;
+    acc[4] += hi.x; acc[5] += hi.y; acc[6] += hi.z; acc[7] += hi.w;
+    src += (int64_t)M * ldw;
+  }
+  T* out = C + (int64_t)m * ldc + n;
+  if (n + 8 <= N && (ldc & 7) == 0 && aligned16_dev(C)) {
+    store_f32<T, 8>(out, acc);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      if (n + e < N) out[e] = from_f32<T>(acc[e]);
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Generic kernel for fp32 operands: element strides for both, fp32 MFMA 32x32x2, 64x64x64 tiles.
 // ------------------------------------------------------------------------------------------
 struct SimpleArgs {
   const void* a; const void* b; void* c; void* pre_act; const void* bias;
@@ -373,6 +647,159 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(SimpleArgs g) {
       const float bval = sb[ks + (lane >> 5)][wn * 32 + (lane & 31)];
       const float aval = sa[ks + (lane >> 5)][wm * 32 + (lane & 31)];
       acc = __builtin_amdgcn_mfma_f32_32x32x2f32(bval, aval, acc, 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+  TO* __restrict__ C = reinterpret_cast<TO*>(g.c);
+  TO* __restrict__ P = reinterpret_cast<TO*>(g.pre_act);
+  const int m = m0 + wm * 32 + (lane & 31);
+  if (m >= g.M) return;
+#pragma unroll
+  for (int rg = 0; rg < 4; ++rg) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int n = n0 + wn * 32 + rg * 8 + (lane >> 5) * 4 + e;
+      if (n >= g.N) continue;
+      float v = acc[rg * 4 + e];
+      if (g.bias) v += load_scalar_f32(g.bias, g.bias_dt, n);
+      if (g.act != AT_ACT_NONE) {
+        if (P) P[(int64_t)m * g.ldp + n] = from_f32<TO>(v);
+        v = act_forward(g.act, v, g.param);
+      }
+      C[(int64_t)m * g.ldc + n] = from_f32<TO>(v);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Generic kernel for 16-bit operands: any strides and extents, 32x32x16 MFMA, tiles of
+// (32 WM) x (32 WN) x 64 staged through registers into LDS rows that are contiguous along the
+// contraction index.  Each operand is fetched with 16-byte loads when its unit-stride dimension
+// allows it and element by element otherwise.
+// ------------------------------------------------------------------------------------------
+constexpr int kSmallPitch = 72;   // 16-bit elements per LDS row: 64 k + 8 of padding (144 bytes)
+
+template <typename T, int R>
+struct SmallTile {   // R outer rows (m or n) x 64 k of one operand
+  static constexpr int NV = R / 32, NS = R / 4;
+  const T* p;
+  int64_t ld;        // stride of the dimension that is not contiguous
+  int o0, o_lim, K;
+  bool outer_fast;   // the outer index (m or n) is the contiguous one
+  bool vec;
+  uint4 v[NV];
+  unsigned short s[NS];
+
+  __device__ __forceinline__ void where_vec(int idx, int& o, int& k) const {
+    if (outer_fast) {
+      // a wave takes 16 k x 4 vectors of 8 outer indices: 64 contiguous bytes per k-row on the
+      // memory side, and LDS writes that spread over the banks (lanes of one k-row would all
+      // fall on two banks)
+      const int lane = idx & 63, blk = idx >> 6;
+      o = ((blk % (R / 32)) * 4 + (lane >> 4)) * 8;
+      k = (blk / (R / 32)) * 16 + (lane & 15);
+    } else {
+      o = idx >> 3;
+      k = (idx & 7) * 8;
+    }
+  }
+  __device__ __forceinline__ void where_one(int e, int& o, int& k) const {
+    if (outer_fast) { o = e % R; k = e / R; } else { o = e >> 6; k = e & 63; }
+  }
+  __device__ __forceinline__ int64_t at(int go, int gk) const {
+    return outer_fast ? (int64_t)gk * ld + go : (int64_t)go * ld + gk;
+  }
+  __device__ __forceinline__ void fetch(int k0) {
+    if (vec) {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        int o, k;
+        where_vec(threadIdx.x + i * 256, o, k);
+        const int go = o0 + o, gk = k0 + k;
+        // the extent along the vector is a multiple of 8, so a vector is inside or outside as a whole
+        v[i] = (go < o_lim && gk < K) ? *reinterpret_cast<const uint4*>(p + at(go, gk)) : make_uint4(0, 0, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NS; ++i) {
+        int o, k;
+        where_one(threadIdx.x + i * 256, o, k);
+        const int go = o0 + o, gk = k0 + k;
+        s[i] = (go < o_lim && gk < K) ? __builtin_bit_cast(unsigned short, p[at(go, gk)]) : (unsigned short)0;
+      }
+    }
+  }
+  __device__ __forceinline__ void stage(unsigned short* lds) const {
+    if (vec) {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        int o, k;
+        where_vec(threadIdx.x + i * 256, o, k);
+        if (!outer_fast) {
+          *reinterpret_cast<uint4*>(lds + o * kSmallPitch + k) = v[i];
+        } else {
+          const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            lds[(o + j) * kSmallPitch + k] = (unsigned short)((j & 1) ? w[j >> 1] >> 16 : w[j >> 1] & 0xffffu);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NS; ++i) {
+        int o, k;
+        where_one(threadIdx.x + i * 256, o, k);
+        lds[o * kSmallPitch + k] = s[i];
+      }
+    }
+  }
+};
+
+template <typename T, typename TO, int WM, int WN>
+__global__ __launch_bounds__(256) void gemm_small16_kernel(SimpleArgs g) {
+  static_assert(WM * WN == 4, "four waves");
+  constexpr int TM = WM * 32, TN = WN * 32, TK = 64;
+  __shared__ __align__(16) unsigned short sa[TM * kSmallPitch];
+  __shared__ __align__(16) unsigned short sb[TN * kSmallPitch];
+  const T* A = reinterpret_cast<const T*>(g.a);
+  const T* B = reinterpret_cast<const T*>(g.b);
+  const int nbn = (g.N + TN - 1) / TN;
+  const int m0 = (blockIdx.x / nbn) * TM, n0 = (blockIdx.x % nbn) * TN;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+
+  SmallTile<T, TM> ta;
+  ta.p = A; ta.o0 = m0; ta.o_lim = g.M; ta.K = g.K;
+  ta.outer_fast = g.sak != 1;
+  ta.ld = ta.outer_fast ? g.sak : g.sam;
+  ta.vec = (ta.ld & 7) == 0 && aligned16_dev(A) && (((ta.outer_fast ? g.M : g.K) & 7) == 0);
+  SmallTile<T, TN> tb;
+  tb.p = B; tb.o0 = n0; tb.o_lim = g.N; tb.K = g.K;
+  tb.outer_fast = g.sbk != 1;
+  tb.ld = tb.outer_fast ? g.sbk : g.sbn;
+  tb.vec = (tb.ld & 7) == 0 && aligned16_dev(B) && (((tb.outer_fast ? g.N : g.K) & 7) == 0);
+
+  f32x16 acc;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+  ta.fetch(0);
+  tb.fetch(0);
+  for (int k0 = 0; k0 < g.K; k0 += TK) {
+    ta.stage(sa);
+    tb.stage(sb);
+    __syncthreads();
+    if (k0 + TK < g.K) {   // the next k-tile travels while this one is multiplied
+      ta.fetch(k0 + TK);
+      tb.fetch(k0 + TK);
+    }
+#pragma unroll
+    for (int ks = 0; ks < TK / 16; ++ks) {
+      const int k = ks * 16 + (lane >> 5) * 8;
+      const uint4 xa = *reinterpret_cast<const uint4*>(sa + (wm * 32 + (lane & 31)) * kSmallPitch + k);
+      const uint4 xb = *reinterpret_cast<const uint4*>(sb + (wn * 32 + (lane & 31)) * kSmallPitch + k);
+      // B first: a lane ends up with 4 consecutive n of one m
+      acc = Mfma16<T>::run(xb, xa, acc);
     }
     __syncthreads();
   }
@@ -519,13 +946,42 @@ inline int dispatch_dtype(int dt, F&& f) {
 
 enum Layout { kFwd = 0, kDx = 1, kDw = 2 };
 
+// Tile choice for a problem the 16-bit kernels can address.  One workgroup of the 256x256
+// kernel occupies a CU, so its time goes in whole rounds of one tile per CU; the 128x128 kernel
+// runs two workgroups per CU at about 60 % of the other's rate (measured: one round of 512
+// tiles takes 0.6 of a round of 256 large ones).
+inline bool prefer_mid_tiles(int64_t M, int64_t N) {
+  const int64_t cus = device_cu_count();
+  const double big = (double)cdiv64(cdiv64(M, BM) * cdiv64(N, BN), cus);
+  double mid = (double)(cdiv64(M, MT) * cdiv64(N, MT)) / (double)(2 * cus);
+  if (mid < 0.6) mid = 0.6;
+  return mid * 0.6 < big;
+}
+
+// Number of splits of the contraction for the weight gradient (a [in, out] tile grid that is
+// small next to the chip, a long contraction over the batch): enough to give every CU two
+// workgroups, each split at least 4 k-tiles long.  1 = no split.
+inline int dw_split_count(int64_t M, int64_t N, int64_t K) {
+  const int64_t tiles = cdiv64(M, MT) * cdiv64(N, MT);
+  const int64_t want = (int64_t)device_cu_count() * 2 / tiles;
+  const int64_t kt = cdiv64(K, BK);
+  int64_t splits = want < kt / 4 ? want : kt / 4;
+  if (splits > 32) splits = 32;
+  if (splits < 2) return 1;
+  const int64_t per = cdiv64(kt, splits);
+  return (int)cdiv64(kt, per);   // no empty split
+}
+
+inline int64_t dw_partial_pitch(int64_t N) { return (N + 7) / 8 * 8; }
+
 // C[M,N] = A(m,k) B(k,n) for the three products of the linear layer.
 //   kFwd: A = [M,K] rows,  B = [K,N] rows          (X, W)
 //   kDx : A = [M,K] rows,  B = [N,K] rows          (dZ, W: contraction over W's columns)
 //   kDw : A = [K,M] rows,  B = [K,N] rows          (X, dZ: contraction over rows of both)
 int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act, const void* bias, int64_t M,
              int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int64_t ldp, int act, float param,
-             int in_dt, int bias_dt, int out_dt, hipStream_t stream) {
+             int in_dt, int bias_dt, int out_dt, hipStream_t stream, void* workspace = nullptr,
+             int64_t workspace_bytes = 0) {
   if (!a || !b || !c) return AT_ERR_NULL;
   if (!dtype_valid(in_dt) || !dtype_valid(out_dt) || (bias && !dtype_valid(bias_dt))) return AT_ERR_DTYPE;
   if (!act_valid(act)) return AT_ERR_ACT;
@@ -535,19 +991,56 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
   if (M == 0) return AT_OK;
 
   const bool a_contig_k = layout != kDw, b_contig_k = layout == kDx;
+  // 16-byte loads need aligned rows; an operand whose rows run along the contraction index also
+  // needs K in whole vectors (the other layout reads whole rows of k, and what a vector picks up
+  // past M or N only reaches outputs that are not stored).
   bool fast = in_dt != AT_DTYPE_F32 && out_dt == in_dt && aligned16(a) && aligned16(b) && (lda % 8) == 0 &&
-              (ldb % 8) == 0 && (K % 8) == 0;
-  if (!a_contig_k) fast = fast && (M % 8) == 0;
-  if (!b_contig_k) fast = fast && (N % 8) == 0;
+              (ldb % 8) == 0;
+  if (a_contig_k || b_contig_k) fast = fast && (K % 8) == 0;
   // buffer descriptors address each operand with 32-bit byte offsets below 2 GiB
   const int64_t a_bytes = (a_contig_k ? M : K) * lda * 2, b_bytes = (b_contig_k ? N : K) * ldb * 2;
   if (a_bytes >= ((int64_t)1 << 31) || b_bytes >= ((int64_t)1 << 31)) fast = false;
-  // Small problems do not fill 256x256 tiles; the generic kernel has finer tiles.
-  if (M * N < (int64_t)BM * BN / 2 || M < 64 || N < 64) fast = false;
+  // Small problems do not fill the tiles of these kernels; the generic kernel has finer ones.
+  if (M * N < (int64_t)MT * MT || M < 64 || N < 64) fast = false;
+
+  const int64_t big_tiles = cdiv64(M, BM) * cdiv64(N, BN);
+  if (fast && prefer_mid_tiles(M, N)) {
+    GemmArgs g{a, b, c, pre_act, bias, (int)M, (int)N, (int)K, lda, ldb, ldc, ldp, act, param, bias_dt, nullptr, 0, 0};
+    const unsigned grid = (unsigned)(cdiv64(M, MT) * cdiv64(N, MT));
+    int splits = 1;
+    if (layout == kDw && workspace) {
+      splits = dw_split_count(M, N, K);
+      if (workspace_bytes < (int64_t)splits * M * dw_partial_pitch(N) * 4) splits = 1;
+    }
+    return dispatch_dtype(in_dt, [&](auto* tp) -> int {
+      typedef std::remove_pointer_t<decltype(tp)> T;
+      if constexpr (std::is_same<T, float>::value) {
+        return AT_ERR_DTYPE;
+      } else {
+        if (splits > 1) {
+          g.partial = (float*)workspace;
+          g.kt_per_split = (int)cdiv64(cdiv64(K, BK), splits);
+          g.ldw = (int)dw_partial_pitch(N);
+          hipLaunchKernelGGL((gemm_mid16_kernel<T, true, false, true>), dim3(grid, splits), dim3(kGemmThreads), 0,
+                             stream, g);
+          const int64_t items = M * (g.ldw / 8);
+          hipLaunchKernelGGL((gemm_split_finish_kernel<T>), dim3((unsigned)cdiv64(items, 256)), dim3(256), 0, stream,
+                             (const float*)workspace, (T*)c, (int)M, (int)N, g.ldw, ldc, splits);
+        } else if (layout == kDx) {
+          hipLaunchKernelGGL((gemm_mid16_kernel<T, false, true, false>), dim3(grid), dim3(kGemmThreads), 0, stream, g);
+        } else if (layout == kDw) {
+          hipLaunchKernelGGL((gemm_mid16_kernel<T, true, false, false>), dim3(grid), dim3(kGemmThreads), 0, stream, g);
+        } else {
+          hipLaunchKernelGGL((gemm_mid16_kernel<T, false, false, false>), dim3(grid), dim3(kGemmThreads), 0, stream, g);
+        }
+        return launch_status();
+      }
+    });
+  }
 
   if (fast) {
-    GemmArgs g{a, b, c, pre_act, bias, (int)M, (int)N, (int)K, lda, ldb, ldc, ldp, act, param, bias_dt};
-    const unsigned grid = (unsigned)(cdiv64(M, BM) * cdiv64(N, BN));
+    GemmArgs g{a, b, c, pre_act, bias, (int)M, (int)N, (int)K, lda, ldb, ldc, ldp, act, param, bias_dt, nullptr, 0, 0};
+    const unsigned grid = (unsigned)big_tiles;
     return dispatch_dtype(in_dt, [&](auto* tp) -> int {
       typedef std::remove_pointer_t<decltype(tp)> T;
       if constexpr (std::is_same<T, float>::value) {
@@ -583,12 +1076,20 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
   SimpleArgs s{a, b, c, pre_act, bias, (int)M, (int)N, (int)K,
                a_contig_k ? lda : 1, a_contig_k ? 1 : lda, b_contig_k ? 1 : ldb, b_contig_k ? ldb : 1,
                ldc, ldp, act, param, bias_dt};
-  const unsigned grid = (unsigned)(cdiv64(M, 64) * cdiv64(N, 64));
   return dispatch_dtype(in_dt, [&](auto* ti) -> int {
     typedef std::remove_pointer_t<decltype(ti)> TI;
     return dispatch_dtype(out_dt, [&](auto* to) -> int {
       typedef std::remove_pointer_t<decltype(to)> TO;
-      hipLaunchKernelGGL((gemm_simple_kernel<TI, TO>), dim3(grid), dim3(256), 0, stream, s);
+      if constexpr (std::is_same<TI, float>::value) {
+        const unsigned grid = (unsigned)(cdiv64(M, 64) * cdiv64(N, 64));
+        hipLaunchKernelGGL((gemm_simple_kernel<TI, TO>), dim3(grid), dim3(256), 0, stream, s);
+      } else if (N <= 32) {   // skinny outputs: all four waves along m
+        const unsigned grid = (unsigned)(cdiv64(M, 128) * cdiv64(N, 32));
+        hipLaunchKernelGGL((gemm_small16_kernel<TI, TO, 4, 1>), dim3(grid), dim3(256), 0, stream, s);
+      } else {
+        const unsigned grid = (unsigned)(cdiv64(M, 64) * cdiv64(N, 64));
+        hipLaunchKernelGGL((gemm_small16_kernel<TI, TO, 2, 2>), dim3(grid), dim3(256), 0, stream, s);
+      }
       return launch_status();
     });
   });
@@ -622,13 +1123,22 @@ int at_linear_bwd_input(const void* pre_act_grad, const void* weight, void* inpu
                   (hipStream_t)stream);
 }
 
-int at_linear_bwd_weight(const void* input, const void* pre_act_grad, void* weight_grad, int64_t batch,
-                         int64_t in_feat, int64_t out_feat, int64_t input_stride, int64_t grad_stride,
-                         int64_t weight_grad_stride, int in_dtype, int out_dtype, at_stream_t stream) {
+int64_t at_linear_bwd_weight_workspace_bytes(int64_t batch, int64_t in_feat, int64_t out_feat, int dtype) {
+  if (batch <= 0 || in_feat <= 0 || out_feat <= 0 || (dtype != AT_DTYPE_F16 && dtype != AT_DTYPE_BF16)) return 0;
+  if (in_feat < 64 || out_feat < 64 || in_feat * out_feat < (int64_t)MT * MT) return 0;
+  if (!prefer_mid_tiles(in_feat, out_feat)) return 0;
+  const int splits = dw_split_count(in_feat, out_feat, batch);
+  return splits > 1 ? (int64_t)splits * in_feat * dw_partial_pitch(out_feat) * 4 : 0;
+}
+
+int at_linear_bwd_weight(const void* input, const void* pre_act_grad, void* weight_grad, void* workspace,
+                         int64_t workspace_bytes, int64_t batch, int64_t in_feat, int64_t out_feat,
+                         int64_t input_stride, int64_t grad_stride, int64_t weight_grad_stride, int in_dtype,
+                         int out_dtype, at_stream_t stream) {
   if (batch <= 0) return AT_ERR_DIM;
   return run_gemm(kDw, input, pre_act_grad, weight_grad, nullptr, nullptr, in_feat, out_feat, batch,
                   input_stride, grad_stride, weight_grad_stride, 0, AT_ACT_NONE, 0.f, in_dtype, 0, out_dtype,
-                  (hipStream_t)stream);
+                  (hipStream_t)stream, workspace, workspace_bytes);
 }
 
 int64_t at_act_bwd_workspace_bytes(int64_t rows, int64_t cols) {

@@ -14,6 +14,7 @@ from typing import Any, Optional, Tuple
 import torch
 from torch import Tensor
 from torch import nn
+from torch.nn import functional as F
 
 from . import _lib
 from .act import act_id, parse_act_func
@@ -27,6 +28,36 @@ def _matrix(tensor: Tensor) -> Tensor:
     if tensor.stride(-1) != 1 or (tensor.shape[0] > 1 and tensor.stride(0) < tensor.shape[1]):
         tensor = tensor.contiguous()
     return tensor
+
+
+def _round_up8(size: int) -> int:
+    return (size + 7) // 8 * 8
+
+
+def _pad_features(batch_dim: int, in_feat_dim: int, out_feat_dim: int, dtype: torch.dtype) -> bool:
+    """
+    Whether the 16-bit operands get zero-padded copies with feature strides in multiples of 8.
+
+    The tiled matrix-core kernels read 16 bytes at a time and need 16-byte aligned rows; other
+    shapes run on the generic kernel, which is several times slower on large problems (a
+    vocabulary of 50257 columns, say).  Copying the operands costs one pass over each, far
+    less than the difference, once the problem is large enough for those kernels at all.
+    """
+    if dtype not in (torch.float16, torch.bfloat16):
+        return False
+    if in_feat_dim % 8 == 0 and out_feat_dim % 8 == 0:
+        return False
+    return (min(batch_dim, in_feat_dim, out_feat_dim) >= 64 and
+            batch_dim * min(in_feat_dim, out_feat_dim) >= 32768)
+
+
+def _zero_pad(matrix: Tensor, rows: int, cols: int) -> Tensor:
+    """
+    Copy of a 2D tensor extended with zeros to [rows, cols] (the tensor itself if it fits already).
+    """
+    if matrix.shape == (rows, cols):
+        return matrix
+    return F.pad(matrix, (0, cols - matrix.shape[1], 0, rows - matrix.shape[0]))
 
 
 class LinearAutoGrad(torch.autograd.Function):
@@ -91,6 +122,12 @@ class LinearAutoGrad(torch.autograd.Function):
         bias_k = None if bias is None else bias.contiguous()
         if bias_k is not None and output_dtype != input.dtype:
             bias_k = bias_k.to(output_dtype)
+        contract_dim = in_feat_dim
+        if _pad_features(batch_dim, in_feat_dim, out_feat_dim, compute_dtype):
+            # zeros along the contraction add nothing; padded output columns are never stored
+            contract_dim = _round_up8(in_feat_dim)
+            input_k = _zero_pad(input_k, batch_dim, contract_dim)
+            weight_k = _zero_pad(weight_k, contract_dim, _round_up8(out_feat_dim))
 
         output = torch.empty((batch_dim, out_feat_dim), device=input.device, dtype=output_dtype)
         pre_act = torch.empty_like(output) if save_pre_act else output
@@ -98,7 +135,7 @@ class LinearAutoGrad(torch.autograd.Function):
         with torch.cuda.device_of(input):
             _lib.check(lib.at_linear_fwd(
                 _lib.ptr(input_k), _lib.ptr(weight_k), _lib.ptr(bias_k), _lib.ptr(pre_act),
-                _lib.ptr(output), batch_dim, in_feat_dim, out_feat_dim, input_k.stride(0),
+                _lib.ptr(output), batch_dim, contract_dim, out_feat_dim, input_k.stride(0),
                 weight_k.stride(0), pre_act.stride(0), output.stride(0), act,
                 0.0 if param is None else param, _lib.dtype_id(compute_dtype),
                 _lib.dtype_id(bias_k.dtype) if bias_k is not None else 0,
@@ -158,25 +195,39 @@ class LinearAutoGrad(torch.autograd.Function):
             # The products run in the output dtype, as under the reference's
             # torch.autocast(dtype=output_dtype) block (linear_layer.py:152-155).
             grad_mm = _matrix(pre_act_grad.to(output_dtype))
+            pad = _pad_features(batch_dim, in_feat_dim, out_feat_dim, output_dtype)
+            contract_dim = out_feat_dim
+            if pad:
+                contract_dim = _round_up8(out_feat_dim)
+                grad_mm = _zero_pad(grad_mm, batch_dim, contract_dim)
             input_grad = weight_grad = None
             if input.requires_grad:
                 weight_mm = _matrix(weight.to(output_dtype))
+                if pad:
+                    weight_mm = _zero_pad(weight_mm, in_feat_dim, contract_dim)
                 input_grad = torch.empty((batch_dim, in_feat_dim), dtype=output_dtype, device=device)
                 _lib.check(lib.at_linear_bwd_input(
                     _lib.ptr(grad_mm), _lib.ptr(weight_mm), _lib.ptr(input_grad), batch_dim,
-                    in_feat_dim, out_feat_dim, grad_mm.stride(0), weight_mm.stride(0),
+                    in_feat_dim, contract_dim, grad_mm.stride(0), weight_mm.stride(0),
                     input_grad.stride(0), _lib.dtype_id(output_dtype),
                     _lib.dtype_id(output_dtype), stream), 'at_linear_bwd_input')
                 input_grad = input_grad.view_as(input)
             if weight.requires_grad:
                 input_mm = _matrix(flattened_input.to(output_dtype))
+                if pad:
+                    input_mm = _zero_pad(input_mm, batch_dim, _round_up8(in_feat_dim))
                 weight_grad = torch.empty((in_feat_dim, out_feat_dim), dtype=output_dtype,
                                           device=device)
                 if batch_dim == 0:
                     weight_grad.zero_()
                 else:
+                    workspace_bytes = lib.at_linear_bwd_weight_workspace_bytes(
+                        batch_dim, in_feat_dim, out_feat_dim, _lib.dtype_id(output_dtype))
+                    workspace = (torch.empty(workspace_bytes, dtype=torch.uint8, device=device)
+                                 if workspace_bytes else None)
                     _lib.check(lib.at_linear_bwd_weight(
-                        _lib.ptr(input_mm), _lib.ptr(grad_mm), _lib.ptr(weight_grad), batch_dim,
+                        _lib.ptr(input_mm), _lib.ptr(grad_mm), _lib.ptr(weight_grad),
+                        _lib.ptr(workspace), workspace_bytes, batch_dim,
                         in_feat_dim, out_feat_dim, input_mm.stride(0), grad_mm.stride(0),
                         weight_grad.stride(0), _lib.dtype_id(output_dtype),
                         _lib.dtype_id(output_dtype), stream), 'at_linear_bwd_weight')

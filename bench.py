@@ -196,9 +196,12 @@ def bench_linear(cfg: str, steps: int, warmup: int, with_cpu: bool) -> Dict:
         raw.check(lib.at_linear_bwd_input(dz.data_ptr(), wd.data_ptr(), dx.data_ptr(), m, k, n, n, n, k, dt, dt,
                                           st()), 'dx')
 
+    dwsb = lib.at_linear_bwd_weight_workspace_bytes(m, k, n, dt)
+    dws = torch.empty(max(dwsb, 1), dtype=torch.uint8, device='cuda')
+
     def k_dw():
-        raw.check(lib.at_linear_bwd_weight(xd.data_ptr(), dz.data_ptr(), dw.data_ptr(), m, k, n, k, n, n, dt, dt,
-                                           st()), 'dw')
+        raw.check(lib.at_linear_bwd_weight(xd.data_ptr(), dz.data_ptr(), dw.data_ptr(), dws.data_ptr(), dwsb,
+                                           m, k, n, k, n, n, dt, dt, st()), 'dw')
 
     def k_db():
         raw.check(lib.at_colsum(dz.data_ptr(), db.data_ptr(), ws.data_ptr(), wsb, m, n, n, dt, dt, st()), 'colsum')

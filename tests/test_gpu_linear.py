@@ -89,3 +89,61 @@ def test_no_grad_path_saves_nothing() -> None:
     y = attorch_amd.LinearAutoGrad.apply(x, w, None, 'relu')
     assert y.grad_fn is None
     torch.testing.assert_close(y, torch.relu(x @ w), rtol=1e-4, atol=1e-4)
+
+
+HALF_DTYPES = [torch.float16, torch.bfloat16]
+
+
+@pytest.mark.parametrize('dtype', HALF_DTYPES)
+@pytest.mark.parametrize('act_func', [None, 'geluapprox'])
+@pytest.mark.parametrize('shape, out_dim', [
+    ((1024, 333), 77),      # both feature sizes odd: the host pads input, weight and gradient
+    ((512, 200), 1001),     # odd output size only (a vocabulary-like head)
+    ((640, 257), 264),      # odd input size only
+    ((4096, 512), 10),      # skinny output: generic 16-bit kernel, all waves along the batch
+    ((96, 1000), 24),       # skinny output, contraction not a multiple of 64
+    ((2048, 512), 384),     # 128x128 tiles
+    ((4096, 256), 256),     # 128x128 tiles, weight gradient split over the batch
+    ((16384, 192), 320),    # split with a ragged last k-tile range
+])
+def test_linear_16bit_kernel_selection(shape, out_dim, act_func, dtype) -> None:
+    run_case(shape, out_dim, True, act_func, dtype)
+
+
+@pytest.mark.parametrize('dtype', HALF_DTYPES)
+@pytest.mark.parametrize('batch, in_dim, out_dim', [(4096, 256, 256), (8000, 320, 136), (1000, 264, 200)])
+def test_weight_grad_split_agrees_with_one_piece(batch, in_dim, out_dim, dtype) -> None:
+    """
+    C ABI: at_linear_bwd_weight with its workspace (batch split into slices, fp32 partial sums)
+    against the same call without one, and against float64.
+    """
+    from attorch_amd import _lib
+    lib = _lib.load()
+    x = randn((batch, in_dim), 1, dtype).cuda()
+    dz = randn((batch, out_dim), 2, dtype).cuda()
+    did = _lib.dtype_id(dtype)
+    stream = _lib.stream_of(x)
+    workspace_bytes = lib.at_linear_bwd_weight_workspace_bytes(batch, in_dim, out_dim, did)
+    if batch >= 4096:
+        assert workspace_bytes > 0
+    results = []
+    for use_workspace in (False, True):
+        dw = torch.full((in_dim, out_dim), float('nan'), dtype=dtype, device='cuda')
+        workspace = torch.empty(max(workspace_bytes, 16), dtype=torch.uint8, device='cuda') if use_workspace else None
+        _lib.check(lib.at_linear_bwd_weight(
+            _lib.ptr(x), _lib.ptr(dz), _lib.ptr(dw), _lib.ptr(workspace), workspace_bytes if use_workspace else 0,
+            batch, in_dim, out_dim, in_dim, out_dim, out_dim, did, did, stream), 'at_linear_bwd_weight')
+        results.append(dw.double().cpu())
+    expected = x.double().cpu().T @ dz.double().cpu()
+    scale = expected.abs().max().item()
+    for got in results:
+        torch.testing.assert_close(got / scale, expected / scale, rtol=2e-2, atol=2e-2 / 8)
+    # both round the same fp32-accurate sums: they differ by an ulp of the 16-bit format at most
+    torch.testing.assert_close(results[0] / scale, results[1] / scale, rtol=2 ** -7, atol=2 ** -9)
+    # a short workspace is not an error: the one-piece path runs
+    dw = torch.empty((in_dim, out_dim), dtype=dtype, device='cuda')
+    tiny = torch.empty(16, dtype=torch.uint8, device='cuda')
+    _lib.check(lib.at_linear_bwd_weight(
+        _lib.ptr(x), _lib.ptr(dz), _lib.ptr(dw), _lib.ptr(tiny), 16, batch, in_dim, out_dim, in_dim, out_dim,
+        out_dim, did, did, stream), 'at_linear_bwd_weight')
+    torch.testing.assert_close(dw.double().cpu(), results[0], rtol=0, atol=0)

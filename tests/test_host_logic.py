@@ -85,6 +85,13 @@ def test_argument_errors_without_gpu() -> None:
     strided = list(good); strided[5] = strided[6] = 4; strided[9] = strided[10] = 2
     assert lib.at_conv2d_bwd_input_workspace_bytes(*strided, 1) == 0
     assert lib.at_conv2d_bwd_weight_workspace_bytes(*good, 0) > 0
+    # weight gradient of the linear layer: slices of the batch only for 16-bit tensors, a long
+    # batch and a weight matrix that is small next to the GPU
+    assert lib.at_linear_bwd_weight_workspace_bytes(16384, 256, 256, 2) >= 2 * 256 * 256 * 4
+    assert lib.at_linear_bwd_weight_workspace_bytes(16384, 256, 256, 0) == 0
+    assert lib.at_linear_bwd_weight_workspace_bytes(64, 256, 256, 2) == 0
+    assert lib.at_linear_bwd_weight_workspace_bytes(16384, 8192, 8192, 2) == 0
+    assert lib.at_linear_bwd_weight(None, p, p, None, 0, 4, 8, 8, 8, 8, 8, 0, 0, None) == -1
     assert lib.at_norm_bwd_workspace_bytes(16, 8, 2) == 16 * 8 * 4 * 2
     assert lib.at_cross_entropy_workspace_bytes(10) == 56
 
