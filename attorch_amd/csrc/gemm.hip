@@ -2,8 +2,8 @@
 //
 // Four kernels:
 //  * gemm_mfma16_kernel — bf16/fp16 operands on v_mfma_f32_32x32x16 (MFMA-bound).  256x256x64
-//    macro-tile per 256-lane workgroup (4 waves, 128x128 each, 256 accumulator registers per
-//    lane), LDS double-buffered, one barrier per k-tile.  Tiles go from global memory straight
+//    macro-tile per 512-lane workgroup (8 waves, 128x64 each, 128 accumulator registers per
+//    lane, two waves per SIMD), LDS double-buffered, one barrier per k-tile.  Tiles go from global memory straight
 //    into LDS (buffer_load ... lds), the loads of tile k+1 in flight while tile k is
 //    multiplied.  An operand whose contraction index is contiguous in memory is kept as
 //    [row][k] with the 16-byte chunk index XOR-swizzled by the row (bank-conflict-free 128-bit
@@ -52,6 +52,14 @@ struct GemmArgs {
 
 constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int kGemmThreads = 256;
+// Waves of the 256x256 kernel: 2 along m (128 rows each) x 4 along n (64 columns each), two per
+// SIMD.  (Four waves of 128x128 read less from LDS per MFMA but leave each SIMD with a single
+// wave and nothing to cover its stalls: measured 10 % slower.)
+constexpr int kBigWaves = 8;
+constexpr int kBigThreads = kBigWaves * 64;
+constexpr int kBigLoads = 32 / kBigWaves;          // wave-wide loads per operand tile and wave
+constexpr int kBigWaveN = BN / (kBigWaves / 2);    // columns per wave
+constexpr int kBigNJ = kBigWaveN / 32;             // 32-column MFMA tiles per wave
 constexpr int kTileBytes = BM * BK * 2;  // one operand tile, 32 KiB
 constexpr int kEpiPitch = BN * 2 + 16;   // bytes per row of the epilogue tile in LDS (padded against bank conflicts)
 constexpr int kEpiBytes = BM * kEpiPitch;
@@ -81,9 +89,9 @@ struct OperandLoader {
     K = K_;
     if (CONTRACT_CONTIG) {
       rsrc = make_buffer_rsrc(base, ((int64_t)(outer_total - 1) * ld + K_) * 2);   // the last row ends at its last element
-      // load i of wave w fills rows 8q .. 8q+7 (q = 8w + i); lane -> (row, position), and the
+      // load i of wave w fills rows 8q .. 8q+7 (q = kBigLoads w + i); lane -> (row, position), and the
       // position holds chunk (position ^ swizzle(row)) so that the reads find chunk c at c ^ swizzle
-      const int row = wave * 64 + (lane >> 3);            // + 8 i
+      const int row = wave * (kBigLoads * 8) + (lane >> 3);   // + 8 i
       k_lane = 0;
       lane_off = (int)(((int64_t)(outer0 + row) * ld) * 2);
       blk_step = (int)(8 * ld * 2);
@@ -92,8 +100,8 @@ struct OperandLoader {
       // up to the end of the 16-byte unit that holds the last element (rows start on such units,
       // and the range check drops a dword that is only partly inside)
       rsrc = make_buffer_rsrc(base, ((int64_t)(K_ - 1) * ld + ((outer_total + 7) & ~7)) * 2);
-      // load i of wave w fills k-rows 2q, 2q+1 (q = 8w + i); lane -> k-row 2q + lane/32, 8 columns at (lane%32)*8
-      const int krow = wave * 16 + (lane >> 5);            // + 2 i
+      // load i of wave w fills k-rows 2q, 2q+1 (q = kBigLoads w + i); lane -> k-row 2q + lane/32, 8 columns at (lane%32)*8
+      const int krow = wave * (kBigLoads * 2) + (lane >> 5);  // + 2 i
       k_lane = 0;
       lane_off = (int)(((int64_t)krow * ld + outer0 + (lane & 31) * 8) * 2);
       blk_step = (int)(2 * ld * 2);
@@ -101,17 +109,17 @@ struct OperandLoader {
     }
   }
 
-  // Issues the 8 loads of this lane for k-tile `kt` into `tile` (LDS).
+  // Issues the loads of this lane for k-tile `kt` into `tile` (LDS).
   __device__ __forceinline__ void issue(int kt, char* tile) const {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) issue_one(kt, tile, i);
+    for (int i = 0; i < kBigLoads; ++i) issue_one(kt, tile, i);
   }
 
-  // Load i (0..7) of this lane for k-tile `kt`.
+  // Load i (0 .. kBigLoads-1) of this lane for k-tile `kt`.
   __device__ __forceinline__ void issue_one(int kt, char* tile, int i) const {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     {
-      const int q = wave * 8 + i;
+      const int q = wave * kBigLoads + i;
       int off;
       char* dst;
       if (CONTRACT_CONTIG) {
@@ -154,9 +162,9 @@ __device__ __forceinline__ uint4 read_frag(const char* tile, int outer_base, int
 }
 
 // ACT is the compile-time activation id of the epilogue (the act switch must fold away: the
-// epilogue is fully unrolled over 256 accumulator registers).
+// epilogue is fully unrolled over the accumulator registers).
 template <typename T, bool A_MC, bool B_KC, int ACT>
-__global__ __launch_bounds__(kGemmThreads) void gemm_mfma16_kernel(GemmArgs g) {
+__global__ __launch_bounds__(kBigThreads) void gemm_mfma16_kernel(GemmArgs g) {
   constexpr bool A_KC = !A_MC;
   constexpr int kATile = operand_tile_bytes<A_KC>(), kBTile = operand_tile_bytes<B_KC>();
   constexpr int kStage = kATile + kBTile;
@@ -183,14 +191,15 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_mfma16_kernel(GemmArgs g) {
   const int n0 = (in_group / gsz) * BN;
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  constexpr int NJ = kBigNJ;
+  const int wm = wave / (kBigWaves / 2), wn = wave % (kBigWaves / 2);
   const int frag_row = lane & 31, frag_half = lane >> 5;
 
-  f32x16 acc[4][4];
+  f32x16 acc[4][NJ];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
@@ -205,24 +214,22 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_mfma16_kernel(GemmArgs g) {
   lds_dma_wait_all();
   __syncthreads();
 
-  auto load_frags = [&](const char* stage, int ks, uint4 (&af)[4], uint4 (&bf)[4]) {
+  auto load_frags = [&](const char* stage, int ks, uint4 (&af)[4], uint4 (&bf)[NJ]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      af[i] = read_frag<A_KC>(stage, wm * 128 + i * 32, ks);
-      bf[i] = read_frag<B_KC>(stage + kATile, wn * 128 + i * 32, ks);
-    }
+    for (int i = 0; i < 4; ++i) af[i] = read_frag<A_KC>(stage, wm * 128 + i * 32, ks);
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) bf[j] = read_frag<B_KC>(stage + kATile, wn * kBigWaveN + j * 32, ks);
   };
 
-  // One k-tile = four k-steps of 16 MFMAs (512 matrix-pipe cycles each).  With a single wave
-  // per SIMD nothing else hides latency, so the other instructions of the iteration are
-  // slotted between MFMAs: the 16 global->LDS loads of the next tile during k-step 0, the
+  // One k-tile = four k-steps of 4 * NJ MFMAs per wave.  The other instructions of the iteration
+  // are slotted between MFMAs: the global->LDS loads of the next tile during k-step 0, the
   // fragment reads of k-step s+1 during k-step s.  The loads of tile kt+1 stay in flight for
   // the whole iteration and are only waited for at the barrier that ends it.
   // (sched_group_barrier masks: 0x8 MFMA, 0x2 VALU, 0x20 VMEM read, 0x100 LDS read.)
   for (int kt = 0; kt < KT; ++kt) {
     char* cur = lds + (kt & 1) * kStage;
     char* nxt = lds + ((kt & 1) ^ 1) * kStage;
-    uint4 af[2][4], bf[2][4];
+    uint4 af[2][4], bf[2][NJ];
     load_frags(cur, 0, af[0], bf[0]);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -231,20 +238,21 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_mfma16_kernel(GemmArgs g) {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          // One global->LDS load of the next tile behind each MFMA of k-step 0.  Unconditional:
-          // past the last k-tile every offset is out of range and the loads write zeros into
-          // a stage nobody reads, so the loop body has no branches.
+        for (int j = 0; j < NJ; ++j) {
+          // One global->LDS load of the next tile behind each MFMA of k-step 0 (2 * kBigLoads =
+          // 4 * NJ of either).  Unconditional: past the last k-tile every offset is out of range
+          // and the loads write zeros into a stage nobody reads, so the loop body has no branches.
           if (ks == 0) {
-            if (i < 2) la.issue_one(kt + 1, nxt, i * 4 + j);
-            else lb.issue_one(kt + 1, nxt + kATile, (i - 2) * 4 + j);
+            const int t = i * NJ + j;
+            if (t < kBigLoads) la.issue_one(kt + 1, nxt, t);
+            else lb.issue_one(kt + 1, nxt + kATile, t - kBigLoads);
           }
           // operands swapped: the accumulator holds C^T, i.e. 4 consecutive n per lane
           acc[i][j] = Mfma16<T>::run(bf[ks & 1][j], af[ks & 1][i], acc[i][j]);
         }
       if (ks < BK / 16 - 1) {
 #pragma unroll
-        for (int q = 0; q < 16; ++q) {
+        for (int q = 0; q < 4 * NJ; ++q) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
@@ -257,7 +265,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_mfma16_kernel(GemmArgs g) {
 
   // ---- epilogue ----
   // A lane holds, for tile (i, j) and register group rg, C[m][n .. n+3] with
-  //   m = wm*128 + i*32 + lane%32,  n = wn*128 + j*32 + rg*8 + (lane/32)*4   (tile-local).
+  //   m = wm*128 + i*32 + lane%32,  n = wn*kBigWaveN + j*32 + rg*8 + (lane/32)*4   (tile-local).
   // Storing that straight to memory touches 32 rows per instruction with 16 bytes each; instead
   // the finished tile goes through LDS (free after the main loop) and leaves as whole rows:
   // 32 lanes x 16 bytes = one 512-byte row segment per half-wave.
@@ -274,10 +282,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_mfma16_kernel(GemmArgs g) {
     if (is_pre && !P) continue;   // uniform
     __syncthreads();              // previous readers of LDS (main loop or previous pass) are done
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
-        const int nl = wn * 128 + j * 32 + rg * 8 + frag_half * 4;
+        const int nl = wn * kBigWaveN + j * 32 + rg * 8 + frag_half * 4;
         float bv[4] = {0.f, 0.f, 0.f, 0.f};
         if (g.bias) {
 #pragma unroll
@@ -297,10 +305,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_mfma16_kernel(GemmArgs g) {
         }
       }
     __syncthreads();
-    // 256 lanes: 8 rows per sweep, 32 lanes x 16 bytes per row
+    // 2 rows per wave and sweep, 32 lanes x 16 bytes per row
     const int rsub = threadIdx.x >> 5, cseg = (threadIdx.x & 31) * 8;
 #pragma unroll 4
-    for (int r0 = 0; r0 < BM; r0 += 8) {
+    for (int r0 = 0; r0 < BM; r0 += kBigThreads / 32) {
       const int ml = r0 + rsub;
       const int m = m0 + ml;
       if (m >= g.M) continue;
@@ -948,14 +956,14 @@ enum Layout { kFwd = 0, kDx = 1, kDw = 2 };
 
 // Tile choice for a problem the 16-bit kernels can address.  One workgroup of the 256x256
 // kernel occupies a CU, so its time goes in whole rounds of one tile per CU; the 128x128 kernel
-// runs two workgroups per CU at about 60 % of the other's rate (measured: one round of 512
-// tiles takes 0.6 of a round of 256 large ones).
+// runs two workgroups per CU at about 65 % of the other's rate (measured: one round of 512
+// tiles takes 0.65 of a round of 256 large ones).
 inline bool prefer_mid_tiles(int64_t M, int64_t N) {
   const int64_t cus = device_cu_count();
   const double big = (double)cdiv64(cdiv64(M, BM) * cdiv64(N, BN), cus);
   double mid = (double)(cdiv64(M, MT) * cdiv64(N, MT)) / (double)(2 * cus);
   if (mid < 0.6) mid = 0.6;
-  return mid * 0.6 < big;
+  return mid * 0.65 < big;
 }
 
 // Number of splits of the contraction for the weight gradient (a [in, out] tile grid that is
@@ -1047,12 +1055,12 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
         return AT_ERR_DTYPE;
       } else {
         if (layout == kDx) {
-          hipLaunchKernelGGL((gemm_mfma16_kernel<T, false, true, AT_ACT_NONE>), dim3(grid), dim3(kGemmThreads), 0, stream, g);
+          hipLaunchKernelGGL((gemm_mfma16_kernel<T, false, true, AT_ACT_NONE>), dim3(grid), dim3(kBigThreads), 0, stream, g);
         } else if (layout == kDw) {
-          hipLaunchKernelGGL((gemm_mfma16_kernel<T, true, false, AT_ACT_NONE>), dim3(grid), dim3(kGemmThreads), 0, stream, g);
+          hipLaunchKernelGGL((gemm_mfma16_kernel<T, true, false, AT_ACT_NONE>), dim3(grid), dim3(kBigThreads), 0, stream, g);
         } else {
           switch (act) {
-#define AT_FWD_CASE(ID) case ID: hipLaunchKernelGGL((gemm_mfma16_kernel<T, false, false, ID>), dim3(grid), dim3(kGemmThreads), 0, stream, g); break;
+#define AT_FWD_CASE(ID) case ID: hipLaunchKernelGGL((gemm_mfma16_kernel<T, false, false, ID>), dim3(grid), dim3(kBigThreads), 0, stream, g); break;
             AT_FWD_CASE(AT_ACT_NONE) AT_FWD_CASE(AT_ACT_RELU) AT_FWD_CASE(AT_ACT_GELUAPPROX)
 #ifndef AT_QUICK_BUILD  // development builds instantiate three epilogues only
             AT_FWD_CASE(AT_ACT_SIGMOID) AT_FWD_CASE(AT_ACT_LOGSIGMOID)
