@@ -33,6 +33,9 @@ PROTOTYPES = {
     'at_cross_entropy_workspace_bytes': (L, [L]),
     'at_cross_entropy_fwd_bwd': (I, [P, P, P, P, P, P, L, L, L, L, L, L, I, I, I, P]),
     'at_cross_entropy_scale_grad': (I, [P, P, L, L, L, I, I, P]),
+    'at_nll_loss_workspace_bytes': (L, [L, L]),
+    'at_nll_loss_fwd': (I, [P, P, P, P, P, P, L, L, L, L, I, I, I, I, P]),
+    'at_nll_loss_bwd': (I, [P, P, P, P, P, L, L, L, I, I, I, I, P]),
     'at_linear_fwd': (I, [P, P, P, P, P, L, L, L, L, L, L, L, I, F, I, I, I, P]),
     'at_linear_bwd_input': (I, [P, P, P, L, L, L, L, L, L, I, I, P]),
     'at_linear_bwd_weight_workspace_bytes': (L, [L, L, L, I]),

@@ -434,6 +434,36 @@ def bench_cross_entropy(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
                                      'cores': torch.get_num_threads(), 'kind': 'port',
                                      'sample': f'first {crow} of {rows_} rows, oracle loss + gradient'}
         results.append(entry)
+
+    # The reference's alternative to the fused loss: LogSoftmax followed by NLLLoss
+    # (weighted mean).  The NLL kernels gather one element per row forward and write the whole
+    # gradient once backward, so their algorithmic traffic is one write of the gradient.
+    logp = torch.log_softmax(logits.float(), dim=1).to(dtype)
+    tgt_valid = torch.where(tgt < 0, torch.zeros_like(tgt), tgt)
+    dlogp = torch.empty_like(logp)
+    sum_weights = torch.empty(1, dtype=torch.float32, device='cuda')
+    nwsb = lib.at_nll_loss_workspace_bytes(rows_, 1)
+    nws = torch.empty(nwsb, dtype=torch.uint8, device='cuda')
+
+    def nll_fwd():
+        raw.check(lib.at_nll_loss_fwd(logp.data_ptr(), tgt_valid.data_ptr(), weight.data_ptr(), loss.data_ptr(),
+                                      sum_weights.data_ptr(), nws.data_ptr(), nwsb, rows_, feat, 1, 1, dt, 0, dt,
+                                      st()), 'nll_fwd')
+
+    def nll_bwd():
+        raw.check(lib.at_nll_loss_bwd(one.data_ptr(), tgt_valid.data_ptr(), weight.data_ptr(),
+                                      sum_weights.data_ptr(), dlogp.data_ptr(), rows_, feat, 1, 1, dt, 0, dt,
+                                      st()), 'nll_bwd')
+    ms_f = gpu_time_ms(nll_fwd, max(5, steps // 2), warmup)
+    ms_b = gpu_time_ms(nll_bwd, max(5, steps // 2), warmup)
+    gbs = tbytes / (ms_f + ms_b) / 1e6
+    results.append({
+        'workload': f'c3: NLLLoss fp16 fwd+bwd log-probabilities[{rows_},{feat}], class-weighted mean',
+        'metric': 'HBM GB/s', 'value': gbs, 'unit': 'GB/s', 'ms_fwd': ms_f, 'ms_bwd': ms_b,
+        'bwd_gbs': tbytes / ms_b / 1e6,
+        'roofline': {'bound': 'hbm', 'achieved': gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                     'frac': gbs / PEAK_HBM_GBS, 'traffic': None},
+    })
     return results
 
 

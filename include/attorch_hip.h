@@ -165,6 +165,38 @@ int at_cross_entropy_scale_grad(void* dlogits, const void* output_grad, int64_t 
                                 int grad_dtype, at_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Negative log likelihood loss — replaces nll_loss_forward_kernel / nll_loss_backward_kernel,
+ * attorch/nll_loss_kernels.py:39-138 and :141-235, and the torch sums and the division by the
+ * summed weights at attorch/nll_loss_layer.py:88-93.
+ * input is contiguous [batch, feat, spatial] log-probabilities, target [batch, spatial].
+ *   forward : l[b, s] = -w[target] * input[b, target, s]  (w = 1 when weight is null)
+ *             AT_REDUCTION_NONE: output[batch, spatial] = l;  _SUM: output[1] = sum(l);
+ *             _MEAN: output[1] = sum(l) / sum(w[target])  (= sum(l) / (batch * spatial) unweighted)
+ *   backward: input_grad[b, c, s] = -output_grad * w[c] / denominator where c == target[b, s],
+ *             zero elsewhere; every element of input_grad is written (no prior zero fill).
+ * output_grad is [batch, spatial] for AT_REDUCTION_NONE and one element otherwise.  The
+ * reductions need at_nll_loss_workspace_bytes bytes of workspace; sum_weights (one fp32,
+ * optional in the forward call) receives sum(w[target]) and is what the backward call of a
+ * weighted mean divides by.  A target outside [0, feat) contributes no loss, weight or gradient
+ * (the reference reads out of bounds there; it has no ignore_index, nll_loss_layer.py:162).
+ * ------------------------------------------------------------------------------------------ */
+#define AT_REDUCTION_NONE 0
+#define AT_REDUCTION_MEAN 1
+#define AT_REDUCTION_SUM 2
+
+int64_t at_nll_loss_workspace_bytes(int64_t batch, int64_t spatial);
+
+int at_nll_loss_fwd(const void* input, const int64_t* target, const void* weight, void* output,
+                    float* sum_weights, void* workspace, int64_t workspace_bytes, int64_t batch,
+                    int64_t feat, int64_t spatial, int reduction, int in_dtype, int weight_dtype,
+                    int out_dtype, at_stream_t stream);
+
+int at_nll_loss_bwd(const void* output_grad, const int64_t* target, const void* weight,
+                    const float* sum_weights, void* input_grad, int64_t batch, int64_t feat,
+                    int64_t spatial, int reduction, int grad_dtype, int weight_dtype,
+                    int out_dtype, at_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
  * Linear — replaces linear_forward_kernel, attorch/linear_kernels.py:59-188 (launched from
  * attorch/linear_layer.py:90-98), act_func_backward_kernel, attorch/act_kernels.py:888-927
  * (launched from linear_layer.py:144-146 and batch_norm_layer.py:204-206), and the torch calls

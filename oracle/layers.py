@@ -272,6 +272,72 @@ def cross_entropy_backward(
 
 
 # ---------------------------------------------------------------------------------------------
+# Negative log likelihood — attorch/nll_loss_kernels.py:39-138, :141-235, nll_loss_layer.py:55-93
+# ---------------------------------------------------------------------------------------------
+def _nll_views(input: Tensor, target: Tensor) -> Tuple[Tensor, Tensor]:
+    """nll_loss_layer.py:58-62: [batch, feat, spatial] and [batch, spatial] views."""
+    flat_input = input.unsqueeze(-1) if input.ndim == 2 else input
+    flat_target = target.unsqueeze(-1) if target.ndim == 1 else target
+    return flat_input.flatten(2, -1), flat_target.flatten(1, -1)
+
+
+def nll_loss_forward(
+    input: Tensor, target: Tensor, weight: Optional[Tensor], reduction: str,
+    output_dtype: torch.dtype, compute: torch.dtype = torch.float32,
+    ) -> Tuple[Tensor, Optional[Tensor]]:
+    """
+    nll_loss_kernels.py:108-138: output[b, s] = -input[b, target[b, s], s], times
+    weight[target[b, s]] when weighted; 'sum' adds all entries; 'mean' divides the sum by
+    batch * spatial (kernel :132-134) or, weighted, by the sum of the selected weights
+    (nll_loss_layer.py:88-93).
+
+    Returns:
+        (loss in output_dtype, sum of the selected weights in `compute` precision or None).
+    """
+    x, t = _nll_views(_c(input, compute), target)
+    picked = x.gather(1, t[:, None, :])[:, 0, :]
+    loss = -picked
+    sum_weights = None
+    if weight is not None:
+        w = _c(weight, compute)[t]
+        loss = loss * w
+        sum_weights = w.sum()
+    if reduction == 'none':
+        return loss.view(target.shape).to(output_dtype), sum_weights
+    total = loss.sum()
+    if reduction == 'mean':
+        total = total / sum_weights if weight is not None else total / t.numel()
+    return total.to(output_dtype), sum_weights
+
+
+def nll_loss_backward(
+    output_grad: Tensor, input_shape: Tuple[int, ...], target: Tensor, weight: Optional[Tensor],
+    reduction: str, output_dtype: torch.dtype, compute: torch.dtype = torch.float32,
+    ) -> Tensor:
+    """
+    nll_loss_kernels.py:207-235 on a zeroed gradient (nll_loss_layer.py:120): at
+    [b, target[b, s], s] the value -output_grad (per entry for 'none', the scalar otherwise),
+    times weight[target] when weighted, divided for 'mean' by the summed selected weights
+    (weighted) or by batch * spatial.
+    """
+    batch, feat = input_shape[:2]
+    flat_target = (target.unsqueeze(-1) if target.ndim == 1 else target).flatten(1, -1)
+    spatial = flat_target.shape[1]
+    g = _c(output_grad, compute)
+    coef = -g.reshape(batch, spatial) if reduction == 'none' else (-g).expand(batch, spatial)
+    if weight is not None:
+        w = _c(weight, compute)[flat_target]
+        coef = coef * w
+        if reduction == 'mean':
+            coef = coef / w.sum()
+    elif reduction == 'mean':
+        coef = coef / (batch * spatial)
+    grad = torch.zeros((batch, feat, spatial), dtype=compute)
+    grad.scatter_(1, flat_target[:, None, :], coef[:, None, :])
+    return grad.view(input_shape).to(output_dtype)
+
+
+# ---------------------------------------------------------------------------------------------
 # Conv2d — attorch/conv_kernels.py:68-207, attorch/conv_layer.py:43-164
 # ---------------------------------------------------------------------------------------------
 def _conv_out(size: int, kernel: int, stride: int, padding: int) -> int:

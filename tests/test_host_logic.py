@@ -72,6 +72,13 @@ def test_argument_errors_without_gpu() -> None:
                                  4, 8, 1, 0.1, 1e-5, 0, 0.0, 0, 1, 0, 0, 0, None) == -5
     assert lib.at_act_dropout_fwd(p, p, 8, 0, 0.0, 1.5, 0, 0, None) == -2
     assert lib.at_act_dropout_bwd(p, None, p, 8, 4, 0.0, 0.0, 0, 0, None) == -1
+    # NLL loss: reductions need their workspace, the reduction id must be known
+    assert lib.at_nll_loss_workspace_bytes(16, 1) > 0
+    assert lib.at_nll_loss_fwd(p, p, None, p, None, None, 0, 4, 8, 1, 1, 0, 0, 0, None) == -5
+    assert lib.at_nll_loss_fwd(p, p, None, p, None, None, 0, 4, 8, 1, 7, 0, 0, 0, None) == -7
+    assert lib.at_nll_loss_fwd(p, None, None, p, None, None, 0, 4, 8, 1, 0, 0, 0, 0, None) == -1
+    assert lib.at_nll_loss_bwd(p, p, p, None, p, 4, 8, 1, 1, 0, 0, 0, None) == -1
+    assert lib.at_nll_loss_bwd(p, p, None, None, p, 4, 0, 1, 1, 0, 0, 0, None) == -2
     # inconsistent convolution geometry
     dims = [1, 4, 8, 8, 4, 9, 9, 3, 3, 1, 1, 1, 1, 1]
     assert lib.at_conv2d_fwd(p, p, None, p, None, 0, *dims, 0, 0, 0, None) == -2

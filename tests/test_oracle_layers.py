@@ -189,6 +189,58 @@ def test_cross_entropy_special_cases() -> None:
     torch.testing.assert_close(grad.sum(dim=1), torch.zeros(4, dtype=D), atol=1e-14, rtol=0)
 
 
+# ------------------------------------------------------------------ NLL loss
+@pytest.mark.parametrize('weighted', [False, True])
+@pytest.mark.parametrize('reduction', ['none', 'mean', 'sum'])
+@pytest.mark.parametrize('shape', [(12, 7), (5, 6, 9), (3, 4, 2, 5)])
+def test_nll_loss_matches_torch(shape, reduction, weighted) -> None:
+    feat = shape[1]
+    x = torch.log_softmax(rand(*shape, seed=1, scale=2.0), dim=1).requires_grad_(True)
+    g = torch.Generator().manual_seed(3)
+    t = torch.randint(0, feat, (shape[0], *shape[2:]), generator=g)
+    w = (0.5 + torch.rand(feat, generator=g, dtype=D)) if weighted else None
+    loss = F.nll_loss(x, t, weight=w, reduction=reduction)
+    dy = rand(*loss.shape, seed=4) if reduction == 'none' else torch.tensor(1.7, dtype=D)
+    (gx,) = torch.autograd.grad(loss, x, dy)
+    out, sum_weights = oracle.nll_loss_forward(x.detach(), t, w, reduction, D, compute=D)
+    torch.testing.assert_close(out, loss.detach(), **TOL)
+    grad = oracle.nll_loss_backward(dy, x.shape, t, w, reduction, D, compute=D)
+    torch.testing.assert_close(grad, gx, **TOL)
+    if weighted:
+        torch.testing.assert_close(sum_weights, w[t].sum(), **TOL)
+
+
+def test_nll_loss_brute_force() -> None:
+    x = rand(3, 4, 2, seed=5)
+    t = torch.tensor([[0, 3], [2, 2], [1, 0]])
+    w = torch.tensor([0.5, 2.0, 1.5, 0.25], dtype=D)
+    total, weights = 0.0, 0.0
+    expected_grad = torch.zeros_like(x)
+    for b in range(3):
+        for s in range(2):
+            c = int(t[b, s])
+            total += -float(x[b, c, s]) * float(w[c])
+            weights += float(w[c])
+    for b in range(3):
+        for s in range(2):
+            c = int(t[b, s])
+            expected_grad[b, c, s] = -2.0 * float(w[c]) / weights
+    out, sum_weights = oracle.nll_loss_forward(x, t, w, 'mean', D, compute=D)
+    assert math.isclose(out.item(), total / weights, rel_tol=1e-12)
+    assert math.isclose(sum_weights.item(), weights, rel_tol=1e-12)
+    grad = oracle.nll_loss_backward(torch.tensor(2.0, dtype=D), x.shape, t, w, 'mean', D, compute=D)
+    torch.testing.assert_close(grad, expected_grad, **TOL)
+    # unweighted mean divides by the number of entries, and log-softmax + NLL is cross entropy
+    out, _ = oracle.nll_loss_forward(x, t, None, 'mean', D, compute=D)
+    assert math.isclose(out.item(), -sum(float(x[b, int(t[b, s]), s]) for b in range(3) for s in range(2)) / 6,
+                        rel_tol=1e-12)
+    logits = rand(6, 5, seed=6)
+    cls = torch.tensor([0, 4, 2, 2, 1, 3])
+    via_nll, _ = oracle.nll_loss_forward(torch.log_softmax(logits, dim=1), cls, None, 'mean', D, compute=D)
+    via_ce, _ = oracle.cross_entropy_forward(logits, cls, None, -100, D, compute=D)
+    torch.testing.assert_close(via_nll, via_ce, **TOL)
+
+
 # ------------------------------------------------------------------ Conv2d
 @pytest.mark.parametrize('kernel, stride, padding, groups',
                          [((3, 3), (1, 1), (1, 1), 1), ((1, 1), (1, 1), (0, 0), 1),
