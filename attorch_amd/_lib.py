@@ -36,6 +36,11 @@ PROTOTYPES = {
     'at_nll_loss_workspace_bytes': (L, [L, L]),
     'at_nll_loss_fwd': (I, [P, P, P, P, P, P, L, L, L, L, I, I, I, I, P]),
     'at_nll_loss_bwd': (I, [P, P, P, P, P, L, L, L, I, I, I, I, P]),
+    'at_p_loss_workspace_bytes': (L, [L]),
+    'at_p_loss_fwd': (I, [P, P, P, P, L, L, I, I, F, I, I, P]),
+    'at_p_loss_bwd': (I, [P, P, P, P, P, L, I, I, F, I, I, I, P]),
+    'at_glu_fwd': (I, [P, P, L, L, I, F, I, P]),
+    'at_glu_bwd': (I, [P, P, P, L, L, I, F, I, P]),
     'at_linear_fwd': (I, [P, P, P, P, P, L, L, L, L, L, L, L, I, F, I, I, I, P]),
     'at_linear_bwd_input': (I, [P, P, P, L, L, L, L, L, L, I, I, P]),
     'at_linear_bwd_weight_workspace_bytes': (L, [L, L, L, I]),

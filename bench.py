@@ -380,6 +380,48 @@ def bench_rows(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
                                      'cores': torch.get_num_threads(), 'kind': 'port',
                                      'sample': f'first {crow} of {rows_} rows, oracle fwd+bwd'}
         results.append(entry)
+
+    # Elementwise layers outside the headline configs, on the same buffers: GLU (sigmoid) gated
+    # along the feature dimension, and the mean squared error with the gradient of the input.
+    half = feat // 2
+    glu_out = [torch.empty((rows_, half), dtype=dtype, device='cuda') for _ in range(nsets)]
+    glu_dy = [gen((rows_, half), 2301 + i, dtype).cuda() for i in range(nsets)]
+
+    def glu_f():
+        i = nxt()
+        raw.check(lib.at_glu_fwd(xs[i].data_ptr(), glu_out[i].data_ptr(), rows_, half, 1, 0.0, dt, st()), 'glu_fwd')
+
+    def glu_b():
+        i = nxt()
+        raw.check(lib.at_glu_bwd(glu_dy[i].data_ptr(), xs[i].data_ptr(), dxs[i].data_ptr(), rows_, half, 1, 0.0, dt,
+                                 st()), 'glu_bwd')
+    loss = torch.empty((), dtype=dtype, device='cuda')
+    one = torch.ones((), dtype=dtype, device='cuda')
+    lwsb = lib.at_p_loss_workspace_bytes(rows_ * feat)
+    lws = torch.empty(lwsb, dtype=torch.uint8, device='cuda')
+
+    def mse_f():
+        i = nxt()
+        raw.check(lib.at_p_loss_fwd(xs[i].data_ptr(), dys[i].data_ptr(), loss.data_ptr(), lws.data_ptr(), lwsb,
+                                    rows_ * feat, 2, 1, 1.0, dt, dt, st()), 'mse_fwd')
+
+    def mse_b():
+        i = nxt()
+        raw.check(lib.at_p_loss_bwd(one.data_ptr(), xs[i].data_ptr(), dys[i].data_ptr(), dxs[i].data_ptr(), None,
+                                    rows_ * feat, 2, 1, 1.0, dt, dt, dt, st()), 'mse_bwd')
+    for name, f, bwd, fwd_units, bwd_units in (('GLU(sigmoid) over the features', glu_f, glu_b, 1.5, 2.5),
+                                               ('MSELoss(mean), input gradient', mse_f, mse_b, 2.0, 3.0)):
+        ms_f = gpu_time_ms(f, iters, warmup)
+        ms_b = gpu_time_ms(bwd, iters, warmup)
+        gbs = (fwd_units + bwd_units) * tbytes / (ms_f + ms_b) / 1e6
+        results.append({
+            'workload': f'c2-shaped: {name} bf16 fwd+bwd X[{rows_},{feat}]', 'metric': 'HBM GB/s', 'value': gbs,
+            'unit': 'GB/s', 'ms_fwd': ms_f, 'ms_bwd': ms_b,
+            'fwd_gbs': fwd_units * tbytes / ms_f / 1e6, 'bwd_gbs': bwd_units * tbytes / ms_b / 1e6,
+            'roofline': {'bound': 'hbm', 'achieved': gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                         'frac': gbs / PEAK_HBM_GBS, 'traffic': None},
+            'elementwise_reference': stream_ref,
+        })
     return results
 
 

@@ -197,6 +197,49 @@ int at_nll_loss_bwd(const void* output_grad, const int64_t* target, const void* 
                     int out_dtype, at_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Regression losses of d = input - target — replace p_loss_forward_kernel /
+ * p_loss_backward_kernel, attorch/p_loss_kernels.py:17-79 and :82-143, and the torch sum at
+ * attorch/p_loss_layers.py:71-73.  The ids are the reference's p_loss integers
+ * (p_loss_layers.py:39-40); param is beta (smooth L1) or delta (Huber).
+ *   forward : AT_REDUCTION_NONE: output[size] = loss(d); _SUM: output[1] = sum; _MEAN: sum / size
+ *   backward: input_grad = output_grad * loss'(d) (/ size for the mean), target_grad = -input_grad;
+ *             either gradient pointer may be null.  At d == 0 the L1-type slope is +1, as in
+ *             the reference (p_loss_kernels.py:128-136).
+ * input and target are contiguous, of one dtype; output_grad is [size] for AT_REDUCTION_NONE
+ * and one element otherwise.  Reductions need at_p_loss_workspace_bytes bytes of workspace.
+ * ------------------------------------------------------------------------------------------ */
+#define AT_P_LOSS_SMOOTH_L1 0
+#define AT_P_LOSS_L1 1
+#define AT_P_LOSS_MSE 2
+#define AT_P_LOSS_HUBER 3
+
+int64_t at_p_loss_workspace_bytes(int64_t size);
+
+int at_p_loss_fwd(const void* input, const void* target, void* output, void* workspace,
+                  int64_t workspace_bytes, int64_t size, int p_loss, int reduction, float param,
+                  int in_dtype, int out_dtype, at_stream_t stream);
+
+int at_p_loss_bwd(const void* output_grad, const void* input, const void* target,
+                  void* input_grad, void* target_grad, int64_t size, int p_loss, int reduction,
+                  float param, int in_dtype, int grad_dtype, int out_dtype, at_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Gated linear unit with an arbitrary activation — replaces glu_forward_kernel /
+ * glu_backward_kernel, attorch/glu_kernels.py:18-57 and :60-105, together with the chunk /
+ * contiguous / concat copies around them (attorch/glu_layer.py:60-62, :113).
+ * input is addressed as [outer][2][half]: for a contiguous tensor gated along dimension d,
+ * outer = product of the sizes before d and half = (size of d / 2) * product of the sizes after d.
+ *   forward : output[outer][half] = x1 * act(x2)
+ *   backward: input_grad[outer][2][half] = (output_grad * act(x2), output_grad * x1 * act'(x2))
+ * act is an AT_ACT_* id other than AT_ACT_NONE.
+ * ------------------------------------------------------------------------------------------ */
+int at_glu_fwd(const void* input, void* output, int64_t outer, int64_t half, int act, float param,
+               int dtype, at_stream_t stream);
+
+int at_glu_bwd(const void* output_grad, const void* input, void* input_grad, int64_t outer,
+               int64_t half, int act, float param, int dtype, at_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
  * Linear — replaces linear_forward_kernel, attorch/linear_kernels.py:59-188 (launched from
  * attorch/linear_layer.py:90-98), act_func_backward_kernel, attorch/act_kernels.py:888-927
  * (launched from linear_layer.py:144-146 and batch_norm_layer.py:204-206), and the torch calls

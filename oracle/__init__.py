@@ -16,7 +16,8 @@ pinned by at least one such check; none is "parity unpinned".
 
 from .acts import ACT_NAMES, act_forward, act_grad, parse_act_func
 from .layers import (act_dropout_backward, act_dropout_forward, batch_norm_backward, batch_norm_forward, conv2d_backward, conv2d_forward,
-                     cross_entropy_backward, cross_entropy_forward, layer_norm_backward,
+                     cross_entropy_backward, cross_entropy_forward, glu_backward, glu_forward,
+                     layer_norm_backward,
                      layer_norm_forward, linear_backward, linear_forward, nll_loss_backward,
-                     nll_loss_forward, rms_norm_backward,
+                     nll_loss_forward, p_loss_backward, p_loss_forward, rms_norm_backward,
                      rms_norm_forward, softmax_backward, softmax_forward)

@@ -545,3 +545,82 @@ def act_dropout_backward(
         g = g * act_grad(input.to(compute), act_func, param)
     dtype = output_grad.dtype if input is None else input.dtype
     return g.to(dtype)
+
+
+# ---------------------------------------------------------------------------------------------
+# Gated linear unit — attorch/glu_kernels.py:18-57, :60-105, attorch/glu_layer.py:60-62, :113
+# ---------------------------------------------------------------------------------------------
+def glu_forward(input: Tensor, dim: int, name: str, param: Optional[float], output_dtype: torch.dtype,
+                compute: torch.dtype = torch.float32) -> Tensor:
+    """
+    glu_layer.py:60 and glu_kernels.py:53-56: the input is cut in two along `dim`;
+    output = first half * act(second half).
+    """
+    x1, x2 = _c(input, compute).chunk(2, dim=dim)
+    return (x1 * act_forward(x2, name, param)).to(output_dtype)
+
+
+def glu_backward(output_grad: Tensor, input: Tensor, dim: int, name: str, param: Optional[float],
+                 output_dtype: torch.dtype, compute: torch.dtype = torch.float32) -> Tensor:
+    """
+    glu_kernels.py:96-104: first-half gradient = output_grad * act(second half), second-half
+    gradient = output_grad * first half * act'(second half); concatenated along `dim`
+    (glu_layer.py:113).
+    """
+    x1, x2 = _c(input, compute).chunk(2, dim=dim)
+    g = _c(output_grad, compute)
+    grad1 = g * act_forward(x2, name, param)
+    grad2 = g * x1 * act_grad(x2, name, param)
+    return torch.concat([grad1, grad2], dim=dim).to(output_dtype)
+
+
+# ---------------------------------------------------------------------------------------------
+# p-norm losses — attorch/p_loss_kernels.py:17-79, :82-143, attorch/p_loss_layers.py:57-76
+# ---------------------------------------------------------------------------------------------
+def p_loss_forward(input: Tensor, target: Tensor, p_loss: int, reduction: str, param: float,
+                   output_dtype: torch.dtype, compute: torch.dtype = torch.float32) -> Tensor:
+    """
+    p_loss_kernels.py:58-79 with diff = input - target: 0 smooth L1 (|d| < beta ? d^2 / (2 beta) :
+    |d| - beta / 2), 1 L1 (|d|), 2 squared L2 (d^2), 3 Huber (|d| < delta ? d^2 / 2 :
+    delta (|d| - delta / 2)); 'mean' divides the sum by the number of elements.
+    """
+    d = _c(input, compute) - _c(target, compute)
+    a = d.abs()
+    if p_loss == 0:
+        error = torch.where(a < param, 0.5 * d * d / param, a - 0.5 * param)
+    elif p_loss == 1:
+        error = a
+    elif p_loss == 2:
+        error = d * d
+    else:
+        error = torch.where(a < param, 0.5 * d * d, param * (a - 0.5 * param))
+    if reduction == 'none':
+        return error.to(output_dtype)
+    total = error.sum()
+    if reduction == 'mean':
+        total = total / error.numel()
+    return total.to(output_dtype)
+
+
+def p_loss_backward(output_grad: Tensor, input: Tensor, target: Tensor, p_loss: int, reduction: str,
+                    param: float, output_dtype: torch.dtype,
+                    compute: torch.dtype = torch.float32) -> Tuple[Tensor, Tensor]:
+    """
+    p_loss_kernels.py:126-143: slope of the loss in diff (sign taken as +1 at diff == 0, :128-136),
+    divided by the number of elements for 'mean', times output_grad; the target's gradient is
+    the negative.
+    """
+    d = _c(input, compute) - _c(target, compute)
+    sign = torch.where(d >= 0, torch.ones_like(d), -torch.ones_like(d))
+    if p_loss == 0:
+        grad = torch.where(d.abs() < param, d / param, sign)
+    elif p_loss == 1:
+        grad = sign
+    elif p_loss == 2:
+        grad = 2 * d
+    else:
+        grad = torch.where(d.abs() < param, d, param * sign)
+    if reduction == 'mean':
+        grad = grad / d.numel()
+    grad = grad * _c(output_grad, compute)
+    return grad.to(output_dtype), (-grad).to(output_dtype)

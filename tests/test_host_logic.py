@@ -79,6 +79,14 @@ def test_argument_errors_without_gpu() -> None:
     assert lib.at_nll_loss_fwd(p, None, None, p, None, None, 0, 4, 8, 1, 0, 0, 0, 0, None) == -1
     assert lib.at_nll_loss_bwd(p, p, p, None, p, 4, 8, 1, 1, 0, 0, 0, None) == -1
     assert lib.at_nll_loss_bwd(p, p, None, None, p, 4, 0, 1, 1, 0, 0, 0, None) == -2
+    # p-norm losses and GLU
+    assert lib.at_p_loss_workspace_bytes(100) > 0
+    assert lib.at_p_loss_fwd(p, p, p, None, 0, 8, 2, 1, 1.0, 0, 0, None) == -5
+    assert lib.at_p_loss_fwd(p, p, p, None, 0, 8, 4, 0, 1.0, 0, 0, None) == -7
+    assert lib.at_p_loss_bwd(p, p, p, None, None, 8, 2, 1, 1.0, 0, 0, 0, None) == -1
+    assert lib.at_glu_fwd(p, p, 4, 8, 0, 0.0, 0, None) == -4            # the gate needs an activation
+    assert lib.at_glu_fwd(p, p, 0, 8, 1, 0.0, 0, None) == 0             # nothing to do
+    assert lib.at_glu_bwd(None, p, p, 4, 8, 1, 0.0, 0, None) == -1
     # inconsistent convolution geometry
     dims = [1, 4, 8, 8, 4, 9, 9, 3, 3, 1, 1, 1, 1, 1]
     assert lib.at_conv2d_fwd(p, p, None, p, None, 0, *dims, 0, 0, 0, None) == -2

@@ -241,6 +241,58 @@ def test_nll_loss_brute_force() -> None:
     torch.testing.assert_close(via_nll, via_ce, **TOL)
 
 
+# ------------------------------------------------------------------ GLU and p-norm losses
+@pytest.mark.parametrize('dim', [-1, 0, 1])
+def test_glu_matches_torch(dim) -> None:
+    x = rand(4, 6, 8, seed=1).requires_grad_(True)
+    y = F.glu(x, dim=dim)                                     # torch's GLU is the sigmoid case
+    dy = rand(*y.shape, seed=2)
+    (gx,) = torch.autograd.grad(y, x, dy)
+    torch.testing.assert_close(oracle.glu_forward(x.detach(), dim, 'sigmoid', None, D, compute=D), y.detach(), **TOL)
+    torch.testing.assert_close(oracle.glu_backward(dy, x.detach(), dim, 'sigmoid', None, D, compute=D), gx, **TOL)
+    # another activation through autograd on the composed expression
+    a, b = x.chunk(2, dim=dim)
+    y2 = a * F.silu(b)
+    (gx2,) = torch.autograd.grad(y2, x, dy)
+    torch.testing.assert_close(oracle.glu_forward(x.detach(), dim, 'silu', None, D, compute=D), y2.detach(), **TOL)
+    torch.testing.assert_close(oracle.glu_backward(dy, x.detach(), dim, 'silu', None, D, compute=D), gx2, **TOL)
+
+
+@pytest.mark.parametrize('reduction', ['none', 'mean', 'sum'])
+@pytest.mark.parametrize('p_loss, torch_fn, param', [
+    (0, lambda x, t, r: F.smooth_l1_loss(x, t, reduction=r, beta=0.7), 0.7),
+    (1, lambda x, t, r: F.l1_loss(x, t, reduction=r), 1.0),
+    (2, lambda x, t, r: F.mse_loss(x, t, reduction=r), 1.0),
+    (3, lambda x, t, r: F.huber_loss(x, t, reduction=r, delta=0.6), 0.6)])
+def test_p_loss_matches_torch(p_loss, torch_fn, param, reduction) -> None:
+    x = rand(5, 7, 3, seed=1).requires_grad_(True)
+    t = rand(5, 7, 3, seed=2).requires_grad_(True)
+    loss = torch_fn(x, t, reduction)
+    dy = rand(*loss.shape, seed=3) if reduction == 'none' else torch.tensor(-1.3, dtype=D)
+    gx, gt = torch.autograd.grad(loss, [x, t], dy)
+    out = oracle.p_loss_forward(x.detach(), t.detach(), p_loss, reduction, param, D, compute=D)
+    torch.testing.assert_close(out, loss.detach(), **TOL)
+    dx, dt = oracle.p_loss_backward(dy, x.detach(), t.detach(), p_loss, reduction, param, D, compute=D)
+    torch.testing.assert_close(dx, gx, **TOL)
+    torch.testing.assert_close(dt, gt, **TOL)
+
+
+def test_p_loss_known_answers() -> None:
+    x = torch.tensor([0.0, 0.25, -2.0, 3.0], dtype=D)
+    t = torch.zeros(4, dtype=D)
+    one = torch.tensor(1.0, dtype=D)
+    assert oracle.p_loss_forward(x, t, 1, 'sum', 1.0, D, compute=D).item() == 5.25
+    assert oracle.p_loss_forward(x, t, 2, 'mean', 1.0, D, compute=D).item() == (0.0625 + 4 + 9) / 4
+    # smooth L1, beta 0.5: 0, 0.0625, 1.75, 2.75;  Huber, delta 0.5: 0, 0.03125, 0.875, 1.375
+    torch.testing.assert_close(oracle.p_loss_forward(x, t, 0, 'none', 0.5, D, compute=D),
+                               torch.tensor([0.0, 0.0625, 1.75, 2.75], dtype=D), **TOL)
+    torch.testing.assert_close(oracle.p_loss_forward(x, t, 3, 'none', 0.5, D, compute=D),
+                               torch.tensor([0.0, 0.03125, 0.875, 1.375], dtype=D), **TOL)
+    # the L1 slope at a zero difference is +1 (p_loss_kernels.py:130), not torch's 0
+    dx, dt = oracle.p_loss_backward(one, x, t, 1, 'sum', 1.0, D, compute=D)
+    assert dx.tolist() == [1.0, 1.0, -1.0, 1.0] and dt.tolist() == [-1.0, -1.0, 1.0, -1.0]
+
+
 # ------------------------------------------------------------------ Conv2d
 @pytest.mark.parametrize('kernel, stride, padding, groups',
                          [((3, 3), (1, 1), (1, 1), 1), ((1, 1), (1, 1), (0, 0), 1),
