@@ -22,7 +22,6 @@
 //  * gemm_simple_kernel — fp32 operands, any strides, fp32 MFMA (32x32x2), 64x64x64 tile, next
 //    k-tile prefetched into registers.
 // All fuse bias, the optional pre-activation store and the activation into the epilogue.
-#include <cstdlib>
 #include <type_traits>
 
 #include "at_act.h"
@@ -161,6 +160,77 @@ __device__ __forceinline__ uint4 read_frag(const char* tile, int outer_base, int
   }
 }
 
+// Epilogue of the 256x256 kernels: bias, optional pre-activation copy and activation, out through LDS.
+template <typename T, int ACT>
+__device__ __forceinline__ void big_tile_epilogue(f32x16 (&acc)[4][kBigNJ], char* lds, const GemmArgs& g, int m0,
+                                                  int n0) {
+  constexpr int NJ = kBigNJ;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave / (kBigWaves / 2), wn = wave % (kBigWaves / 2);
+  const int frag_row = lane & 31, frag_half = lane >> 5;
+  // A lane holds, for tile (i, j) and register group rg, C[m][n .. n+3] with
+  //   m = wm*128 + i*32 + lane%32,  n = wn*kBigWaveN + j*32 + rg*8 + (lane/32)*4   (tile-local).
+  // Storing that straight to memory touches 32 rows per instruction with 16 bytes each; instead
+  // the finished tile goes through LDS (free after the main loop) and leaves as whole rows:
+  // 32 lanes x 16 bytes = one 512-byte row segment per half-wave.
+  T* __restrict__ C = reinterpret_cast<T*>(g.c);
+  T* __restrict__ P = reinterpret_cast<T*>(g.pre_act);
+  const bool rows16 = ((g.ldc & 7) == 0) && aligned16_dev(C) && (n0 + BN <= g.N) &&
+                      (!P || (((g.ldp & 7) == 0) && aligned16_dev(P)));
+  constexpr int n_out = ACT != AT_ACT_NONE ? 2 : 1;
+#pragma unroll
+  for (int pass = 0; pass < n_out; ++pass) {
+    const bool is_pre = (n_out == 2 && pass == 0);
+    T* __restrict__ dst = is_pre ? P : C;
+    const int64_t ldd = is_pre ? g.ldp : g.ldc;
+    if (is_pre && !P) continue;   // uniform
+    __syncthreads();              // previous readers of LDS (main loop or previous pass) are done
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        const int nl = wn * kBigWaveN + j * 32 + rg * 8 + frag_half * 4;
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (g.bias) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n0 + nl + e < g.N) bv[e] = load_scalar_f32(g.bias, g.bias_dt, n0 + nl + e);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            v[e] = acc[i][j][rg * 4 + e] + bv[e];
+            if (ACT != AT_ACT_NONE && !is_pre) v[e] = act_forward(ACT, v[e], g.param);
+          }
+          const int ml = wm * 128 + i * 32 + frag_row;
+          store_f32<T, 4>(reinterpret_cast<T*>(lds + ml * kEpiPitch) + nl, v);
+        }
+      }
+    __syncthreads();
+    // 2 rows per wave and sweep, 32 lanes x 16 bytes per row
+    const int rsub = threadIdx.x >> 5, cseg = (threadIdx.x & 31) * 8;
+#pragma unroll 4
+    for (int r0 = 0; r0 < BM; r0 += kBigThreads / 32) {
+      const int ml = r0 + rsub;
+      const int m = m0 + ml;
+      if (m >= g.M) continue;
+      const uint4 v = *reinterpret_cast<const uint4*>(lds + ml * kEpiPitch + cseg * 2);
+      T* out = dst + (int64_t)m * ldd + n0 + cseg;
+      if (rows16) {
+        *reinterpret_cast<uint4*>(out) = v;
+      } else {
+        union { uint4 raw; T e[8]; } u;
+        u.raw = v;
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (n0 + cseg + e < g.N) out[e] = u.e[e];
+      }
+    }
+  }
+}
+
 // ACT is the compile-time activation id of the epilogue (the act switch must fold away: the
 // epilogue is fully unrolled over the accumulator registers).
 template <typename T, bool A_MC, bool B_KC, int ACT>
@@ -263,68 +333,7 @@ __global__ __launch_bounds__(kBigThreads) void gemm_mfma16_kernel(GemmArgs g) {
     __syncthreads();      // ... and so has everybody else's; the current stage may be overwritten
   }
 
-  // ---- epilogue ----
-  // A lane holds, for tile (i, j) and register group rg, C[m][n .. n+3] with
-  //   m = wm*128 + i*32 + lane%32,  n = wn*kBigWaveN + j*32 + rg*8 + (lane/32)*4   (tile-local).
-  // Storing that straight to memory touches 32 rows per instruction with 16 bytes each; instead
-  // the finished tile goes through LDS (free after the main loop) and leaves as whole rows:
-  // 32 lanes x 16 bytes = one 512-byte row segment per half-wave.
-  T* __restrict__ C = reinterpret_cast<T*>(g.c);
-  T* __restrict__ P = reinterpret_cast<T*>(g.pre_act);
-  const bool rows16 = ((g.ldc & 7) == 0) && aligned16_dev(C) && (n0 + BN <= g.N) &&
-                      (!P || (((g.ldp & 7) == 0) && aligned16_dev(P)));
-  constexpr int n_out = ACT != AT_ACT_NONE ? 2 : 1;
-#pragma unroll
-  for (int pass = 0; pass < n_out; ++pass) {
-    const bool is_pre = (n_out == 2 && pass == 0);
-    T* __restrict__ dst = is_pre ? P : C;
-    const int64_t ldd = is_pre ? g.ldp : g.ldc;
-    if (is_pre && !P) continue;   // uniform
-    __syncthreads();              // previous readers of LDS (main loop or previous pass) are done
-#pragma unroll
-    for (int j = 0; j < NJ; ++j)
-#pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        const int nl = wn * kBigWaveN + j * 32 + rg * 8 + frag_half * 4;
-        float bv[4] = {0.f, 0.f, 0.f, 0.f};
-        if (g.bias) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (n0 + nl + e < g.N) bv[e] = load_scalar_f32(g.bias, g.bias_dt, n0 + nl + e);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          float v[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            v[e] = acc[i][j][rg * 4 + e] + bv[e];
-            if (ACT != AT_ACT_NONE && !is_pre) v[e] = act_forward(ACT, v[e], g.param);
-          }
-          const int ml = wm * 128 + i * 32 + frag_row;
-          store_f32<T, 4>(reinterpret_cast<T*>(lds + ml * kEpiPitch) + nl, v);
-        }
-      }
-    __syncthreads();
-    // 2 rows per wave and sweep, 32 lanes x 16 bytes per row
-    const int rsub = threadIdx.x >> 5, cseg = (threadIdx.x & 31) * 8;
-#pragma unroll 4
-    for (int r0 = 0; r0 < BM; r0 += kBigThreads / 32) {
-      const int ml = r0 + rsub;
-      const int m = m0 + ml;
-      if (m >= g.M) continue;
-      const uint4 v = *reinterpret_cast<const uint4*>(lds + ml * kEpiPitch + cseg * 2);
-      T* out = dst + (int64_t)m * ldd + n0 + cseg;
-      if (rows16) {
-        *reinterpret_cast<uint4*>(out) = v;
-      } else {
-        union { uint4 raw; T e[8]; } u;
-        u.raw = v;
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (n0 + cseg + e < g.N) out[e] = u.e[e];
-      }
-    }
-  }
+  big_tile_epilogue<T, ACT>(acc, lds, g, m0, n0);
 }
 
 // ------------------------------------------------------------------------------------------
