@@ -37,13 +37,17 @@ PEAK_MFMA_FP32_TFLOPS = 157.3    # dense fp32 MFMA
 # taken in separate profiling runs, so these are recorded measurements, not live ones; reads that
 # the 256 MB Infinity Cache serves are included.
 MEASURED_TRAFFIC_BYTES = {
-    'c4_linear_fwd': 4331900620,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.09 GiB read, 1.0 GiB written
-    'c2_layer_norm': 387451410,       # norm_fwd + norm_bwd + reduce_partials
-    'c2_rms_norm': 378432107,
-    'c2_softmax': 335719684,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
-    'c3_cross_entropy': 1609265111,   # ce_row_kernel (ignored rows are not read)
-    'c5_conv': 644439252,             # 2 window kernels + weight gradient + 2 layout copies + weight reorders
-    'c5_batch_norm': 616866723,       # stats + apply + backward reduce + backward apply
+    'c4_linear_fwd': 4298750121,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.0 GiB read, 1.0 GiB written
+    'c2_layer_norm': 387451134,       # norm_fwd + norm_bwd + reduce_partials
+    'c2_rms_norm': 378435064,
+    'c2_softmax': 335718756,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
+    'c2_act_dropout': 336050223,      # act_dropout forward + backward
+    'c2_glu': 269041120,              # glu forward + backward
+    'c2_mse': 335722766,              # p_loss forward + backward
+    'c3_cross_entropy': 1610209101,   # ce_row_kernel (ignored rows are not read)
+    'c3_nll_loss': 827006662,         # nll forward (a gather) + the single-pass gradient write
+    'c5_conv': 644303338,             # 2 window kernels + weight gradient + 2 layout copies + weight reorders
+    'c5_batch_norm': 616867814,       # stats + apply + backward reduce + backward apply
 }
 
 
@@ -358,7 +362,7 @@ def bench_rows(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
         oracle.act_dropout_backward(dyc[:crow], xc[:crow], 'geluapprox', None, dropped, 0.1)
 
     traffic_key = {'LayerNorm': 'c2_layer_norm', 'RMSNorm': 'c2_rms_norm', 'Softmax': 'c2_softmax',
-                   'LogSoftmax': 'c2_softmax', 'GELU(tanh)+Dropout(0.1) layer': None}
+                   'LogSoftmax': 'c2_softmax', 'GELU(tanh)+Dropout(0.1) layer': 'c2_act_dropout'}
     for name, f, bwd, cpu in (('LayerNorm', ln_f, ln_b, cpu_ln), ('RMSNorm', rms_f, rms_b, cpu_rms),
                               ('Softmax', sm_f, sm_b, cpu_sm(False)), ('LogSoftmax', lsm_f, lsm_b, cpu_sm(True)),
                               ('GELU(tanh)+Dropout(0.1) layer', act_f, act_b, cpu_act)):
@@ -419,7 +423,8 @@ def bench_rows(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
             'unit': 'GB/s', 'ms_fwd': ms_f, 'ms_bwd': ms_b,
             'fwd_gbs': fwd_units * tbytes / ms_f / 1e6, 'bwd_gbs': bwd_units * tbytes / ms_b / 1e6,
             'roofline': {'bound': 'hbm', 'achieved': gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
-                         'frac': gbs / PEAK_HBM_GBS, 'traffic': None},
+                         'frac': gbs / PEAK_HBM_GBS,
+                         'traffic': MEASURED_TRAFFIC_BYTES['c2_glu' if name.startswith('GLU') else 'c2_mse']},
             'elementwise_reference': stream_ref,
         })
     return results
@@ -504,7 +509,7 @@ def bench_cross_entropy(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
         'metric': 'HBM GB/s', 'value': gbs, 'unit': 'GB/s', 'ms_fwd': ms_f, 'ms_bwd': ms_b,
         'bwd_gbs': tbytes / ms_b / 1e6,
         'roofline': {'bound': 'hbm', 'achieved': gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
-                     'frac': gbs / PEAK_HBM_GBS, 'traffic': None},
+                     'frac': gbs / PEAK_HBM_GBS, 'traffic': MEASURED_TRAFFIC_BYTES['c3_nll_loss']},
     })
     return results
 
