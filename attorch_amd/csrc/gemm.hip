@@ -906,18 +906,56 @@ __global__ __launch_bounds__(256) void act_bwd_kernel(
 }
 
 // Column sums of a [M, N] matrix: partial[slice, n] over a slice of rows, then a fixed-order
-// reduction; grid = (ceil(N / 256), slices).
-template <typename T>
+// reduction.  A workgroup is CT column lanes (8 columns each, one 16-byte load per row) times
+// 256 / CT row lanes that stride the rows of the slice; the row lanes are folded through LDS in
+// a fixed order.  grid = (ceil(N / (8 CT)), slices).
+template <typename T, bool VEC_OK>
 __global__ __launch_bounds__(256) void colsum_partial_kernel(const T* __restrict__ x, float* __restrict__ part,
-                                                            int64_t M, int N, int64_t xs,
-                                                            int64_t rows_per_slice) {
-  const int n = blockIdx.x * 256 + threadIdx.x;
-  if (n >= N) return;
+                                                            int64_t M, int N, int64_t xs, int64_t rows_per_slice,
+                                                            int ct_log2) {
+  constexpr int VEC = 8;
+  __shared__ float sm[256 * VEC];
+  const int CT = 1 << ct_log2, RT = 256 >> ct_log2;
+  const int cx = threadIdx.x & (CT - 1), ry = threadIdx.x >> ct_log2;
+  const int c = (blockIdx.x * CT + cx) * VEC;
   const int64_t r0 = (int64_t)blockIdx.y * rows_per_slice;
   const int64_t r1 = r0 + rows_per_slice < M ? r0 + rows_per_slice : M;
-  float s = 0.f;
-  for (int64_t r = r0; r < r1; ++r) s += to_f32(x[r * xs + n]);
-  part[(int64_t)blockIdx.y * N + n] = s;
+  float s[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) s[j] = 0.f;
+  if (c < N) {
+    auto add_row = [&](int64_t r) {
+      const T* p = x + r * xs + c;
+      float v[VEC];
+      if (VEC_OK) {
+        load_f32<T, VEC>(p, v);
+      } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = c + j < N ? to_f32(p[j]) : 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) s[j] += v[j];
+    };
+    int64_t r = r0 + ry;
+    for (; r + 3 * RT < r1; r += 4 * RT) {   // four independent loads in flight
+      add_row(r);
+      add_row(r + RT);
+      add_row(r + 2 * RT);
+      add_row(r + 3 * RT);
+    }
+    for (; r < r1; r += RT) add_row(r);
+  }
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) sm[(ry * CT + cx) * VEC + j] = s[j];
+  __syncthreads();
+  if (ry == 0 && c < N) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      float t = 0.f;
+      for (int q = 0; q < RT; ++q) t += sm[(q * CT + cx) * VEC + j];
+      if (c + j < N) part[(int64_t)blockIdx.y * N + c + j] = t;
+    }
+  }
 }
 
 // out[n] = sum over slices of part[slice][n], fixed order.  A workgroup owns 16 columns: 4 column
@@ -1112,7 +1150,7 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
   });
 }
 
-constexpr int kColsumSlices = 64;
+constexpr int kColsumSlices = 256;   // at most; fewer when the columns alone fill the GPU
 constexpr int kActBwdMaxSlices = 512;
 
 }  // namespace
@@ -1219,14 +1257,25 @@ int at_colsum(const void* x, void* out, void* workspace, int64_t workspace_bytes
   if (!dtype_valid(x_dtype) || !dtype_valid(out_dtype)) return AT_ERR_DTYPE;
   if (rows <= 0 || cols <= 0 || cols > INT32_MAX || x_stride < cols) return AT_ERR_DIM;
   if (!workspace || workspace_bytes < at_colsum_workspace_bytes(rows, cols)) return AT_ERR_WORKSPACE;
-  int slices = (int)(rows < kColsumSlices ? rows : kColsumSlices);
+  // column lanes: enough for the columns, at most a whole workgroup; slices: about 1024 workgroups
+  int ct_log2 = 0;
+  while (ct_log2 < 8 && ((int64_t)8 << ct_log2) < cols) ++ct_log2;
+  const unsigned gx = (unsigned)cdiv64(cols, (int64_t)8 << ct_log2);
+  int64_t want = cdiv64(1024, gx);
+  if (want < 16) want = 16;
+  if (want > kColsumSlices) want = kColsumSlices;
+  int slices = (int)(rows < want ? rows : want);
   const int64_t rows_per_slice = cdiv64(rows, slices);
   slices = (int)cdiv64(rows, rows_per_slice);
-  const unsigned gx = (unsigned)cdiv64(cols, 256);
+  const bool vec_ok = cols % 8 == 0 && x_stride % 8 == 0 && aligned16(x);
   int rc = dispatch_dtype(x_dtype, [&](auto* tp) -> int {
     typedef std::remove_pointer_t<decltype(tp)> T;
-    hipLaunchKernelGGL((colsum_partial_kernel<T>), dim3(gx, slices), dim3(256), 0, (hipStream_t)stream,
-                       (const T*)x, (float*)workspace, rows, (int)cols, x_stride, rows_per_slice);
+    if (vec_ok)
+      hipLaunchKernelGGL((colsum_partial_kernel<T, true>), dim3(gx, slices), dim3(256), 0, (hipStream_t)stream,
+                         (const T*)x, (float*)workspace, rows, (int)cols, x_stride, rows_per_slice, ct_log2);
+    else
+      hipLaunchKernelGGL((colsum_partial_kernel<T, false>), dim3(gx, slices), dim3(256), 0, (hipStream_t)stream,
+                         (const T*)x, (float*)workspace, rows, (int)cols, x_stride, rows_per_slice, ct_log2);
     return launch_status();
   });
   if (rc) return rc;
