@@ -56,7 +56,9 @@ class NLLLossAutoGrad(torch.autograd.Function):
         _lib.require_gpu(input, 'NLLLoss')
         lib = _lib.load()
         batch_dim, feat_dim = input.shape[:2]
-        spatial_dim = target[0].numel() if target.ndim > 1 else 1
+        spatial_dim = 1
+        for size in target.shape[1:]:
+            spatial_dim *= size
         output_dtype = get_output_dtype(input.dtype, autocast='fp32')
         device = input.device
 

@@ -103,3 +103,5 @@ def test_empty_batch() -> None:
     assert x.grad.shape == (0, 5)
     assert attorch_amd.NLLLoss(reduction='none')(x, target).shape == (0,)
     assert torch.isnan(attorch_amd.NLLLoss(reduction='mean')(x, target))
+    spatial = torch.empty((0, 5, 3), device='cuda')
+    assert attorch_amd.NLLLoss(reduction='none')(spatial, torch.empty((0, 3), dtype=torch.int64, device='cuda')).shape == (0, 3)
