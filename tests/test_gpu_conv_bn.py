@@ -135,6 +135,55 @@ def test_conv_matrix_core_path_agrees_with_generic_kernel(dtype) -> None:
                                     *dims, dt, stream) == -5
 
 
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('n, c, h, w, o, pad, groups, bias', [
+    (44, 64, 56, 56, 64, 1, 1, False),     # the ResNet 3x3 / 64-channel layer, whole 16-byte output segments
+    (40, 64, 57, 59, 96, 1, 1, True),      # odd image (element stores), second channel tile partly empty
+    (44, 128, 56, 56, 128, 1, 2, True),    # two groups of 64 channels
+    (44, 64, 58, 58, 64, 0, 1, False),     # no padding: output smaller than the input
+    (41, 64, 56, 56, 64, 2, 1, False),     # padding wider than the filter reach (forward only)
+])
+def test_conv_window_kernel_agrees_with_generic_kernel_at_size(n, c, h, w, o, pad, groups, bias, dtype) -> None:
+    """
+    ResNet-sized 3x3 layers (hundreds of tiles per CU, image borders, odd images, groups, a partly
+    empty channel tile): the matrix-core window kernel, forward and input gradient, must agree with
+    the generic gather kernel (same C ABI call without workspace) to 16-bit rounding.
+    """
+    from attorch_amd import _lib
+    lib = _lib.load()
+    k = 3
+    oh, ow = h + 2 * pad - k + 1, w + 2 * pad - k + 1
+    dims = (n, c, h, w, o, oh, ow, k, k, 1, 1, pad, pad, groups)
+    dt = _lib.dtype_id(dtype)
+    x = randn((n, c, h, w), 1, dtype).cuda()
+    wt = randn((o, c // groups, k, k), 2, dtype, (c // groups * k * k) ** -0.5).cuda()
+    b = randn((o,), 4, dtype).cuda() if bias else None
+    dy = randn((n, o, oh, ow), 3, dtype).cuda()
+    stream = _lib.stream_of(x)
+    nb_f = lib.at_conv2d_fwd_workspace_bytes(*dims, dt, dt)
+    assert nb_f > 0
+    ws_f = torch.empty(nb_f, dtype=torch.uint8, device='cuda')
+    y_fast = torch.full_like(dy, float('nan'))
+    y_slow = torch.empty_like(dy)
+    _lib.check(lib.at_conv2d_fwd(_lib.ptr(x), _lib.ptr(wt), _lib.ptr(b), _lib.ptr(y_fast), _lib.ptr(ws_f), nb_f,
+                                 *dims, dt, dt, dt, stream), 'fwd')
+    _lib.check(lib.at_conv2d_fwd(_lib.ptr(x), _lib.ptr(wt), _lib.ptr(b), _lib.ptr(y_slow), None, 0,
+                                 *dims, dt, dt, dt, stream), 'fwd')
+    assert_close(y_fast, y_slow.cpu(), dtype, 'output', normalize=True)
+    nb_x = lib.at_conv2d_bwd_input_workspace_bytes(*dims, dt)
+    if pad > k - 1:
+        assert nb_x == 0                    # the input gradient as a convolution needs pad <= k - 1
+        return
+    ws_x = torch.empty(nb_x, dtype=torch.uint8, device='cuda')
+    dx_fast = torch.full_like(x, float('nan'))
+    dx_slow = torch.empty_like(x)
+    _lib.check(lib.at_conv2d_bwd_input(_lib.ptr(dy), None, _lib.ptr(wt), _lib.ptr(dx_fast), _lib.ptr(ws_x), nb_x,
+                                       *dims, dt, stream), 'dx')
+    _lib.check(lib.at_conv2d_bwd_input(_lib.ptr(dy), None, _lib.ptr(wt), _lib.ptr(dx_slow), None, 0,
+                                       *dims, dt, stream), 'dx')
+    assert_close(dx_fast, dx_slow.cpu(), dtype, 'input_grad', normalize=True)
+
+
 BN_SHAPES = [(6, 5), (128, 1024), (2048, 768), (8, 960, 196), (2048, 64, 16), (2, 3, 224, 224),
              (16, 64, 56, 56), (32, 128, 7, 7), (3, 7, 3, 5)]
 
