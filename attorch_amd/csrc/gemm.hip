@@ -1,6 +1,6 @@
 // Linear layer GEMMs: Y = act(X W + b) and the two backward products, fp32 accumulate.
 //
-// Four kernels:
+// Five kernels:
 //  * gemm_mfma16_kernel — bf16/fp16 operands on v_mfma_f32_32x32x16 (MFMA-bound).  256x256x64
 //    macro-tile per 512-lane workgroup (8 waves, 128x64 each, 128 accumulator registers per
 //    lane, two waves per SIMD), LDS double-buffered, one barrier per k-tile.  Tiles go from global memory straight
@@ -19,6 +19,8 @@
 //  * gemm_small16_kernel — bf16/fp16 operands with any strides and extents (16-byte loads where
 //    an operand allows them, element loads otherwise), 64x64 or 128x32 tiles: skinny outputs,
 //    small problems, rows that are not 16-byte aligned.
+//  * gemm_f32_kernel — fp32 operands with 16-byte aligned rows on v_mfma_f32_32x32x2f32: 128x128x16
+//    (or 64x64x16) tiles straight from global memory into LDS, two stages.
 //  * gemm_simple_kernel — fp32 operands, any strides, fp32 MFMA (32x32x2), 64x64x64 tile, next
 //    k-tile prefetched into registers.
 // All fuse bias, the optional pre-activation store and the activation into the epilogue.
@@ -596,6 +598,219 @@ __global__ __launch_bounds__(256) void gemm_split_finish_kernel(const float* __r
 }
 
 // ------------------------------------------------------------------------------------------
+// fp32 operands on v_mfma_f32_32x32x2f32 (MFMA-bound: one MFMA is 64 cycles for 512 bytes of
+// operands, so LDS and the loads have time to spare).  (64 WT) x (64 WT) x 16 tiles, 2x2 waves,
+// tiles straight from global memory into LDS, two stages, one barrier per k-tile.  The MFMA
+// takes one value per lane and operand, so either memory layout is read with plain ds_read_b32:
+//  * rows along the contraction ([outer][k]): 64-byte rows of 16 k, the 16-byte chunk index
+//    XORed with (row / 4) % 4 so that 16 consecutive rows read at one k fall on different banks;
+//  * the other way round ([k][outer]): rows of 64 WT * 4 bytes as loaded, consecutive lanes
+//    read consecutive addresses.
+// ------------------------------------------------------------------------------------------
+constexpr int FK = 16;   // k per tile (the swizzle below is written for 64-byte rows)
+
+template <int WT, bool CONTRACT_CONTIG>
+struct F32Loader {
+  static constexpr int TILE = 64 * WT;
+  static constexpr int kBytes = TILE * FK * 4;
+  static constexpr int kLoads = kBytes / 1024 / 4;   // wave-wide loads per wave
+  i32x4 rsrc;
+  int lane_off, blk_step, k_step, k_lane, K;
+
+  __device__ __forceinline__ void init(const float* base, int64_t ld, int outer0, int outer_total, int K_) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    K = K_;
+    if (CONTRACT_CONTIG) {
+      rsrc = make_buffer_rsrc(base, ((int64_t)(outer_total - 1) * ld + K_) * 4);
+      // a wave-wide load fills 16 rows of 64 bytes: lane -> row lane / 4, position lane % 4
+      const int row = wave * (kLoads * 16) + (lane >> 2);          // + 16 i
+      k_lane = ((lane & 3) ^ ((row >> 2) & 3)) * 4;                // the same for row + 16
+      lane_off = (int)(((int64_t)(outer0 + row) * ld) * 4) + k_lane * 4;
+      blk_step = (int)(16 * ld * 4);
+      k_step = FK * 4;
+    } else {
+      rsrc = make_buffer_rsrc(base, ((int64_t)(K_ - 1) * ld + ((outer_total + 3) & ~3)) * 4);
+      // a wave-wide load fills 1024 / (4 TILE) k-rows: lane -> k-row lane / TILE', 4 columns
+      constexpr int LPR = TILE / 4;                                // lanes per k-row
+      constexpr int RPL = 64 / LPR;                                // k-rows per load
+      const int krow = wave * (kLoads * RPL) + lane / LPR;         // + RPL i
+      k_lane = 0;
+      lane_off = (int)(((int64_t)krow * ld + outer0 + (lane % LPR) * 4) * 4);
+      blk_step = (int)(RPL * ld * 4);
+      k_step = (int)(FK * ld * 4);
+    }
+  }
+  __device__ __forceinline__ void issue(int kt, char* tile) const {
+    const int wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+      int off;
+      if (CONTRACT_CONTIG) off = kt * FK + k_lane < K ? lane_off + i * blk_step + kt * k_step : kOobOffset;
+      else off = lane_off + i * blk_step + kt * k_step;          // k-rows past K fall out of range
+      lds_dma_16(rsrc, off, tile + (wave * kLoads + i) * 1024);
+    }
+  }
+  // value (outer, k) of the tile
+  static __device__ __forceinline__ float read(const char* tile, int outer, int k) {
+    if (CONTRACT_CONTIG)
+      return *reinterpret_cast<const float*>(tile + outer * 64 + ((((k >> 2) ^ (outer >> 2)) & 3) << 4) + (k & 3) * 4);
+    else
+      return *reinterpret_cast<const float*>(tile + k * (TILE * 4) + outer * 4);
+  }
+};
+
+template <int WT, bool A_MC, bool B_KC>
+__global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g) {
+  constexpr int TILE = 64 * WT;
+  constexpr int kTile = TILE * FK * 4, kStage = 2 * kTile;
+  // ring of NS stages, NS - 1 k-tiles of loads in flight: small tiles have little work per k-tile
+  // to cover the load latency with, so they look further ahead
+  constexpr int NS = WT == 1 ? 6 : 3;
+  constexpr int kLoadsPerIter = 2 * (kTile / 1024 / 4);
+  __shared__ __attribute__((aligned(1024))) char lds[NS * kStage];
+  const float* __restrict__ A = reinterpret_cast<const float*>(g.a);
+  const float* __restrict__ B = reinterpret_cast<const float*>(g.b);
+
+  const int nbm = (g.M + TILE - 1) / TILE, nbn = (g.N + TILE - 1) / TILE;
+  const int total = nbm * nbn;
+  int logical;
+  {
+    const int bid = blockIdx.x, xcd = bid & 7, idx = bid >> 3;
+    const int q = total >> 3, rem = total & 7;
+    logical = xcd * q + (xcd < rem ? xcd : rem) + idx;
+  }
+  constexpr int GROUP = 8;
+  const int per_group = GROUP * nbn;
+  const int first_m = (logical / per_group) * GROUP;
+  const int gsz = nbm - first_m < GROUP ? nbm - first_m : GROUP;
+  const int in_group = logical % per_group;
+  const int m0 = (first_m + in_group % gsz) * TILE;
+  const int n0 = (in_group / gsz) * TILE;
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  f32x16 acc[WT][WT];
+#pragma unroll
+  for (int i = 0; i < WT; ++i)
+#pragma unroll
+    for (int j = 0; j < WT; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  F32Loader<WT, !A_MC> la;
+  F32Loader<WT, B_KC> lb;
+  la.init(A, g.lda, m0, g.M, g.K);
+  lb.init(B, g.ldb, n0, g.N, g.K);
+  const int KT = (g.K + FK - 1) / FK;
+  // loads past the last k-tile are issued all the same (they are out of range and write zeros into
+  // stages nobody reads), so the number of loads in flight is the same in every iteration
+#pragma unroll
+  for (int t = 0; t < NS - 1; ++t) {
+    la.issue(t, lds + t * kStage);
+    lb.issue(t, lds + t * kStage + kTile);
+  }
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadsPerIter * (NS - 2)) : "memory");   // k-tile 0 has landed
+  __syncthreads();
+
+  int cur_stage = 0;
+  for (int kt = 0; kt < KT; ++kt) {
+    const char* cur = lds + cur_stage * kStage;
+    {
+      const int fill = cur_stage == 0 ? NS - 1 : cur_stage - 1;   // the stage the previous iteration left
+      la.issue(kt + NS - 1, lds + fill * kStage);
+      lb.issue(kt + NS - 1, lds + fill * kStage + kTile);
+    }
+    cur_stage = cur_stage + 1 == NS ? 0 : cur_stage + 1;
+#pragma unroll
+    for (int ks = 0; ks < FK / 2; ++ks) {
+      const int k = ks * 2 + (lane >> 5);
+      float av[WT], bv[WT];
+#pragma unroll
+      for (int i = 0; i < WT; ++i) {
+        av[i] = F32Loader<WT, !A_MC>::read(cur, wm * 32 * WT + i * 32 + (lane & 31), k);
+        bv[i] = F32Loader<WT, B_KC>::read(cur + kTile, wn * 32 * WT + i * 32 + (lane & 31), k);
+      }
+#pragma unroll
+      for (int i = 0; i < WT; ++i)
+#pragma unroll
+        for (int j = 0; j < WT; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j], av[i], acc[i][j], 0, 0, 0);   // C^T: 4 consecutive n per lane
+    }
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadsPerIter * (NS - 2)) : "memory");   // k-tile kt + 1 has landed
+    __syncthreads();
+  }
+  lds_dma_wait_all();   // the zero-fill loads past the end: the epilogue reuses the stages
+  __syncthreads();
+
+  // Epilogue.  A lane holds, for tile (i, j) and register group rg, C[m][n .. n+3] with
+  //   m = wm*32*WT + i*32 + lane%32,  n = wn*32*WT + j*32 + rg*8 + (lane/32)*4   (tile-local).
+  // Each wave passes its 32 x (32 WT) block of rows through a private piece of LDS and finishes it
+  // in a rolled loop (bias, pre-activation copy, activation chosen at run time, 16-byte stores of
+  // whole row segments), so the activation code exists once instead of once per accumulator.
+  constexpr int W = 32 * WT, kPitch = W + 4;
+  static_assert(4 * 32 * kPitch * 4 <= NS * kStage, "the wave blocks fit in the stages");
+  float* block = reinterpret_cast<float*>(lds) + wave * 32 * kPitch;
+  float* __restrict__ C = reinterpret_cast<float*>(g.c);
+  float* __restrict__ P = g.act != AT_ACT_NONE ? reinterpret_cast<float*>(g.pre_act) : nullptr;
+  const bool vec_c = (g.ldc & 3) == 0 && aligned16_dev(C), vec_p = P && (g.ldp & 3) == 0 && aligned16_dev(P);
+  constexpr int SEGS = W / 4, ROWS_PER_IT = 64 / SEGS;
+  const int seg = lane % SEGS, rsub = lane / SEGS;
+  const int n = n0 + wn * W + seg * 4;
+  float bias4[4] = {0.f, 0.f, 0.f, 0.f};
+  if (g.bias) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (n + e < g.N) bias4[e] = load_scalar_f32(g.bias, g.bias_dt, n + e);
+  }
+#pragma unroll
+  for (int i = 0; i < WT; ++i) {
+#pragma unroll
+    for (int jj = 0; jj < WT; ++jj)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        const f32x16& a = acc[i][jj];
+        *reinterpret_cast<float4*>(block + (lane & 31) * kPitch + jj * 32 + rg * 8 + (lane >> 5) * 4) =
+            make_float4(a[rg * 4 + 0], a[rg * 4 + 1], a[rg * 4 + 2], a[rg * 4 + 3]);
+      }
+    // same wave: LDS operations complete in order; only the compiler has to keep them in place
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll 1
+    for (int it = 0; it < 32 / ROWS_PER_IT; ++it) {
+      const int r = it * ROWS_PER_IT + rsub;
+      const int m = m0 + wm * W + i * 32 + r;
+      const float4 raw = *reinterpret_cast<const float4*>(block + r * kPitch + seg * 4);
+      if (m >= g.M || n >= g.N) continue;
+      float v[4] = {raw.x + bias4[0], raw.y + bias4[1], raw.z + bias4[2], raw.w + bias4[3]};
+      const bool whole = n + 4 <= g.N;
+      if (P) {
+        float* out = P + (int64_t)m * g.ldp + n;
+        if (whole && vec_p) {
+          *reinterpret_cast<float4*>(out) = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < g.N) out[e] = v[e];
+        }
+      }
+      if (g.act != AT_ACT_NONE) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = act_forward(g.act, v[e], g.param);
+      }
+      float* out = C + (int64_t)m * g.ldc + n;
+      if (whole && vec_c) {
+        *reinterpret_cast<float4*>(out) = make_float4(v[0], v[1], v[2], v[3]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (n + e < g.N) out[e] = v[e];
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // Generic kernel for fp32 operands: element strides for both, fp32 MFMA 32x32x2, 64x64x64 tiles.
 // ------------------------------------------------------------------------------------------
 struct SimpleArgs {
@@ -1126,6 +1341,25 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
         return launch_status();
       }
     });
+  }
+
+  // fp32 tensors whose rows allow 16-byte loads: the tiled fp32 MFMA kernel
+  if (in_dt == AT_DTYPE_F32 && out_dt == AT_DTYPE_F32 && aligned16(a) && aligned16(b) && (lda % 4) == 0 &&
+      (ldb % 4) == 0 && (!(a_contig_k || b_contig_k) || (K % 4) == 0) && M >= 32 && N >= 32 &&
+      (a_contig_k ? M : K) * lda * 4 < ((int64_t)1 << 31) && (b_contig_k ? N : K) * ldb * 4 < ((int64_t)1 << 31)) {
+    GemmArgs g{a, b, c, pre_act, bias, (int)M, (int)N, (int)K, lda, ldb, ldc, ldp, act, param, bias_dt, nullptr, 0, 0};
+    // 128x128 tiles once they give every CU a workgroup, 64x64 tiles below that
+    const bool big = cdiv64(M, 128) * cdiv64(N, 128) >= device_cu_count();
+    const unsigned grid = (unsigned)(big ? cdiv64(M, 128) * cdiv64(N, 128) : cdiv64(M, 64) * cdiv64(N, 64));
+#define AT_F32_LAUNCH(WT)                                                                                     \
+  {                                                                                                           \
+    if (layout == kDx) hipLaunchKernelGGL((gemm_f32_kernel<WT, false, true>), dim3(grid), dim3(256), 0, stream, g);       \
+    else if (layout == kDw) hipLaunchKernelGGL((gemm_f32_kernel<WT, true, false>), dim3(grid), dim3(256), 0, stream, g);  \
+    else hipLaunchKernelGGL((gemm_f32_kernel<WT, false, false>), dim3(grid), dim3(256), 0, stream, g);                    \
+  }
+    if (big) AT_F32_LAUNCH(2) else AT_F32_LAUNCH(1)
+#undef AT_F32_LAUNCH
+    return launch_status();
   }
 
   SimpleArgs s{a, b, c, pre_act, bias, (int)M, (int)N, (int)K,
