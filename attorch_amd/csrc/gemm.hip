@@ -810,6 +810,53 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g) {
   }
 }
 
+// Epilogue of the generic kernels: one 32x32 accumulator tile per wave (register r of a lane =
+// C[m = lane % 32][n = (r / 4) * 8 + (lane / 32) * 4 + r % 4]) goes through a wave-private block
+// of LDS (32 rows of 36 floats) and is finished in a rolled loop, so that the run-time activation
+// switch exists once and not once per accumulator register.  `block` must not be in use by
+// anybody else; rows are stored as segments of 4 consecutive columns.
+template <typename TO, typename ARGS>
+__device__ __forceinline__ void wave_tile_epilogue(const f32x16& acc, float* block, const ARGS& g, int m_base,
+                                                   int n_base) {
+  constexpr int kPitch = 36;
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int rg = 0; rg < 4; ++rg)
+    *reinterpret_cast<float4*>(block + (lane & 31) * kPitch + rg * 8 + (lane >> 5) * 4) =
+        make_float4(acc[rg * 4 + 0], acc[rg * 4 + 1], acc[rg * 4 + 2], acc[rg * 4 + 3]);
+  __builtin_amdgcn_wave_barrier();   // same wave: LDS operations complete in order
+  TO* __restrict__ C = reinterpret_cast<TO*>(g.c);
+  TO* __restrict__ P = g.act != AT_ACT_NONE ? reinterpret_cast<TO*>(g.pre_act) : nullptr;
+  const int seg = lane & 7, rsub = lane >> 3;
+  const int n = n_base + seg * 4;
+  float bias4[4] = {0.f, 0.f, 0.f, 0.f};
+  if (g.bias) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (n + e < g.N) bias4[e] = load_scalar_f32(g.bias, g.bias_dt, n + e);
+  }
+#pragma unroll 1
+  for (int it = 0; it < 4; ++it) {
+    const int r = it * 8 + rsub;
+    const int m = m_base + r;
+    const float4 raw = *reinterpret_cast<const float4*>(block + r * kPitch + seg * 4);
+    if (m >= g.M || n >= g.N) continue;
+    float v[4] = {raw.x + bias4[0], raw.y + bias4[1], raw.z + bias4[2], raw.w + bias4[3]};
+    if (P) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (n + e < g.N) P[(int64_t)m * g.ldp + n + e] = from_f32<TO>(v[e]);
+    }
+    if (g.act != AT_ACT_NONE) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = act_forward(g.act, v[e], g.param);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (n + e < g.N) C[(int64_t)m * g.ldc + n + e] = from_f32<TO>(v[e]);
+  }
+}
+
 // ------------------------------------------------------------------------------------------
 // Generic kernel for fp32 operands: element strides for both, fp32 MFMA 32x32x2, 64x64x64 tiles.
 // ------------------------------------------------------------------------------------------
@@ -824,8 +871,10 @@ template <typename TI, typename TO>
 __global__ __launch_bounds__(256) void gemm_simple_kernel(SimpleArgs g) {
   constexpr int TM = 64, TN = 64, TK = 64;
   constexpr int PER = TM * TK / 256;   // elements of each operand tile per lane
-  __shared__ float sa[TK][TM + 1];
-  __shared__ float sb[TK][TN + 1];
+  __shared__ float smem[2][TK][TM + 1];   // A and B tiles; reused by the epilogue
+  float (*sa)[TM + 1] = smem[0];
+  float (*sb)[TN + 1] = smem[1];
+  static_assert(TM == TN, "one array for both tiles");
   const TI* __restrict__ A = reinterpret_cast<const TI*>(g.a);
   const TI* __restrict__ B = reinterpret_cast<const TI*>(g.b);
   const int nbn = (g.N + TN - 1) / TN;
@@ -883,25 +932,9 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(SimpleArgs g) {
     __syncthreads();
   }
 
-  TO* __restrict__ C = reinterpret_cast<TO*>(g.c);
-  TO* __restrict__ P = reinterpret_cast<TO*>(g.pre_act);
-  const int m = m0 + wm * 32 + (lane & 31);
-  if (m >= g.M) return;
-#pragma unroll
-  for (int rg = 0; rg < 4; ++rg) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int n = n0 + wn * 32 + rg * 8 + (lane >> 5) * 4 + e;
-      if (n >= g.N) continue;
-      float v = acc[rg * 4 + e];
-      if (g.bias) v += load_scalar_f32(g.bias, g.bias_dt, n);
-      if (g.act != AT_ACT_NONE) {
-        if (P) P[(int64_t)m * g.ldp + n] = from_f32<TO>(v);
-        v = act_forward(g.act, v, g.param);
-      }
-      C[(int64_t)m * g.ldc + n] = from_f32<TO>(v);
-    }
-  }
+  // the operand tiles are dead (barrier above): 32 x 36 floats of them per wave for the epilogue
+  static_assert(4 * 32 * 36 * 4 <= (int)sizeof(smem), "epilogue blocks fit in the tiles");
+  wave_tile_epilogue<TO>(acc, &smem[0][0][0] + wave * 32 * 36, g, m0 + wm * 32, n0 + wn * 32);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -992,8 +1025,9 @@ template <typename T, typename TO, int WM, int WN>
 __global__ __launch_bounds__(256) void gemm_small16_kernel(SimpleArgs g) {
   static_assert(WM * WN == 4, "four waves");
   constexpr int TM = WM * 32, TN = WN * 32, TK = 64;
-  __shared__ __align__(16) unsigned short sa[TM * kSmallPitch];
-  __shared__ __align__(16) unsigned short sb[TN * kSmallPitch];
+  __shared__ __align__(16) unsigned short smem[(TM + TN) * kSmallPitch];   // A and B tiles; reused by the epilogue
+  unsigned short* const sa = smem;
+  unsigned short* const sb = smem + TM * kSmallPitch;
   const T* A = reinterpret_cast<const T*>(g.a);
   const T* B = reinterpret_cast<const T*>(g.b);
   const int nbn = (g.N + TN - 1) / TN;
@@ -1036,25 +1070,9 @@ __global__ __launch_bounds__(256) void gemm_small16_kernel(SimpleArgs g) {
     __syncthreads();
   }
 
-  TO* __restrict__ C = reinterpret_cast<TO*>(g.c);
-  TO* __restrict__ P = reinterpret_cast<TO*>(g.pre_act);
-  const int m = m0 + wm * 32 + (lane & 31);
-  if (m >= g.M) return;
-#pragma unroll
-  for (int rg = 0; rg < 4; ++rg) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int n = n0 + wn * 32 + rg * 8 + (lane >> 5) * 4 + e;
-      if (n >= g.N) continue;
-      float v = acc[rg * 4 + e];
-      if (g.bias) v += load_scalar_f32(g.bias, g.bias_dt, n);
-      if (g.act != AT_ACT_NONE) {
-        if (P) P[(int64_t)m * g.ldp + n] = from_f32<TO>(v);
-        v = act_forward(g.act, v, g.param);
-      }
-      C[(int64_t)m * g.ldc + n] = from_f32<TO>(v);
-    }
-  }
+  // the operand tiles are dead (barrier above): 32 x 36 floats of them per wave for the epilogue
+  static_assert(4 * 32 * 36 * 4 <= (int)sizeof(smem), "epilogue blocks fit in the tiles");
+  wave_tile_epilogue<TO>(acc, reinterpret_cast<float*>(smem) + wave * 32 * 36, g, m0 + wm * 32, n0 + wn * 32);
 }
 
 // ------------------------------------------------------------------------------------------
