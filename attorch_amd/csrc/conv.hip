@@ -36,6 +36,37 @@ struct ConvArgs {
 
 constexpr int TM = 64, TN = 64, TK = 16;
 
+// A position a * (nb * nc) + b * nc + c, moved forward by a fixed step with two carries.
+struct MixedRadix {
+  int a, b, c;
+  int da, db, dc;
+  __device__ __forceinline__ void init(int64_t pos, int nb, int nc) {
+    c = (int)(pos % nc);
+    const int64_t t = pos / nc;
+    b = (int)(t % nb);
+    a = (int)(t / nb);
+  }
+  __device__ __forceinline__ void set_step(int step, int nb, int nc) {
+    dc = step % nc;
+    const int t = step / nc;
+    db = t % nb;
+    da = t / nb;
+  }
+  __device__ __forceinline__ void advance(int nb, int nc) {
+    c += dc;
+    if (c >= nc) { c -= nc; ++b; }
+    b += db;
+    if (b >= nb) { b -= nb; ++a; }
+    a += da;
+  }
+  __device__ __forceinline__ void next(int nb, int nc) {
+    if (++c >= nc) {
+      c = 0;
+      if (++b >= nb) { b = 0; ++a; }
+    }
+  }
+};
+
 template <int MODE, typename TI, typename TO>
 __global__ __launch_bounds__(256) void conv_gemm_kernel(ConvArgs g) {
   __shared__ float sa[TK][TM + 1];
@@ -56,105 +87,150 @@ __global__ __launch_bounds__(256) void conv_gemm_kernel(ConvArgs g) {
     k_end = k_begin + g.k_per_split < g.K ? k_begin + g.k_per_split : g.K;
   }
 
-  // Per-thread tile coordinates.  For fwd/dx the m index (fast across lanes, contiguous in
-  // memory along the image row) is fixed per thread; its decomposition is hoisted.
-  const int mm_fast = threadIdx.x & 63, kk_slow = threadIdx.x >> 6;   // e = tid + 256 i -> kk = kk_slow + 4 i
-  const int kk_fast = threadIdx.x & 15, xx_slow = threadIdx.x >> 4;   // e = tid + 256 i -> xx = xx_slow + 16 i
+  // Tile elements per thread.  "Gather" operands (the A tile of fwd / dx: contiguous along the image
+  // row, i.e. along m) give a thread one m and four consecutive k; "k-fast" operands (contiguous
+  // along k) give it one k and four rows 16 apart.  The (channel, kh, kw) or (n, oh, ow) split of a
+  // thread's k is carried from k-tile to k-tile by adding the split of TK with two carries
+  // (MixedRadix), so the main loop holds no integer division.
+  const int tid = threadIdx.x;
+  const int m_lane = tid & 63, kq = tid >> 6;
+  const int k_lane = tid & 15, x_lane = tid >> 4;
 
-  int a_n = 0, a_p = 0, a_q = 0;  // (n, oh, ow) for fwd, (n, ih, iw) for dx
+  // fwd / dx gather state
   bool a_row_ok = false;
+  int a_n = 0, a_p = 0, a_q = 0;  // (n, oh, ow) for fwd, (n, ih, iw) for dx
+  int64_t a_base = 0;
+  MixedRadix ga{};                // (channel, kh, kw) of k0 + 4 kq
+  // fwd: k of the B element; dx: (co, tap) of it; dw: (n, oh, ow) of both operands' k
+  int64_t k_cur = k_begin + k_lane;
+  MixedRadix gb{};
+  int dw_c[4] = {0, 0, 0, 0}, dw_kh[4] = {0, 0, 0, 0}, dw_kw[4] = {0, 0, 0, 0};
+  bool dw_ok[4] = {false, false, false, false};
+
   if (MODE != kConvDw) {
-    const int64_t m = m0 + mm_fast;
+    const int64_t m = m0 + m_lane;
     a_row_ok = m < g.M;
     const int pw_ = MODE == kConvFwd ? g.OW : g.W, ph_ = MODE == kConvFwd ? g.OH : g.H;
     const int64_t t = a_row_ok ? m : 0;
     a_q = (int)(t % pw_);
     a_p = (int)((t / pw_) % ph_);
     a_n = (int)(t / ((int64_t)pw_ * ph_));
+    ga.init(k_begin + 4 * kq, g.KH, g.KW);
+    ga.set_step(TK, g.KH, g.KW);
+    if (MODE == kConvFwd) {
+      // X[n, grp*Cg + c, a_p*sh - ph + kh, a_q*sw - pw + kw] = X[a_base + (c*H + kh)*W + kw]
+      a_base = (((int64_t)a_n * g.C + grp * g.Cg) * g.H + (a_p * g.sh - g.ph)) * g.W + (a_q * g.sw - g.pw);
+    } else {
+      gb.init(k_begin + k_lane, 1, KK);
+      gb.set_step(TK, 1, KK);
+    }
+  } else {
+    gb.init(k_begin + k_lane, g.OH, g.OW);
+    gb.set_step(TK, g.OH, g.OW);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int j = n0 + x_lane + 16 * i;
+      dw_ok[i] = j < g.cols;
+      const int jj = dw_ok[i] ? j : 0;
+      const int r = jj % KK;
+      dw_c[i] = jj / KK;
+      dw_kh[i] = r / g.KW;
+      dw_kw[i] = r % g.KW;
+    }
   }
+
+  // Loads one k-tile's elements of both operands into registers and moves the state on by TK.
+  auto fetch = [&](float (&ra)[4], float (&rb)[4]) {
+    if (MODE == kConvFwd) {
+      MixedRadix e = ga;
+      const int ih0 = a_p * g.sh - g.ph, iw0 = a_q * g.sw - g.pw;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v = 0.f;
+        if (a_row_ok && e.a < g.Cg && (unsigned)(ih0 + e.b) < (unsigned)g.H && (unsigned)(iw0 + e.c) < (unsigned)g.W)
+          v = to_f32(A[a_base + ((int64_t)e.a * g.H + e.b) * g.W + e.c]);
+        ra[i] = v;
+        e.next(g.KH, g.KW);
+      }
+      ga.advance(g.KH, g.KW);
+      // B(k, co) = W[co, k], contiguous over k
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int co = n0 + x_lane + 16 * i;
+        rb[i] = (co < g.Og && k_cur < k_end) ? to_f32(B[((int64_t)grp * g.Og + co) * g.K + k_cur]) : 0.f;
+      }
+    } else if (MODE == kConvDx) {
+      MixedRadix e = ga;
+      const int th0 = a_p + g.ph, tw0 = a_q + g.pw;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v = 0.f;
+        int oh = th0 - e.b, ow = tw0 - e.c;
+        bool ok = a_row_ok && e.a < g.Og && oh >= 0 && ow >= 0;
+        if (g.sh != 1) {
+          const int q = oh / g.sh;
+          ok = ok && q * g.sh == oh;
+          oh = q;
+        }
+        if (g.sw != 1) {
+          const int q = ow / g.sw;
+          ok = ok && q * g.sw == ow;
+          ow = q;
+        }
+        if (ok && oh < g.OH && ow < g.OW)
+          v = to_f32(A[(((int64_t)a_n * g.O + grp * g.Og + e.a) * g.OH + oh) * g.OW + ow]);
+        ra[i] = v;
+        e.next(g.KH, g.KW);
+      }
+      ga.advance(g.KH, g.KW);
+      // B(k = (co, tap), c) = W[co, c, tap]
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int c = n0 + x_lane + 16 * i;
+        rb[i] = (c < g.Cg && gb.a < g.Og)
+                    ? to_f32(B[(((int64_t)grp * g.Og + gb.a) * g.Cg + c) * KK + gb.c]) : 0.f;
+      }
+      gb.advance(1, KK);
+    } else {
+      const bool k_ok = k_cur < k_end;
+      // A(co, k) = dY[n, co, oh, ow]
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int co = (int)m0 + x_lane + 16 * i;
+        ra[i] = (k_ok && co < g.Og)
+                    ? to_f32(A[(((int64_t)gb.a * g.O + grp * g.Og + co) * g.OH + gb.b) * g.OW + gb.c]) : 0.f;
+      }
+      // B(k, j = (c, kh, kw)) = X[n, c, oh*s-p+kh, ow*s-p+kw]
+      const int ih0 = gb.b * g.sh - g.ph, iw0 = gb.c * g.sw - g.pw;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int ih = ih0 + dw_kh[i], iw = iw0 + dw_kw[i];
+        float v = 0.f;
+        if (k_ok && dw_ok[i] && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W)
+          v = to_f32(B[(((int64_t)gb.a * g.C + grp * g.Cg + dw_c[i]) * g.H + ih) * g.W + iw]);
+        rb[i] = v;
+      }
+      gb.advance(g.OH, g.OW);
+    }
+    k_cur += TK;
+  };
 
   f32x16 acc;
 #pragma unroll
   for (int e = 0; e < 16; ++e) acc[e] = 0.f;
 
+  float ra[4], rb[4];
+  if (k_begin < k_end) fetch(ra, rb);
   for (int64_t k0 = k_begin; k0 < k_end; k0 += TK) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      // ---- A tile ----
-      if (MODE == kConvFwd) {
-        const int kk = kk_slow + 4 * i;
-        const int64_t k = k0 + kk;
-        float v = 0.f;
-        if (a_row_ok && k < k_end) {
-          const int c = (int)(k / KK), r = (int)(k % KK), kh = r / g.KW, kw = r % g.KW;
-          const int ih = a_p * g.sh - g.ph + kh, iw = a_q * g.sw - g.pw + kw;
-          if (ih >= 0 && ih < g.H && iw >= 0 && iw < g.W)
-            v = to_f32(A[(((int64_t)a_n * g.C + grp * g.Cg + c) * g.H + ih) * g.W + iw]);
-        }
-        sa[kk][mm_fast] = v;
-      } else if (MODE == kConvDx) {
-        const int kk = kk_slow + 4 * i;
-        const int64_t k = k0 + kk;
-        float v = 0.f;
-        if (a_row_ok && k < k_end) {
-          const int co = (int)(k / KK), r = (int)(k % KK), kh = r / g.KW, kw = r % g.KW;
-          const int th = a_p + g.ph - kh, tw = a_q + g.pw - kw;
-          if (th >= 0 && tw >= 0 && th % g.sh == 0 && tw % g.sw == 0) {
-            const int oh = th / g.sh, ow = tw / g.sw;
-            if (oh < g.OH && ow < g.OW)
-              v = to_f32(A[(((int64_t)a_n * g.O + grp * g.Og + co) * g.OH + oh) * g.OW + ow]);
-          }
-        }
-        sa[kk][mm_fast] = v;
-      } else {
-        // dw: A(co, k) = dY[n, co, oh, ow], k = (n, oh, ow) contiguous over (oh, ow)
-        const int kk = kk_fast, mm = xx_slow + 16 * i;
-        const int64_t k = k0 + kk;
-        const int co = (int)m0 + mm;
-        float v = 0.f;
-        if (co < g.Og && k < k_end) {
-          const int64_t hw = (int64_t)g.OH * g.OW;
-          const int64_t n = k / hw, r = k % hw;
-          v = to_f32(A[(n * g.O + grp * g.Og + co) * hw + r]);
-        }
-        sa[kk][mm] = v;
-      }
-      // ---- B tile ----
-      if (MODE == kConvFwd) {
-        // B(k, co) = W[co, k], contiguous over k
-        const int kk = kk_fast, nn = xx_slow + 16 * i;
-        const int64_t k = k0 + kk;
-        const int co = n0 + nn;
-        sb[kk][nn] = (co < g.Og && k < k_end) ? to_f32(B[((int64_t)grp * g.Og + co) * g.K + k]) : 0.f;
-      } else if (MODE == kConvDx) {
-        // B(k = (co, kh, kw), c) = W[co, c, kh, kw]
-        const int kk = kk_fast, nn = xx_slow + 16 * i;
-        const int64_t k = k0 + kk;
-        const int c = n0 + nn;
-        float v = 0.f;
-        if (c < g.Cg && k < k_end) {
-          const int co = (int)(k / KK), r = (int)(k % KK);
-          v = to_f32(B[(((int64_t)grp * g.Og + co) * g.Cg + c) * KK + r]);
-        }
-        sb[kk][nn] = v;
-      } else {
-        // dw: B(k = (n, oh, ow), j = (c, kh, kw)) = X[n, c, oh*s-p+kh, ow*s-p+kw]
-        const int kk = kk_fast, nn = xx_slow + 16 * i;
-        const int64_t k = k0 + kk;
-        const int j = n0 + nn;
-        float v = 0.f;
-        if (j < g.cols && k < k_end) {
-          const int c = j / KK, r = j % KK, kh = r / g.KW, kw = r % g.KW;
-          const int ow = (int)(k % g.OW), oh = (int)((k / g.OW) % g.OH);
-          const int64_t n = k / ((int64_t)g.OW * g.OH);
-          const int ih = oh * g.sh - g.ph + kh, iw = ow * g.sw - g.pw + kw;
-          if (ih >= 0 && ih < g.H && iw >= 0 && iw < g.W)
-            v = to_f32(B[((n * g.C + grp * g.Cg + c) * g.H + ih) * g.W + iw]);
-        }
-        sb[kk][nn] = v;
-      }
+      if (MODE == kConvDw) sa[k_lane][x_lane + 16 * i] = ra[i];
+      else sa[4 * kq + i][m_lane] = ra[i];
+      sb[k_lane][x_lane + 16 * i] = rb[i];
     }
     __syncthreads();
+    // the next tile's loads are in flight while this one is multiplied
+    if (k0 + TK < k_end) fetch(ra, rb);
 #pragma unroll
     for (int ks = 0; ks < TK; ks += 2) {
       const float av = sa[ks + (lane >> 5)][wm * 32 + (lane & 31)];
