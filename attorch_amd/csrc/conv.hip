@@ -276,8 +276,146 @@ __global__ void conv_dw_reduce_kernel(const float* __restrict__ part, TO* __rest
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= total) return;
   float s = 0.f;
+#pragma unroll 8
   for (int p = 0; p < splits; ++p) s += part[(int64_t)p * total + i];
   out[i] = from_f32<TO>(s);
+}
+
+// ------------------------------------------------------------------------------------------
+// Thin groups (depthwise convolutions, pooling written as a convolution, a three-channel input
+// gradient): 64-wide matrix tiles would be mostly padding, so a lane owns one output element and
+// walks the few channels and taps of its group in fp32.
+// ------------------------------------------------------------------------------------------
+constexpr int kThinFeat = 8;         // at most this many output columns of the implicit GEMM
+constexpr int kThinWalkFwd = 512;    // channels x taps walked per output element (fwd, dw)
+constexpr int kThinWalkDx = 4096;    // output channels x taps walked per input-gradient element
+constexpr int kThinTaps = 16;        // taps accumulated at once per lane in the weight gradient
+
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void conv_direct_fwd_kernel(ConvArgs g) {
+  const TI* __restrict__ X = reinterpret_cast<const TI*>(g.a);
+  const TI* __restrict__ Wt = reinterpret_cast<const TI*>(g.b);
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= g.M) return;  // M = N * O * OH * OW
+  const int ow = (int)(idx % g.OW);
+  int64_t t = idx / g.OW;
+  const int oh = (int)(t % g.OH);
+  t /= g.OH;
+  const int co = (int)(t % g.O);
+  const int64_t n = t / g.O;
+  const int grp = co / g.Og;
+  const TI* xg = X + (n * g.C + (int64_t)grp * g.Cg) * g.H * g.W;
+  const TI* wg = Wt + (int64_t)co * g.Cg * g.KH * g.KW;
+  const int ih0 = oh * g.sh - g.ph, iw0 = ow * g.sw - g.pw;
+  float acc = 0.f;
+  for (int c = 0; c < g.Cg; ++c) {
+    for (int kh = 0; kh < g.KH; ++kh) {
+      const int ih = ih0 + kh;
+      if ((unsigned)ih >= (unsigned)g.H) continue;
+      const TI* xr = xg + ((int64_t)c * g.H + ih) * g.W;
+      const TI* wr = wg + (c * g.KH + kh) * g.KW;
+#pragma unroll 4
+      for (int kw = 0; kw < g.KW; ++kw) {
+        const int iw = iw0 + kw;
+        if ((unsigned)iw < (unsigned)g.W) acc = fmaf(to_f32(xr[iw]), to_f32(wr[kw]), acc);
+      }
+    }
+  }
+  if (g.bias) acc += load_scalar_f32(g.bias, g.bias_dt, co);
+  reinterpret_cast<TO*>(g.out)[idx] = from_f32<TO>(acc);
+}
+
+// grid (N * C, cdiv(H * W, 256)): a workgroup stays inside one input-gradient plane, so the
+// Og x KH x KW weights that plane needs are staged in LDS once.
+template <typename T>
+__global__ __launch_bounds__(256) void conv_direct_dx_kernel(ConvArgs g) {
+  __shared__ float wl[kThinWalkDx];
+  const T* __restrict__ dY = reinterpret_cast<const T*>(g.a);
+  const T* __restrict__ Wt = reinterpret_cast<const T*>(g.b);
+  const int c = blockIdx.x % g.C;
+  const int64_t n = blockIdx.x / g.C;
+  const int grp = c / g.Cg, cl = c % g.Cg;
+  const int KK = g.KH * g.KW;
+  for (int i = threadIdx.x; i < g.Og * KK; i += 256) {
+    const int co = i / KK, tap = i % KK;
+    wl[i] = to_f32(Wt[(((int64_t)grp * g.Og + co) * g.Cg + cl) * KK + tap]);
+  }
+  __syncthreads();
+  const int pix = blockIdx.y * 256 + threadIdx.x;
+  if (pix >= g.H * g.W) return;
+  const int ih = pix / g.W, iw = pix % g.W;
+  const int64_t plane = (int64_t)g.OH * g.OW;
+  const T* dyg = dY + (n * g.O + (int64_t)grp * g.Og) * plane;
+  float acc = 0.f;
+  // only the taps kh = (ih + ph) mod sh, + sh, ... reach an output row, which then steps down by one
+  const int th = ih + g.ph, tw = iw + g.pw;
+  const int kh0 = th % g.sh, kw0 = tw % g.sw, oh0 = th / g.sh, ow0 = tw / g.sw;
+  for (int kh = kh0, oh = oh0; kh < g.KH && oh >= 0; kh += g.sh, --oh) {
+    if (oh >= g.OH) continue;
+    for (int kw = kw0, ow = ow0; kw < g.KW && ow >= 0; kw += g.sw, --ow) {
+      if (ow >= g.OW) continue;
+      const T* dyp = dyg + (int64_t)oh * g.OW + ow;
+      const float* wp = wl + kh * g.KW + kw;
+      // independent loads in flight together: one at a time the walk is bound by memory latency
+#pragma unroll 8
+      for (int co = 0; co < g.Og; ++co) acc = fmaf(to_f32(dyp[co * plane]), wp[co * KK], acc);
+    }
+  }
+  reinterpret_cast<T*>(g.out)[((n * g.C + c) * g.H) * g.W + pix] = from_f32<T>(acc);
+}
+
+// grid (O * Cg, splits): a workgroup sums one filter plane dW[co, c, :, :] over its share of the
+// batch x space positions and writes the fp32 partial [split][O][Cg * KH * KW].
+template <typename T>
+__global__ __launch_bounds__(256) void conv_direct_dw_kernel(ConvArgs g) {
+  __shared__ float fold[4][kThinTaps];
+  const T* __restrict__ dY = reinterpret_cast<const T*>(g.a);
+  const T* __restrict__ X = reinterpret_cast<const T*>(g.b);
+  float* __restrict__ part = reinterpret_cast<float*>(g.out);
+  const int co = blockIdx.x / g.Cg, cl = blockIdx.x % g.Cg;
+  const int c = (co / g.Og) * g.Cg + cl;
+  const int KK = g.KH * g.KW;
+  const int64_t p_begin = (int64_t)blockIdx.y * g.k_per_split;
+  const int64_t p_end = p_begin + g.k_per_split < g.K ? p_begin + g.k_per_split : g.K;  // K = N * OH * OW
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float* out = part + (((int64_t)blockIdx.y * g.O + co) * g.Cg + cl) * KK;
+
+  for (int t0 = 0; t0 < KK; t0 += kThinTaps) {
+    int tkh[kThinTaps], tkw[kThinTaps];
+#pragma unroll
+    for (int j = 0; j < kThinTaps; ++j) {
+      const int tap = t0 + j < KK ? t0 + j : 0;
+      tkh[j] = tap / g.KW;
+      tkw[j] = tap % g.KW;
+    }
+    float acc[kThinTaps];
+#pragma unroll
+    for (int j = 0; j < kThinTaps; ++j) acc[j] = 0.f;
+    for (int64_t p = p_begin + threadIdx.x; p < p_end; p += 256) {
+      const int ow = (int)(p % g.OW);
+      const int64_t q = p / g.OW;
+      const int oh = (int)(q % g.OH);
+      const int64_t n = q / g.OH;
+      const float dv = to_f32(dY[((n * g.O + co) * g.OH + oh) * g.OW + ow]);
+      const T* xp = X + (n * g.C + c) * g.H * g.W;
+      const int ih0 = oh * g.sh - g.ph, iw0 = ow * g.sw - g.pw;
+#pragma unroll
+      for (int j = 0; j < kThinTaps; ++j) {
+        const int ih = ih0 + tkh[j], iw = iw0 + tkw[j];
+        if (t0 + j < KK && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W)
+          acc[j] = fmaf(dv, to_f32(xp[(int64_t)ih * g.W + iw]), acc[j]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kThinTaps; ++j) {
+      const float v = wave_reduce(acc[j], kWave, SumOp());
+      if (lane == 0) fold[wave][j] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x < kThinTaps && t0 + threadIdx.x < KK)
+      out[t0 + threadIdx.x] = (fold[0][threadIdx.x] + fold[1][threadIdx.x]) + (fold[2][threadIdx.x] + fold[3][threadIdx.x]);
+    __syncthreads();
+  }
 }
 
 // Per-channel sum over batch and space of a [N, C, S] tensor (bias gradient).
@@ -395,6 +533,19 @@ int at_conv2d_fwd(const void* input, const void* weight, const void* bias, void*
   ConvArgs g = base_args(s);
   g.a = input; g.b = weight; g.out = output; g.bias = bias; g.bias_dt = bias_dtype;
   g.M = s.N * s.OH * s.OW; g.K = (int64_t)g.Cg * g.KH * g.KW; g.cols = g.Og;
+  if (g.Og <= kThinFeat && g.K <= kThinWalkFwd) {
+    g.M = s.N * s.O * s.OH * s.OW;
+    if (cdiv64(g.M, 256) > INT32_MAX) return AT_ERR_DIM;
+    return dispatch_dtype(in_dtype, [&](auto* ti) -> int {
+      typedef std::remove_pointer_t<decltype(ti)> TI;
+      return dispatch_dtype(out_dtype, [&](auto* to) -> int {
+        typedef std::remove_pointer_t<decltype(to)> TO;
+        hipLaunchKernelGGL((conv_direct_fwd_kernel<TI, TO>), dim3((unsigned)cdiv64(g.M, 256)), dim3(256), 0,
+                           (hipStream_t)stream, g);
+        return launch_status();
+      });
+    });
+  }
   const dim3 grid((unsigned)(cdiv64(g.M, TM) * cdiv64(g.cols, TN)), 1, (unsigned)g.groups);
   return dispatch_dtype(in_dtype, [&](auto* ti) -> int {
     typedef std::remove_pointer_t<decltype(ti)> TI;
@@ -438,6 +589,15 @@ int at_conv2d_bwd_input(const void* output_grad, const void* output_grad_nhwc, c
   ConvArgs g = base_args(s);
   g.a = output_grad; g.b = weight; g.out = input_grad;
   g.M = s.N * s.H * s.W; g.K = (int64_t)g.Og * g.KH * g.KW; g.cols = g.Cg;
+  if (g.Cg <= kThinFeat && g.K <= kThinWalkDx) {
+    if (s.N * s.C > INT32_MAX || s.H * s.W > (int64_t)65535 * 256) return AT_ERR_DIM;
+    return dispatch_dtype(dtype, [&](auto* tp) -> int {
+      typedef std::remove_pointer_t<decltype(tp)> T;
+      hipLaunchKernelGGL((conv_direct_dx_kernel<T>), dim3((unsigned)(s.N * s.C), (unsigned)cdiv64(s.H * s.W, 256)),
+                         dim3(256), 0, (hipStream_t)stream, g);
+      return launch_status();
+    });
+  }
   const dim3 grid((unsigned)(cdiv64(g.M, TM) * cdiv64(g.cols, TN)), 1, (unsigned)g.groups);
   return dispatch_dtype(dtype, [&](auto* tp) -> int {
     typedef std::remove_pointer_t<decltype(tp)> T;
@@ -480,8 +640,31 @@ int at_conv2d_bwd_weight(const void* output_grad, const void* output_grad_nhwc, 
                            (hipStream_t)stream);
   }
   ConvArgs g = base_args(s);
-  const int splits = dw_splits(s);
   const int64_t total = s.O * g.Cg * s.KH * s.KW;
+  if (g.Og <= kThinFeat && g.Cg <= kThinFeat && (int64_t)g.Cg * g.KH * g.KW <= kThinWalkFwd) {
+    // one workgroup per filter plane and slice of the batch x space positions
+    const int64_t positions = s.N * s.OH * s.OW, planes = s.O * g.Cg;
+    int64_t want = cdiv64((int64_t)device_cu_count() * 4, planes);
+    const int64_t by_work = cdiv64(positions, 1024);
+    if (want > by_work) want = by_work;
+    if (want > kDwMaxSplits) want = kDwMaxSplits;
+    if (want < 1) want = 1;
+    g.k_per_split = cdiv64(positions, want);
+    const int thin_splits = (int)cdiv64(positions, g.k_per_split);
+    if (!workspace || workspace_bytes < (int64_t)thin_splits * total * (int64_t)sizeof(float)) return AT_ERR_WORKSPACE;
+    g.a = output_grad; g.b = input; g.out = workspace; g.K = positions;
+    return dispatch_dtype(dtype, [&](auto* tp) -> int {
+      typedef std::remove_pointer_t<decltype(tp)> T;
+      hipLaunchKernelGGL((conv_direct_dw_kernel<T>), dim3((unsigned)planes, (unsigned)thin_splits), dim3(256), 0,
+                         (hipStream_t)stream, g);
+      int rc2 = launch_status();
+      if (rc2) return rc2;
+      hipLaunchKernelGGL((conv_dw_reduce_kernel<T>), dim3((unsigned)cdiv64(total, 256)), dim3(256), 0,
+                         (hipStream_t)stream, (const float*)workspace, (T*)weight_grad, thin_splits, total);
+      return launch_status();
+    });
+  }
+  const int splits = dw_splits(s);
   if (!workspace || workspace_bytes < (int64_t)splits * total * (int64_t)sizeof(float)) return AT_ERR_WORKSPACE;
   g.a = output_grad; g.b = input; g.out = workspace;
   g.M = g.Og; g.K = s.N * s.OH * s.OW; g.cols = g.Cg * g.KH * g.KW;

@@ -31,6 +31,13 @@ CONV_CASES = [
     ((2, 128, 9, 8), 64, (1, 1), (1, 1), (0, 0), 1),
     ((1, 64, 12, 10), 64, (5, 3), (1, 1), (2, 0), 1),
     ((5, 64, 20, 24), 64, (3, 3), (1, 1), (1, 1), 1),
+    # thin groups take the direct kernels: depthwise with a channel multiplier and more taps than
+    # one accumulation pass holds, a pooling-shaped depthwise layer, a three-channel stem (input
+    # gradient only), and few output channels without groups
+    ((3, 12, 17, 15), 24, (5, 5), (2, 1), (2, 2), 12),
+    ((4, 32, 30, 30), 32, (2, 2), (2, 2), (0, 0), 32),
+    ((2, 3, 20, 20), 40, (7, 7), (2, 2), (3, 3), 1),
+    ((2, 20, 13, 13), 6, (3, 3), (1, 1), (1, 1), 1),
 ]
 
 
