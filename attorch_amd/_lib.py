@@ -144,3 +144,15 @@ def rows(tensor: Tensor) -> Tensor:
     if tensor.stride(-1) != 1 or (tensor.shape[0] > 1 and tensor.stride(0) < tensor.shape[1]):
         tensor = tensor.contiguous()
     return tensor
+
+
+def row_stride(tensor: Tensor) -> int:
+    """
+    Row stride of a [rows, feat] matrix in elements, as the kernels expect it.  PyTorch leaves
+    the stride of an extent-1 dimension arbitrary (a [1, feat] or [feat, 1].T tensor counts as
+    contiguous whatever stride(0) says), so a single row reports its extent instead.
+    """
+    if tensor.shape[0] <= 1:
+        return max(int(tensor.shape[1]), 1)
+    return int(tensor.stride(0))
+

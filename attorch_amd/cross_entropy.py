@@ -65,7 +65,7 @@ class CrossEntropyLossAutoGrad(torch.autograd.Function):
             _lib.check(lib.at_cross_entropy_fwd_bwd(
                 _lib.ptr(logits), _lib.ptr(target_k), _lib.ptr(weight_k), _lib.ptr(output),
                 _lib.ptr(input_grad), _lib.ptr(workspace), workspace_bytes, batch_dim, feat_dim,
-                logits.stride(0), feat_dim, ignore_index, _lib.dtype_id(logits.dtype),
+                _lib.row_stride(logits), feat_dim, ignore_index, _lib.dtype_id(logits.dtype),
                 _lib.dtype_id(weight_k.dtype) if weight_k is not None else 0,
                 _lib.dtype_id(output_dtype), _lib.stream_of(input)), 'at_cross_entropy_fwd_bwd')
 
@@ -94,7 +94,7 @@ class CrossEntropyLossAutoGrad(torch.autograd.Function):
         with torch.cuda.device_of(input_grad):
             _lib.check(lib.at_cross_entropy_scale_grad(
                 _lib.ptr(input_grad), _lib.ptr(output_grad), batch_dim, feat_dim,
-                input_grad.stride(0), _lib.dtype_id(input_grad.dtype),
+                _lib.row_stride(input_grad), _lib.dtype_id(input_grad.dtype),
                 _lib.dtype_id(output_grad.dtype), _lib.stream_of(input_grad)),
                 'at_cross_entropy_scale_grad')
 

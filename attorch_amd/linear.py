@@ -135,8 +135,8 @@ class LinearAutoGrad(torch.autograd.Function):
         with torch.cuda.device_of(input):
             _lib.check(lib.at_linear_fwd(
                 _lib.ptr(input_k), _lib.ptr(weight_k), _lib.ptr(bias_k), _lib.ptr(pre_act),
-                _lib.ptr(output), batch_dim, contract_dim, out_feat_dim, input_k.stride(0),
-                weight_k.stride(0), pre_act.stride(0), output.stride(0), act,
+                _lib.ptr(output), batch_dim, contract_dim, out_feat_dim, _lib.row_stride(input_k),
+                _lib.row_stride(weight_k), _lib.row_stride(pre_act), _lib.row_stride(output), act,
                 0.0 if param is None else param, _lib.dtype_id(compute_dtype),
                 _lib.dtype_id(bias_k.dtype) if bias_k is not None else 0,
                 _lib.dtype_id(output_dtype), _lib.stream_of(input)), 'at_linear_fwd')
@@ -187,8 +187,8 @@ class LinearAutoGrad(torch.autograd.Function):
                 _lib.check(lib.at_act_bwd(
                     _lib.ptr(output_grad), _lib.ptr(pre_act), _lib.ptr(pre_act_grad),
                     _lib.ptr(bias_grad), _lib.ptr(workspace), workspace_bytes or 0,
-                    batch_dim, out_feat_dim, output_grad.stride(0), pre_act.stride(0),
-                    pre_act_grad.stride(0), ctx.act, 0.0 if ctx.param is None else ctx.param,
+                    batch_dim, out_feat_dim, _lib.row_stride(output_grad), _lib.row_stride(pre_act),
+                    _lib.row_stride(pre_act_grad), ctx.act, 0.0 if ctx.param is None else ctx.param,
                     _lib.dtype_id(output_grad.dtype), _lib.dtype_id(pre_act.dtype),
                     _lib.dtype_id(pre_act.dtype), stream), 'at_act_bwd')
 
@@ -208,8 +208,8 @@ class LinearAutoGrad(torch.autograd.Function):
                 input_grad = torch.empty((batch_dim, in_feat_dim), dtype=output_dtype, device=device)
                 _lib.check(lib.at_linear_bwd_input(
                     _lib.ptr(grad_mm), _lib.ptr(weight_mm), _lib.ptr(input_grad), batch_dim,
-                    in_feat_dim, contract_dim, grad_mm.stride(0), weight_mm.stride(0),
-                    input_grad.stride(0), _lib.dtype_id(output_dtype),
+                    in_feat_dim, contract_dim, _lib.row_stride(grad_mm), _lib.row_stride(weight_mm),
+                    _lib.row_stride(input_grad), _lib.dtype_id(output_dtype),
                     _lib.dtype_id(output_dtype), stream), 'at_linear_bwd_input')
                 input_grad = input_grad.view_as(input)
             if weight.requires_grad:
@@ -228,8 +228,8 @@ class LinearAutoGrad(torch.autograd.Function):
                     _lib.check(lib.at_linear_bwd_weight(
                         _lib.ptr(input_mm), _lib.ptr(grad_mm), _lib.ptr(weight_grad),
                         _lib.ptr(workspace), workspace_bytes, batch_dim,
-                        in_feat_dim, out_feat_dim, input_mm.stride(0), grad_mm.stride(0),
-                        weight_grad.stride(0), _lib.dtype_id(output_dtype),
+                        in_feat_dim, out_feat_dim, _lib.row_stride(input_mm), _lib.row_stride(grad_mm),
+                        _lib.row_stride(weight_grad), _lib.dtype_id(output_dtype),
                         _lib.dtype_id(output_dtype), stream), 'at_linear_bwd_weight')
             if ctx.bias_requires_grad and bias_grad is None:
                 bias_grad = torch.empty(out_feat_dim, dtype=pre_act_grad.dtype, device=device)
@@ -240,7 +240,7 @@ class LinearAutoGrad(torch.autograd.Function):
                     workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=device)
                     _lib.check(lib.at_colsum(
                         _lib.ptr(pre_act_grad), _lib.ptr(bias_grad), _lib.ptr(workspace),
-                        workspace_bytes, batch_dim, out_feat_dim, pre_act_grad.stride(0),
+                        workspace_bytes, batch_dim, out_feat_dim, _lib.row_stride(pre_act_grad),
                         _lib.dtype_id(pre_act_grad.dtype), _lib.dtype_id(bias_grad.dtype), stream),
                         'at_colsum')
 

@@ -84,7 +84,7 @@ class LayerNormAutoGrad(torch.autograd.Function):
             _lib.check(lib.at_layer_norm_fwd(
                 _lib.ptr(flattened_input), _lib.ptr(weight_k), _lib.ptr(bias_k),
                 _lib.ptr(mean), _lib.ptr(inv_std), _lib.ptr(output),
-                batch_dim, feat_dim, flattened_input.stride(0), output.stride(0), eps,
+                batch_dim, feat_dim, _lib.row_stride(flattened_input), _lib.row_stride(output), eps,
                 _lib.dtype_id(input.dtype),
                 _lib.dtype_id(weight_k.dtype) if scale_by_weight else 0,
                 _lib.dtype_id(output_dtype), _lib.stream_of(input)), 'at_layer_norm_fwd')
@@ -133,7 +133,8 @@ class LayerNormAutoGrad(torch.autograd.Function):
                 _lib.ptr(mean), _lib.ptr(inv_std), _lib.ptr(weight_k),
                 _lib.ptr(input_grad), _lib.ptr(weight_grad), _lib.ptr(bias_grad),
                 _lib.ptr(workspace), workspace_bytes, batch_dim, feat_dim,
-                flattened_output_grad.stride(0), flattened_input.stride(0), input_grad.stride(0),
+                _lib.row_stride(flattened_output_grad), _lib.row_stride(flattened_input),
+                _lib.row_stride(input_grad),
                 _lib.dtype_id(flattened_output_grad.dtype), _lib.dtype_id(flattened_input.dtype),
                 _lib.dtype_id(weight_k.dtype) if scale_by_weight else 0,
                 _lib.dtype_id(input_grad.dtype), _lib.stream_of(flattened_input)),
@@ -220,7 +221,7 @@ class RMSNormAutoGrad(torch.autograd.Function):
         with torch.cuda.device_of(input):
             _lib.check(lib.at_rms_norm_fwd(
                 _lib.ptr(flattened_input), _lib.ptr(weight_k), _lib.ptr(inv_rms), _lib.ptr(output),
-                batch_dim, feat_dim, flattened_input.stride(0), output.stride(0), eps,
+                batch_dim, feat_dim, _lib.row_stride(flattened_input), _lib.row_stride(output), eps,
                 _lib.dtype_id(input.dtype),
                 _lib.dtype_id(weight_k.dtype) if scale_by_weight else 0,
                 _lib.dtype_id(output.dtype), _lib.stream_of(input)), 'at_rms_norm_fwd')
@@ -263,7 +264,8 @@ class RMSNormAutoGrad(torch.autograd.Function):
                 _lib.ptr(flattened_output_grad), _lib.ptr(flattened_input), _lib.ptr(inv_rms),
                 _lib.ptr(weight_k), _lib.ptr(input_grad), _lib.ptr(weight_grad),
                 _lib.ptr(workspace), workspace_bytes, batch_dim, feat_dim,
-                flattened_output_grad.stride(0), flattened_input.stride(0), input_grad.stride(0),
+                _lib.row_stride(flattened_output_grad), _lib.row_stride(flattened_input),
+                _lib.row_stride(input_grad),
                 _lib.dtype_id(flattened_output_grad.dtype), _lib.dtype_id(flattened_input.dtype),
                 _lib.dtype_id(weight_k.dtype) if scale_by_weight else 0,
                 _lib.dtype_id(input_grad.dtype), _lib.stream_of(flattened_input)),

@@ -49,7 +49,7 @@ class SoftmaxAutoGrad(torch.autograd.Function):
         with torch.cuda.device_of(input):
             _lib.check(lib.at_softmax_fwd(
                 _lib.ptr(flattened_input), _lib.ptr(output), batch_dim, feat_dim,
-                flattened_input.stride(0), output.stride(0), int(neg), int(log),
+                _lib.row_stride(flattened_input), _lib.row_stride(output), int(neg), int(log),
                 _lib.dtype_id(input.dtype), _lib.dtype_id(output_dtype),
                 _lib.stream_of(input)), 'at_softmax_fwd')
 
@@ -77,8 +77,8 @@ class SoftmaxAutoGrad(torch.autograd.Function):
         with torch.cuda.device_of(output):
             _lib.check(lib.at_softmax_bwd(
                 _lib.ptr(flattened_output_grad), _lib.ptr(output), _lib.ptr(input_grad),
-                batch_dim, feat_dim, flattened_output_grad.stride(0), output.stride(0),
-                input_grad.stride(0), int(ctx.neg), int(ctx.log),
+                batch_dim, feat_dim, _lib.row_stride(flattened_output_grad), _lib.row_stride(output),
+                _lib.row_stride(input_grad), int(ctx.neg), int(ctx.log),
                 _lib.dtype_id(flattened_output_grad.dtype), _lib.dtype_id(output.dtype),
                 _lib.dtype_id(input_grad.dtype), _lib.stream_of(output)), 'at_softmax_bwd')
 

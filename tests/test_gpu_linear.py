@@ -147,3 +147,37 @@ def test_weight_grad_split_agrees_with_one_piece(batch, in_dim, out_dim, dtype) 
         _lib.ptr(x), _lib.ptr(dz), _lib.ptr(dw), _lib.ptr(tiny), 16, batch, in_dim, out_dim, in_dim, out_dim,
         out_dim, did, did, stream), 'at_linear_bwd_weight')
     torch.testing.assert_close(dw.double().cpu(), results[0], rtol=0, atol=0)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+def test_extent_one_dimensions_with_arbitrary_strides(dtype) -> None:
+    """
+    PyTorch leaves the stride of an extent-1 dimension arbitrary: the [1, out] weight of a layer
+    with one input feature is a transposed [out, 1] tensor whose stride(0) is 1, and a [feat, 1]
+    tensor transposed to one row of feat elements reports a row stride of 1 as well.
+    """
+    lin = attorch_amd.Linear(1, 63, device='cuda', dtype=dtype)
+    assert tuple(lin.weight.shape) == (1, 63) and lin.weight.stride(0) < 63
+    x = randn((2048, 1), 1, dtype).cuda().requires_grad_(True)
+    dy = randn((2048, 63), 2, dtype).cuda()
+    y = lin(x)
+    y.backward(dy)
+    w, b = lin.weight.detach().double(), lin.bias.detach().double()
+    assert_close(y, x.detach().double() @ w + b, dtype, 'output')
+    assert_close(x.grad, dy.double() @ w.T, dtype, 'input_grad', normalize=True)
+    assert_close(lin.weight.grad, x.detach().double().T @ dy.double(), dtype, 'weight_grad', normalize=True)
+    assert_close(lin.bias.grad, dy.double().sum(0), dtype, 'bias_grad', normalize=True)
+
+    row = randn((300, 1), 3, dtype).cuda().T            # one row of 300 elements, stride(0) == 1
+    assert tuple(row.shape) == (1, 300) and row.stride(0) == 1
+    row.requires_grad_(True)
+    out = attorch_amd.Softmax(dim=-1)(row)
+    out.backward(torch.ones_like(out) * torch.arange(300, device='cuda', dtype=dtype))
+    ref_in = row.detach().double().requires_grad_(True)
+    ref = torch.softmax(ref_in, dim=-1)
+    ref.backward(torch.arange(300, device='cuda', dtype=dtype).double().expand(1, 300))
+    assert_close(out, ref, dtype, 'softmax of one strided row')
+    assert_close(row.grad, ref_in.grad, dtype, 'softmax input_grad', normalize=True)
+    norm = attorch_amd.LayerNorm(300, device='cuda', dtype=dtype)
+    assert_close(norm(row), torch.nn.functional.layer_norm(row.detach().double(), (300,), norm.weight.double(),
+                                                           norm.bias.double(), norm.eps), dtype, 'layer norm')
