@@ -240,6 +240,39 @@ def test_batch_norm_training(shape, dtype, affine, residual, act_func) -> None:
         assert_close(rd.grad, dres_ref, dtype, 'residual_grad')
 
 
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('act_func', [None, 'relu'])
+def test_batch_norm_eval_backward_follows_the_reference(act_func, dtype) -> None:
+    """
+    In eval mode the reference's backward (batch_norm_layer.py:191-245, no is_train argument)
+    still applies the batch-statistics formula, with the running statistics in the place of the
+    batch ones; torch treats them as constants.  The kernels keep the reference's result.
+    """
+    shape, feat = (6, 10, 7, 5), 10
+    x, w, b = randn(shape, 1, dtype), randn((feat,), 2, dtype), randn((feat,), 3, dtype)
+    res, dy = randn(shape, 4, dtype), randn(shape, 5, dtype)
+    running_mean, running_var = randn((feat,), 6) * 0.1, randn((feat,), 7).abs() + 0.5
+    cd = compute_dtype(dtype)
+    name, param = oracle.parse_act_func(act_func)
+    y_ref, _, mean, inv_std, rm_ref, rv_ref = oracle.batch_norm_forward(
+        x, False, w, b, running_mean, running_var, 0.1, 1e-5, True, res, name, param, compute=cd)
+    xd, rd = x.cuda().requires_grad_(True), res.cuda().requires_grad_(True)
+    wd, bd = w.cuda().requires_grad_(True), b.cuda().requires_grad_(True)
+    rm, rv = running_mean.cuda(), running_var.cuda()
+    y = attorch_amd.BatchNormAutoGrad.apply(xd, False, wd, bd, rm, rv, 0.1, 1e-5, True, rd, act_func)
+    saved = [None if t is None else t.detach().cpu() for t in y.grad_fn.saved_tensors]
+    y.backward(dy.cuda())
+    assert_close(y, y_ref, dtype, 'output')
+    torch.testing.assert_close(rm.cpu(), running_mean), torch.testing.assert_close(rv.cpu(), running_var)
+    assert_close(saved[1], running_mean, torch.float32, 'saved mean = running mean')
+    dx_ref, dw_ref, db_ref, dres_ref = oracle.batch_norm_backward(
+        dy, x, saved[1], saved[2], w, True, saved[4] if name is not None else None, name, param, compute=cd)
+    assert_close(xd.grad, dx_ref, dtype, 'input_grad', normalize=True)
+    assert_close(wd.grad, dw_ref.to(dtype), dtype, 'weight_grad', normalize=True)
+    assert_close(bd.grad, db_ref.to(dtype), dtype, 'bias_grad', normalize=True)
+    assert_close(rd.grad, dres_ref, dtype, 'residual_grad')
+
+
 @pytest.mark.parametrize('track_running_stats', [False, True])
 def test_batch_norm_modules_train_then_eval(track_running_stats) -> None:
     torch.manual_seed(0)
