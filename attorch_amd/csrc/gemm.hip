@@ -18,7 +18,10 @@
 //    gemm_split_finish_kernel adds up in a fixed order.
 //  * gemm_small16_kernel — bf16/fp16 operands with any strides and extents (16-byte loads where
 //    an operand allows them, element loads otherwise), 64x64 or 128x32 tiles: skinny outputs,
-//    small problems, rows that are not 16-byte aligned.
+//    small problems, rows that are not 16-byte aligned; 32x32 tiles with the contraction split
+//    over the four waves when the larger tiles would leave most CUs idle.
+//  * gemm_skinny.h — at most 16 output features (classifier heads): vector-ALU kernels bound by
+//    one pass over the wide operand.
 //  * gemm_f32_kernel — fp32 operands with 16-byte aligned rows on v_mfma_f32_32x32x2f32: 128x128x16
 //    (or 64x64x16) tiles straight from global memory into LDS, two stages.
 //  * gemm_simple_kernel — fp32 operands, any strides, fp32 MFMA (32x32x2), 64x64x64 tile, next
@@ -28,6 +31,7 @@
 
 #include "at_act.h"
 #include "at_mfma.h"
+#include "gemm_skinny.h"
 
 namespace at_hip {
 namespace {
@@ -581,6 +585,7 @@ __global__ __launch_bounds__(256) void gemm_split_finish_kernel(const float* __r
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
   const float* src = partial + (int64_t)m * ldw + n;
+#pragma unroll 4
   for (int sidx = 0; sidx < splits; ++sidx) {
     const float4 lo = *reinterpret_cast<const float4*>(src), hi = *reinterpret_cast<const float4*>(src + 4);
     acc[0] += lo.x; acc[1] += lo.y; acc[2] += lo.z; acc[3] += lo.w;
@@ -1021,11 +1026,17 @@ struct SmallTile {   // R outer rows (m or n) x 64 k of one operand
   }
 };
 
-template <typename T, typename TO, int WM, int WN>
+// KSPLIT: the four waves share one 32x32 output tile and each multiplies a quarter of every
+// k-tile; their accumulators are added through LDS at the end.  Four times the workgroups of the
+// 64x64 arrangement, for outputs too small to occupy the GPU otherwise (a 10-class head).
+template <typename T, typename TO, int WM, int WN, bool KSPLIT = false>
 __global__ __launch_bounds__(256) void gemm_small16_kernel(SimpleArgs g) {
-  static_assert(WM * WN == 4, "four waves");
+  static_assert(KSPLIT ? (WM == 1 && WN == 1) : WM * WN == 4, "four waves");
   constexpr int TM = WM * 32, TN = WN * 32, TK = 64;
-  __shared__ __align__(16) unsigned short smem[(TM + TN) * kSmallPitch];   // A and B tiles; reused by the epilogue
+  constexpr int kTileShorts = (TM + TN) * kSmallPitch;
+  constexpr int kFoldShorts = KSPLIT ? 4 * 64 * 16 * 2 : 0;   // four waves x 16 fp32 registers per lane
+  // A and B tiles; reused by the epilogue
+  __shared__ __align__(16) unsigned short smem[kTileShorts > kFoldShorts ? kTileShorts : kFoldShorts];
   unsigned short* const sa = smem;
   unsigned short* const sb = smem + TM * kSmallPitch;
   const T* A = reinterpret_cast<const T*>(g.a);
@@ -1033,7 +1044,7 @@ __global__ __launch_bounds__(256) void gemm_small16_kernel(SimpleArgs g) {
   const int nbn = (g.N + TN - 1) / TN;
   const int m0 = (blockIdx.x / nbn) * TM, n0 = (blockIdx.x % nbn) * TN;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int wm = wave / WN, wn = wave % WN;
+  const int wm = KSPLIT ? 0 : wave / WN, wn = KSPLIT ? 0 : wave % WN;
 
   SmallTile<T, TM> ta;
   ta.p = A; ta.o0 = m0; ta.o_lim = g.M; ta.K = g.K;
@@ -1061,6 +1072,7 @@ __global__ __launch_bounds__(256) void gemm_small16_kernel(SimpleArgs g) {
     }
 #pragma unroll
     for (int ks = 0; ks < TK / 16; ++ks) {
+      if (KSPLIT && ks != wave) continue;
       const int k = ks * 16 + (lane >> 5) * 8;
       const uint4 xa = *reinterpret_cast<const uint4*>(sa + (wm * 32 + (lane & 31)) * kSmallPitch + k);
       const uint4 xb = *reinterpret_cast<const uint4*>(sb + (wn * 32 + (lane & 31)) * kSmallPitch + k);
@@ -1070,8 +1082,21 @@ __global__ __launch_bounds__(256) void gemm_small16_kernel(SimpleArgs g) {
     __syncthreads();
   }
 
-  // the operand tiles are dead (barrier above): 32 x 36 floats of them per wave for the epilogue
-  static_assert(4 * 32 * 36 * 4 <= (int)sizeof(smem), "epilogue blocks fit in the tiles");
+  // the operand tiles are dead (barrier above)
+  if (KSPLIT) {
+    float* fold = reinterpret_cast<float*>(smem);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) fold[(r * 4 + wave) * 64 + lane] = acc[r];
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      acc[r] = (fold[(r * 4 + 0) * 64 + lane] + fold[(r * 4 + 1) * 64 + lane]) +
+               (fold[(r * 4 + 2) * 64 + lane] + fold[(r * 4 + 3) * 64 + lane]);
+    __builtin_amdgcn_wave_barrier();
+  }
+  // 32 x 36 floats of the tiles per wave for the epilogue
+  static_assert((KSPLIT ? 1 : 4) * 32 * 36 * 4 <= (int)sizeof(smem), "epilogue blocks fit in the tiles");
   wave_tile_epilogue<TO>(acc, reinterpret_cast<float*>(smem) + wave * 32 * 36, g, m0 + wm * 32, n0 + wn * 32);
 }
 
@@ -1361,6 +1386,46 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
     });
   }
 
+  // Classifier heads (at most 16 output features) on the vector ALUs.
+  if (layout == kFwd && N <= kSkinnyCols && skinny_rows_ok(a, K, lda, in_dt)) {
+    SkinnyArgs sk{a, b, nullptr, c, pre_act, bias, bias_dt, (int)M, (int)N, (int)K, lda, ldb, 0, ldc, ldp, act, param, 0};
+    return dispatch_dtype(in_dt, [&](auto* ti) -> int {
+      typedef std::remove_pointer_t<decltype(ti)> TI;
+      return dispatch_dtype(out_dt, [&](auto* to) -> int {
+        typedef std::remove_pointer_t<decltype(to)> TO;
+        hipLaunchKernelGGL((skinny_fwd_kernel<TI, TO>), dim3((unsigned)cdiv64(M, kSkinnyRowsFwd)), dim3(256), 0, stream, sk);
+        return launch_status();
+      });
+    });
+  }
+  if (layout == kDx && K <= kSkinnyCols && in_dt == out_dt && skinny_rows_ok(c, N, ldc, out_dt)) {
+    // dX[M, N] = dZ[M, K] W[N, K]^T with the narrow dimension contracted
+    SkinnyArgs sk{nullptr, b, a, c, nullptr, nullptr, 0, (int)M, (int)K, (int)N, 0, ldb, lda, ldc, 0, AT_ACT_NONE, 0.f, 0};
+    return dispatch_dtype(in_dt, [&](auto* tp) -> int {
+      typedef std::remove_pointer_t<decltype(tp)> T;
+      hipLaunchKernelGGL((skinny_dx_kernel<T>), dim3((unsigned)cdiv64(M, kSkinnyRowsDx)), dim3(256), 0, stream, sk);
+      return launch_status();
+    });
+  }
+  if (layout == kDw && N <= kSkinnyCols && in_dt == out_dt && skinny_rows_ok(a, M, lda, in_dt) && workspace &&
+      workspace_bytes >= skinny_dw_workspace_bytes(K, M)) {
+    // dW[M, N] = X[K, M]^T dZ[K, N]: the batch (K here) is cut into slices of rows
+    const int64_t rows_per_slice = skinny_rows_per_slice(K);
+    const int slices = (int)cdiv64(K, rows_per_slice);
+    SkinnyArgs sk{a, nullptr, b, workspace, nullptr, nullptr, 0, (int)K, (int)N, (int)M, lda, 0, ldb, 0, 0,
+                  AT_ACT_NONE, 0.f, (int)rows_per_slice};
+    return dispatch_dtype(in_dt, [&](auto* tp) -> int {
+      typedef std::remove_pointer_t<decltype(tp)> T;
+      constexpr int VEC = 16 / (int)sizeof(T);
+      hipLaunchKernelGGL((skinny_dw_kernel<T>), dim3((unsigned)cdiv64(M, 64 * VEC), (unsigned)slices), dim3(256), 0,
+                         stream, sk);
+      const int64_t items = M * (kSkinnyCols / 8);
+      hipLaunchKernelGGL((gemm_split_finish_kernel<T>), dim3((unsigned)cdiv64(items, 256)), dim3(256), 0, stream,
+                         (const float*)workspace, (T*)c, (int)M, (int)N, kSkinnyCols, ldc, slices);
+      return launch_status();
+    });
+  }
+
   // fp32 tensors whose rows allow 16-byte loads: the tiled fp32 MFMA kernel
   if (in_dt == AT_DTYPE_F32 && out_dt == AT_DTYPE_F32 && aligned16(a) && aligned16(b) && (lda % 4) == 0 &&
       (ldb % 4) == 0 && (!(a_contig_k || b_contig_k) || (K % 4) == 0) && M >= 32 && N >= 32 &&
@@ -1390,12 +1455,18 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
       if constexpr (std::is_same<TI, float>::value) {
         const unsigned grid = (unsigned)(cdiv64(M, 64) * cdiv64(N, 64));
         hipLaunchKernelGGL((gemm_simple_kernel<TI, TO>), dim3(grid), dim3(256), 0, stream, s);
-      } else if (N <= 32) {   // skinny outputs: all four waves along m
-        const unsigned grid = (unsigned)(cdiv64(M, 128) * cdiv64(N, 32));
-        hipLaunchKernelGGL((gemm_small16_kernel<TI, TO, 4, 1>), dim3(grid), dim3(256), 0, stream, s);
       } else {
-        const unsigned grid = (unsigned)(cdiv64(M, 64) * cdiv64(N, 64));
-        hipLaunchKernelGGL((gemm_small16_kernel<TI, TO, 2, 2>), dim3(grid), dim3(256), 0, stream, s);
+        // skinny outputs put all four waves along m; outputs that leave most CUs without a
+        // workgroup split the contraction over the waves instead (four times the workgroups)
+        const int64_t blocks = N <= 32 ? cdiv64(M, 128) * cdiv64(N, 32) : cdiv64(M, 64) * cdiv64(N, 64);
+        if (blocks * 2 <= device_cu_count() && K >= 256) {
+          const unsigned grid = (unsigned)(cdiv64(M, 32) * cdiv64(N, 32));
+          hipLaunchKernelGGL((gemm_small16_kernel<TI, TO, 1, 1, true>), dim3(grid), dim3(256), 0, stream, s);
+        } else if (N <= 32) {
+          hipLaunchKernelGGL((gemm_small16_kernel<TI, TO, 4, 1>), dim3((unsigned)blocks), dim3(256), 0, stream, s);
+        } else {
+          hipLaunchKernelGGL((gemm_small16_kernel<TI, TO, 2, 2>), dim3((unsigned)blocks), dim3(256), 0, stream, s);
+        }
       }
       return launch_status();
     });
@@ -1431,7 +1502,9 @@ int at_linear_bwd_input(const void* pre_act_grad, const void* weight, void* inpu
 }
 
 int64_t at_linear_bwd_weight_workspace_bytes(int64_t batch, int64_t in_feat, int64_t out_feat, int dtype) {
-  if (batch <= 0 || in_feat <= 0 || out_feat <= 0 || (dtype != AT_DTYPE_F16 && dtype != AT_DTYPE_BF16)) return 0;
+  if (batch <= 0 || in_feat <= 0 || out_feat <= 0 || !dtype_valid(dtype)) return 0;
+  if (out_feat <= kSkinnyCols) return skinny_dw_workspace_bytes(batch, in_feat);
+  if (dtype != AT_DTYPE_F16 && dtype != AT_DTYPE_BF16) return 0;
   if (in_feat < 64 || out_feat < 64 || in_feat * out_feat < (int64_t)MT * MT) return 0;
   if (!prefer_mid_tiles(in_feat, out_feat)) return 0;
   const int splits = dw_split_count(in_feat, out_feat, batch);

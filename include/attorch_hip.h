@@ -274,8 +274,9 @@ int at_linear_bwd_input(const void* pre_act_grad, const void* weight, void* inpu
 
 /* Scratch for at_linear_bwd_weight: with it, a weight gradient whose [in_feat, out_feat] tile
  * grid is small next to the GPU is computed in several slices of the batch at once (fp32 partial
- * sums, added in a fixed order).  0 when the product runs in one piece anyway.  The workspace is
- * optional: NULL (or a short one) selects the one-piece path. */
+ * sums, added in a fixed order); so is the weight gradient of a layer with at most 16 output
+ * features.  0 when the product runs in one piece anyway.  The workspace is optional: NULL (or a
+ * short one) selects the one-piece path. */
 int64_t at_linear_bwd_weight_workspace_bytes(int64_t batch, int64_t in_feat, int64_t out_feat,
                                              int dtype);
 

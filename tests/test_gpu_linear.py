@@ -181,3 +181,17 @@ def test_extent_one_dimensions_with_arbitrary_strides(dtype) -> None:
     norm = attorch_amd.LayerNorm(300, device='cuda', dtype=dtype)
     assert_close(norm(row), torch.nn.functional.layer_norm(row.detach().double(), (300,), norm.weight.double(),
                                                            norm.bias.double(), norm.eps), dtype, 'layer norm')
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('act_func', [None, 'relu', 'geluapprox'])
+@pytest.mark.parametrize('shape, out_dim', [((4096, 2048), 10), ((1000, 512), 1), ((37, 264), 16),
+                                            ((3, 5, 1024), 7), ((130, 256), 13), ((2050, 768), 2)])
+def test_linear_classifier_heads(shape, out_dim, act_func, dtype) -> None:
+    """
+    At most 16 output features with a wide, 16-byte aligned input: the three products run on the
+    vector-ALU kernels (row counts that do not fill a workgroup, one to sixteen columns, several
+    chunks of the contraction).
+    """
+    run_case(shape, out_dim, True, act_func, dtype)
+    run_case(shape, out_dim, False, act_func, dtype)
