@@ -97,6 +97,69 @@ def _conv_case(rng: random.Random, index: int) -> None:
         assert_close(layer.bias.grad, br.grad, dtype, what + ' bias_grad', normalize=True)
 
 
+FEATS = [1, 2, 3, 5, 8, 15, 16, 31, 33, 64, 100, 127, 128, 255, 256, 300, 511, 512, 1000, 1024, 2047, 2048,
+         4096, 5000, 8192, 10000, 20000, 50257, 70001]
+ROWS = [1, 2, 3, 7, 16, 33, 100, 257, 1000, 1025, 4096]
+
+
+def _row_case(rng: random.Random, index: int) -> None:
+    kind = rng.choice(['layer_norm', 'rms_norm', 'softmax', 'log_softmax', 'softmin', 'cross_entropy'])
+    dtype = rng.choice(DTYPES)
+    rows, feat = rng.choice(ROWS), rng.choice(FEATS)
+    if rows * feat > 2e7:
+        rows = max(1, int(2e7 // feat))
+    what = f'row case {index}: {kind} [{rows}, {feat}] {dtype}'
+    gen = torch.Generator().manual_seed(index)
+    if kind == 'cross_entropy':
+        feat = max(feat, 2)
+        x = (2 * torch.randn(rows, feat, generator=gen)).to(dtype).cuda().requires_grad_(True)
+        target = torch.randint(0, feat, (rows,), generator=gen).cuda()
+        if rows > 1:   # an all-ignored batch is 0 / 0 in both implementations
+            target[torch.rand(rows, generator=gen).cuda() < 0.3] = -100
+            target[0] = 0
+        weight = (0.5 + torch.rand(feat, generator=gen)).to(dtype).cuda() if rng.random() < 0.5 else None
+        xr = x.detach().double().requires_grad_(True)
+        y = attorch_amd.CrossEntropyLoss(weight=weight)(x, target)
+        yr = F.cross_entropy(xr, target, weight=None if weight is None else weight.double(), ignore_index=-100)
+        y.backward()
+        yr.backward()
+        assert_close(y, yr.to(y.dtype), dtype, what + ' loss')
+        assert_close(x.grad, xr.grad, dtype, what + ' input_grad', normalize=True)
+        return
+    wide = rng.random() < 0.3   # rows longer than the features: row stride > feat
+    base = torch.randn(rows, feat + (rng.choice([1, 3, 8]) if wide else 0), generator=gen).to(dtype).cuda()
+    x = base[:, :feat].detach().requires_grad_(True)
+    xr = x.detach().double().requires_grad_(True)
+    dy = torch.randn(rows, feat, generator=gen).to(dtype).cuda()
+    if kind == 'layer_norm':
+        layer = attorch_amd.LayerNorm(feat, device='cuda', dtype=dtype)
+        with torch.no_grad():
+            layer.weight.normal_(1, 0.2), layer.bias.normal_(0, 0.2)
+        yr = F.layer_norm(xr, (feat,), layer.weight.double(), layer.bias.double(), layer.eps)
+    elif kind == 'rms_norm':
+        layer = attorch_amd.RMSNorm(feat, eps=1e-5, device='cuda', dtype=dtype)
+        with torch.no_grad():
+            layer.weight.normal_(1, 0.2)
+        yr = xr * torch.rsqrt(xr.pow(2).mean(-1, keepdim=True) + 1e-5) * layer.weight.double()
+    else:
+        layer = {'softmax': attorch_amd.Softmax, 'log_softmax': attorch_amd.LogSoftmax,
+                 'softmin': attorch_amd.Softmin}[kind](dim=-1)
+        yr = {'softmax': F.softmax, 'log_softmax': F.log_softmax, 'softmin': F.softmin}[kind](xr, dim=-1)
+    y = layer(x)
+    y.backward(dy)
+    yr.backward(dy.double())
+    assert_close(y, yr, dtype, what + ' output', normalize=True)
+    # a row of one feature has a zero gradient up to rounding of inv_std * (g - g)
+    assert_close(x.grad, xr.grad, dtype, what + ' input_grad', normalize=True, atol_scale=1.0 if feat > 1 else 100.0)
+
+
+@pytest.mark.parametrize('chunk', range(3))
+def test_row_kernels_random_shapes(chunk) -> None:
+    rng = random.Random(3000 + chunk)
+    for index in range(chunk * 30, chunk * 30 + 30):
+        _row_case(rng, index)
+
+
 @pytest.mark.parametrize('chunk', range(4))
 def test_linear_random_shapes(chunk) -> None:
     rng = random.Random(1000 + chunk)

@@ -182,3 +182,16 @@ def test_product_never_imports_the_oracle() -> None:
     for path in (ROOT / 'attorch_amd').rglob('*.py'):
         text = path.read_text()
         assert 'import oracle' not in text and 'from oracle' not in text, path
+
+
+def test_row_stride_of_extent_one_dimensions() -> None:
+    """
+    PyTorch leaves the stride of an extent-1 dimension arbitrary; the C ABI checks strides against
+    the row length, so a single row reports its length.
+    """
+    from attorch_amd import _lib
+    assert _lib.row_stride(torch.zeros(5, 7)) == 7
+    assert _lib.row_stride(torch.zeros(5, 12)[:, :7]) == 12
+    weight = torch.zeros(63, 1).T.contiguous()            # shape [1, 63], stride(0) stays 1
+    assert tuple(weight.shape) == (1, 63) and _lib.row_stride(weight) == 63
+    assert _lib.row_stride(torch.zeros(0, 7)) == 7
