@@ -30,9 +30,23 @@ __global__ __launch_bounds__(1024) void ce_denominator_kernel(
     float* __restrict__ denom_out, int64_t batch, int feat, int64_t ignore_index) {
   __shared__ float scratch[16];
   float s = 0.f;
-  for (int64_t i = threadIdx.x; i < batch; i += blockDim.x) {
-    const int64_t t = target[i];
-    if (target_kept(t, ignore_index, feat)) s += weight ? load_scalar_f32(weight, wdt, t) : 1.f;
+  // targets first, then the weights they select: two rounds of independent loads per batch of
+  // rows instead of a dependent pair per row (the pass is pure memory latency)
+  constexpr int U = 8;
+  for (int64_t base = threadIdx.x; base < batch; base += (int64_t)blockDim.x * U) {
+    int64_t t[U];
+    bool kept[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t i = base + (int64_t)u * blockDim.x;
+      t[u] = i < batch ? target[i] : 0;
+      kept[u] = i < batch && target_kept(t[u], ignore_index, feat);
+    }
+    float w[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) w[u] = kept[u] ? (weight ? load_scalar_f32(weight, wdt, t[u]) : 1.f) : 0.f;
+#pragma unroll
+    for (int u = 0; u < U; ++u) s += w[u];
   }
   s = group_reduce(s, (int)blockDim.x, scratch, SumOp(), 0.f);
   if (threadIdx.x == 0) denom_out[0] = s;
@@ -43,6 +57,7 @@ __global__ __launch_bounds__(1024) void ce_finalize_kernel(
     int out_dt, int64_t batch) {
   __shared__ float scratch[16];
   float s = 0.f;
+#pragma unroll 8
   for (int64_t i = threadIdx.x; i < batch; i += blockDim.x) s += row_loss[i];
   s = group_reduce(s, (int)blockDim.x, scratch, SumOp(), 0.f);
   if (threadIdx.x == 0) store_scalar_f32(loss, out_dt, 0, s / denom[0]);
