@@ -644,6 +644,162 @@ __global__ __launch_bounds__(256) void conv_dw_kernel(DwArgs g) {
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Weight gradient of 3x3 / stride 1 / padding 1 layers with rows of at most 64 pixels: all nine
+// taps in one workgroup.  A k-tile is TR whole output rows of one image (TR * OW <= 64 pixels,
+// padded with zero rows of dY to 64); the input rows they touch, TR + 2 rows of W + 2 pixels with
+// the out-of-image positions as zeros, sit in LDS once and every tap reads its operand fragments
+// from them at shifted positions.  Against one workgroup per tap this moves a third of the bytes
+// into LDS and multiplies nine times as much per barrier.
+// ------------------------------------------------------------------------------------------
+constexpr int kRowsWinMax = 208;                              // window pixels at most
+constexpr int kRowsSlots = 36;                                // wave-wide loads per k-tile: 8 + 26 + 2 spare
+constexpr int kRowsStage = kRowsSlots * 1024;                 // dY tile, then the window (+ spare rows)
+constexpr int kRowsStages = 4;                                // k-tiles in LDS: one multiplied, three in flight
+
+struct DwRowsArgs {
+  const void* dy;     // [N*OH*OW][Otot]
+  const void* x;      // [N][H][W][Ctot]
+  float* part;        // [splits][Otot][9 * Cg]
+  int H, W, Ctot, Otot, Cg, Og;
+  int TR;             // output rows per k-tile
+  int Wp;             // W + 2
+  int win_px;         // (TR + 2) * Wp
+  int tiles_per_image, total_tiles, tiles_per_split, splits;
+  int K;              // 9 * Cg
+  int mtiles, ctiles;
+  int64_t dy_bytes, x_bytes;
+  FastDiv div_ow, div_wp, div_tpi;
+};
+
+// Six waves: wave = (32-channel half of the tile's 64 input channels) x (filter row kh); it holds
+// 64 output channels x 32 input channels x 3 taps (six accumulator tiles) and reads two dY
+// fragments and three window fragments per k-step for six MFMAs.  The transposing LDS reads bound
+// this kernel, so the fragments are shared as widely as the register file allows.
+constexpr int kRowsWaves = 6;
+
+template <typename T>
+__global__ __launch_bounds__(kRowsWaves * 64) void conv_dw_rows_kernel(DwRowsArgs g) {
+  __shared__ __attribute__((aligned(1024))) char lds[kRowsStages * kRowsStage];
+  const int grp = blockIdx.z;
+  const int tiles = g.mtiles * g.ctiles;
+  const int xcd = blockIdx.x & 7, pos = blockIdx.x >> 3;
+  const int split = xcd + 8 * (pos / tiles);
+  if (split >= g.splits) return;   // padding of the grid, uniform for the workgroup
+  const int tile = pos % tiles;
+  const int tile_m = tile / g.ctiles;
+  const int co0 = tile_m * 64, c0 = (tile - tile_m * g.ctiles) * 64;   // within the group
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wn = wave & 1, kh = wave >> 1;
+
+  const int t_begin = split * g.tiles_per_split;
+  const int t_end = t_begin + g.tiles_per_split < g.total_tiles ? t_begin + g.tiles_per_split : g.total_tiles;
+
+  const i32x4 ra = make_buffer_rsrc(g.dy, g.dy_bytes);
+  const i32x4 rb = make_buffer_rsrc(g.x, g.x_bytes);
+  // Every wave issues exactly kRowsSlots / kRowsWaves loads per k-tile (slots past the data fetch
+  // zeros into spare rows), so that "k-tile t has landed" is a fixed count of outstanding loads.
+  auto issue = [&](int t, char* stage) {
+    const bool live = t < t_end;
+    const int n = fast_div(t, g.div_tpi);
+    const int oh0 = (t - n * g.tiles_per_image) * g.TR;
+#pragma unroll
+    for (int i = 0; i < kRowsSlots / kRowsWaves; ++i) {
+      const int slot = wave + kRowsWaves * i;
+      int off = kOobOffset;
+      if (slot < 8) {
+        // dY tile: pixel k of the k-tile is (row k / OW, column k % OW); rows past TR are zeros
+        const int k = slot * 8 + (lane >> 3);
+        const int r = fast_div(k, g.div_ow), ow = k - r * g.W;
+        const int chunk = (lane & 7) ^ dw_chunk_swizzle(k);
+        const int oh = oh0 + r;
+        if (live && r < g.TR && oh < g.H && co0 + chunk * 8 < g.Og)
+          off = (((n * g.H + oh) * g.W + ow) * g.Otot + grp * g.Og + co0 + chunk * 8) * 2;
+        lds_dma_16(ra, off, stage + slot * 1024);
+      } else {
+        const int j = (slot - 8) * 8 + (lane >> 3);           // window pixel
+        const int chunk = (lane & 7) ^ dw_chunk_swizzle(j);
+        const int wr = fast_div(j, g.div_wp), wc = j - wr * g.Wp;
+        const int ih = oh0 - 1 + wr, iw = wc - 1;
+        if (live && j < g.win_px && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W &&
+            c0 + chunk * 8 < g.Cg)
+          off = (((n * g.H + ih) * g.W + iw) * g.Ctot + grp * g.Cg + c0 + chunk * 8) * 2;
+        lds_dma_16(rb, off, stage + slot * 1024);
+      }
+    }
+  };
+
+  // Window rows of the 8 pixels whose values this lane collects per k-tile, for this wave's filter
+  // row and kw = 0: pixel k -> (row r, column ow) -> (r + kh) * Wp + ow; padding pixels (their dY is
+  // zero) stay inside the window.
+  const int li = lane & 15, gq = lane >> 4;
+  int base_row[4][2];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int k = ks * 16 + (gq >> 1) * 8 + (li >> 2) + h * 4;
+      int r = fast_div(k, g.div_ow);
+      const int ow = k - r * g.W;
+      if (r >= g.TR) r = g.TR - 1;
+      base_row[ks][h] = (r + kh) * g.Wp + ow;
+    }
+  const int b_byte = (wn * 32 + (gq & 1) * 16 + (li & 3) * 4) * 2;   // channel bytes of this lane
+
+  f32x16 acc[2][3];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int t = 0; t < 3; ++t)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][t][e] = 0.f;
+
+#pragma unroll
+  for (int d = 0; d < kRowsStages - 1; ++d) issue(t_begin + d, lds + d * kRowsStage);
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  for (int t = t_begin; t < t_end; ++t) {
+    const int st = (t - t_begin) % kRowsStages;
+    // loads are answered in order: all but the two younger k-tiles' loads of this wave are done
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kRowsStages - 2) * (kRowsSlots / kRowsWaves)) : "memory");
+    __syncthreads();   // k-tile t is in LDS for everybody, and nobody reads k-tile t - 1 any more
+    issue(t + kRowsStages - 1, lds + ((st + kRowsStages - 1) % kRowsStages) * kRowsStage);
+    const char* cur = lds + st * kRowsStage;
+    const char* win = cur + kDwTile;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const uint4 a0 = read_frag_tr(cur, 0, ks), a1 = read_frag_tr(cur, 32, ks);
+#pragma unroll
+      for (int kw = 0; kw < 3; ++kw) {
+        const int r0 = base_row[ks][0] + kw, r1 = base_row[ks][1] + kw;
+        const int in0 = (((b_byte >> 4) ^ dw_chunk_swizzle(r0)) << 4) + (b_byte & 15);
+        const int in1 = (((b_byte >> 4) ^ dw_chunk_swizzle(r1)) << 4) + (b_byte & 15);
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(win + r0 * 128 + in0));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(win + r1 * 128 + in1));
+        const uint2 x0 = __builtin_bit_cast(uint2, lo), x1 = __builtin_bit_cast(uint2, hi);
+        const uint4 b = make_uint4(x0.x, x0.y, x1.x, x1.y);
+        acc[0][kw] = Mfma16<T>::run(a0, b, acc[0][kw]);
+        acc[1][kw] = Mfma16<T>::run(a1, b, acc[1][kw]);
+      }
+    }
+  }
+  lds_dma_wait_all();   // the loads issued past the end of the range have nothing to deliver, but must land
+
+  // register r of a 32 x 32 accumulator = output channel (r/4)*8 + (lane/32)*4 + r%4, column lane%32
+  float* part = g.part + (int64_t)split * g.Otot * g.K;
+  const int c = c0 + wn * 32 + (lane & 31);
+  if (c < g.Cg) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int kw = 0; kw < 3; ++kw)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int co = co0 + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+          if (co < g.Og) part[(int64_t)(grp * g.Og + co) * g.K + (kh * 3 + kw) * g.Cg + c] = acc[i][kw][r];
+        }
+  }
+}
+
 // dW[o][c][tap] = sum over splits of part[split][o][tap * Cg + c], fixed order.  A workgroup
 // owns 64 consecutive partial columns; its four waves each sum every fourth split.
 template <typename T>
@@ -897,6 +1053,46 @@ int conv_igemm_dw(const ConvProblem& p, const void* dy, const void* dy_nhwc, con
     xh = dst;
   }
   if (rc) return rc;
+  if (p.KH == 3 && p.KW == 3 && p.sh == 1 && p.sw == 1 && p.ph == 1 && p.pw == 1 && p.OW <= 64) {
+    DwRowsArgs r{};
+    r.dy = dyh; r.x = xh; r.part = part;
+    r.H = (int)p.H; r.W = (int)p.W; r.Ctot = (int)p.C; r.Otot = (int)p.O; r.Cg = (int)(p.C / p.groups);
+    r.Og = (int)(p.O / p.groups);
+    r.TR = (int)(64 / p.OW < p.OH ? 64 / p.OW : p.OH);
+    r.Wp = (int)p.W + 2;
+    r.win_px = (r.TR + 2) * r.Wp;
+    if (r.win_px <= kRowsWinMax) {
+      r.tiles_per_image = (int)cdiv64(p.OH, r.TR);
+      r.total_tiles = (int)(p.N * r.tiles_per_image);
+      r.K = 9 * r.Cg;
+      r.mtiles = (int)cdiv64(r.Og, 64);
+      r.ctiles = (int)cdiv64(r.Cg, 64);
+      // two workgroups per CU over the whole grid, at least four k-tiles each
+      int64_t want = cdiv64((int64_t)device_cu_count() * 2, (int64_t)r.mtiles * r.ctiles * p.groups);
+      const int64_t by_len = cdiv64(r.total_tiles, 4);
+      if (want > by_len) want = by_len;
+      if (want > kDwMaxSplits) want = kDwMaxSplits;
+      if (want < 1) want = 1;
+      r.tiles_per_split = (int)cdiv64(r.total_tiles, want);
+      r.splits = (int)cdiv64(r.total_tiles, r.tiles_per_split);
+      r.dy_bytes = p.N * p.O * p.OH * p.OW * 2;
+      r.x_bytes = p.N * p.C * p.H * p.W * 2;
+      r.div_ow = make_fastdiv(p.OW);
+      r.div_wp = make_fastdiv(r.Wp);
+      r.div_tpi = make_fastdiv(r.tiles_per_image);
+      const dim3 grid((unsigned)(r.mtiles * r.ctiles * (cdiv64(r.splits, 8) * 8)), 1, (unsigned)p.groups);
+      const int64_t total = p.O * (int64_t)r.K;
+      return dispatch16(p.dtype, [&](auto* tp) -> int {
+        typedef std::remove_pointer_t<decltype(tp)> T;
+        hipLaunchKernelGGL((conv_dw_rows_kernel<T>), grid, dim3(kRowsWaves * 64), 0, stream, r);
+        int rc2 = launch_status();
+        if (rc2) return rc2;
+        hipLaunchKernelGGL((conv_dw_finish_kernel<T>), dim3((unsigned)cdiv64(total, 64)), dim3(256), 0, stream,
+                           (const float*)part, (T*)dw, r.splits, r.Cg, 9, total);
+        return launch_status();
+      });
+    }
+  }
   DwArgs g{};
   g.dy = dyh; g.x = xh; g.part = part;
   g.H = (int)p.H; g.W = (int)p.W; g.Ctot = (int)p.C; g.Otot = (int)p.O; g.Cg = (int)(p.C / p.groups);

@@ -177,6 +177,14 @@ def test_conv_window_kernel_agrees_with_generic_kernel_at_size(n, c, h, w, o, pa
     _lib.check(lib.at_conv2d_fwd(_lib.ptr(x), _lib.ptr(wt), _lib.ptr(b), _lib.ptr(y_slow), None, 0,
                                  *dims, dt, dt, dt, stream), 'fwd')
     assert_close(y_fast, y_slow.cpu(), dtype, 'output', normalize=True)
+    # weight gradient: the matrix-core path (all taps per workgroup for pad 1) against torch in fp32
+    nb_w = lib.at_conv2d_bwd_weight_workspace_bytes(*dims, dt)
+    ws_w = torch.empty(nb_w, dtype=torch.uint8, device='cuda')
+    dw_fast = torch.full_like(wt, float('nan'))
+    _lib.check(lib.at_conv2d_bwd_weight(_lib.ptr(dy), None, _lib.ptr(x), None, _lib.ptr(dw_fast), _lib.ptr(ws_w),
+                                        nb_w, *dims, dt, stream), 'dw')
+    dw_ref = torch.nn.grad.conv2d_weight(x.float(), wt.shape, dy.float(), stride=1, padding=pad, groups=groups)
+    assert_close(dw_fast, dw_ref.cpu(), dtype, 'weight_grad', normalize=True)
     nb_x = lib.at_conv2d_bwd_input_workspace_bytes(*dims, dt)
     if pad > k - 1:
         assert nb_x == 0                    # the input gradient as a convolution needs pad <= k - 1
