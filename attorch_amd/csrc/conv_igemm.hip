@@ -672,11 +672,13 @@ struct DwRowsArgs {
   FastDiv div_ow, div_wp, div_tpi;
 };
 
-// Six waves: wave = (32-channel half of the tile's 64 input channels) x (filter row kh); it holds
-// 64 output channels x 32 input channels x 3 taps (six accumulator tiles) and reads two dY
-// fragments and three window fragments per k-step for six MFMAs.  The transposing LDS reads bound
-// this kernel, so the fragments are shared as widely as the register file allows.
-constexpr int kRowsWaves = 6;
+// Twelve waves: wave = (k-steps 0-1 | 2-3 of every k-tile) x (filter row kh) x (32-channel half of
+// the tile's 64 input channels); it holds 64 output channels x 32 input channels x 3 taps (six
+// accumulator tiles) and reads two dY fragments and three window fragments per k-step for six
+// MFMAs.  The transposing LDS reads bound this kernel: the fragments are shared as widely as the
+// register file allows, and the k-steps are split over two sets of waves (added through LDS at the
+// end) only to have enough waves asking for them.
+constexpr int kRowsWaves = 12;
 
 template <typename T>
 __global__ __launch_bounds__(kRowsWaves * 64) void conv_dw_rows_kernel(DwRowsArgs g) {
@@ -690,7 +692,8 @@ __global__ __launch_bounds__(kRowsWaves * 64) void conv_dw_rows_kernel(DwRowsArg
   const int tile_m = tile / g.ctiles;
   const int co0 = tile_m * 64, c0 = (tile - tile_m * g.ctiles) * 64;   // within the group
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int wn = wave & 1, kh = wave >> 1;
+  const int khalf = wave / 6, w6 = wave % 6;   // which k-steps; position among the six accumulator owners
+  const int wn = w6 & 1, kh = w6 >> 1;
 
   const int t_begin = split * g.tiles_per_split;
   const int t_end = t_begin + g.tiles_per_split < g.total_tiles ? t_begin + g.tiles_per_split : g.total_tiles;
@@ -733,16 +736,16 @@ __global__ __launch_bounds__(kRowsWaves * 64) void conv_dw_rows_kernel(DwRowsArg
   // row and kw = 0: pixel k -> (row r, column ow) -> (r + kh) * Wp + ow; padding pixels (their dY is
   // zero) stay inside the window.
   const int li = lane & 15, gq = lane >> 4;
-  int base_row[4][2];
+  int base_row[2][2];
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks)
+  for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      const int k = ks * 16 + (gq >> 1) * 8 + (li >> 2) + h * 4;
+      const int k = (khalf * 2 + kk) * 16 + (gq >> 1) * 8 + (li >> 2) + h * 4;
       int r = fast_div(k, g.div_ow);
       const int ow = k - r * g.W;
       if (r >= g.TR) r = g.TR - 1;
-      base_row[ks][h] = (r + kh) * g.Wp + ow;
+      base_row[kk][h] = (r + kh) * g.Wp + ow;
     }
   const int b_byte = (wn * 32 + (gq & 1) * 16 + (li & 3) * 4) * 2;   // channel bytes of this lane
 
@@ -766,11 +769,12 @@ __global__ __launch_bounds__(kRowsWaves * 64) void conv_dw_rows_kernel(DwRowsArg
     const char* cur = lds + st * kRowsStage;
     const char* win = cur + kDwTile;
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
+    for (int kk = 0; kk < 2; ++kk) {
+      const int ks = khalf * 2 + kk;
       const uint4 a0 = read_frag_tr(cur, 0, ks), a1 = read_frag_tr(cur, 32, ks);
 #pragma unroll
       for (int kw = 0; kw < 3; ++kw) {
-        const int r0 = base_row[ks][0] + kw, r1 = base_row[ks][1] + kw;
+        const int r0 = base_row[kk][0] + kw, r1 = base_row[kk][1] + kw;
         const int in0 = (((b_byte >> 4) ^ dw_chunk_swizzle(r0)) << 4) + (b_byte & 15);
         const int in1 = (((b_byte >> 4) ^ dw_chunk_swizzle(r1)) << 4) + (b_byte & 15);
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(win + r0 * 128 + in0));
@@ -783,6 +787,27 @@ __global__ __launch_bounds__(kRowsWaves * 64) void conv_dw_rows_kernel(DwRowsArg
     }
   }
   lds_dma_wait_all();   // the loads issued past the end of the range have nothing to deliver, but must land
+  // The waves of the second k-step set hand their sums to their partners through LDS, one
+  // 32-output-channel half (48 floats per lane) at a time.
+  float* fold = reinterpret_cast<float*>(lds);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    __syncthreads();
+    if (khalf == 1) {
+#pragma unroll
+      for (int kw = 0; kw < 3; ++kw)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) fold[((w6 * 48 + kw * 16 + r) << 6) + lane] = acc[i][kw][r];
+    }
+    __syncthreads();
+    if (khalf == 0) {
+#pragma unroll
+      for (int kw = 0; kw < 3; ++kw)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][kw][r] += fold[((w6 * 48 + kw * 16 + r) << 6) + lane];
+    }
+  }
+  if (khalf == 1) return;
 
   // register r of a 32 x 32 accumulator = output channel (r/4)*8 + (lane/32)*4 + r%4, column lane%32
   float* part = g.part + (int64_t)split * g.Otot * g.K;
