@@ -702,52 +702,74 @@ __global__ __launch_bounds__(kRowsWaves * 64) void conv_dw_rows_kernel(DwRowsArg
   const i32x4 rb = make_buffer_rsrc(g.x, g.x_bytes);
   // Every wave issues exactly kRowsSlots / kRowsWaves loads per k-tile (slots past the data fetch
   // zeros into spare rows), so that "k-tile t has landed" is a fixed count of outstanding loads.
+  // What a lane fetches differs between k-tiles only by the tile's first pixel (n, oh0, 0): the rest
+  // of the byte offset, and whether the position exists at all, are fixed per slot.
+  constexpr int kLoads = kRowsSlots / kRowsWaves;
+  int slot_const[kLoads], slot_row[kLoads], slot_pitch[kLoads];
+  bool slot_ok[kLoads];
+#pragma unroll
+  for (int i = 0; i < kLoads; ++i) {
+    const int slot = wave + kRowsWaves * i;
+    if (slot < 8) {
+      // dY tile: pixel k of the k-tile is (row k / OW, column k % OW); rows past TR are zeros
+      const int k = slot * 8 + (lane >> 3);
+      const int r = fast_div(k, g.div_ow), ow = k - r * g.W;
+      const int chunk = (lane & 7) ^ dw_chunk_swizzle(k);
+      slot_ok[i] = r < g.TR && co0 + chunk * 8 < g.Og;
+      slot_row[i] = r;
+      slot_pitch[i] = g.Otot * 2;
+      slot_const[i] = ((r * g.W + ow) * g.Otot + grp * g.Og + co0 + chunk * 8) * 2;
+    } else {
+      const int j = (slot - 8) * 8 + (lane >> 3);           // window pixel
+      const int chunk = (lane & 7) ^ dw_chunk_swizzle(j);
+      const int wr = fast_div(j, g.div_wp), wc = j - wr * g.Wp;
+      slot_ok[i] = j < g.win_px && (unsigned)(wc - 1) < (unsigned)g.W && c0 + chunk * 8 < g.Cg;
+      slot_row[i] = wr - 1;
+      slot_pitch[i] = g.Ctot * 2;
+      slot_const[i] = (((wr - 1) * g.W + wc - 1) * g.Ctot + grp * g.Cg + c0 + chunk * 8) * 2;
+    }
+  }
   auto issue = [&](int t, char* stage) {
     const bool live = t < t_end;
     const int n = fast_div(t, g.div_tpi);
     const int oh0 = (t - n * g.tiles_per_image) * g.TR;
+    const int first_px = (n * g.H + oh0) * g.W;
 #pragma unroll
-    for (int i = 0; i < kRowsSlots / kRowsWaves; ++i) {
+    for (int i = 0; i < kLoads; ++i) {
       const int slot = wave + kRowsWaves * i;
-      int off = kOobOffset;
-      if (slot < 8) {
-        // dY tile: pixel k of the k-tile is (row k / OW, column k % OW); rows past TR are zeros
-        const int k = slot * 8 + (lane >> 3);
-        const int r = fast_div(k, g.div_ow), ow = k - r * g.W;
-        const int chunk = (lane & 7) ^ dw_chunk_swizzle(k);
-        const int oh = oh0 + r;
-        if (live && r < g.TR && oh < g.H && co0 + chunk * 8 < g.Og)
-          off = (((n * g.H + oh) * g.W + ow) * g.Otot + grp * g.Og + co0 + chunk * 8) * 2;
-        lds_dma_16(ra, off, stage + slot * 1024);
-      } else {
-        const int j = (slot - 8) * 8 + (lane >> 3);           // window pixel
-        const int chunk = (lane & 7) ^ dw_chunk_swizzle(j);
-        const int wr = fast_div(j, g.div_wp), wc = j - wr * g.Wp;
-        const int ih = oh0 - 1 + wr, iw = wc - 1;
-        if (live && j < g.win_px && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W &&
-            c0 + chunk * 8 < g.Cg)
-          off = (((n * g.H + ih) * g.W + iw) * g.Ctot + grp * g.Cg + c0 + chunk * 8) * 2;
-        lds_dma_16(rb, off, stage + slot * 1024);
-      }
+      const bool ok = live && slot_ok[i] && (unsigned)(oh0 + slot_row[i]) < (unsigned)g.H;
+      const int off = ok ? first_px * slot_pitch[i] + slot_const[i] : kOobOffset;
+      if (slot < 8) lds_dma_16(ra, off, stage + slot * 1024);   // uniform for the wave
+      else lds_dma_16(rb, off, stage + slot * 1024);
     }
   };
 
-  // Window rows of the 8 pixels whose values this lane collects per k-tile, for this wave's filter
-  // row and kw = 0: pixel k -> (row r, column ow) -> (r + kh) * Wp + ow; padding pixels (their dY is
-  // zero) stay inside the window.
+  // LDS positions (relative to a stage) of the fragments this lane reads per k-tile; they do not
+  // change from k-tile to k-tile.  dY fragments as in read_frag_tr.  Window fragments: pixel k ->
+  // (row r, column ow) -> window row (r + kh) * Wp + ow + kw; padding pixels (their dY is zero) are
+  // kept inside the window.
   const int li = lane & 15, gq = lane >> 4;
-  int base_row[2][2];
+  int a_rel[2][2][2], b_rel[2][3][2];
 #pragma unroll
   for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int k = (khalf * 2 + kk) * 16 + (gq >> 1) * 8 + (li >> 2) + h * 4;
+#pragma unroll
+      for (int f = 0; f < 2; ++f) {
+        const int byte = (f * 32 + (gq & 1) * 16 + (li & 3) * 4) * 2;
+        a_rel[kk][f][h] = k * 128 + (((byte >> 4) ^ dw_chunk_swizzle(k)) << 4) + (byte & 15);
+      }
       int r = fast_div(k, g.div_ow);
       const int ow = k - r * g.W;
       if (r >= g.TR) r = g.TR - 1;
-      base_row[kk][h] = (r + kh) * g.Wp + ow;
+      const int byte = (wn * 32 + (gq & 1) * 16 + (li & 3) * 4) * 2;
+#pragma unroll
+      for (int kw = 0; kw < 3; ++kw) {
+        const int row = (r + kh) * g.Wp + ow + kw;
+        b_rel[kk][kw][h] = kDwTile + row * 128 + (((byte >> 4) ^ dw_chunk_swizzle(row)) << 4) + (byte & 15);
+      }
     }
-  const int b_byte = (wn * 32 + (gq & 1) * 16 + (li & 3) * 4) * 2;   // channel bytes of this lane
 
   f32x16 acc[2][3];
 #pragma unroll
@@ -767,20 +789,18 @@ __global__ __launch_bounds__(kRowsWaves * 64) void conv_dw_rows_kernel(DwRowsArg
     __syncthreads();   // k-tile t is in LDS for everybody, and nobody reads k-tile t - 1 any more
     issue(t + kRowsStages - 1, lds + ((st + kRowsStages - 1) % kRowsStages) * kRowsStage);
     const char* cur = lds + st * kRowsStage;
-    const char* win = cur + kDwTile;
+    auto frag = [&](const int (&rel)[2]) {
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(cur + rel[0]));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(cur + rel[1]));
+      const uint2 x0 = __builtin_bit_cast(uint2, lo), x1 = __builtin_bit_cast(uint2, hi);
+      return make_uint4(x0.x, x0.y, x1.x, x1.y);
+    };
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
-      const int ks = khalf * 2 + kk;
-      const uint4 a0 = read_frag_tr(cur, 0, ks), a1 = read_frag_tr(cur, 32, ks);
+      const uint4 a0 = frag(a_rel[kk][0]), a1 = frag(a_rel[kk][1]);
 #pragma unroll
       for (int kw = 0; kw < 3; ++kw) {
-        const int r0 = base_row[kk][0] + kw, r1 = base_row[kk][1] + kw;
-        const int in0 = (((b_byte >> 4) ^ dw_chunk_swizzle(r0)) << 4) + (b_byte & 15);
-        const int in1 = (((b_byte >> 4) ^ dw_chunk_swizzle(r1)) << 4) + (b_byte & 15);
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(win + r0 * 128 + in0));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(win + r1 * 128 + in1));
-        const uint2 x0 = __builtin_bit_cast(uint2, lo), x1 = __builtin_bit_cast(uint2, hi);
-        const uint4 b = make_uint4(x0.x, x0.y, x1.x, x1.y);
+        const uint4 b = frag(b_rel[kk][kw]);
         acc[0][kw] = Mfma16<T>::run(a0, b, acc[0][kw]);
         acc[1][kw] = Mfma16<T>::run(a1, b, acc[1][kw]);
       }
