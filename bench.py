@@ -37,17 +37,17 @@ PEAK_MFMA_FP32_TFLOPS = 157.3    # dense fp32 MFMA
 # taken in separate profiling runs, so these are recorded measurements, not live ones; reads that
 # the 256 MB Infinity Cache serves are included.
 MEASURED_TRAFFIC_BYTES = {
-    'c4_linear_fwd': 4298346833,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.0 GiB read, 1.0 GiB written
-    'c2_layer_norm': 387442735,       # norm_fwd + norm_bwd + reduce_partials
-    'c2_rms_norm': 378444348,
-    'c2_softmax': 335725000,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
-    'c2_act_dropout': 336063645,      # act_dropout forward + backward
-    'c2_glu': 269042882,              # glu forward + backward
-    'c2_mse': 335730416,              # p_loss forward + backward
-    'c3_cross_entropy': 1610248667,   # ce_row_kernel (ignored rows are not read)
-    'c3_nll_loss': 827006774,         # nll forward (a gather) + the single-pass gradient write
-    'c5_conv': 644367335,             # 2 window kernels + weight gradient + 2 layout copies + weight reorders
-    'c5_batch_norm': 616878257,       # stats + apply + backward reduce + backward apply
+    'c4_linear_fwd': 4298071383,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.0 GiB read, 1.0 GiB written
+    'c2_layer_norm': 387439942,       # norm_fwd + norm_bwd + reduce_partials
+    'c2_rms_norm': 378441942,
+    'c2_softmax': 335723463,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
+    'c2_act_dropout': 336052762,      # act_dropout forward + backward
+    'c2_glu': 269041149,              # glu forward + backward
+    'c2_mse': 335729135,              # p_loss forward + backward
+    'c3_cross_entropy': 1610279799,   # ce_row_kernel (ignored rows are not read)
+    'c3_nll_loss': 827002516,         # nll forward (a gather) + the single-pass gradient write
+    'c5_conv': 687515005,             # 2 window kernels + weight gradient + 2 layout copies + weight reorders
+    'c5_batch_norm': 616874527,       # stats + apply + backward reduce + backward apply
 }
 
 
