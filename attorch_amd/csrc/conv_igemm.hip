@@ -137,24 +137,35 @@ __global__ void conv_weight_taps_kernel(const T* __restrict__ w, T* __restrict__
   }
 }
 
-// wt[groups * Og][K] -> fragment-major copy for the kernel that reads the weights straight into
-// registers: the 64 lanes x 16 bytes of one operand fragment (32 output channels x 16 k) are
-// contiguous, ordered [group][channel tile of 32][k / 16][lane]; channels past Og are zeros.
+// W[O][Cg][KH][KW] -> fragment-major copy of wt (as defined above) for the kernel that reads the
+// weights straight into registers: the 64 lanes x 16 bytes of one operand fragment (32 rows x 16 k)
+// are contiguous, ordered [group][row tile of 32][k / 16][lane]; rows past Og are zeros.
+// k = tap * Cg + c for the forward product (flip = 0); for the input gradient (flip = 1) the roles
+// of the channel counts are swapped and the taps mirrored.  Cg = contraction channels per group (a
+// multiple of 8), Og = rows per group.
 template <typename T>
-__global__ void conv_weight_frags_kernel(const T* __restrict__ wt, T* __restrict__ wf, int Og, int K, int ntiles,
-                                         int64_t total_chunks) {
+__global__ void conv_weight_frags_direct_kernel(const T* __restrict__ w, T* __restrict__ wf, int Cg, int Og, int taps,
+                                                int flip, int ntiles, int64_t total_chunks) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= total_chunks) return;
   const int lane = (int)(i & 63);
   const int64_t frag = i >> 6;
-  const int ksteps = K / 16;
+  const int ksteps = taps * Cg / 16;
   const int kstep = (int)(frag % ksteps);
   const int tile = (int)((frag / ksteps) % ntiles);
   const int grp = (int)(frag / ((int64_t)ksteps * ntiles));
   const int co = tile * 32 + (lane & 31);
-  uint4 v = make_uint4(0, 0, 0, 0);
-  if (co < Og) v = *reinterpret_cast<const uint4*>(wt + (int64_t)(grp * Og + co) * K + kstep * 16 + (lane >> 5) * 8);
-  reinterpret_cast<uint4*>(wf)[i] = v;
+  const int k0 = kstep * 16 + (lane >> 5) * 8;
+  const int tap = k0 / Cg, c = k0 - tap * Cg;
+  union { uint4 raw; T e[8]; } u;
+  u.raw = make_uint4(0, 0, 0, 0);
+  if (co < Og) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      u.e[e] = flip ? w[(((int64_t)grp * Cg + c + e) * Og + co) * taps + (taps - 1 - tap)]
+                    : w[(((int64_t)grp * Og + co) * Cg + c + e) * taps + tap];
+  }
+  reinterpret_cast<uint4*>(wf)[i] = u.raw;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -945,7 +956,8 @@ int64_t halo_rows_needed(const IgemmArgs& g, int64_t n_img, int64_t OH, int KH) 
 }
 
 // One product out[(n,oh,ow), co] over channels-last `act`; see IgemmArgs for the meaning of the fields.
-int run_igemm(IgemmArgs g, int64_t n_img, int64_t OH, int groups, int dt, hipStream_t stream) {
+int run_igemm(IgemmArgs g, const void* w, const ConvProblem& p, int flip, int64_t n_img, int64_t OH, int groups,
+              int dt, hipStream_t stream) {
   g.OHW = (int)(OH * g.OW);
   g.M = (int)(n_img * g.OHW);
   g.K = g.KT * 64;
@@ -963,10 +975,12 @@ int run_igemm(IgemmArgs g, int64_t n_img, int64_t OH, int groups, int dt, hipStr
     if (resident) {
       const int ntiles = (g.Og + 31) / 32;
       const int64_t chunks = (int64_t)groups * ntiles * (g.K / 16) * 64;
-      hipLaunchKernelGGL((conv_weight_frags_kernel<T>), dim3((unsigned)cdiv64(chunks, 256)), dim3(256), 0, stream,
-                         (const T*)g.wt, (T*)g.wf, g.Og, g.K, ntiles, chunks);
+      hipLaunchKernelGGL((conv_weight_frags_direct_kernel<T>), dim3((unsigned)cdiv64(chunks, 256)), dim3(256), 0,
+                         stream, (const T*)w, (T*)g.wf, g.Cg, g.Og, (int)(p.KH * p.KW), flip, ntiles, chunks);
       hipLaunchKernelGGL((conv_igemm_halo_kernel<T>), grid, dim3(256), 0, stream, g);
     } else {
+      const int rc = weight_taps(w, const_cast<void*>(g.wt), p, flip, stream);
+      if (rc) return rc;
       hipLaunchKernelGGL((conv_igemm_kernel<T>), grid, dim3(256), 0, stream, g);
     }
     return launch_status();
@@ -1034,8 +1048,6 @@ int conv_igemm_fwd(const ConvProblem& p, const void* x, const void* w, const voi
   void* wt = ws + round256(p.N * p.C * p.H * p.W * 2);
   int rc = to_nhwc(x, xh, p.N, p.C, p.H * p.W, p.dtype, stream);
   if (rc) return rc;
-  rc = weight_taps(w, wt, p, 0, stream);
-  if (rc) return rc;
   IgemmArgs g{};
   g.act = xh; g.wt = wt; g.out = y; g.bias = bias; g.bias_dt = bias_dt;
   g.wf = static_cast<char*>(wt) + round256(p.O * (p.C / p.groups) * p.KH * p.KW * 2);
@@ -1044,7 +1056,7 @@ int conv_igemm_fwd(const ConvProblem& p, const void* x, const void* w, const voi
   g.KT = (int)(p.KH * p.KW * (g.Cg / 64));
   g.act_bytes = p.N * p.C * p.H * p.W * 2;
   g.wt_bytes = p.O * g.Cg * p.KH * p.KW * 2;
-  return run_igemm(g, p.N, p.OH, (int)p.groups, p.dtype, stream);
+  return run_igemm(g, w, p, 0, p.N, p.OH, (int)p.groups, p.dtype, stream);
 }
 
 int conv_nchw_to_nhwc(const void* src, void* dst, int64_t N, int64_t C, int64_t HW, int dtype,
@@ -1065,8 +1077,6 @@ int conv_igemm_dx(const ConvProblem& p, const void* dy, const void* dy_nhwc, con
     dyh = ws;
   }
   if (rc) return rc;
-  rc = weight_taps(w, wt, p, 1, stream);
-  if (rc) return rc;
   // dX[n, c, ih, iw] = sum_{taps', o} dY[n, ih + kh' - (KH-1-ph), iw + kw' - (KW-1-pw), o] * W[o, c, mirrored tap]
   IgemmArgs g{};
   g.act = dyh; g.wt = wt; g.out = dx; g.bias = nullptr; g.bias_dt = 0;
@@ -1076,7 +1086,7 @@ int conv_igemm_dx(const ConvProblem& p, const void* dy, const void* dy_nhwc, con
   g.KT = (int)(p.KH * p.KW * (g.Cg / 64));
   g.act_bytes = p.N * p.O * p.OH * p.OW * 2;
   g.wt_bytes = p.O * (p.C / p.groups) * p.KH * p.KW * 2;
-  return run_igemm(g, p.N, p.H, (int)p.groups, p.dtype, stream);
+  return run_igemm(g, w, p, 1, p.N, p.H, (int)p.groups, p.dtype, stream);
 }
 
 int conv_igemm_dw(const ConvProblem& p, const void* dy, const void* dy_nhwc, const void* x, const void* x_nhwc,
