@@ -37,17 +37,17 @@ PEAK_MFMA_FP32_TFLOPS = 157.3    # dense fp32 MFMA
 # taken in separate profiling runs, so these are recorded measurements, not live ones; reads that
 # the 256 MB Infinity Cache serves are included.
 MEASURED_TRAFFIC_BYTES = {
-    'c4_linear_fwd': 4298071383,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.0 GiB read, 1.0 GiB written
-    'c2_layer_norm': 387439942,       # norm_fwd + norm_bwd + reduce_partials
-    'c2_rms_norm': 378441942,
-    'c2_softmax': 335723463,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
-    'c2_act_dropout': 336052762,      # act_dropout forward + backward
-    'c2_glu': 269041149,              # glu forward + backward
-    'c2_mse': 335729135,              # p_loss forward + backward
-    'c3_cross_entropy': 1610279799,   # ce_row_kernel (ignored rows are not read)
-    'c3_nll_loss': 827002516,         # nll forward (a gather) + the single-pass gradient write
-    'c5_conv': 687515005,             # 2 window kernels + weight gradient + 2 layout copies + weight reorders
-    'c5_batch_norm': 616874527,       # stats + apply + backward reduce + backward apply
+    'c4_linear_fwd': 4299419969,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.0 GiB read, 1.0 GiB written
+    'c2_layer_norm': 387435537,       # norm_fwd + norm_bwd + reduce_partials
+    'c2_rms_norm': 378436585,
+    'c2_softmax': 335720132,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
+    'c2_act_dropout': 336053007,      # act_dropout forward + backward
+    'c2_glu': 269037744,              # glu forward + backward
+    'c2_mse': 335722286,              # p_loss forward + backward
+    'c3_cross_entropy': 1610258526,   # ce_row_kernel (ignored rows are not read)
+    'c3_nll_loss': 827004360,         # nll forward (a gather) + the single-pass gradient write
+    'c5_conv': 687076692,             # 2 window kernels + weight gradient + 2 layout copies + weight reorders
+    'c5_batch_norm': 616867690,       # stats + apply + backward reduce + backward apply
 }
 
 
