@@ -1130,6 +1130,11 @@ int conv_igemm_dw(const ConvProblem& p, const void* dy, const void* dy_nhwc, con
       if (want < 1) want = 1;
       r.tiles_per_split = (int)cdiv64(r.total_tiles, want);
       r.splits = (int)cdiv64(r.total_tiles, r.tiles_per_split);
+    }
+    // small problems give this kernel too few workgroups (one per pixel range and 64 x 64 tile of
+    // all taps); the per-tap kernel below has nine times as many
+    if (r.win_px <= kRowsWinMax &&
+        (int64_t)r.mtiles * r.ctiles * p.groups * r.splits * 2 >= device_cu_count()) {
       r.dy_bytes = p.N * p.O * p.OH * p.OW * 2;
       r.x_bytes = p.N * p.C * p.H * p.W * 2;
       r.div_ow = make_fastdiv(p.OW);

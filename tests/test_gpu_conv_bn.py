@@ -149,6 +149,8 @@ def test_conv_matrix_core_path_agrees_with_generic_kernel(dtype) -> None:
     (44, 128, 56, 56, 128, 1, 2, True),    # two groups of 64 channels
     (44, 64, 58, 58, 64, 0, 1, False),     # no padding: output smaller than the input
     (41, 64, 56, 56, 64, 2, 1, False),     # padding wider than the filter reach (forward only)
+    (96, 64, 23, 23, 64, 1, 1, False),     # two output rows per k-tile of the weight gradient, odd row count
+    (128, 128, 7, 7, 192, 1, 1, True),     # whole 7x7 images per k-tile, several channel tiles
 ])
 def test_conv_window_kernel_agrees_with_generic_kernel_at_size(n, c, h, w, o, pad, groups, bias, dtype) -> None:
     """
@@ -197,6 +199,33 @@ def test_conv_window_kernel_agrees_with_generic_kernel_at_size(n, c, h, w, o, pa
     _lib.check(lib.at_conv2d_bwd_input(_lib.ptr(dy), None, _lib.ptr(wt), _lib.ptr(dx_slow), None, 0,
                                        *dims, dt, stream), 'dx')
     assert_close(dx_fast, dx_slow.cpu(), dtype, 'input_grad', normalize=True)
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('n, c, h, w, o, groups', [
+    (64, 72, 14, 14, 40, 1),       # channel counts that are multiples of 8 only: partly empty 64-wide tiles
+    (48, 48, 30, 20, 96, 2),       # two groups, three output rows per k-tile, rows do not divide the image
+    (256, 8, 9, 64, 16, 1),        # a full 64-pixel row per k-tile, very few channels
+])
+def test_conv_weight_gradient_all_taps_kernel(n, c, h, w, o, groups, dtype) -> None:
+    """
+    3x3 / stride 1 / padding 1 weight gradients large enough for the kernel that handles all taps
+    in one workgroup, at channel counts and image shapes its tiles do not divide, against torch in
+    fp32 from the same operands.
+    """
+    from attorch_amd import _lib
+    lib = _lib.load()
+    dims = (n, c, h, w, o, h, w, 3, 3, 1, 1, 1, 1, groups)
+    dt = _lib.dtype_id(dtype)
+    x = randn((n, c, h, w), 1, dtype).cuda()
+    dy = randn((n, o, h, w), 3, dtype).cuda()
+    nb = lib.at_conv2d_bwd_weight_workspace_bytes(*dims, dt)
+    ws = torch.empty(nb, dtype=torch.uint8, device='cuda')
+    dw = torch.full((o, c // groups, 3, 3), float('nan'), dtype=dtype, device='cuda')
+    _lib.check(lib.at_conv2d_bwd_weight(_lib.ptr(dy), None, _lib.ptr(x), None, _lib.ptr(dw), _lib.ptr(ws), nb,
+                                        *dims, dt, _lib.stream_of(x)), 'dw')
+    ref = torch.nn.grad.conv2d_weight(x.float(), dw.shape, dy.float(), stride=1, padding=1, groups=groups)
+    assert_close(dw, ref.cpu(), dtype, 'weight_grad', normalize=True)
 
 
 BN_SHAPES = [(6, 5), (128, 1024), (2048, 768), (8, 960, 196), (2048, 64, 16), (2, 3, 224, 224),
