@@ -120,7 +120,8 @@ struct OperandLoader {
     for (int i = 0; i < kBigLoads; ++i) issue_one(kt, tile, i);
   }
 
-  // Load i (0 .. kBigLoads-1) of this lane for k-tile `kt`.
+  // Load i (0 .. kBigLoads-1) of this lane for k-tile `kt`; kt < 0 gives an offset that is out of
+  // range (the load writes zeros).
   __device__ __forceinline__ void issue_one(int kt, char* tile, int i) const {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     {
@@ -131,10 +132,10 @@ struct OperandLoader {
         const int row = q * 8 + (lane >> 3);
         const int chunk = (lane & 7) ^ ((row ^ (row >> 3)) & 7);
         const int k = kt * BK + chunk * 8;
-        off = k < K ? lane_off + i * blk_step + k * 2 : kOobOffset;   // K tail reads as zeros
+        off = (kt >= 0 && k < K) ? lane_off + i * blk_step + k * 2 : kOobOffset;   // K tail reads as zeros
         dst = tile + q * 1024;
       } else {
-        off = lane_off + i * blk_step + kt * k_step;                  // k-rows past K fall out of range
+        off = kt >= 0 ? lane_off + i * blk_step + kt * k_step : kOobOffset;        // k-rows past K fall out of range
         dst = tile + q * kPairPitch;
       }
       lds_dma_16(rsrc, off, dst);
@@ -285,11 +286,6 @@ __global__ __launch_bounds__(kBigThreads) void gemm_mfma16_kernel(GemmArgs g) {
   lb.init(B, g.ldb, n0, g.N, g.K);
   const int KT = (g.K + BK - 1) / BK;
 
-  la.issue(0, lds);
-  lb.issue(0, lds + kATile);
-  lds_dma_wait_all();
-  __syncthreads();
-
   auto load_frags = [&](const char* stage, int ks, uint4 (&af)[4], uint4 (&bf)[NJ]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) af[i] = read_frag<A_KC>(stage, wm * 128 + i * 32, ks);
@@ -297,47 +293,66 @@ __global__ __launch_bounds__(kBigThreads) void gemm_mfma16_kernel(GemmArgs g) {
     for (int j = 0; j < NJ; ++j) bf[j] = read_frag<B_KC>(stage + kATile, wn * kBigWaveN + j * 32, ks);
   };
 
-  // One k-tile = four k-steps of 4 * NJ MFMAs per wave.  The other instructions of the iteration
-  // are slotted between MFMAs: the global->LDS loads of the next tile during k-step 0, the
-  // fragment reads of k-step s+1 during k-step s.  The loads of tile kt+1 stay in flight for
-  // the whole iteration and are only waited for at the barrier that ends it.
+  la.issue(0, lds);
+  lb.issue(0, lds + kATile);
+  lds_dma_wait_all();
+  __syncthreads();
+  la.issue(1, lds + kStage);   // k-tile 1 travels while k-tile 0 is multiplied (zeros when there is none)
+  lb.issue(1, lds + kStage + kATile);
+  uint4 af[2][4], bf[2][NJ];
+  load_frags(lds, 0, af[0], bf[0]);
+
+  // One k-tile = four k-steps of 4 * NJ MFMAs per wave, the other instructions slotted between
+  // them.  K-steps 0..2 multiply while the fragments of the following k-step are read.  Before
+  // k-step 3 every fragment of the current stage is in registers, so the one barrier of the
+  // iteration both publishes k-tile kt+1 (issued a whole iteration earlier) and frees the
+  // current stage: k-step 3 multiplies while the loads of k-tile kt+2 are issued into it and the
+  // first fragments of k-tile kt+1 are read, so the MFMAs run on across the barrier.
   // (sched_group_barrier masks: 0x8 MFMA, 0x2 VALU, 0x20 VMEM read, 0x100 LDS read.)
   for (int kt = 0; kt < KT; ++kt) {
     char* cur = lds + (kt & 1) * kStage;
     char* nxt = lds + ((kt & 1) ^ 1) * kStage;
-    uint4 af[2][4], bf[2][NJ];
-    load_frags(cur, 0, af[0], bf[0]);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
-      if (ks + 1 < BK / 16) load_frags(cur, ks + 1, af[(ks + 1) & 1], bf[(ks + 1) & 1]);
+    for (int ks = 0; ks < BK / 16 - 1; ++ks) {
+      load_frags(cur, ks + 1, af[(ks + 1) & 1], bf[(ks + 1) & 1]);
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-          // One global->LDS load of the next tile behind each MFMA of k-step 0 (2 * kBigLoads =
-          // 4 * NJ of either).  Unconditional: past the last k-tile every offset is out of range
-          // and the loads write zeros into a stage nobody reads, so the loop body has no branches.
-          if (ks == 0) {
-            const int t = i * NJ + j;
-            if (t < kBigLoads) la.issue_one(kt + 1, nxt, t);
-            else lb.issue_one(kt + 1, nxt + kATile, t - kBigLoads);
-          }
+        for (int j = 0; j < NJ; ++j)
           // operands swapped: the accumulator holds C^T, i.e. 4 consecutive n per lane
           acc[i][j] = Mfma16<T>::run(bf[ks & 1][j], af[ks & 1][i], acc[i][j]);
-        }
-      if (ks < BK / 16 - 1) {
 #pragma unroll
-        for (int q = 0; q < 4 * NJ; ++q) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
+      for (int q = 0; q < 4 * NJ; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    lds_dma_wait_all();   // this wave's part of the next stage has landed
-    __syncthreads();      // ... and so has everybody else's; the current stage may be overwritten
+    lds_dma_wait_all();   // k-tile kt+1: this wave's part has landed
+    __syncthreads();      // ... and everybody's; nobody reads the current stage any more
+    // Past the last k-tile the loads are issued all the same, with offsets that are out of range:
+    // they write zeros into a stage nobody reads, and the loop body has no branches.
+    const int kt2 = kt + 2 < KT ? kt + 2 : -1;
+    load_frags(nxt, 0, af[0], bf[0]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        // one global->LDS load behind each MFMA (2 * kBigLoads = 4 * NJ of either)
+        const int t = i * NJ + j;
+        if (t < kBigLoads) la.issue_one(kt2, cur, t);
+        else lb.issue_one(kt2, cur + kATile, t - kBigLoads);
+        acc[i][j] = Mfma16<T>::run(bf[1][j], af[1][i], acc[i][j]);
+      }
+#pragma unroll
+    for (int q = 0; q < 4 * NJ; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
   }
+  lds_dma_wait_all();   // the zero-fill loads past the end: the epilogue reuses the stages
 
   big_tile_epilogue<T, ACT>(acc, lds, g, m0, n0);
 }
