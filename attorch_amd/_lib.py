@@ -32,6 +32,7 @@ PROTOTYPES = {
     'at_softmax_bwd': (I, [P, P, P, L, L, L, L, L, I, I, I, I, I, P]),
     'at_cross_entropy_workspace_bytes': (L, [L]),
     'at_cross_entropy_fwd_bwd': (I, [P, P, P, P, P, P, L, L, L, L, L, L, I, I, I, P]),
+    'at_cross_entropy_bwd': (I, [P, P, P, P, P, P, L, L, L, L, L, I, I, I, I, I, P]),
     'at_cross_entropy_scale_grad': (I, [P, P, L, L, L, I, I, P]),
     'at_nll_loss_workspace_bytes': (L, [L, L]),
     'at_nll_loss_fwd': (I, [P, P, P, P, P, P, L, L, L, L, I, I, I, I, P]),
@@ -132,6 +133,21 @@ def require_gpu(tensor: Tensor, what: str) -> None:
     if not tensor.is_cuda:
         raise RuntimeError(f'{what}: expected a tensor on a HIP device (device type "cuda"), '
                            f'received one on {tensor.device}; there is no CPU path')
+
+
+def require_same_device(what: str, reference: Tensor, *others: Optional[Tensor]) -> None:
+    """
+    Every tensor whose address goes to a kernel must live on the device of `reference` (the
+    tensor whose device the launch runs on): a host pointer, or one of another GPU, handed to a
+    kernel ends in a memory fault instead of an error.  Absent optionals (None) are skipped.
+    """
+    require_gpu(reference, what)
+    for other in others:
+        if other is None:
+            continue
+        if other.device != reference.device:
+            raise RuntimeError(f'{what}: expected all tensors on {reference.device}, '
+                               f'received one on {other.device}')
 
 
 def rows(tensor: Tensor) -> Tensor:

@@ -4,7 +4,8 @@ Cross entropy loss with PyTorch autodiff support, running on the fused gfx950 ke
 API mirrors attorch/cross_entropy_loss_layer.py (mean reduction only, no label smoothing,
 optional class weights) and adds what the reference lacks: ignore_index.  The forward pass
 reads the logits once and produces both the loss and, when the logits require a gradient,
-the gradient for an upstream gradient of one; backward only rescales it.
+the gradient for an upstream gradient of one; backward hands that gradient out when the
+upstream gradient is one and recomputes it from the logits otherwise.
 """
 
 from typing import Any, Optional, Tuple
@@ -47,10 +48,16 @@ class CrossEntropyLossAutoGrad(torch.autograd.Function):
         assert weight is None or len(weight) == input.shape[1], \
             f'Dimensionality of weight vector ({len(weight)}) and input features ({input.shape[1]}) not equal'
 
-        _lib.require_gpu(input, 'CrossEntropyLoss')
+        _lib.require_same_device('CrossEntropyLoss', input, target, weight)
         lib = _lib.load()
         batch_dim, feat_dim = input.shape
         output_dtype = get_output_dtype(input.dtype, autocast='fp32')
+
+        if batch_dim == 0:
+            # mean over no rows, as torch: nan loss, empty gradient; nothing is launched
+            ctx.empty = True
+            ctx.grad_shape_dtype = (input.shape, output_dtype, input.device)
+            return torch.full((), float('nan'), dtype=output_dtype, device=input.device)
 
         logits = input if input.stride(1) == 1 and input.stride(0) >= feat_dim else input.contiguous()
         target_k = target.to(torch.int64).contiguous()
@@ -69,9 +76,17 @@ class CrossEntropyLossAutoGrad(torch.autograd.Function):
                 _lib.dtype_id(weight_k.dtype) if weight_k is not None else 0,
                 _lib.dtype_id(output_dtype), _lib.stream_of(input)), 'at_cross_entropy_fwd_bwd')
 
+        ctx.empty = False
         ctx.output_dtype = output_dtype
+        ctx.ignore_index = ignore_index
+        ctx.has_weight = weight_k is not None
+        # the gradient computed above may be handed to autograd once; see backward
+        ctx.unit_grad_available = input.requires_grad
         if input.requires_grad:
-            ctx.save_for_backward(input_grad)
+            saved = [logits, target_k, workspace, input_grad]
+            if weight_k is not None:
+                saved.append(weight_k)
+            ctx.save_for_backward(*saved)
 
         return output
 
@@ -81,22 +96,42 @@ class CrossEntropyLossAutoGrad(torch.autograd.Function):
         output_grad: Tensor,
         ) -> Tuple[Optional[Tensor], ...]:
         """
-        Gradient of the logits: the one computed in forward, times the upstream gradient
-        (read on the device; nothing is rewritten when it is exactly one).
+        Gradient of the logits, output_grad * (softmax - onehot) * weight[target] / divisor
+        (attorch/cross_entropy_loss_layer.py:85-121).  The first call returns the buffer the
+        forward pass filled for an upstream gradient of one: the kernel leaves it as it is when
+        the upstream value (read on the device) is exactly one and recomputes it from the
+        logits otherwise, the upstream value multiplied in before the one rounding.  That
+        buffer then belongs to autograd, so any later call (retain_graph) computes into a
+        fresh one.
         """
+        if ctx.empty:
+            shape, dtype, device = ctx.grad_shape_dtype
+            return torch.empty(shape, dtype=dtype, device=device), None, None, None
+
         lib = _lib.load()
-        (input_grad,) = ctx.saved_tensors
-        batch_dim, feat_dim = input_grad.shape
+        logits, target_k, workspace, unit_grad = ctx.saved_tensors[:4]
+        weight_k = ctx.saved_tensors[4] if ctx.has_weight else None
+        batch_dim, feat_dim = logits.shape
+        _lib.require_same_device('CrossEntropyLoss backward', logits, output_grad)
         output_grad = output_grad.contiguous()
         if output_grad.dtype not in _lib.DTYPE_IDS:
             output_grad = output_grad.float()
 
-        with torch.cuda.device_of(input_grad):
-            _lib.check(lib.at_cross_entropy_scale_grad(
-                _lib.ptr(input_grad), _lib.ptr(output_grad), batch_dim, feat_dim,
-                _lib.row_stride(input_grad), _lib.dtype_id(input_grad.dtype),
-                _lib.dtype_id(output_grad.dtype), _lib.stream_of(input_grad)),
-                'at_cross_entropy_scale_grad')
+        if ctx.unit_grad_available:
+            input_grad, holds_unit_grad = unit_grad, 1
+            ctx.unit_grad_available = False
+        else:
+            input_grad, holds_unit_grad = torch.empty_like(unit_grad), 0
+
+        with torch.cuda.device_of(logits):
+            _lib.check(lib.at_cross_entropy_bwd(
+                _lib.ptr(logits), _lib.ptr(target_k), _lib.ptr(weight_k), _lib.ptr(output_grad),
+                _lib.ptr(workspace), _lib.ptr(input_grad), batch_dim, feat_dim,
+                _lib.row_stride(logits), feat_dim, ctx.ignore_index, holds_unit_grad,
+                _lib.dtype_id(logits.dtype),
+                _lib.dtype_id(weight_k.dtype) if weight_k is not None else 0,
+                _lib.dtype_id(output_grad.dtype), _lib.dtype_id(input_grad.dtype),
+                _lib.stream_of(logits)), 'at_cross_entropy_bwd')
 
         return input_grad, None, None, None
 

@@ -8,8 +8,14 @@
 // fp16 logits makes every other row start on an odd element): a row is addressed through
 // the 16-byte grid of its own address space, interior vectors move with 128-bit accesses and
 // only the first and last vector of a row fall back to guarded element accesses.  The
-// gradient row must sit at the same phase of the 16-byte grid as the logits row for this
-// path; anything else (or a different gradient dtype) takes the streaming kernel.
+// gradient may be stored in the dtype of the logits or in fp32 (16-bit logits under autocast);
+// its rows must sit at the phase of the 16-byte grid that matches the logits row for this
+// path, anything else takes the streaming kernel.
+//
+// The same kernels serve the backward entry point: with an upstream gradient pointer they
+// skip the loss, multiply the scale by the upstream value in fp32 before the one rounding
+// (as the reference's backward kernel does) and, when told that the destination already holds
+// the gradient for an upstream value of one, return at once if the value is exactly one.
 #include <type_traits>
 
 #include "at_common.h"
@@ -63,27 +69,53 @@ __global__ __launch_bounds__(1024) void ce_finalize_kernel(
   if (threadIdx.x == 0) store_scalar_f32(loss, out_dt, 0, s / denom[0]);
 }
 
-// Register-cached row kernel.  T is the dtype of both the logits and the gradient.
+// Stores the 16 / sizeof(T) gradient values of interior vector v of a row; `base` is the address of
+// the row's first interior element in the gradient (16-byte aligned, host check).
+template <typename T, typename TO>
+__device__ __forceinline__ void store_grad_vec(TO* __restrict__ base, int v, const float (&f)[16 / sizeof(T)]) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  if constexpr (std::is_same<T, TO>::value) {
+    reinterpret_cast<uint4*>(base)[v] = pack16<T>(f);
+  } else {   // fp32 gradient of 16-bit logits: 32 contiguous bytes per lane
+    float4* dst = reinterpret_cast<float4*>(base + (int64_t)v * VEC);
+    dst[0] = make_float4(f[0], f[1], f[2], f[3]);
+    dst[1] = make_float4(f[4], f[5], f[6], f[7]);
+  }
+}
+
+// Upstream gradient of the backward entry point: 1 in the forward call (no pointer).  Returns false
+// when nothing has to be computed (the destination already holds the gradient for the value 1).
+__device__ __forceinline__ bool read_upstream(const void* upstream, int gdt, int skip_if_one, float& g) {
+  g = 1.f;
+  if (!upstream) return true;
+  g = load_scalar_f32(upstream, gdt, 0);
+  return !(skip_if_one && g == 1.f);
+}
+
+// Register-cached row kernel.  T is the dtype of the logits, TO of the gradient (T or float).
 // A row is split into "interior" 16-byte vectors (fully inside the row, 128-bit accesses) and
 // at most 7 + 7 "edge" elements before the first and after the last interior vector, each
 // owned by one of the first 16 lanes and moved with element accesses.
-template <typename T, int CACHE_VECS>
+template <typename T, typename TO, int CACHE_VECS>
 __global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_kernel(
     const T* __restrict__ logits, const int64_t* __restrict__ target, const void* __restrict__ weight,
-    int wdt, const float* __restrict__ denom, float* __restrict__ row_loss, T* __restrict__ dlogits,
-    int feat, int64_t xs, int64_t ds, int64_t ignore_index) {
+    int wdt, const float* __restrict__ denom, float* __restrict__ row_loss, TO* __restrict__ dlogits,
+    int feat, int64_t xs, int64_t ds, int64_t ignore_index, const void* __restrict__ upstream, int gdt,
+    int skip_if_one) {
   constexpr int VEC = 16 / (int)sizeof(T);
   __shared__ float scratch[16];
+  float up;
+  if (!read_upstream(upstream, gdt, skip_if_one, up)) return;
   const int tid = threadIdx.x;
   const int64_t row = blockIdx.x;
   const T* xr = logits + row * xs;
-  T* dr = dlogits ? dlogits + row * ds : nullptr;
+  TO* dr = dlogits ? dlogits + row * ds : nullptr;
   const int off = (int)((reinterpret_cast<uintptr_t>(xr) & 15u) / sizeof(T));
   const int head_n = off ? (VEC - off < feat ? VEC - off : feat) : 0;  // row elements [0, head_n)
   const int n_int = (feat - head_n) / VEC;                             // interior vectors
   const int tail0 = head_n + n_int * VEC;                              // row elements [tail0, feat)
   const uint4* xv = reinterpret_cast<const uint4*>(xr + head_n);       // 16-byte aligned
-  uint4* dv = dr ? reinterpret_cast<uint4*>(dr + head_n) : nullptr;    // same phase (host check)
+  TO* dv = dr ? dr + head_n : nullptr;                                 // 16-byte aligned too (host check)
   // edge element owned by this lane, -1 if none
   const int edge = tid < 8 ? (tid < head_n ? tid : -1)
                            : (tid < 16 && tail0 + tid - 8 < feat ? tail0 + tid - 8 : -1);
@@ -91,10 +123,13 @@ __global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_k
   const bool kept = target_kept(t, ignore_index, feat);
 
   if (!kept) {
-    if (tid == 0) row_loss[row] = 0.f;
+    if (tid == 0 && row_loss) row_loss[row] = 0.f;
     if (dr) {
-      for (int v = tid; v < n_int; v += kCeBlock) dv[v] = make_uint4(0, 0, 0, 0);
-      if (edge >= 0) dr[edge] = from_f32<T>(0.f);
+      float zero[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) zero[j] = 0.f;
+      for (int v = tid; v < n_int; v += kCeBlock) store_grad_vec<T, TO>(dv, v, zero);
+      if (edge >= 0) dr[edge] = from_f32<TO>(0.f);
     }
     return;
   }
@@ -153,10 +188,10 @@ __global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_k
 
   const float wt = weight ? load_scalar_f32(weight, wdt, t) : 1.f;
   const float x_t = to_f32(xr[t]);
-  if (tid == 0) row_loss[row] = (__logf(s) - x_t + m) * wt;
+  if (tid == 0 && row_loss) row_loss[row] = (__logf(s) - x_t + m) * wt;
   if (!dr) return;
 
-  const float scale = wt / denom[0];
+  const float scale = wt / denom[0] * up;
   const float k = scale / s;
 #pragma unroll
   for (int i = 0; i < CACHE_VECS; ++i) {
@@ -166,15 +201,15 @@ __global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_k
       unpack16<T>(cache[i], f);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) f[j] *= k;
-      dv[v] = pack16<T>(f);
+      store_grad_vec<T, TO>(dv, v, f);
     }
   }
-  if (edge >= 0) dr[edge] = from_f32<T>(edge_e * k);
+  if (edge >= 0) dr[edge] = from_f32<TO>(edge_e * k);
   // The target column gets softmax - 1: the lane that stored the column overwrites it (stores of
   // one lane to one address stay in order).
   const int tv = (int)t - head_n;   // target position relative to the first interior element
   const bool owner = (tv >= 0 && tv < n_int * VEC) ? ((tv / VEC) % kCeBlock == tid) : (edge == (int)t);
-  if (owner) dr[t] = from_f32<T>(fmaf(__builtin_amdgcn_exp2f(fmaf(x_t, kLog2e, -m2)), k, -scale));
+  if (owner) dr[t] = from_f32<TO>(fmaf(__builtin_amdgcn_exp2f(fmaf(x_t, kLog2e, -m2)), k, -scale));
 }
 
 // Streaming kernel: any dtypes, any alignment, any width; the row is read twice (online
@@ -183,15 +218,18 @@ template <typename T, typename TO>
 __global__ __launch_bounds__(1024) void ce_row_stream_kernel(
     const T* __restrict__ logits, const int64_t* __restrict__ target, const void* __restrict__ weight,
     int wdt, const float* __restrict__ denom, float* __restrict__ row_loss, TO* __restrict__ dlogits,
-    int feat, int64_t xs, int64_t ds, int64_t ignore_index) {
+    int feat, int64_t xs, int64_t ds, int64_t ignore_index, const void* __restrict__ upstream, int gdt,
+    int skip_if_one) {
   __shared__ float scratch[16];
+  float up;
+  if (!read_upstream(upstream, gdt, skip_if_one, up)) return;
   const int64_t row = blockIdx.x;
   const T* xr = logits + row * xs;
   TO* dr = dlogits ? dlogits + row * ds : nullptr;
   const int64_t t = target[row];
   const bool kept = target_kept(t, ignore_index, feat);
   if (!kept) {
-    if (threadIdx.x == 0) row_loss[row] = 0.f;
+    if (threadIdx.x == 0 && row_loss) row_loss[row] = 0.f;
     if (dr)
       for (int c = threadIdx.x; c < feat; c += blockDim.x) dr[c] = from_f32<TO>(0.f);
     return;
@@ -203,9 +241,9 @@ __global__ __launch_bounds__(1024) void ce_row_stream_kernel(
   for (int c = threadIdx.x; c < feat; c += blockDim.x) s += __expf(to_f32(xr[c]) - m);
   s = group_reduce(s, (int)blockDim.x, scratch, SumOp(), 0.f);
   const float wt = weight ? load_scalar_f32(weight, wdt, t) : 1.f;
-  if (threadIdx.x == 0) row_loss[row] = (__logf(s) - to_f32(xr[t]) + m) * wt;
+  if (threadIdx.x == 0 && row_loss) row_loss[row] = (__logf(s) - to_f32(xr[t]) + m) * wt;
   if (!dr) return;
-  const float scale = wt / denom[0];
+  const float scale = wt / denom[0] * up;
   const float k = scale / s;
   for (int c = threadIdx.x; c < feat; c += blockDim.x) {
     float g = __expf(to_f32(xr[c]) - m) * k;
@@ -259,6 +297,82 @@ inline int dispatch_one(int dt, F&& f) {
   return AT_ERR_DTYPE;
 }
 
+// One row kernel launch: loss and/or gradient rows.  upstream == nullptr: forward call.
+int launch_ce_rows(const void* logits, const int64_t* target, const void* weight, const float* denom,
+                   float* row_loss, void* dlogits, int64_t batch, int64_t feat, int64_t logits_stride,
+                   int64_t dlogits_stride, int64_t ignore_index, int logits_dtype, int weight_dtype,
+                   int out_dtype, const void* upstream, int grad_dtype, int skip_if_one, hipStream_t stream) {
+  const int es = dtype_size(logits_dtype), os = dtype_size(out_dtype);
+  const int vec = 16 / es;
+  const int64_t max_vecs = cdiv64(feat, vec);
+  // The gradient row must reach a 16-byte boundary at the same element as the logits row does.
+  const uintptr_t la = reinterpret_cast<uintptr_t>(logits), da = reinterpret_cast<uintptr_t>(dlogits);
+  bool same_phase = true;
+  if (dlogits) {
+    const int64_t unit = 16 / os;   // elements of the gradient per 16 bytes
+    same_phase = (la % es) == 0 && (da % os) == 0 &&
+                 ((int64_t)(da / os) - (int64_t)(la / es)) % unit == 0 && (dlogits_stride - logits_stride) % unit == 0;
+  }
+  const bool cached = same_phase && max_vecs <= (int64_t)kCeBlock * 16 && (la % es) == 0;
+
+  return dispatch_one(logits_dtype, [&](auto* tp) -> int {
+    typedef std::remove_pointer_t<decltype(tp)> T;
+    auto run = [&](auto* top) -> int {
+      typedef std::remove_pointer_t<decltype(top)> TO;
+      if (cached) {
+        const int per_lane = (int)cdiv64(max_vecs, kCeBlock);
+#define AT_CE_LAUNCH(CV)                                                                              \
+  hipLaunchKernelGGL((ce_row_kernel<T, TO, CV>), dim3((unsigned)batch), dim3(kCeBlock), 0, stream,    \
+                     (const T*)logits, target, weight, weight_dtype, denom, row_loss, (TO*)dlogits,   \
+                     (int)feat, logits_stride, dlogits_stride, ignore_index, upstream, grad_dtype, skip_if_one)
+        if (per_lane <= 2) AT_CE_LAUNCH(2);
+        else if (per_lane <= 4) AT_CE_LAUNCH(4);
+        else if (per_lane <= 8) AT_CE_LAUNCH(8);
+        else if (per_lane <= 13) AT_CE_LAUNCH(13);   // up to 13 vectors: registers for three workgroups per CU
+        else AT_CE_LAUNCH(16);
+#undef AT_CE_LAUNCH
+      } else {
+        hipLaunchKernelGGL((ce_row_stream_kernel<T, TO>), dim3((unsigned)batch), dim3(1024), 0, stream,
+                           (const T*)logits, target, weight, weight_dtype, denom, row_loss, (TO*)dlogits,
+                           (int)feat, logits_stride, dlogits_stride, ignore_index, upstream, grad_dtype,
+                           skip_if_one);
+      }
+      return launch_status();
+    };
+    if (out_dtype == logits_dtype) return run((T*)0);
+    return run((float*)0);
+  });
+}
+
+int check_ce_args(const void* logits, const int64_t* target, const void* weight, int64_t batch, int64_t feat,
+                  int64_t logits_stride, const void* dlogits, int64_t dlogits_stride, int logits_dtype,
+                  int weight_dtype, int out_dtype) {
+  if (!logits || !target) return AT_ERR_NULL;
+  if (!dtype_valid(logits_dtype) || !dtype_valid(out_dtype) || (weight && !dtype_valid(weight_dtype)))
+    return AT_ERR_DTYPE;
+  if (!(out_dtype == logits_dtype || out_dtype == AT_DTYPE_F32)) return AT_ERR_DTYPE;
+  if (batch <= 0 || feat <= 0 || feat > ((int64_t)1 << 30)) return AT_ERR_DIM;
+  if (logits_stride < feat || (dlogits && dlogits_stride < feat)) return AT_ERR_DIM;
+  return AT_OK;
+}
+
+// Forward call on a given workspace.
+int ce_fwd_bwd(const void* logits, const int64_t* target, const void* weight, void* loss, void* dlogits,
+               float* workspace, int64_t batch, int64_t feat, int64_t logits_stride, int64_t dlogits_stride,
+               int64_t ignore_index, int logits_dtype, int weight_dtype, int out_dtype, hipStream_t stream) {
+  float* denom = workspace;
+  float* row_loss = denom + 4;
+  hipLaunchKernelGGL(ce_denominator_kernel, dim3(1), dim3(1024), 0, stream, target, weight, weight_dtype,
+                     denom, batch, (int)feat, ignore_index);
+  int rc = launch_ce_rows(logits, target, weight, denom, row_loss, dlogits, batch, feat, logits_stride,
+                          dlogits_stride, ignore_index, logits_dtype, weight_dtype, out_dtype, nullptr, 0, 0,
+                          stream);
+  if (rc) return rc;
+  hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(1024), 0, stream, row_loss, denom, loss, out_dtype,
+                     batch);
+  return launch_status();
+}
+
 }  // namespace
 }  // namespace at_hip
 
@@ -276,59 +390,30 @@ int at_cross_entropy_fwd_bwd(const void* logits, const int64_t* target, const vo
                              int64_t feat, int64_t logits_stride, int64_t dlogits_stride,
                              int64_t ignore_index, int logits_dtype, int weight_dtype, int out_dtype,
                              at_stream_t stream_) {
-  hipStream_t stream = (hipStream_t)stream_;
-  if (!logits || !target || !loss) return AT_ERR_NULL;
-  if (!dtype_valid(logits_dtype) || !dtype_valid(out_dtype) || (weight && !dtype_valid(weight_dtype)))
-    return AT_ERR_DTYPE;
-  if (!(out_dtype == logits_dtype || out_dtype == AT_DTYPE_F32)) return AT_ERR_DTYPE;
-  if (batch <= 0 || feat <= 0 || feat > ((int64_t)1 << 30)) return AT_ERR_DIM;
-  if (logits_stride < feat || (dlogits && dlogits_stride < feat)) return AT_ERR_DIM;
+  if (!loss) return AT_ERR_NULL;
+  int rc = check_ce_args(logits, target, weight, batch, feat, logits_stride, dlogits, dlogits_stride,
+                         logits_dtype, weight_dtype, out_dtype);
+  if (rc) return rc;
   if (!workspace || workspace_bytes < at_cross_entropy_workspace_bytes(batch)) return AT_ERR_WORKSPACE;
   if ((reinterpret_cast<uintptr_t>(workspace) & 3u) != 0) return AT_ERR_ALIGN;
+  return ce_fwd_bwd(logits, target, weight, loss, dlogits, (float*)workspace, batch, feat, logits_stride,
+                    dlogits_stride, ignore_index, logits_dtype, weight_dtype, out_dtype, (hipStream_t)stream_);
+}
 
-  float* denom = (float*)workspace;
-  float* row_loss = denom + 4;
-  hipLaunchKernelGGL(ce_denominator_kernel, dim3(1), dim3(1024), 0, stream, target, weight, weight_dtype,
-                     denom, batch, (int)feat, ignore_index);
-
-  const int es = dtype_size(logits_dtype);
-  const int vec = 16 / es;
-  const int64_t max_vecs = cdiv64(feat, vec);
-  const bool same_phase =
-      !dlogits || (((reinterpret_cast<uintptr_t>(dlogits) ^ reinterpret_cast<uintptr_t>(logits)) & 15u) == 0 &&
-                   ((dlogits_stride - logits_stride) * es) % 16 == 0);
-  const bool cached = out_dtype == logits_dtype && same_phase && max_vecs <= (int64_t)kCeBlock * 16 &&
-                      (reinterpret_cast<uintptr_t>(logits) % es) == 0;
-
-  int rc = dispatch_one(logits_dtype, [&](auto* tp) -> int {
-    typedef std::remove_pointer_t<decltype(tp)> T;
-    if (cached) {
-      const int per_lane = (int)cdiv64(max_vecs, kCeBlock);
-#define AT_CE_LAUNCH(CV)                                                                          \
-  hipLaunchKernelGGL((ce_row_kernel<T, CV>), dim3((unsigned)batch), dim3(kCeBlock), 0, stream,    \
-                     (const T*)logits, target, weight, weight_dtype, denom, row_loss, (T*)dlogits, \
-                     (int)feat, logits_stride, dlogits_stride, ignore_index)
-      if (per_lane <= 2) AT_CE_LAUNCH(2);
-      else if (per_lane <= 4) AT_CE_LAUNCH(4);
-      else if (per_lane <= 8) AT_CE_LAUNCH(8);
-      else if (per_lane <= 13) AT_CE_LAUNCH(13);   // up to 13 vectors: registers for three workgroups per CU
-      else AT_CE_LAUNCH(16);
-#undef AT_CE_LAUNCH
-    } else if (out_dtype == logits_dtype) {
-      hipLaunchKernelGGL((ce_row_stream_kernel<T, T>), dim3((unsigned)batch), dim3(1024), 0, stream,
-                         (const T*)logits, target, weight, weight_dtype, denom, row_loss, (T*)dlogits,
-                         (int)feat, logits_stride, dlogits_stride, ignore_index);
-    } else {
-      hipLaunchKernelGGL((ce_row_stream_kernel<T, float>), dim3((unsigned)batch), dim3(1024), 0, stream,
-                         (const T*)logits, target, weight, weight_dtype, denom, row_loss, (float*)dlogits,
-                         (int)feat, logits_stride, dlogits_stride, ignore_index);
-    }
-    return launch_status();
-  });
+int at_cross_entropy_bwd(const void* logits, const int64_t* target, const void* weight,
+                         const void* output_grad, const void* workspace, void* dlogits, int64_t batch,
+                         int64_t feat, int64_t logits_stride, int64_t dlogits_stride, int64_t ignore_index,
+                         int holds_unit_grad, int logits_dtype, int weight_dtype, int grad_dtype,
+                         int out_dtype, at_stream_t stream_) {
+  if (!output_grad || !workspace || !dlogits) return AT_ERR_NULL;
+  int rc = check_ce_args(logits, target, weight, batch, feat, logits_stride, dlogits, dlogits_stride,
+                         logits_dtype, weight_dtype, out_dtype);
   if (rc) return rc;
-  hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(1024), 0, stream, row_loss, denom, loss, out_dtype,
-                     batch);
-  return launch_status();
+  if (!dtype_valid(grad_dtype)) return AT_ERR_DTYPE;
+  if ((reinterpret_cast<uintptr_t>(workspace) & 3u) != 0) return AT_ERR_ALIGN;
+  return launch_ce_rows(logits, target, weight, (const float*)workspace, nullptr, dlogits, batch, feat,
+                        logits_stride, dlogits_stride, ignore_index, logits_dtype, weight_dtype, out_dtype,
+                        output_grad, grad_dtype, holds_unit_grad ? 1 : 0, (hipStream_t)stream_);
 }
 
 int at_cross_entropy_scale_grad(void* dlogits, const void* output_grad, int64_t batch, int64_t feat,

@@ -148,9 +148,18 @@ int at_softmax_bwd(const void* dy, const void* y, void* dx, int64_t batch, int64
  * Rows whose target equals ignore_index — or lies outside [0, feat) — contribute nothing and
  * get an all-zero gradient row. loss is one element of out_dtype; workspace needs
  * at_cross_entropy_workspace_bytes(batch) bytes; on return workspace[0] (fp32) holds denom.
- * at_cross_entropy_scale_grad multiplies dlogits in place by the upstream gradient, read on
- * the device as one element of grad_dtype (cross_entropy_loss_kernels.py:155); it returns
- * without touching memory when that value is exactly 1.
+ * dlogits may have the dtype of the logits or be fp32 (the reference's autocast policy returns
+ * an fp32 loss and gradient for 16-bit logits, cross_entropy_loss_layer.py:59,108).
+ * at_cross_entropy_bwd is the reference's backward kernel (cross_entropy_loss_kernels.py:96-172):
+ * dlogits = output_grad * (softmax - onehot) * w[target] / denom, recomputed from the logits,
+ * with output_grad read on the device as one element of grad_dtype (:155) and multiplied in
+ * fp32 before the one rounding.  `workspace` is the one the forward call filled (it only reads
+ * workspace[0], the divisor).  holds_unit_grad != 0 states that dlogits already holds the
+ * gradient the forward call produced (upstream gradient 1): the call then leaves it untouched
+ * when output_grad is exactly 1 and overwrites it otherwise.
+ * at_cross_entropy_scale_grad multiplies dlogits in place by the upstream gradient (it returns
+ * without touching memory when that value is exactly 1); the product is rounded from the
+ * already rounded gradient, so prefer at_cross_entropy_bwd for 16-bit gradients.
  * ------------------------------------------------------------------------------------------ */
 int64_t at_cross_entropy_workspace_bytes(int64_t batch);
 
@@ -159,6 +168,13 @@ int at_cross_entropy_fwd_bwd(const void* logits, const int64_t* target, const vo
                              int64_t batch, int64_t feat, int64_t logits_stride,
                              int64_t dlogits_stride, int64_t ignore_index, int logits_dtype,
                              int weight_dtype, int out_dtype, at_stream_t stream);
+
+int at_cross_entropy_bwd(const void* logits, const int64_t* target, const void* weight,
+                         const void* output_grad, const void* workspace, void* dlogits,
+                         int64_t batch, int64_t feat, int64_t logits_stride,
+                         int64_t dlogits_stride, int64_t ignore_index, int holds_unit_grad,
+                         int logits_dtype, int weight_dtype, int grad_dtype, int out_dtype,
+                         at_stream_t stream);
 
 int at_cross_entropy_scale_grad(void* dlogits, const void* output_grad, int64_t batch,
                                 int64_t feat, int64_t dlogits_stride, int dlogits_dtype,

@@ -110,3 +110,118 @@ def test_unaligned_base_pointer() -> None:
     assert_close(loss, ref, torch.float16, 'loss')
     grad_ref = oracle.cross_entropy_backward(torch.tensor(1.0), x.cpu(), target.cpu(), None, -100, torch.float16)
     assert_close(xd.grad.float() * 8, grad_ref.float() * 8, torch.float16, 'input_grad')
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+def test_backward_twice_through_a_retained_graph(dtype) -> None:
+    # every backward through a retained graph gives output_grad times the unit gradient, whatever
+    # came before; the tensor a call returned is never written again
+    x = randn((48, 1000), 1, dtype, 2.0)
+    target = make_targets(48, 1000, 2, 0.1)
+    cd = compute_dtype(dtype)
+    xd = x.cuda().requires_grad_(True)
+    loss = attorch_amd.CrossEntropyLossAutoGrad.apply(xd, target.cuda(), None, -100)
+    kept = float((target != -100).sum())
+    results = []
+    for upstream in (3.0, 3.0, 1.0, 0.25):
+        (grad,) = torch.autograd.grad(loss, xd, torch.tensor(upstream, dtype=loss.dtype, device='cuda'),
+                                      retain_graph=True)
+        ref = oracle.cross_entropy_backward(torch.tensor(upstream), x, target, None, -100, dtype, compute=cd)
+        results.append((grad, grad.clone(), ref))
+    for grad, snapshot, ref in results:
+        assert torch.equal(grad, snapshot), 'a gradient handed out earlier was modified by a later call'
+        assert_close(grad * kept, ref.to(cd) * kept, dtype, 'input_grad')
+    assert len({g.data_ptr() for g, _, _ in results}) == len(results), 'calls must not share a buffer'
+
+
+def test_backward_with_upstream_one_returns_the_forward_gradient_without_a_copy() -> None:
+    x = randn((16, 512), 1, torch.float32, 2.0)
+    target = make_targets(16, 512, 2, 0.0)
+    xd = x.cuda().requires_grad_(True)
+    loss = attorch_amd.CrossEntropyLossAutoGrad.apply(xd, target.cuda(), None, -100)
+    loss.backward()
+    ref = oracle.cross_entropy_backward(torch.tensor(1.0), x, target, None, -100, torch.float32,
+                                        compute=torch.float64)
+    assert_close(xd.grad * 16, ref * 16, torch.float32, 'input_grad')
+
+
+def test_fp16_loss_scale_is_applied_before_rounding() -> None:
+    # vocabulary-wide rows: probability / rows is far below fp16's smallest subnormal, so a
+    # gradient rounded at upstream 1 and scaled afterwards would be all zeros off the target column
+    rows, vocab, scale = 1024, 50257, 32768.0   # the largest power of two below fp16's maximum
+    x = randn((rows, vocab), 1, torch.float16, 2.0)
+    target = make_targets(rows, vocab, 2, 0.05)
+    xd = x.cuda().requires_grad_(True)
+    loss = attorch_amd.CrossEntropyLossAutoGrad.apply(xd, target.cuda(), None, -100)
+    loss.backward(torch.tensor(scale, dtype=torch.float16, device='cuda'))
+    ref = oracle.cross_entropy_backward(torch.tensor(scale), x, target, None, -100, torch.float16)
+    kept = target != -100
+    got = xd.grad.cpu()
+    assert torch.all(got[~kept] == 0)
+    nonzero_ref = (ref[kept] != 0).float().mean().item()
+    nonzero_got = (got[kept] != 0).float().mean().item()
+    assert nonzero_ref > 0.5, 'the case must exercise values that survive only with the scale applied first'
+    assert abs(nonzero_got - nonzero_ref) < 0.01
+    mass_ref, mass_got = ref.float().abs().sum().item(), got.float().abs().sum().item()
+    assert abs(mass_got - mass_ref) < 2e-2 * mass_ref
+    per_row = float(kept.sum()) / scale
+    assert_close(got.float() * per_row, ref.float() * per_row, torch.float16, 'input_grad')
+
+
+def test_autocast_at_vocabulary_width() -> None:
+    # the reference's policy: fp16 logits under autocast give an fp32 loss and an fp32 gradient
+    rows, vocab = 8192, 50257
+    x = randn((rows, vocab), 3001, torch.float16, 2.0)
+    gen = torch.Generator().manual_seed(3002)
+    target = torch.randint(0, vocab, (rows,), generator=gen)
+    target[torch.rand(rows, generator=gen) < 0.05] = -100
+    xd = x.cuda().requires_grad_(True)
+    with torch.autocast('cuda', dtype=torch.float16):
+        loss = attorch_amd.CrossEntropyLoss()(xd, target.cuda())
+    loss.backward()
+    assert loss.dtype is torch.float32 and xd.grad.dtype is torch.float16   # autograd casts to the leaf's dtype
+    keep = target != -100
+    denom = float(keep.sum())
+    total = torch.zeros((), dtype=torch.float64)
+    for start in range(0, rows, 1024):
+        sl = slice(start, start + 1024)
+        part, part_denom = oracle.cross_entropy_forward(x[sl], target[sl], None, -100, torch.float64)
+        total += part * part_denom.double()
+    assert_close(loss, (total / denom).float(), torch.float32, 'loss')
+    # the fp32 gradient itself (autograd casts it to the leaf's dtype): the same call through the C ABI
+    from attorch_amd import _lib
+    lib = _lib.load()
+    logits_d, target_d = x.cuda(), target.cuda()
+    grad = torch.empty(rows, vocab, dtype=torch.float32, device='cuda')
+    loss32 = torch.empty((), dtype=torch.float32, device='cuda')
+    ws_bytes = lib.at_cross_entropy_workspace_bytes(rows)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device='cuda')
+    _lib.check(lib.at_cross_entropy_fwd_bwd(
+        logits_d.data_ptr(), target_d.data_ptr(), None, loss32.data_ptr(), grad.data_ptr(), ws.data_ptr(), ws_bytes,
+        rows, vocab, vocab, vocab, -100, _lib.dtype_id(torch.float16), 0, _lib.dtype_id(torch.float32),
+        _lib.stream_of(logits_d)), 'at_cross_entropy_fwd_bwd')
+    assert torch.equal(loss32, loss.detach())
+    for start in (0, 4096, 8192 - 128):
+        sl = slice(start, start + 128)
+        local = float(keep[sl].sum())
+        ref = oracle.cross_entropy_backward(torch.tensor(local / denom), x[sl], target[sl], None, -100,
+                                            torch.float32, compute=torch.float64)
+        assert_close(grad[sl] * denom, ref * denom, torch.float32, 'input_grad slice', atol_scale=10)
+    assert torch.all(grad[(~keep).cuda()] == 0)
+    assert_close(xd.grad[:256].float() * denom, grad[:256] * denom, torch.float16, 'gradient cast to the leaf dtype')
+
+
+def test_empty_batch_gives_nan_loss_and_empty_gradient() -> None:
+    x = torch.empty(0, 7, device='cuda', requires_grad=True)
+    loss = attorch_amd.CrossEntropyLoss()(x, torch.empty(0, dtype=torch.int64, device='cuda'))
+    assert math.isnan(loss.item())
+    loss.backward()
+    assert x.grad.shape == (0, 7)
+
+
+def test_host_tensors_raise_instead_of_faulting() -> None:
+    x = randn((4, 9), 1).cuda().requires_grad_(True)
+    with pytest.raises(RuntimeError, match='expected all tensors on'):
+        attorch_amd.CrossEntropyLoss()(x, torch.zeros(4, dtype=torch.int64))          # target on the host
+    with pytest.raises(RuntimeError, match='expected all tensors on'):
+        attorch_amd.CrossEntropyLoss(weight=torch.ones(9))(x, torch.zeros(4, dtype=torch.int64, device='cuda'))
