@@ -297,6 +297,10 @@ inline int dispatch_one(int dt, F&& f) {
   return AT_ERR_DTYPE;
 }
 
+// Per-device address of the library's own workspace for the allocation-free entry point.
+constexpr int64_t kCeStaticMaxBatch = 65536;
+constexpr int kCeMaxDevices = 64;
+
 // One row kernel launch: loss and/or gradient rows.  upstream == nullptr: forward call.
 int launch_ce_rows(const void* logits, const int64_t* target, const void* weight, const float* denom,
                    float* row_loss, void* dlogits, int64_t batch, int64_t feat, int64_t logits_stride,
@@ -356,7 +360,7 @@ int check_ce_args(const void* logits, const int64_t* target, const void* weight,
   return AT_OK;
 }
 
-// Forward call on a given workspace.
+// Forward call on a given workspace (the caller's or the library's own).
 int ce_fwd_bwd(const void* logits, const int64_t* target, const void* weight, void* loss, void* dlogits,
                float* workspace, int64_t batch, int64_t feat, int64_t logits_stride, int64_t dlogits_stride,
                int64_t ignore_index, int logits_dtype, int weight_dtype, int out_dtype, hipStream_t stream) {
@@ -378,6 +382,12 @@ int ce_fwd_bwd(const void* logits, const int64_t* target, const void* weight, vo
 
 using namespace at_hip;
 
+// Workspace of at_cross_entropy_fwd_bwd_static: the divisor and one loss per row (65536 rows at
+// most, 256 KiB).  Device memory of the library itself: every GPU the library runs on holds its own
+// copy until the process ends.  In host code this name is only a handle for hipGetSymbolAddress;
+// kernels receive the address that call returns for the current device.
+static __device__ __align__(256) float ce_static_scratch[4 + 65536];
+
 extern "C" {
 
 int64_t at_cross_entropy_workspace_bytes(int64_t batch) {
@@ -397,6 +407,40 @@ int at_cross_entropy_fwd_bwd(const void* logits, const int64_t* target, const vo
   if (!workspace || workspace_bytes < at_cross_entropy_workspace_bytes(batch)) return AT_ERR_WORKSPACE;
   if ((reinterpret_cast<uintptr_t>(workspace) & 3u) != 0) return AT_ERR_ALIGN;
   return ce_fwd_bwd(logits, target, weight, loss, dlogits, (float*)workspace, batch, feat, logits_stride,
+                    dlogits_stride, ignore_index, logits_dtype, weight_dtype, out_dtype, (hipStream_t)stream_);
+}
+
+int64_t at_cross_entropy_static_max_batch(void) { return kCeStaticMaxBatch; }
+
+int at_cross_entropy_fwd_bwd_static(const void* logits, const int64_t* target, const void* weight, void* loss,
+                                    void* dlogits, int64_t batch, int64_t feat, int64_t logits_stride,
+                                    int64_t dlogits_stride, int64_t ignore_index, int logits_dtype,
+                                    int weight_dtype, int out_dtype, at_stream_t stream_) {
+  if (!loss) return AT_ERR_NULL;
+  int rc = check_ce_args(logits, target, weight, batch, feat, logits_stride, dlogits, dlogits_stride,
+                         logits_dtype, weight_dtype, out_dtype);
+  if (rc) return rc;
+  if (batch > kCeStaticMaxBatch) return AT_ERR_WORKSPACE;   // the library's own workspace holds 65536 rows
+  // Address of this device's copy of the workspace, looked up once per device (the lookup does
+  // not allocate: the array is part of the loaded code object).  Racing first calls store the
+  // same value.
+  static float* scratch_of_device[kCeMaxDevices] = {};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kCeMaxDevices) return AT_ERR_UNSUPPORTED;
+  float* scratch = scratch_of_device[dev];
+  if (!scratch) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(ce_static_scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!p) return AT_ERR_UNSUPPORTED;
+    scratch = (float*)p;
+    scratch_of_device[dev] = scratch;
+  }
+  // every element the kernels read from the workspace is written earlier in this call (the divisor
+  // by the first launch, one loss per row by the row kernel), so nothing has to be cleared
+  return ce_fwd_bwd(logits, target, weight, loss, dlogits, scratch, batch, feat, logits_stride,
                     dlogits_stride, ignore_index, logits_dtype, weight_dtype, out_dtype, (hipStream_t)stream_);
 }
 

@@ -180,6 +180,23 @@ int at_cross_entropy_scale_grad(void* dlogits, const void* output_grad, int64_t 
                                 int64_t feat, int64_t dlogits_stride, int dlogits_dtype,
                                 int grad_dtype, at_stream_t stream);
 
+/* at_cross_entropy_fwd_bwd without a workspace argument and without any allocation.  It has no
+ * counterpart in the reference: it is for callers that cannot allocate device memory (code
+ * under HIP graph capture, serving loops, harnesses that forbid hipMalloc).  The divisor and
+ * the per-row losses live in a 256 KiB device array inside the library (one copy per GPU,
+ * held until the process ends), so batch is limited to at_cross_entropy_static_max_batch()
+ * = 65536 rows; larger batches return AT_ERR_WORKSPACE.  Every call on a GPU shares that
+ * GPU's array: calls that overlap in time on one GPU (two streams) race; calls ordered on one
+ * stream do not.  Arguments and results otherwise as at_cross_entropy_fwd_bwd. */
+int64_t at_cross_entropy_static_max_batch(void);
+
+int at_cross_entropy_fwd_bwd_static(const void* logits, const int64_t* target,
+                                    const void* weight, void* loss, void* dlogits,
+                                    int64_t batch, int64_t feat, int64_t logits_stride,
+                                    int64_t dlogits_stride, int64_t ignore_index,
+                                    int logits_dtype, int weight_dtype, int out_dtype,
+                                    at_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * Negative log likelihood loss — replaces nll_loss_forward_kernel / nll_loss_backward_kernel,
  * attorch/nll_loss_kernels.py:39-138 and :141-235, and the torch sums and the division by the
