@@ -34,6 +34,7 @@ def _launch_forward(input: Tensor, act: int, param: float, drop_p: float, seed: 
 def _launch_backward(output_grad: Tensor, input: Optional[Tensor], act: int, param: float,
                      drop_p: float, seed: int) -> Tensor:
     reference = output_grad if input is None else input
+    _lib.require_same_device('activation / dropout backward', output_grad, input)
     flattened_grad = output_grad.to(reference.dtype).contiguous().view(-1)
     flattened_input = None if input is None else input.contiguous().view(-1)
     input_grad = torch.empty_like(flattened_grad)

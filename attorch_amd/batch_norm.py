@@ -70,7 +70,7 @@ class BatchNormAutoGrad(torch.autograd.Function):
         Returns:
             Normalized (+ residual, activated) input, same shape and dtype as input.
         """
-        _lib.require_gpu(input, 'BatchNorm')
+        _lib.require_same_device('BatchNorm', input, weight, bias, running_mean, running_var, pre_act_add)
         lib = _lib.load()
         act_func, param = parse_act_func(act_func)
         act = act_id(act_func, param)
@@ -135,6 +135,7 @@ class BatchNormAutoGrad(torch.autograd.Function):
         """
         lib = _lib.load()
         (input, mean, inv_std, weight, pre_act) = ctx.saved_tensors
+        _lib.require_same_device('BatchNorm backward', input, output_grad)
         batch_dim, feat_dim, spatial_dim = _dims(input)
         device = input.device
 

@@ -90,7 +90,7 @@ class Conv2dAutoGrad(torch.autograd.Function):
         assert bias is None or weight.shape[0] == bias.shape[0], \
             f'Incompatible weights ({weight.shape}) and bias ({bias.shape}) shape'
 
-        _lib.require_gpu(input, 'Conv2d')
+        _lib.require_same_device('Conv2d', input, weight, bias)
         lib = _lib.load()
         batch_dim, in_feat_dim, in_height, in_width = input.shape
         out_feat_dim, _, kernel_height, kernel_width = weight.shape
@@ -145,6 +145,7 @@ class Conv2dAutoGrad(torch.autograd.Function):
         """
         lib = _lib.load()
         input, weight = ctx.saved_tensors
+        _lib.require_same_device('Conv2d backward', input, output_grad)
         output_dtype = ctx.output_dtype
         device = input.device
         dims = ctx.dims

@@ -139,16 +139,27 @@ __global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_k
   const int n_iter = (n_int + kCeBlock - 1) / kCeBlock;
   constexpr float kLog2e = 1.4426950408889634f;
 
+  // All loads of the row are issued back to back and without a branch (the register writes on the
+  // other side of a branch would have to wait for the load): a lane with no vector at position v
+  // reads the aligned 16 bytes that hold the first element of the row instead (the same page as
+  // that element, so always mapped), and what it read is replaced by the padding afterwards.
   uint4 cache[CACHE_VECS];
+  // xr - off is on the 16-byte grid whatever the row looks like (xv is only when the row reaches
+  // its first boundary, i.e. when it has interior vectors at all)
+  const uint4* const safe = reinterpret_cast<const uint4*>(xr - off);
 #pragma unroll
   for (int i = 0; i < CACHE_VECS; ++i) {
     const int v = tid + i * kCeBlock;
-    constexpr uint32_t P = Word<T>::kNegInf;
-    cache[i] = v < n_int ? xv[v] : make_uint4(P, P, P, P);
+    cache[i] = *(v < n_int ? xv + v : safe);
   }
-  const float edge_x = edge >= 0 ? to_f32(xr[edge]) : -INFINITY;
+  const float edge_x = to_f32(xr[edge >= 0 ? edge : 0]);
+#pragma unroll
+  for (int i = 0; i < CACHE_VECS; ++i) {
+    constexpr uint32_t P = Word<T>::kNegInf;
+    if (tid + i * kCeBlock >= n_int) cache[i] = make_uint4(P, P, P, P);
+  }
 
-  float m = edge_x;
+  float m = edge >= 0 ? edge_x : -INFINITY;
 #pragma unroll
   for (int i = 0; i < CACHE_VECS; ++i) {
     if (i < n_iter) {
@@ -167,7 +178,7 @@ __global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_k
   // Second sweep: e = exp(x - max) replaces x in the cache (in the storage format: the gradient
   // is rounded to it anyway), so the third sweep is a multiplication.
   const float m2 = m * kLog2e;
-  const float edge_e = exp2f(fmaf(edge_x, kLog2e, -m2));   // exp2(-inf) = 0 without an edge
+  const float edge_e = edge >= 0 ? exp2f(fmaf(edge_x, kLog2e, -m2)) : 0.f;
   float s = edge_e;
 #pragma unroll
   for (int i = 0; i < CACHE_VECS; ++i) {

@@ -140,16 +140,25 @@ __device__ __forceinline__ void group_sum2(float& a, float& b, int group, float 
 template <typename T, int VEC, int ITERS>
 struct RowCache {
   Chunk<T, VEC> ch[ITERS];
-  // Issues the loads of this lane's chunks of `row`.  Nothing is read for an invalid row or past
-  // the end of the row; those chunks hold `pad`.
+  // Issues the loads of this lane's chunks of `row`, without a branch: an invalid row reads row 0
+  // and a chunk past the end of the row reads chunk 0 (both exist), and mask() replaces what
+  // they brought by the padding value once the row is about to be used.  A load inside a
+  // divergent branch would be waited for at the end of that branch, i.e. before the next load is
+  // even issued.
   __device__ __forceinline__ void load(const T* __restrict__ base, int64_t row, int64_t stride,
-                                       bool valid, int lane, int group, int chunks, float pad) {
+                                       bool valid, int lane, int group, int chunks) {
     const T* r = base + (valid ? row : 0) * stride;
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int c = lane + it * group;
-      if (valid && c < chunks) ch[it].load(r + (int64_t)c * VEC);
-      else ch[it].fill(pad);
+      ch[it].load(r + (int64_t)(c < chunks ? c : 0) * VEC);
+    }
+  }
+  __device__ __forceinline__ void mask(bool valid, int lane, int group, int chunks, float pad) {
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int c = lane + it * group;
+      if (!(valid && c < chunks)) ch[it].fill(pad);
     }
   }
   __device__ __forceinline__ void pin() {
@@ -165,7 +174,9 @@ struct RowCache {
 // are issued before the current one is reduced and written, which keeps reads and writes of
 // different rows in flight together.  Memory operations retire in order per wave, so nothing
 // that the current row waits on may be issued after the prefetch: parameters are held in
-// registers (packed) and per-row statistics travel with the prefetch.
+// registers (packed) and per-row statistics travel with the prefetch.  The two row-blocks live
+// in two register sets that swap roles from one iteration to the next (the loop body exists
+// twice): copying the prefetched set into the current one would have to wait for its loads.
 
 // ------------------------------------------------------------------------------------------
 // Norm forward.  LAYER = true: LayerNorm (mean subtracted, optional bias); false: RMSNorm.
@@ -203,16 +214,16 @@ __global__ __launch_bounds__(512) void norm_fwd_kernel(
     }
   }
 
-  RowCache<TX, VEC, ITERS> cur, nxt;
+  RowCache<TX, VEC, ITERS> set_a, set_b;
   {
     const int64_t row0 = (int64_t)blockIdx.x * rpb + rib;
-    cur.load(x, row0, xs, row0 < batch, lane, group, chunks, 0.f);
+    set_a.load(x, row0, xs, row0 < batch, lane, group, chunks);
   }
-#pragma unroll 1
-  for (int64_t rb = blockIdx.x; rb < row_blocks; rb += gridDim.x) {
+  auto step = [&](int64_t rb, RowCache<TX, VEC, ITERS>& cur, RowCache<TX, VEC, ITERS>& nxt) {
     const int64_t row = rb * rpb + rib;
     const bool valid = row < batch;
-    nxt.load(x, row + row_step, xs, row + row_step < batch, lane, group, chunks, 0.f);
+    nxt.load(x, row + row_step, xs, row + row_step < batch, lane, group, chunks);
+    cur.mask(valid, lane, group, chunks, 0.f);
     if (HOIST) {   // opaque per iteration: otherwise their widening to fp32 is hoisted out of the loop
 #pragma unroll
       for (int it = 0; it < ITERS; ++it) {
@@ -285,8 +296,11 @@ __global__ __launch_bounds__(512) void norm_fwd_kernel(
         }
       }
     }
-    cur = nxt;
-    cur.pin();
+  };
+#pragma unroll 1
+  for (int64_t rb = blockIdx.x; rb < row_blocks; rb += 2 * (int64_t)gridDim.x) {
+    step(rb, set_a, set_b);
+    if (rb + gridDim.x < row_blocks) step(rb + gridDim.x, set_b, set_a);
   }
 }
 
@@ -359,7 +373,9 @@ __global__ __launch_bounds__(1024) void norm_fwd_stream_kernel(
 // Dynamic LDS: blockDim.x * VEC floats (only used when a workgroup holds several rows).
 // ------------------------------------------------------------------------------------------
 template <bool LAYER, typename TDY, typename TX, typename TDX, typename TW, int VEC, int ITERS>
-__global__ __launch_bounds__(512) void norm_bwd_kernel(
+// RMSNorm with at most two chunks per lane fits 128 registers, i.e. two workgroups per CU; the
+// LayerNorm instance (bias gradient accumulators on top) would spill there and runs one per CU.
+__global__ __launch_bounds__(512, (ITERS <= 2 && !LAYER ? 4 : 1)) void norm_bwd_kernel(
     const TDY* __restrict__ dy, const TX* __restrict__ x, const float* __restrict__ mean_in,
     const float* __restrict__ rstd_in, const TW* __restrict__ w, TDX* __restrict__ dx,
     float* __restrict__ part_w, float* __restrict__ part_b, int64_t batch, int feat,
@@ -397,36 +413,30 @@ __global__ __launch_bounds__(512) void norm_bwd_kernel(
   }
 
   // the row stays in registers in its storage format between the two sweeps
-  RowCache<TDY, VEC, ITERS> cdy, ndy;
-  RowCache<TX, VEC, ITERS> cx, nx;
-  float mean = 0.f, rstd = 0.f, nmean = 0.f, nrstd = 0.f;
+  struct RowSet {
+    RowCache<TDY, VEC, ITERS> dy;
+    RowCache<TX, VEC, ITERS> x;
+    float mean, rstd;   // of an invalid row: those of row 0 (finite; its dy is masked to zero)
+  };
+  RowSet set_a, set_b;
   int parity = 0;
-  {
-    const int64_t row0 = (int64_t)blockIdx.x * rpb + rib;
-    const bool v0 = row0 < batch;
-    if (v0) {
-      if (LAYER) mean = mean_in[row0];
-      rstd = rstd_in[row0];
-    }
-    cdy.load(dy, row0, dys, v0, lane, group, chunks, 0.f);
-    cx.load(x, row0, xs, v0, lane, group, chunks, 0.f);
-  }
-#pragma unroll 1
-  for (int64_t rb = blockIdx.x; rb < row_blocks; rb += gridDim.x) {
+  auto fetch = [&](RowSet& t, int64_t row) {
+    const bool v = row < batch;
+    t.mean = LAYER ? mean_in[v ? row : 0] : 0.f;
+    t.rstd = rstd_in[v ? row : 0];
+    t.dy.load(dy, row, dys, v, lane, group, chunks);
+    t.x.load(x, row, xs, v, lane, group, chunks);
+  };
+  fetch(set_a, (int64_t)blockIdx.x * rpb + rib);
+  auto step = [&](int64_t rb, RowSet& cur, RowSet& nxt) {
     const int64_t row = rb * rpb + rib;
     const bool valid = row < batch;
-    {
-      const int64_t nrow = row + row_step;
-      const bool nv = nrow < batch;
-      nmean = 0.f;
-      nrstd = 0.f;
-      if (nv) {
-        if (LAYER) nmean = mean_in[nrow];
-        nrstd = rstd_in[nrow];
-      }
-      ndy.load(dy, nrow, dys, nv, lane, group, chunks, 0.f);
-      nx.load(x, nrow, xs, nv, lane, group, chunks, 0.f);
-    }
+    fetch(nxt, row + row_step);
+    RowCache<TDY, VEC, ITERS>& cdy = cur.dy;
+    RowCache<TX, VEC, ITERS>& cx = cur.x;
+    const float mean = cur.mean, rstd = cur.rstd;
+    const float shift = -mean * rstd;
+    cdy.mask(valid, lane, group, chunks, 0.f);
     if (HOIST) {   // opaque per iteration: otherwise their widening to fp32 is hoisted out of the loop
 #pragma unroll
       for (int it = 0; it < ITERS; ++it) pw[HOIST ? it : 0].pin();
@@ -450,7 +460,9 @@ __global__ __launch_bounds__(512) void norm_bwd_kernel(
       }
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        const float h = (xv[j] - mean) * rstd;
+        // (x - mean) * rstd; one fma where the input has 16 bits anyway (the rounded product
+        // mean * rstd costs accuracy when |mean| is large next to the spread of the row)
+        const float h = sizeof(TX) == 2 ? fmaf(xv[j], rstd, shift) : (xv[j] - mean) * rstd;
         const float gg = dv[j] * wv[j];
         s1 += h * gg;
         s2 += gg;
@@ -501,7 +513,7 @@ __global__ __launch_bounds__(512) void norm_bwd_kernel(
             }
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
-              const float h = (xv[j] - mean) * rstd;
+              const float h = sizeof(TX) == 2 ? fmaf(xv[j], rstd, shift) : (xv[j] - mean) * rstd;
               o[j] = fmaf(dv[j] * wv[j], rstd, -fmaf(h, s1, s2));
             }
           }
@@ -510,12 +522,11 @@ __global__ __launch_bounds__(512) void norm_bwd_kernel(
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    cdy = ndy;
-    cx = nx;
-    mean = nmean;
-    rstd = nrstd;
-    cdy.pin();
-    cx.pin();
+  };
+#pragma unroll 1
+  for (int64_t rb = blockIdx.x; rb < row_blocks; rb += 2 * (int64_t)gridDim.x) {
+    step(rb, set_a, set_b);
+    if (rb + gridDim.x < row_blocks) step(rb + gridDim.x, set_b, set_a);
   }
 
   if (!part_w && !part_b) return;
@@ -663,11 +674,17 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(
 // ------------------------------------------------------------------------------------------
 // Softmax family.
 // ------------------------------------------------------------------------------------------
-template <typename TX, typename TY, int VEC, int ITERS>
-__global__ __launch_bounds__(1024) void softmax_fwd_kernel(
+// MAXB: largest workgroup the instance is launched with (256 leaves the compiler 256 registers per lane).
+template <typename TX, typename TY, int VEC, int ITERS, int MAXB>
+__global__ __launch_bounds__(MAXB) void softmax_fwd_kernel(
     const TX* __restrict__ x, TY* __restrict__ y, int64_t batch, int feat, int64_t xs, int64_t ys,
     int neg, int log, int group_log2) {
   static_assert(ITERS > 0, "rows are cached in registers");
+  // With few enough elements per lane the exponentials of the second sweep (the shifted logits for
+  // log-softmax) stay in registers as fp32 and the third sweep is one multiplication per element;
+  // otherwise the third sweep computes them again from the cached row.
+  constexpr bool KEEP = ITERS * VEC <= (MAXB <= 256 ? 32 : 16);
+  constexpr float kLog2e = 1.4426950408889634f, kLn2 = 0.6931471805599453f;
   __shared__ float slots[2][16];
   int parity = 0;
   const int group = 1 << group_log2;
@@ -676,20 +693,21 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
   const int rib = threadIdx.x >> group_log2;
   const int chunks = feat / VEC;
   const float sign = neg ? -1.f : 1.f;
+  const float scale = sign * kLog2e;    // exponentials in base 2: exp(s x - m) = exp2(x * scale - m * log2(e))
   const float pad = -sign * INFINITY;   // padding never wins the max and adds exp(-inf) = 0
   const int64_t row_blocks = (batch + rpb - 1) / rpb;
   const int64_t row_step = (int64_t)gridDim.x * rpb;
 
-  RowCache<TX, VEC, ITERS> cur, nxt;
+  RowCache<TX, VEC, ITERS> set_a, set_b;
   {
     const int64_t row0 = (int64_t)blockIdx.x * rpb + rib;
-    cur.load(x, row0, xs, row0 < batch, lane, group, chunks, pad);
+    set_a.load(x, row0, xs, row0 < batch, lane, group, chunks);
   }
-#pragma unroll 1
-  for (int64_t rb = blockIdx.x; rb < row_blocks; rb += gridDim.x) {
+  auto step = [&](int64_t rb, RowCache<TX, VEC, ITERS>& cur, RowCache<TX, VEC, ITERS>& nxt) {
     const int64_t row = rb * rpb + rib;
     const bool valid = row < batch;
-    nxt.load(x, row + row_step, xs, row + row_step < batch, lane, group, chunks, pad);
+    nxt.load(x, row + row_step, xs, row + row_step < batch, lane, group, chunks);
+    cur.mask(valid, lane, group, chunks, pad);
     __builtin_amdgcn_sched_barrier(0);
 
     float m = -INFINITY;
@@ -704,16 +722,23 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
     if (!valid) m = 0.f;   // an invalid row is all padding: keep its arithmetic finite
     cur.pin();
 
+    const float m2 = m * kLog2e;
     float s = 0.f;
+    float kept[KEEP ? ITERS : 1][VEC];
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       float v[VEC];
       cur.ch[it].get(v);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) s += __expf(v[j] * sign - m);
+      for (int j = 0; j < VEC; ++j) {
+        const float t = fmaf(v[j], scale, -m2);          // (s x - m) * log2(e); -inf for padding
+        const float e = __builtin_amdgcn_exp2f(t);
+        s += e;
+        if (KEEP) kept[KEEP ? it : 0][j] = log ? t : e;
+      }
     }
     s = group_reduce_alt(s, group, slots, parity, SumOp(), 0.f);
-    cur.pin();
+    if (!KEEP) cur.pin();
 
     if (valid) {
       const float inv = 1.0f / s;
@@ -724,18 +749,27 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
         const int c = lane + it * group;
         if (c < chunks) {
           float v[VEC];
-          cur.ch[it].get(v);
+          if (KEEP) {
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) {
-            const float d = v[j] * sign - m;
-            v[j] = log ? d - lg : __expf(d) * inv;
+            for (int j = 0; j < VEC; ++j)
+              v[j] = log ? fmaf(kept[KEEP ? it : 0][j], kLn2, -lg) : kept[KEEP ? it : 0][j] * inv;
+          } else {
+            cur.ch[it].get(v);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+              const float t = fmaf(v[j], scale, -m2);
+              v[j] = log ? fmaf(t, kLn2, -lg) : __builtin_amdgcn_exp2f(t) * inv;
+            }
           }
           store_f32<TY, VEC>(yr + (int64_t)c * VEC, v);
         }
       }
     }
-    cur = nxt;
-    cur.pin();
+  };
+#pragma unroll 1
+  for (int64_t rb = blockIdx.x; rb < row_blocks; rb += 2 * (int64_t)gridDim.x) {
+    step(rb, set_a, set_b);
+    if (rb + gridDim.x < row_blocks) step(rb + gridDim.x, set_b, set_a);
   }
 }
 
@@ -796,19 +830,25 @@ __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
   const int64_t row_blocks = (batch + rpb - 1) / rpb;
   const int64_t row_step = (int64_t)gridDim.x * rpb;
 
-  RowCache<TDY, VEC, ITERS> cdy, ndy;
-  RowCache<TY, VEC, ITERS> cy, ny;
+  struct RowSet {
+    RowCache<TDY, VEC, ITERS> dy;
+    RowCache<TY, VEC, ITERS> y;
+  };
+  RowSet set_a, set_b;
   {
     const int64_t row0 = (int64_t)blockIdx.x * rpb + rib;
-    cdy.load(dy, row0, dys, row0 < batch, lane, group, chunks, 0.f);
-    cy.load(y, row0, ys, row0 < batch, lane, group, chunks, 0.f);
+    set_a.dy.load(dy, row0, dys, row0 < batch, lane, group, chunks);
+    set_a.y.load(y, row0, ys, row0 < batch, lane, group, chunks);
   }
-#pragma unroll 1
-  for (int64_t rb = blockIdx.x; rb < row_blocks; rb += gridDim.x) {
+  auto step = [&](int64_t rb, RowSet& cur, RowSet& nxt) {
     const int64_t row = rb * rpb + rib;
     const bool valid = row < batch;
-    ndy.load(dy, row + row_step, dys, row + row_step < batch, lane, group, chunks, 0.f);
-    ny.load(y, row + row_step, ys, row + row_step < batch, lane, group, chunks, 0.f);
+    nxt.dy.load(dy, row + row_step, dys, row + row_step < batch, lane, group, chunks);
+    nxt.y.load(y, row + row_step, ys, row + row_step < batch, lane, group, chunks);
+    RowCache<TDY, VEC, ITERS>& cdy = cur.dy;
+    RowCache<TY, VEC, ITERS>& cy = cur.y;
+    cdy.mask(valid, lane, group, chunks, 0.f);   // dy = 0 makes every product of the padding vanish
+    cy.mask(valid, lane, group, chunks, 0.f);
     __builtin_amdgcn_sched_barrier(0);
 
     float s = 0.f;
@@ -840,10 +880,11 @@ __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
         }
       }
     }
-    cdy = ndy;
-    cy = ny;
-    cdy.pin();
-    cy.pin();
+  };
+#pragma unroll 1
+  for (int64_t rb = blockIdx.x; rb < row_blocks; rb += 2 * (int64_t)gridDim.x) {
+    step(rb, set_a, set_b);
+    if (rb + gridDim.x < row_blocks) step(rb + gridDim.x, set_b, set_a);
   }
 }
 
@@ -969,8 +1010,9 @@ int norm_fwd(const void* x, const void* weight, const void* bias, float* mean, f
                          rows_vectorizable(y, ys, ydt) && (!weight || aligned16(weight)) &&
                          (!bias || aligned16(bias));
   if (!vector_ok) vec = 1;
-  // few chunks per lane: many resident waves hide the latency of the row reductions
-  const RowPlan p = plan_rows(feat, vec, 256, 2, 512);
+  // up to four chunks per lane before a row spreads over more than one wave: fewer waves share
+  // each reduction, and enough of them stay resident to hide its latency
+  const RowPlan p = plan_rows(feat, vec, 256, 4, 512);
   return dispatch_pair(xdt, ydt, [&](auto* tx, auto* ty) -> int {
     typedef std::remove_pointer_t<decltype(tx)> TX;
     typedef std::remove_pointer_t<decltype(ty)> TY;
@@ -1163,7 +1205,8 @@ int at_softmax_fwd(const void* x, void* y, int64_t batch, int64_t feat, int64_t 
   int vec = narrow_vec(x_dtype, y_dtype, AT_DTYPE_F32);
   if (!(feat % vec == 0 && rows_vectorizable(x, x_stride, x_dtype) && rows_vectorizable(y, y_stride, y_dtype)))
     vec = 1;
-  const RowPlan p = plan_rows(feat, vec, 256, 4, 1024);
+  // one wave per row up to eight chunks per lane (no workgroup barrier in the reductions)
+  const RowPlan p = plan_rows(feat, vec, 256, 8, 1024);
   return dispatch_pair(x_dtype, y_dtype, [&](auto* tx, auto* ty) -> int {
     typedef std::remove_pointer_t<decltype(tx)> TX;
     typedef std::remove_pointer_t<decltype(ty)> TY;
@@ -1178,14 +1221,18 @@ int at_softmax_fwd(const void* x, void* y, int64_t batch, int64_t feat, int64_t 
       return launch_status();
     }
     const int64_t row_blocks = cdiv64(batch, p.block >> p.group_log2);
-#define AT_SOFTMAX_FWD_LAUNCH(VV)                                                                        \
+#define AT_SOFTMAX_FWD_LAUNCH(VV, MAXB)                                                                  \
   AT_DISPATCH_ITERS(p.iters, {                                                                           \
-    auto kernel = softmax_fwd_kernel<TX, TY, VV, ITERS>;                                                 \
+    auto kernel = softmax_fwd_kernel<TX, TY, VV, ITERS, MAXB>;                                           \
     const unsigned grid = persistent_grid((const void*)kernel, p.block, 0, row_blocks, 0);               \
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(p.block), 0, stream, (const TX*)x, (TY*)y, batch,        \
                        (int)feat, x_stride, y_stride, neg, log, p.group_log2);                           \
   })
-    if (vec != 1) { AT_SOFTMAX_FWD_LAUNCH(VECW); } else { AT_SOFTMAX_FWD_LAUNCH(1); }
+    if (p.block <= 256) {
+      if (vec != 1) { AT_SOFTMAX_FWD_LAUNCH(VECW, 256); } else { AT_SOFTMAX_FWD_LAUNCH(1, 256); }
+    } else {
+      if (vec != 1) { AT_SOFTMAX_FWD_LAUNCH(VECW, 1024); } else { AT_SOFTMAX_FWD_LAUNCH(1, 1024); }
+    }
 #undef AT_SOFTMAX_FWD_LAUNCH
     return launch_status();
   });

@@ -91,6 +91,7 @@ class GLUAutoGrad(torch.autograd.Function):
         """
         lib = _lib.load()
         (input_k,) = ctx.saved_tensors
+        _lib.require_same_device('GLU backward', input_k, output_grad)
         outer, half = ctx.geometry
         output_grad = output_grad.contiguous()
         input_grad = torch.empty_like(input_k)

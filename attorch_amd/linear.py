@@ -99,7 +99,7 @@ class LinearAutoGrad(torch.autograd.Function):
         assert bias is None or weight.shape[1] == bias.shape[0], \
             f'Incompatible weights ({weight.shape}) and bias ({bias.shape}) shape'
 
-        _lib.require_gpu(input, 'Linear')
+        _lib.require_same_device('Linear', input, weight, bias)
         lib = _lib.load()
         act_func, param = parse_act_func(act_func)
         act = act_id(act_func, param)
@@ -161,6 +161,7 @@ class LinearAutoGrad(torch.autograd.Function):
         """
         lib = _lib.load()
         input, pre_act, weight = ctx.saved_tensors
+        _lib.require_same_device('Linear backward', input, output_grad)
         output_dtype = ctx.output_dtype
         device = input.device
 

@@ -53,7 +53,7 @@ class NLLLossAutoGrad(torch.autograd.Function):
             f'Dimensionality of weight vector ({len(weight)}) and input features ({input.shape[1]}) not equal'
         assert reduction in REDUCTIONS, f'Reduction must be one of {tuple(REDUCTIONS)}, received {reduction}'
 
-        _lib.require_gpu(input, 'NLLLoss')
+        _lib.require_same_device('NLLLoss', input, target, weight)
         lib = _lib.load()
         batch_dim, feat_dim = input.shape[:2]
         spatial_dim = 1
@@ -105,6 +105,7 @@ class NLLLossAutoGrad(torch.autograd.Function):
         """
         lib = _lib.load()
         target_k, weight_k, sum_weights = ctx.saved_tensors
+        _lib.require_same_device('NLLLoss backward', target_k, output_grad)
         batch_dim, feat_dim = ctx.input_shape[:2]
         input_grad = torch.empty(ctx.input_shape, dtype=ctx.output_dtype, device=target_k.device)
         if input_grad.numel() > 0:

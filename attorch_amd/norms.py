@@ -55,7 +55,7 @@ class LayerNormAutoGrad(torch.autograd.Function):
         Returns:
             Normalized input, same shape as input.
         """
-        _lib.require_gpu(input, 'LayerNorm')
+        _lib.require_same_device('LayerNorm', input, weight, bias)
         lib = _lib.load()
         flattened_input = _lib.rows(input)
         batch_dim, feat_dim = flattened_input.shape
@@ -110,6 +110,7 @@ class LayerNormAutoGrad(torch.autograd.Function):
         lib = _lib.load()
         scale_by_weight, add_bias = ctx.scale_by_weight, ctx.add_bias
         (flattened_input, mean, inv_std, weight) = ctx.saved_tensors
+        _lib.require_same_device('LayerNorm backward', flattened_input, output_grad)
         flattened_output_grad = _lib.rows(output_grad.reshape(flattened_input.shape)
                                           .to(ctx.output_dtype))
         batch_dim, feat_dim = flattened_output_grad.shape
@@ -204,7 +205,7 @@ class RMSNormAutoGrad(torch.autograd.Function):
         Returns:
             Normalized input, same shape and dtype as input.
         """
-        _lib.require_gpu(input, 'RMSNorm')
+        _lib.require_same_device('RMSNorm', input, weight)
         lib = _lib.load()
         flattened_input = _lib.rows(input)
         batch_dim, feat_dim = flattened_input.shape
@@ -244,6 +245,7 @@ class RMSNormAutoGrad(torch.autograd.Function):
         lib = _lib.load()
         scale_by_weight = ctx.scale_by_weight
         (flattened_input, inv_rms, weight) = ctx.saved_tensors
+        _lib.require_same_device('RMSNorm backward', flattened_input, output_grad)
         flattened_output_grad = _lib.rows(output_grad.reshape(flattened_input.shape)
                                           .to(flattened_input.dtype))
         batch_dim, feat_dim = flattened_output_grad.shape

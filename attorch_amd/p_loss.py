@@ -46,7 +46,7 @@ class PLossAutoGrad(torch.autograd.Function):
         assert input.shape == target.shape, \
             f'Input shape {input.shape} and target shape {target.shape} not equal'
         assert reduction in REDUCTIONS, f'Reduction must be one of {tuple(REDUCTIONS)}, received {reduction}'
-        _lib.require_gpu(input, 'p-norm loss')
+        _lib.require_same_device('p-norm loss', input, target)
         lib = _lib.load()
         output_dtype = get_output_dtype(input.dtype, autocast='fp32')
         device = input.device
@@ -89,6 +89,7 @@ class PLossAutoGrad(torch.autograd.Function):
         """
         lib = _lib.load()
         input_k, target_k = ctx.saved_tensors
+        _lib.require_same_device('p-norm loss backward', input_k, output_grad)
         needs_input, needs_target = ctx.needs
         size = input_k.numel()
         input_grad = torch.empty_like(input_k, dtype=ctx.output_dtype) if needs_input else None

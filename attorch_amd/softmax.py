@@ -70,6 +70,7 @@ class SoftmaxAutoGrad(torch.autograd.Function):
         """
         lib = _lib.load()
         (output,) = ctx.saved_tensors
+        _lib.require_same_device('Softmax backward', output, output_grad)
         flattened_output_grad = _lib.rows(output_grad.reshape(output.shape).to(output.dtype))
         batch_dim, feat_dim = output.shape
         input_grad = torch.empty_like(output)

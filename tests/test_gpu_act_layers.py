@@ -173,3 +173,27 @@ def test_act_dropout_argument_errors() -> None:
     assert lib.at_act_dropout_fwd(p, p, 8, 0, 0.0, 0.0, 0, 7, st) == -3
     assert lib.at_act_dropout_bwd(p, None, p, 8, 4, 0.0, 0.0, 0, 0, st) == -1   # activation needs its input
     assert lib.at_act_dropout_fwd(p, p, 0, 0, 0.0, 0.0, 0, 0, st) == 0
+
+
+def test_host_tensors_raise_instead_of_faulting() -> None:
+    # a host pointer handed to a kernel is a memory fault; every layer checks all its tensors first
+    x = torch.randn(8, 16, device='cuda', requires_grad=True)
+    with pytest.raises(RuntimeError, match='expected all tensors on'):
+        attorch_amd.Linear(16, 4, device='cpu')(x)
+    with pytest.raises(RuntimeError, match='expected all tensors on'):
+        attorch_amd.LayerNorm(16, device='cpu')(x)
+    with pytest.raises(RuntimeError, match='expected all tensors on'):
+        attorch_amd.RMSNorm(16, device='cpu')(x)
+    with pytest.raises(RuntimeError, match='expected all tensors on'):
+        attorch_amd.BatchNorm1d(16, device='cpu')(x)
+    with pytest.raises(RuntimeError, match='expected all tensors on'):
+        attorch_amd.Conv2d(16, 4, 1, device='cpu')(x.view(8, 16, 1, 1))
+    with pytest.raises(RuntimeError, match='expected all tensors on'):
+        attorch_amd.NLLLoss()(torch.log_softmax(x, dim=1), torch.zeros(8, dtype=torch.int64))
+    with pytest.raises(RuntimeError, match='expected all tensors on'):
+        attorch_amd.MSELoss()(x, torch.zeros(8, 16))
+    y = attorch_amd.Softmax(dim=-1)(x)
+    with pytest.raises(RuntimeError):                      # autograd's own device check comes first here
+        torch.autograd.grad(y, x, torch.ones(8, 16))       # upstream gradient on the host
+    with pytest.raises(RuntimeError, match='there is no CPU path'):
+        attorch_amd.Softmax(dim=-1)(torch.zeros(2, 3))
