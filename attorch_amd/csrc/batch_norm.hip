@@ -3,11 +3,14 @@
 //
 // HBM-bound.  The reference gives one program to each channel (C workgroups, a quarter of the
 // chip for C = 64); here every pass is spread over C x P workgroups:
-//   forward : partial (count, mean, M2) per (channel, split) -> per-channel finalize (Chan
-//             merge in fixed order, running-stat EMA) -> elementwise apply
+//   forward : partial (count, mean, M2) per (channel, split) -> elementwise apply
 //   backward: partial (sum g, sum g*x_hat) per (channel, split), writing g = dy * act'(z) on
-//             the way -> per-channel finalize (weight/bias gradients, coefficients) ->
-//             elementwise input gradient
+//             the way -> elementwise input gradient
+// Two launches per direction: every workgroup of an apply pass merges the partials of its
+// channel itself (a few dozen values, in a fixed order, so all of them get the same bits), and
+// the workgroup that owns the channel's first plane also writes the per-channel outputs
+// (statistics, running-statistics update, weight / bias gradients).  Each lane keeps several
+// independent 16-byte loads in flight: these passes are bound by memory latency otherwise.
 // All cross-workgroup combination goes through small fp32 workspaces and is order-fixed.
 #include <type_traits>
 
@@ -70,6 +73,20 @@ __device__ __forceinline__ void for_channel_chunks(int c, int p, int P, int64_t 
   }
 }
 
+// Raw 16-byte (or narrower) image of VEC elements, widened on use: loads are issued into these
+// so that nothing has to wait before the next load is issued.
+template <typename T, int VEC>
+struct RawVec {
+  typename raw_vec<(int)sizeof(T) * VEC>::type r;
+  __device__ __forceinline__ void load(const T* p) { r = *reinterpret_cast<const decltype(r)*>(p); }
+  __device__ __forceinline__ void get(float (&f)[VEC]) const {
+    union { decltype(r) raw; T e[VEC]; } u;
+    u.raw = r;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) f[j] = to_f32(u.e[j]);
+  }
+};
+
 template <typename T, int VEC>
 __global__ __launch_bounds__(kBnBlock) void bn_stats_kernel(const T* __restrict__ x, float* __restrict__ part,
                                                            int64_t N, int C, int S, int P) {
@@ -100,82 +117,123 @@ __global__ __launch_bounds__(kBnBlock) void bn_stats_kernel(const T* __restrict_
   }
 }
 
-// One wave per channel: merges the P partials, derives mean / inv_std, updates the running
-// statistics (unbiased variance) and leaves {mean, inv_std} in stat[c].
-__global__ __launch_bounds__(64) void bn_stats_finalize_kernel(
-    const float* __restrict__ part, int P, float* __restrict__ stat, float* __restrict__ mean_out,
-    float* __restrict__ inv_std_out, void* __restrict__ running_mean, void* __restrict__ running_var,
-    int rdt, float momentum, float eps) {
-  const int c = blockIdx.x;
-  Welford acc{0.f, 0.f, 0.f};
-  for (int p = threadIdx.x; p < P; p += 64) {
-    const float* src = part + ((int64_t)c * P + p) * 3;
-    acc = wf_merge(acc, Welford{src[0], src[1], src[2]});
+// Statistics of channel c for an apply workgroup.  Every thread of the workgroup calls this.
+//   part != nullptr: wave 0 merges the P partial (count, mean, M2) triples with three sums over the
+//     wave (total count; count-weighted mean; M2 plus count * squared distance of each partial
+//     mean from the merged one) — the same order in every workgroup, so all of them get the same
+//     bits — and the result travels through LDS; `count` receives the number of elements.
+//   part == nullptr: the running statistics (evaluation mode).
+__device__ __forceinline__ void channel_stats(const float* __restrict__ part, int P, int c,
+                                              const void* __restrict__ running_mean,
+                                              const void* __restrict__ running_var, int rdt,
+                                              float* smem /* 4 floats */, float& mean, float& var, float& count) {
+  if (!part) {
+    mean = load_scalar_f32(running_mean, rdt, c);
+    var = load_scalar_f32(running_var, rdt, c);
+    count = 0.f;
+    return;
   }
-  for (int o = 32; o > 0; o >>= 1) {
-    Welford other{__shfl_xor(acc.n, o, 64), __shfl_xor(acc.mean, o, 64), __shfl_xor(acc.m2, o, 64)};
-    acc = (threadIdx.x & o) ? wf_merge(other, acc) : wf_merge(acc, other);
-  }
-  if (threadIdx.x == 0) {
-    const float var = acc.m2 / acc.n;
-    const float inv_std = rsqrtf(var + eps);
-    stat[2 * c] = acc.mean;
-    stat[2 * c + 1] = inv_std;
-    if (mean_out) mean_out[c] = acc.mean;
-    if (inv_std_out) inv_std_out[c] = inv_std;
-    if (running_mean && running_var) {
-      const float rm = load_scalar_f32(running_mean, rdt, c), rv = load_scalar_f32(running_var, rdt, c);
-      store_scalar_f32(running_mean, rdt, c, (1.f - momentum) * rm + momentum * acc.mean);
-      store_scalar_f32(running_var, rdt, c, (1.f - momentum) * rv + momentum * var * acc.n / (acc.n - 1.f));
+  __syncthreads();   // previous readers of smem are done
+  if (threadIdx.x < 64) {
+    float n = 0.f, nm = 0.f;
+    for (int p = threadIdx.x; p < P; p += 64) {
+      const float* src = part + ((int64_t)c * P + p) * 3;
+      n += src[0];
+      nm += src[0] * src[1];
+    }
+    n = wave_reduce(n, 64, SumOp());
+    nm = wave_reduce(nm, 64, SumOp());
+    const float m = nm / n;
+    float m2 = 0.f;
+    for (int p = threadIdx.x; p < P; p += 64) {
+      const float* src = part + ((int64_t)c * P + p) * 3;
+      const float d = src[1] - m;
+      m2 += src[2] + src[0] * d * d;
+    }
+    m2 = wave_reduce(m2, 64, SumOp());
+    if (threadIdx.x == 0) {
+      smem[0] = m;
+      smem[1] = m2 / n;
+      smem[2] = n;
     }
   }
-}
-
-__global__ void bn_eval_stats_kernel(const void* __restrict__ running_mean, const void* __restrict__ running_var,
-                                     int rdt, float* __restrict__ stat, float* __restrict__ mean_out,
-                                     float* __restrict__ inv_std_out, int C, float eps) {
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= C) return;
-  const float m = load_scalar_f32(running_mean, rdt, c);
-  const float r = rsqrtf(load_scalar_f32(running_var, rdt, c) + eps);
-  stat[2 * c] = m;
-  stat[2 * c + 1] = r;
-  if (mean_out) mean_out[c] = m;
-  if (inv_std_out) inv_std_out[c] = r;
+  __syncthreads();
+  mean = smem[0];
+  var = smem[1];
+  count = smem[2];
 }
 
 // y = act(w * (x - mean) * inv_std + b (+ residual)); one workgroup per slice of a plane.
-// grid.x = planes (n * C + c), grid.y = slices of the plane.
+// grid.x = planes (n * C + c), grid.y = slices of the plane.  The workgroup of slice 0 of a
+// channel's first plane (n = 0) also writes mean / inv_std and updates the running statistics
+// (unbiased variance) of that channel.
 template <typename T, int VEC, int ACT>
 __global__ __launch_bounds__(kBnBlock) void bn_apply_kernel(
     const T* __restrict__ x, const T* __restrict__ res, T* __restrict__ pre_act, T* __restrict__ y,
-    const float* __restrict__ stat, const void* __restrict__ w, const void* __restrict__ b, int wdt,
-    int C, int S, float param, int64_t total_planes) {
+    const float* __restrict__ part, int P, float* __restrict__ mean_out, float* __restrict__ inv_std_out,
+    void* __restrict__ running_mean, void* __restrict__ running_var, int rdt, int update_running,
+    float momentum, float eps, const void* __restrict__ w, const void* __restrict__ b, int wdt, int C, int S,
+    float param, int64_t total_planes) {
+  __shared__ float smem[4];
   const int sp = S / VEC;
+  const int step = gridDim.y * kBnBlock;
   for (int64_t plane = blockIdx.x; plane < total_planes; plane += gridDim.x) {
     const int c = (int)(plane % C);
-    const float mean = stat[2 * c], inv_std = stat[2 * c + 1];
+    const int64_t base = plane * (int64_t)S;
+    // Two chunks per lane and pass, their loads (input and residual) issued together; those of the
+    // first pass go out before the statistics of the channel are merged, so both latencies overlap.
+    int i0 = blockIdx.y * kBnBlock + threadIdx.x;
+    bool has1;
+    int64_t off[2];
+    RawVec<T, VEC> xin[2], rin[2];
+    auto issue = [&](int i) {   // i < sp
+      has1 = i + step < sp;
+      off[0] = base + (int64_t)i * VEC;
+      off[1] = base + (int64_t)(has1 ? i + step : i) * VEC;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        xin[u].load(x + off[u]);
+        if (res) rin[u].load(res + off[u]);   // uniform
+      }
+    };
+    issue(i0 < sp ? i0 : 0);
+    float mean, var, count;
+    channel_stats(part, P, c, running_mean, running_var, rdt, smem, mean, var, count);
+    const float inv_std = rsqrtf(var + eps);
+    if (plane < C && blockIdx.y == 0 && threadIdx.x == 0) {
+      if (mean_out) mean_out[c] = mean;
+      if (inv_std_out) inv_std_out[c] = inv_std;
+      if (update_running) {
+        const float rm = load_scalar_f32(running_mean, rdt, c), rv = load_scalar_f32(running_var, rdt, c);
+        store_scalar_f32(running_mean, rdt, c, (1.f - momentum) * rm + momentum * mean);
+        store_scalar_f32(running_var, rdt, c, (1.f - momentum) * rv + momentum * var * count / (count - 1.f));
+      }
+    }
     const float wt = w ? load_scalar_f32(w, wdt, c) : 1.f;
     const float bs = b ? load_scalar_f32(b, wdt, c) : 0.f;
-    const int64_t base = plane * (int64_t)S;
-    for (int i = blockIdx.y * kBnBlock + threadIdx.x; i < sp; i += gridDim.y * kBnBlock) {
-      const int64_t off = base + (int64_t)i * VEC;
-      float v[VEC];
-      load_f32<T, VEC>(x + off, v);
+    while (i0 < sp) {
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) v[j] = wt * (v[j] - mean) * inv_std + bs;
-      if (res) {
-        float r[VEC];
-        load_f32<T, VEC>(res + off, r);
+      for (int u = 0; u < 2; ++u) {
+        if (u == 1 && !has1) break;
+        float v[VEC];
+        xin[u].get(v);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) v[j] += r[j];
+        for (int j = 0; j < VEC; ++j) v[j] = wt * (v[j] - mean) * inv_std + bs;
+        if (res) {
+          float r[VEC];
+          rin[u].get(r);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) v[j] += r[j];
+        }
+        if (ACT != AT_ACT_NONE) {
+          if (pre_act) store_f32<T, VEC>(pre_act + off[u], v);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) v[j] = act_forward(ACT, v[j], param);
+        }
+        store_f32<T, VEC>(y + off[u], v);
       }
-      if (ACT != AT_ACT_NONE) {
-        if (pre_act) store_f32<T, VEC>(pre_act + off, v);
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) v[j] = act_forward(ACT, v[j], param);
-      }
-      store_f32<T, VEC>(y + off, v);
+      i0 += 2 * step;
+      if (i0 < sp) issue(i0);
     }
   }
 }
@@ -219,47 +277,74 @@ __global__ __launch_bounds__(kBnBlock) void bn_bwd_reduce_kernel(
   }
 }
 
-__global__ __launch_bounds__(64) void bn_bwd_finalize_kernel(
-    const float* __restrict__ part, int P, const void* __restrict__ w, int wdt, float count,
-    float* __restrict__ coef, float* __restrict__ weight_grad, float* __restrict__ bias_grad) {
-  const int c = blockIdx.x;
-  float s1 = 0.f, s2 = 0.f;
-  for (int p = threadIdx.x; p < P; p += 64) {
-    s1 += part[((int64_t)c * P + p) * 2];
-    s2 += part[((int64_t)c * P + p) * 2 + 1];
-  }
-  s1 = wave_reduce(s1, 64, SumOp());
-  s2 = wave_reduce(s2, 64, SumOp());
-  if (threadIdx.x == 0) {
-    const float wt = w ? load_scalar_f32(w, wdt, c) : 1.f;
-    coef[2 * c] = s1 * wt / count;
-    coef[2 * c + 1] = s2 * wt / count;
-    if (weight_grad) weight_grad[c] = s1;
-    if (bias_grad) bias_grad[c] = s2;
-  }
-}
-
+// input_grad = inv_std * (w * g - (t1 * x_hat + t2)) with t1 = w * sum(g x_hat) / count and
+// t2 = w * sum(g) / count.  Every workgroup sums the P partial pairs of its channel itself (wave 0,
+// lane-strided then a tree: the same order everywhere); the workgroup of slice 0 of the channel's
+// first plane also writes the weight and bias gradients.
 template <typename T, int VEC>
 __global__ __launch_bounds__(kBnBlock) void bn_bwd_apply_kernel(
     const T* __restrict__ g, const T* __restrict__ x, T* __restrict__ dx, const float* __restrict__ mean_in,
-    const float* __restrict__ inv_std_in, const float* __restrict__ coef, const void* __restrict__ w, int wdt,
+    const float* __restrict__ inv_std_in, const float* __restrict__ part, int P, float count,
+    float* __restrict__ weight_grad, float* __restrict__ bias_grad, const void* __restrict__ w, int wdt,
     int C, int S, int64_t total_planes) {
+  __shared__ float smem[2];
   const int sp = S / VEC;
+  const int step = gridDim.y * kBnBlock;
   for (int64_t plane = blockIdx.x; plane < total_planes; plane += gridDim.x) {
     const int c = (int)(plane % C);
-    const float mean = mean_in[c], inv_std = inv_std_in[c];
-    const float t1 = coef[2 * c], t2 = coef[2 * c + 1];
-    const float wt = w ? load_scalar_f32(w, wdt, c) : 1.f;
     const int64_t base = plane * (int64_t)S;
-    for (int i = blockIdx.y * kBnBlock + threadIdx.x; i < sp; i += gridDim.y * kBnBlock) {
-      const int64_t off = base + (int64_t)i * VEC;
-      float gv[VEC], xv[VEC];
-      load_f32<T, VEC>(g + off, gv);
-      load_f32<T, VEC>(x + off, xv);
+    int i0 = blockIdx.y * kBnBlock + threadIdx.x;
+    bool has1;
+    int64_t off[2];
+    RawVec<T, VEC> gin[2], xin[2];
+    auto issue = [&](int i) {   // i < sp
+      has1 = i + step < sp;
+      off[0] = base + (int64_t)i * VEC;
+      off[1] = base + (int64_t)(has1 ? i + step : i) * VEC;
 #pragma unroll
-      for (int j = 0; j < VEC; ++j)
-        gv[j] = inv_std * (wt * gv[j] - (t1 * (xv[j] - mean) * inv_std + t2));
-      store_f32<T, VEC>(dx + off, gv);
+      for (int u = 0; u < 2; ++u) {
+        gin[u].load(g + off[u]);
+        xin[u].load(x + off[u]);
+      }
+    };
+    issue(i0 < sp ? i0 : 0);   // in flight while the partial sums of the channel are added up
+    __syncthreads();   // previous readers of smem are done
+    if (threadIdx.x < 64) {
+      float s1 = 0.f, s2 = 0.f;
+      for (int p = threadIdx.x; p < P; p += 64) {
+        s1 += part[((int64_t)c * P + p) * 2];
+        s2 += part[((int64_t)c * P + p) * 2 + 1];
+      }
+      s1 = wave_reduce(s1, 64, SumOp());
+      s2 = wave_reduce(s2, 64, SumOp());
+      if (threadIdx.x == 0) {
+        smem[0] = s1;
+        smem[1] = s2;
+      }
+    }
+    __syncthreads();
+    const float s1 = smem[0], s2 = smem[1];
+    if (plane < C && blockIdx.y == 0 && threadIdx.x == 0) {
+      if (weight_grad) weight_grad[c] = s1;
+      if (bias_grad) bias_grad[c] = s2;
+    }
+    const float mean = mean_in[c], inv_std = inv_std_in[c];
+    const float wt = w ? load_scalar_f32(w, wdt, c) : 1.f;
+    const float t1 = s1 * wt / count, t2 = s2 * wt / count;
+    while (i0 < sp) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        if (u == 1 && !has1) break;
+        float gv[VEC], xv[VEC];
+        gin[u].get(gv);
+        xin[u].get(xv);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+          gv[j] = inv_std * (wt * gv[j] - (t1 * (xv[j] - mean) * inv_std + t2));
+        store_f32<T, VEC>(dx + off[u], gv);
+      }
+      i0 += 2 * step;
+      if (i0 < sp) issue(i0);
     }
   }
 }
@@ -344,7 +429,6 @@ int at_batch_norm_fwd(const void* input, const void* weight, const void* bias, f
   if (pre_act == output) pre_act = nullptr;
 
   float* part = (float*)workspace;
-  float* stat = part + feat * (int64_t)kMaxSplits * 3;
   const int C = (int)feat, S = (int)spatial;
   const int es = dtype_size(dtype);
   const int vfull = 16 / es;
@@ -354,33 +438,33 @@ int at_batch_norm_fwd(const void* input, const void* weight, const void* bias, f
   return dispatch_dtype(dtype, [&](auto* tp) -> int {
     typedef std::remove_pointer_t<decltype(tp)> T;
     constexpr int VEC = 16 / (int)sizeof(T);
+    int P = 0;
     if (batch_stats) {
-      const int P = bn_splits(batch, C);
+      P = bn_splits(batch, C);
       if (vec_ok)
         hipLaunchKernelGGL((bn_stats_kernel<T, VEC>), dim3(C, P), dim3(kBnBlock), 0, stream, (const T*)input,
                            part, batch, C, S, P);
       else
         hipLaunchKernelGGL((bn_stats_kernel<T, 1>), dim3(C, P), dim3(kBnBlock), 0, stream, (const T*)input,
                            part, batch, C, S, P);
-      const bool update = track_running_stats && is_train && running_mean && running_var;
-      hipLaunchKernelGGL(bn_stats_finalize_kernel, dim3(C), dim3(64), 0, stream, part, P, stat, mean, inv_std,
-                         update ? running_mean : nullptr, update ? running_var : nullptr, running_dtype,
-                         momentum, eps);
-    } else {
-      hipLaunchKernelGGL(bn_eval_stats_kernel, dim3((unsigned)cdiv64(C, 256)), dim3(256), 0, stream,
-                         running_mean, running_var, running_dtype, stat, mean, inv_std, C, eps);
     }
+    const int update = batch_stats && track_running_stats && is_train && running_mean && running_var;
+    const float* part_in = batch_stats ? part : nullptr;   // null: the apply pass reads the running statistics
     dim3 grid;
     const int64_t planes = batch * feat;
     apply_grid(planes, S, vec_ok ? VEC : 1, &grid);
     if (vec_ok) {
       AT_BN_ACT_SWITCH(act, hipLaunchKernelGGL((bn_apply_kernel<T, VEC, ACT>), grid, dim3(kBnBlock), 0, stream,
                                                (const T*)input, (const T*)pre_act_add, (T*)pre_act, (T*)output,
-                                               stat, weight, bias, param_dtype, C, S, param, planes));
+                                               part_in, P, mean, inv_std, running_mean, running_var,
+                                               running_dtype, update, momentum, eps, weight, bias, param_dtype, C,
+                                               S, param, planes));
     } else {
       AT_BN_ACT_SWITCH(act, hipLaunchKernelGGL((bn_apply_kernel<T, 1, ACT>), grid, dim3(kBnBlock), 0, stream,
                                                (const T*)input, (const T*)pre_act_add, (T*)pre_act, (T*)output,
-                                               stat, weight, bias, param_dtype, C, S, param, planes));
+                                               part_in, P, mean, inv_std, running_mean, running_var,
+                                               running_dtype, update, momentum, eps, weight, bias, param_dtype, C,
+                                               S, param, planes));
     }
     return launch_status();
   });
@@ -400,7 +484,6 @@ int at_batch_norm_bwd(const void* output_grad, const void* pre_act, const void* 
   if (!workspace || workspace_bytes < at_batch_norm_workspace_bytes(feat)) return AT_ERR_WORKSPACE;
 
   float* part = (float*)workspace;
-  float* coef = part + feat * (int64_t)kMaxSplits * 3;
   const int C = (int)feat, S = (int)spatial;
   const int vfull = 16 / dtype_size(dtype);
   const bool vec_ok = S % vfull == 0 && aligned16(output_grad) && aligned16(input) && aligned16(input_grad) &&
@@ -420,17 +503,18 @@ int at_batch_norm_bwd(const void* output_grad, const void* pre_act, const void* 
                                                stream, (const T*)output_grad, (const T*)pre_act, (const T*)input,
                                                (T*)pre_act_grad, mean, inv_std, part, batch, C, S, P, param));
     }
-    hipLaunchKernelGGL(bn_bwd_finalize_kernel, dim3(C), dim3(64), 0, stream, part, P, weight, param_dtype,
-                       (float)(batch * spatial), coef, weight_grad, bias_grad);
     dim3 grid;
     const int64_t planes = batch * feat;
     apply_grid(planes, S, vec_ok ? VEC : 1, &grid);
+    const float count = (float)(batch * spatial);
     if (vec_ok)
       hipLaunchKernelGGL((bn_bwd_apply_kernel<T, VEC>), grid, dim3(kBnBlock), 0, stream, (const T*)g_for_apply,
-                         (const T*)input, (T*)input_grad, mean, inv_std, coef, weight, param_dtype, C, S, planes);
+                         (const T*)input, (T*)input_grad, mean, inv_std, part, P, count, weight_grad, bias_grad,
+                         weight, param_dtype, C, S, planes);
     else
       hipLaunchKernelGGL((bn_bwd_apply_kernel<T, 1>), grid, dim3(kBnBlock), 0, stream, (const T*)g_for_apply,
-                         (const T*)input, (T*)input_grad, mean, inv_std, coef, weight, param_dtype, C, S, planes);
+                         (const T*)input, (T*)input_grad, mean, inv_std, part, P, count, weight_grad, bias_grad,
+                         weight, param_dtype, C, S, planes);
     return launch_status();
   });
 }
