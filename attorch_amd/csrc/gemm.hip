@@ -958,6 +958,103 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(SimpleArgs g) {
 }
 
 // ------------------------------------------------------------------------------------------
+// fp32 operands, outputs too small to give every CU a 64x64 tile (a 512 x 256 layer): 32x32 output
+// tiles, four times as many workgroups, and the four waves of a workgroup share the contraction —
+// wave w multiplies k-steps w, w + 4, ... of every 64-wide k-tile — so the serial chain of MFMAs
+// per wave is a quarter as long; the four accumulators are added through LDS in a fixed order.
+// Tiles are fetched with 16-byte loads along the contiguous index of each operand, the next
+// k-tile travelling in registers while the current one is multiplied.
+// ------------------------------------------------------------------------------------------
+// TK (the k-tile) is 256 for long contractions: with so little arithmetic per byte an iteration
+// lasts about as long as its loads take to arrive, so fewer, larger iterations are faster.
+template <bool A_MC, bool B_KC, int TK>
+__global__ __launch_bounds__(256) void gemm_f32_split_kernel(GemmArgs g) {
+  constexpr int TM = 32;
+  constexpr int NV = TK / 32;           // 16-byte vectors per lane, operand and k-tile
+  // LDS image of a tile: as in memory, rows padded by 4 floats (16-byte aligned rows, and the 32
+  // lanes of a fragment read spread over the banks): [outer][TK + 4] for an operand whose rows
+  // run along the contraction, [k][32 + 4] for the other layout.
+  constexpr int kPitchK = TK + 4, kPitchO = TM + 4;
+  constexpr int kTileFloats = TM * kPitchK > TK * kPitchO ? TM * kPitchK : TK * kPitchO;
+  __shared__ __align__(16) float smem[2 * kTileFloats > 4 * 64 * 16 ? 2 * kTileFloats : 4 * 64 * 16];
+  float* const sa = smem;
+  float* const sb = smem + kTileFloats;
+  const float* __restrict__ A = reinterpret_cast<const float*>(g.a);
+  const float* __restrict__ B = reinterpret_cast<const float*>(g.b);
+  const int nbn = (g.N + TM - 1) / TM;
+  const int m0 = (blockIdx.x / nbn) * TM, n0 = (blockIdx.x % nbn) * TM;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+  // Each lane fetches NV 16-byte vectors per operand and k-tile: 4 consecutive k of one outer index
+  // or 4 consecutive outer indices of one k, whichever is contiguous in memory.  Extents along the
+  // vectors are multiples of 4 (host check), so a vector is inside or outside as a whole.
+  float4 ra[NV], rb[NV];
+  auto where = [&](bool outer_contig, int idx, int& o, int& k) {
+    if (outer_contig) { k = idx >> 3; o = (idx & 7) * 4; } else { o = idx / (TK / 4); k = (idx % (TK / 4)) * 4; }
+  };
+  auto fetch_one = [&](const float* base, int64_t ld, bool outer_contig, int o0, int o_lim, int k0, int idx) {
+    int o, k;
+    where(outer_contig, idx, o, k);
+    const int go = o0 + o, gk = k0 + k;
+    if (go >= o_lim || gk >= g.K) return make_float4(0.f, 0.f, 0.f, 0.f);
+    return *reinterpret_cast<const float4*>(base + (outer_contig ? (int64_t)gk * ld + go : (int64_t)go * ld + gk));
+  };
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      ra[i] = fetch_one(A, g.lda, A_MC, m0, g.M, k0, threadIdx.x + i * 256);
+      rb[i] = fetch_one(B, g.ldb, !B_KC, n0, g.N, k0, threadIdx.x + i * 256);
+    }
+  };
+  auto stage_one = [&](float* tile, bool outer_contig, const float4& v, int idx) {
+    int o, k;
+    where(outer_contig, idx, o, k);
+    *reinterpret_cast<float4*>(tile + (outer_contig ? k * kPitchO + o : o * kPitchK + k)) = v;
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      stage_one(sa, A_MC, ra[i], threadIdx.x + i * 256);
+      stage_one(sb, !B_KC, rb[i], threadIdx.x + i * 256);
+    }
+  };
+  auto value = [&](const float* tile, bool outer_contig, int o, int k) {
+    return tile[outer_contig ? k * kPitchO + o : o * kPitchK + k];
+  };
+
+  f32x16 acc;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+  fetch(0);
+  for (int k0 = 0; k0 < g.K; k0 += TK) {
+    stage();
+    __syncthreads();
+    if (k0 + TK < g.K) fetch(k0 + TK);
+#pragma unroll
+    for (int q = 0; q < TK / 8; ++q) {
+      const int k = (q * 4 + wave) * 2 + (lane >> 5);   // k-step q * 4 + wave of this tile
+      // operands swapped so that a lane ends up with 4 consecutive n of one m
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(value(sb, !B_KC, lane & 31, k), value(sa, A_MC, lane & 31, k), acc, 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+  // the operand tiles are dead (barrier above): add the four partial accumulators in wave order
+  float* fold = smem;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) fold[(r * 4 + wave) * 64 + lane] = acc[r];
+  __syncthreads();
+  if (wave != 0) return;
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    acc[r] = (fold[(r * 4 + 0) * 64 + lane] + fold[(r * 4 + 1) * 64 + lane]) +
+             (fold[(r * 4 + 2) * 64 + lane] + fold[(r * 4 + 3) * 64 + lane]);
+  __builtin_amdgcn_wave_barrier();
+  static_assert(32 * 36 <= 4 * 64 * 16, "the epilogue block fits");
+  wave_tile_epilogue<float>(acc, smem, g, m0, n0);
+}
+
+// ------------------------------------------------------------------------------------------
 // Generic kernel for 16-bit operands: any strides and extents, 32x32x16 MFMA, tiles of
 // (32 WM) x (32 WN) x 64 staged through registers into LDS rows that are contiguous along the
 // contraction index.  Each operand is fetched with 16-byte loads when its unit-stride dimension
@@ -1446,6 +1543,19 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
       (ldb % 4) == 0 && (!(a_contig_k || b_contig_k) || (K % 4) == 0) && M >= 32 && N >= 32 &&
       (a_contig_k ? M : K) * lda * 4 < ((int64_t)1 << 31) && (b_contig_k ? N : K) * ldb * 4 < ((int64_t)1 << 31)) {
     GemmArgs g{a, b, c, pre_act, bias, (int)M, (int)N, (int)K, lda, ldb, ldc, ldp, act, param, bias_dt, nullptr, 0, 0};
+    // outputs with fewer 64x64 tiles than CUs: 32x32 tiles, the contraction shared by the waves
+    if (cdiv64(M, 64) * cdiv64(N, 64) < device_cu_count() && K >= 128 && (M % 4) == 0 && (N % 4) == 0) {
+      const unsigned grid = (unsigned)(cdiv64(M, 32) * cdiv64(N, 32));
+#define AT_SPLIT_LAUNCH(TK)                                                                                              \
+  {                                                                                                                      \
+    if (layout == kDx) hipLaunchKernelGGL((gemm_f32_split_kernel<false, true, TK>), dim3(grid), dim3(256), 0, stream, g);       \
+    else if (layout == kDw) hipLaunchKernelGGL((gemm_f32_split_kernel<true, false, TK>), dim3(grid), dim3(256), 0, stream, g);  \
+    else hipLaunchKernelGGL((gemm_f32_split_kernel<false, false, TK>), dim3(grid), dim3(256), 0, stream, g);                    \
+  }
+      if (K >= 512) AT_SPLIT_LAUNCH(256) else AT_SPLIT_LAUNCH(64)
+#undef AT_SPLIT_LAUNCH
+      return launch_status();
+    }
     // 128x128 tiles once they give every CU a workgroup, 64x64 tiles below that
     const bool big = cdiv64(M, 128) * cdiv64(N, 128) >= device_cu_count();
     const unsigned grid = (unsigned)(big ? cdiv64(M, 128) * cdiv64(N, 128) : cdiv64(M, 64) * cdiv64(N, 64));
