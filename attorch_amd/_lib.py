@@ -31,11 +31,11 @@ PROTOTYPES = {
     'at_softmax_fwd': (I, [P, P, L, L, L, L, I, I, I, I, P]),
     'at_softmax_bwd': (I, [P, P, P, L, L, L, L, L, I, I, I, I, I, P]),
     'at_cross_entropy_workspace_bytes': (L, [L]),
-    'at_cross_entropy_fwd_bwd': (I, [P, P, P, P, P, P, L, L, L, L, L, L, I, I, I, P]),
+    'at_cross_entropy_fwd_bwd': (I, [P, P, P, P, P, P, L, L, L, L, L, L, I, I, I, I, P]),
     'at_cross_entropy_bwd': (I, [P, P, P, P, P, P, L, L, L, L, L, I, I, I, I, I, P]),
     'at_cross_entropy_scale_grad': (I, [P, P, L, L, L, I, I, P]),
     'at_cross_entropy_static_max_batch': (L, []),
-    'at_cross_entropy_fwd_bwd_static': (I, [P, P, P, P, P, L, L, L, L, L, I, I, I, P]),
+    'at_cross_entropy_fwd_bwd_static': (I, [P, P, P, P, P, L, L, L, L, L, I, I, I, I, P]),
     'at_nll_loss_workspace_bytes': (L, [L, L]),
     'at_nll_loss_fwd': (I, [P, P, P, P, P, P, L, L, L, L, I, I, I, I, P]),
     'at_nll_loss_bwd': (I, [P, P, P, P, P, L, L, L, I, I, I, I, P]),

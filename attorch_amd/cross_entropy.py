@@ -56,14 +56,19 @@ class CrossEntropyLossAutoGrad(torch.autograd.Function):
         if batch_dim == 0:
             # mean over no rows, as torch: nan loss, empty gradient; nothing is launched
             ctx.empty = True
-            ctx.grad_shape_dtype = (input.shape, output_dtype, input.device)
+            ctx.grad_shape_dtype = (input.shape, input.dtype, input.device)
             return torch.full((), float('nan'), dtype=output_dtype, device=input.device)
 
         logits = input if input.stride(1) == 1 and input.stride(0) >= feat_dim else input.contiguous()
         target_k = target.to(torch.int64).contiguous()
         weight_k = None if weight is None else weight.contiguous()
         output = torch.empty((), dtype=output_dtype, device=input.device)
-        input_grad = (torch.empty((batch_dim, feat_dim), dtype=output_dtype, device=input.device)
+        # The gradient is computed in float32 and rounded once, straight to the dtype of the
+        # logits: under autocast the reference produces a float32 gradient that autograd then
+        # casts to that dtype (attorch/cross_entropy_loss_layer.py:24, custom_fwd with
+        # cast_inputs), which is the same single rounding after a float32 round trip
+        # through memory.
+        input_grad = (torch.empty((batch_dim, feat_dim), dtype=input.dtype, device=input.device)
                       if input.requires_grad else None)
         workspace_bytes = lib.at_cross_entropy_workspace_bytes(batch_dim)
         workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=input.device)
@@ -74,7 +79,8 @@ class CrossEntropyLossAutoGrad(torch.autograd.Function):
                 _lib.ptr(input_grad), _lib.ptr(workspace), workspace_bytes, batch_dim, feat_dim,
                 _lib.row_stride(logits), feat_dim, ignore_index, _lib.dtype_id(logits.dtype),
                 _lib.dtype_id(weight_k.dtype) if weight_k is not None else 0,
-                _lib.dtype_id(output_dtype), _lib.stream_of(input)), 'at_cross_entropy_fwd_bwd')
+                _lib.dtype_id(input.dtype), _lib.dtype_id(output_dtype), _lib.stream_of(input)),
+                'at_cross_entropy_fwd_bwd')
 
         ctx.empty = False
         ctx.output_dtype = output_dtype

@@ -374,7 +374,9 @@ int check_ce_args(const void* logits, const int64_t* target, const void* weight,
 // Forward call on a given workspace (the caller's or the library's own).
 int ce_fwd_bwd(const void* logits, const int64_t* target, const void* weight, void* loss, void* dlogits,
                float* workspace, int64_t batch, int64_t feat, int64_t logits_stride, int64_t dlogits_stride,
-               int64_t ignore_index, int logits_dtype, int weight_dtype, int out_dtype, hipStream_t stream) {
+               int64_t ignore_index, int logits_dtype, int weight_dtype, int out_dtype, int loss_dtype,
+               hipStream_t stream) {
+  if (!dtype_valid(loss_dtype)) return AT_ERR_DTYPE;
   float* denom = workspace;
   float* row_loss = denom + 4;
   hipLaunchKernelGGL(ce_denominator_kernel, dim3(1), dim3(1024), 0, stream, target, weight, weight_dtype,
@@ -383,7 +385,7 @@ int ce_fwd_bwd(const void* logits, const int64_t* target, const void* weight, vo
                           dlogits_stride, ignore_index, logits_dtype, weight_dtype, out_dtype, nullptr, 0, 0,
                           stream);
   if (rc) return rc;
-  hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(1024), 0, stream, row_loss, denom, loss, out_dtype,
+  hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(1024), 0, stream, row_loss, denom, loss, loss_dtype,
                      batch);
   return launch_status();
 }
@@ -410,7 +412,7 @@ int at_cross_entropy_fwd_bwd(const void* logits, const int64_t* target, const vo
                              void* dlogits, void* workspace, int64_t workspace_bytes, int64_t batch,
                              int64_t feat, int64_t logits_stride, int64_t dlogits_stride,
                              int64_t ignore_index, int logits_dtype, int weight_dtype, int out_dtype,
-                             at_stream_t stream_) {
+                             int loss_dtype, at_stream_t stream_) {
   if (!loss) return AT_ERR_NULL;
   int rc = check_ce_args(logits, target, weight, batch, feat, logits_stride, dlogits, dlogits_stride,
                          logits_dtype, weight_dtype, out_dtype);
@@ -418,7 +420,8 @@ int at_cross_entropy_fwd_bwd(const void* logits, const int64_t* target, const vo
   if (!workspace || workspace_bytes < at_cross_entropy_workspace_bytes(batch)) return AT_ERR_WORKSPACE;
   if ((reinterpret_cast<uintptr_t>(workspace) & 3u) != 0) return AT_ERR_ALIGN;
   return ce_fwd_bwd(logits, target, weight, loss, dlogits, (float*)workspace, batch, feat, logits_stride,
-                    dlogits_stride, ignore_index, logits_dtype, weight_dtype, out_dtype, (hipStream_t)stream_);
+                    dlogits_stride, ignore_index, logits_dtype, weight_dtype, out_dtype, loss_dtype,
+                    (hipStream_t)stream_);
 }
 
 int64_t at_cross_entropy_static_max_batch(void) { return kCeStaticMaxBatch; }
@@ -426,7 +429,7 @@ int64_t at_cross_entropy_static_max_batch(void) { return kCeStaticMaxBatch; }
 int at_cross_entropy_fwd_bwd_static(const void* logits, const int64_t* target, const void* weight, void* loss,
                                     void* dlogits, int64_t batch, int64_t feat, int64_t logits_stride,
                                     int64_t dlogits_stride, int64_t ignore_index, int logits_dtype,
-                                    int weight_dtype, int out_dtype, at_stream_t stream_) {
+                                    int weight_dtype, int out_dtype, int loss_dtype, at_stream_t stream_) {
   if (!loss) return AT_ERR_NULL;
   int rc = check_ce_args(logits, target, weight, batch, feat, logits_stride, dlogits, dlogits_stride,
                          logits_dtype, weight_dtype, out_dtype);
@@ -452,7 +455,8 @@ int at_cross_entropy_fwd_bwd_static(const void* logits, const int64_t* target, c
   // every element the kernels read from the workspace is written earlier in this call (the divisor
   // by the first launch, one loss per row by the row kernel), so nothing has to be cleared
   return ce_fwd_bwd(logits, target, weight, loss, dlogits, scratch, batch, feat, logits_stride,
-                    dlogits_stride, ignore_index, logits_dtype, weight_dtype, out_dtype, (hipStream_t)stream_);
+                    dlogits_stride, ignore_index, logits_dtype, weight_dtype, out_dtype, loss_dtype,
+                    (hipStream_t)stream_);
 }
 
 int at_cross_entropy_bwd(const void* logits, const int64_t* target, const void* weight,

@@ -1233,14 +1233,38 @@ __global__ __launch_bounds__(256) void act_bwd_kernel(
   constexpr int ROWS = 4;  // rows in flight per lane
   for (int64_t rb = r0; rb < r1; rb += ROWS) {
     float d[ROWS][VEC], zz[ROWS][VEC];
+    if (VEC_OK) {
+      // all loads of the row block first, none inside a branch: a row past the slice reads the last
+      // row of the slice again (its values are not used), so no load waits for another
+      constexpr int ND = (int)sizeof(TDY) * VEC / 16, NZ = (int)sizeof(TZ) * VEC / 16;   // 16-byte vectors per row
+      uint4 rd[ROWS][ND], rz[ROWS][NZ];
 #pragma unroll
-    for (int u = 0; u < ROWS; ++u) {
-      const int64_t r = rb + u;
-      if (r < r1) {
-        if (VEC_OK) {
-          load_f32<TDY, VEC>(dy + r * dys + c, d[u]);
-          load_f32<TZ, VEC>(z + r * zs + c, zz[u]);
-        } else {
+      for (int u = 0; u < ROWS; ++u) {
+        const int64_t r = rb + u < r1 ? rb + u : r1 - 1;
+#pragma unroll
+        for (int q = 0; q < ND; ++q) rd[u][q] = reinterpret_cast<const uint4*>(dy + r * dys + c)[q];
+#pragma unroll
+        for (int q = 0; q < NZ; ++q) rz[u][q] = reinterpret_cast<const uint4*>(z + r * zs + c)[q];
+      }
+#pragma unroll
+      for (int u = 0; u < ROWS; ++u) {
+        union { uint4 raw[ND]; TDY e[VEC]; } ud;
+        union { uint4 raw[NZ]; TZ e[VEC]; } uz;
+#pragma unroll
+        for (int q = 0; q < ND; ++q) ud.raw[q] = rd[u][q];
+#pragma unroll
+        for (int q = 0; q < NZ; ++q) uz.raw[q] = rz[u][q];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          d[u][j] = to_f32(ud.e[j]);
+          zz[u][j] = to_f32(uz.e[j]);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < ROWS; ++u) {
+        const int64_t r = rb + u;
+        if (r < r1) {
 #pragma unroll
           for (int j = 0; j < VEC; ++j) {
             const bool ok = c + j < N;

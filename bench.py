@@ -23,7 +23,7 @@ import json
 import os
 import sys
 import time
-from typing import Callable, Dict, List, Tuple
+from typing import Callable, Dict, List, Optional, Tuple
 
 import torch
 
@@ -35,7 +35,10 @@ PEAK_MFMA_FP32_TFLOPS = 157.3    # dense fp32 MFMA
 # multi-kernel workloads), from the rocprofv3 FETCH_SIZE / WRITE_SIZE passes summarised in
 # profiles/bench_all_configs.hbm_traffic.txt (scaled there by a copy of known size).  Counters are
 # taken in separate profiling runs, so these are recorded measurements, not live ones; reads that
-# the 256 MB Infinity Cache serves are included.
+# the 256 MB Infinity Cache serves are included.  They belong to the kernel sources whose digest is
+# TRAFFIC_SOURCE_DIGEST: when the sources of the loaded library differ, `traffic` is reported as
+# null and the recorded figure moves to `traffic_recorded` (stale until the profile is redone).
+TRAFFIC_SOURCE_DIGEST = 'unset'
 MEASURED_TRAFFIC_BYTES = {
     'c4_linear_fwd': 4299419969,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.0 GiB read, 1.0 GiB written
     'c2_layer_norm': 387435537,       # norm_fwd + norm_bwd + reduce_partials
@@ -45,10 +48,48 @@ MEASURED_TRAFFIC_BYTES = {
     'c2_glu': 269037744,              # glu forward + backward
     'c2_mse': 335722286,              # p_loss forward + backward
     'c3_cross_entropy': 1610258526,   # ce_row_kernel (ignored rows are not read)
+    'c3_cross_entropy_autocast': None,
     'c3_nll_loss': 827004360,         # nll forward (a gather) + the single-pass gradient write
     'c5_conv': 687076692,             # 2 window kernels + weight gradient + 2 layout copies + weight reorders
     'c5_batch_norm': 616867690,       # stats + apply + backward reduce + backward apply
 }
+
+
+def kernel_source_digest() -> str:
+    """
+    Digest of the kernel sources (csrc/*.hip, csrc/*.h, include/*.h) the library is built from.
+    """
+    import hashlib
+    root = os.path.dirname(os.path.abspath(__file__))
+    h = hashlib.sha256()
+    files = []
+    for sub in ('attorch_amd/csrc', 'include'):
+        d = os.path.join(root, sub)
+        files += [os.path.join(d, f) for f in os.listdir(d) if f.endswith(('.hip', '.h'))]
+    for f in sorted(files):
+        h.update(os.path.basename(f).encode())
+        with open(f, 'rb') as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+_DIGEST_MATCHES = None
+
+
+def traffic_fields(key: str) -> Dict:
+    """
+    {'traffic': bytes or None} for a roofline object, plus provenance when a figure is recorded.
+    """
+    global _DIGEST_MATCHES
+    if _DIGEST_MATCHES is None:
+        _DIGEST_MATCHES = kernel_source_digest() == TRAFFIC_SOURCE_DIGEST
+    recorded = MEASURED_TRAFFIC_BYTES.get(key)
+    if recorded is None:
+        return {'traffic': None}
+    if _DIGEST_MATCHES:
+        return {'traffic': recorded, 'traffic_source': 'profiles/bench_all_configs.hbm_traffic.txt'}
+    return {'traffic': None, 'traffic_recorded': recorded,
+            'traffic_note': 'recorded for other kernel sources than the ones loaded; see profiles/'}
 
 
 def parse_args() -> argparse.Namespace:
@@ -94,6 +135,59 @@ def wall_time_ms(fn: Callable[[], None], steps: int, warmup: int) -> float:
         fn()
     torch.cuda.synchronize()
     return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def module_times_ms(forward: Callable[[int], torch.Tensor], backward: Callable[[torch.Tensor, int], None],
+                    iters: int, warmup: int, sets: int = 1) -> Dict:
+    """
+    Timings of a layer called the way a user calls it (nn.Module + autograd, allocations and
+    host work included): forward alone, forward + backward, and their difference.
+    forward(i) runs the layer on input set i and returns its output; backward(out, i)
+    back-propagates from it.  Wall-clock over `iters` calls bracketed by device syncs.
+    """
+    count = [0]
+
+    def fwd_only():
+        count[0] += 1
+        forward(count[0] % sets)
+
+    def fwd_bwd():
+        count[0] += 1
+        i = count[0] % sets
+        backward(forward(i), i)
+    ms_f = wall_time_ms(fwd_only, iters, warmup)
+    ms_fb = wall_time_ms(fwd_bwd, iters, warmup)
+
+    # The same forward + backward calls captured once into a HIP graph (one pass over every input
+    # set) and replayed: what the module path costs on the GPU with the host out of the way.
+    def all_sets():
+        for i in range(sets):
+            backward(forward(i), i)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            all_sets()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        all_sets()
+    ms_graph = gpu_time_ms(graph.replay, max(2, iters // sets), 2) / sets
+    del graph
+    return {'ms_fwd': ms_f, 'ms_bwd': ms_fb - ms_f, 'ms_fwd_bwd': ms_fb, 'ms_fwd_bwd_hip_graph': ms_graph,
+            'note': 'nn.Module + autograd calls with their allocations and casts: wall clock per eager call '
+                    '(host-bound below about 0.1 ms), and per replay of the same calls captured in a HIP graph'}
+
+
+def functional_cpu_entry(fn: Callable[[], None], units: float, unit: str, sample: str, dtype) -> Dict:
+    """
+    torch's own CPU kernels (torch.nn.functional, forward + backward through autograd) in the
+    workload's dtype on all host threads torch uses: `units` of work per call of fn.
+    """
+    sec = cpu_time_s(fn)
+    return {'value': units / sec, 'unit': unit, 'cores': torch.get_num_threads(),
+            'kind': 'torch.nn.functional on the CPU', 'dtype': str(dtype).replace('torch.', ''), 'sample': sample}
 
 
 def cpu_time_s(fn: Callable[[], None], reps: int = 3) -> float:
@@ -226,7 +320,7 @@ def bench_linear(cfg: str, steps: int, warmup: int, with_cpu: bool) -> Dict:
                           for kk in ('linear_fwd', 'linear_bwd_input', 'linear_bwd_weight')},
         'roofline': {'bound': 'mfma', 'kernel': 'linear_fwd (GEMM + bias + activation epilogue)',
                      'achieved': fwd_tflops, 'peak': peak, 'unit': 'TFLOP/s', 'frac': fwd_tflops / peak,
-                     'traffic': MEASURED_TRAFFIC_BYTES['c4_linear_fwd'] if cfg == 'c4' else None},
+                     **(traffic_fields('c4_linear_fwd') if cfg == 'c4' else {'traffic': None})},
         'frac_of_peak_step': flop / ms_step / 1e9 / peak,
     }
     if with_cpu:
@@ -244,6 +338,16 @@ def bench_linear(cfg: str, steps: int, warmup: int, with_cpu: bool) -> Dict:
         out['cpu_baseline'] = {'value': 6.0 * rows * k * n / sec / 1e12, 'unit': 'TFLOP/s',
                                'cores': torch.get_num_threads(), 'kind': 'port',
                                'sample': f'first {rows} of {m} rows, full K and N, oracle fwd+bwd in fp32 compute'}
+        F = torch.nn.functional
+        xg = xs.clone().requires_grad_(True)
+        wg, bg = w.T.contiguous().requires_grad_(True), b.clone().requires_grad_(True)
+        act_fn = (lambda t: F.gelu(t, approximate='tanh')) if name == 'geluapprox' else F.relu
+
+        def cpu_functional():
+            xg.grad = wg.grad = bg.grad = None
+            act_fn(F.linear(xg, wg, bg)).backward(dys)
+        out['cpu_functional'] = functional_cpu_entry(
+            cpu_functional, 6.0 * rows * k * n / 1e12, 'TFLOP/s', f'first {rows} of {m} rows, full K and N', dtype)
     return out
 
 
@@ -361,6 +465,45 @@ def bench_rows(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
         oracle.act_dropout_forward(xc[:crow], 'geluapprox', None, dropped, 0.1)
         oracle.act_dropout_backward(dyc[:crow], xc[:crow], 'geluapprox', None, dropped, 0.1)
 
+    # the same layers as a user calls them: nn.Module + autograd on the rotating inputs
+    import attorch_amd
+    F = torch.nn.functional
+    xins = [x.clone().requires_grad_(True) for x in xs]
+    ln_mod = attorch_amd.LayerNorm(feat, dtype=dtype, device='cuda')
+    rms_mod = attorch_amd.RMSNorm(feat, eps=1e-5, dtype=dtype, device='cuda')
+    act_mod = attorch_amd.GELU(approximate='tanh', drop_p=0.1)
+    with torch.no_grad():
+        ln_mod.weight.copy_(w), ln_mod.bias.copy_(b), rms_mod.weight.copy_(w)
+    modules = {'LayerNorm': ln_mod, 'RMSNorm': rms_mod, 'Softmax': attorch_amd.Softmax(dim=-1),
+               'LogSoftmax': attorch_amd.LogSoftmax(dim=-1), 'GELU(tanh)+Dropout(0.1) layer': act_mod}
+
+    def module_level(mod):
+        def fwd(i):
+            return mod(xins[i])
+
+        def bwd(out, i):
+            xins[i].grad = None
+            for prm in mod.parameters():
+                prm.grad = None
+            out.backward(dys[i])
+        return module_times_ms(fwd, bwd, iters, warmup, nsets)
+
+    xg = xc[:crow].clone().requires_grad_(True)
+    wg, bg = wc.clone().requires_grad_(True), bc.clone().requires_grad_(True)
+    functional = {
+        'LayerNorm': lambda: F.layer_norm(xg, (feat,), wg, bg, 1e-5),
+        'RMSNorm': lambda: F.rms_norm(xg, (feat,), wg, 1e-5),
+        'Softmax': lambda: F.softmax(xg, dim=-1),
+        'LogSoftmax': lambda: F.log_softmax(xg, dim=-1),
+        'GELU(tanh)+Dropout(0.1) layer': lambda: F.dropout(F.gelu(xg, approximate='tanh'), 0.1),
+    }
+
+    def cpu_functional(name):
+        def f():
+            xg.grad = wg.grad = bg.grad = None
+            functional[name]().backward(dyc[:crow])
+        return f
+
     traffic_key = {'LayerNorm': 'c2_layer_norm', 'RMSNorm': 'c2_rms_norm', 'Softmax': 'c2_softmax',
                    'LogSoftmax': 'c2_softmax', 'GELU(tanh)+Dropout(0.1) layer': 'c2_act_dropout'}
     for name, f, bwd, cpu in (('LayerNorm', ln_f, ln_b, cpu_ln), ('RMSNorm', rms_f, rms_b, cpu_rms),
@@ -374,15 +517,18 @@ def bench_rows(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
             'unit': 'GB/s', 'ms_fwd': ms_f, 'ms_bwd': ms_b,
             'fwd_gbs': 2 * tbytes / ms_f / 1e6, 'bwd_gbs': 3 * tbytes / ms_b / 1e6,
             'roofline': {'bound': 'hbm', 'achieved': gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
-                         'frac': gbs / PEAK_HBM_GBS, 'traffic': MEASURED_TRAFFIC_BYTES.get(traffic_key[name])},
+                         'frac': gbs / PEAK_HBM_GBS, **traffic_fields(traffic_key[name])},
             'buffer_rotation': f'{nsets} sets of X/dY/Y/dX (64 MiB each)',
             'elementwise_reference': stream_ref,
+            'module_level': module_level(modules[name]),
         }
         if with_cpu:
             sec = cpu_time_s(cpu)
             entry['cpu_baseline'] = {'value': 5 * crow * feat * 2 / sec / 1e9, 'unit': 'GB/s',
                                      'cores': torch.get_num_threads(), 'kind': 'port',
                                      'sample': f'first {crow} of {rows_} rows, oracle fwd+bwd'}
+            entry['cpu_functional'] = functional_cpu_entry(
+                cpu_functional(name), 5 * crow * feat * 2 / 1e9, 'GB/s', f'first {crow} of {rows_} rows', dtype)
         results.append(entry)
 
     # Elementwise layers outside the headline configs, on the same buffers: GLU (sigmoid) gated
@@ -424,7 +570,7 @@ def bench_rows(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
             'fwd_gbs': fwd_units * tbytes / ms_f / 1e6, 'bwd_gbs': bwd_units * tbytes / ms_b / 1e6,
             'roofline': {'bound': 'hbm', 'achieved': gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
                          'frac': gbs / PEAK_HBM_GBS,
-                         'traffic': MEASURED_TRAFFIC_BYTES['c2_glu' if name.startswith('GLU') else 'c2_mse']},
+                         **traffic_fields('c2_glu' if name.startswith('GLU') else 'c2_mse')},
             'elementwise_reference': stream_ref,
         })
     return results
@@ -453,21 +599,49 @@ def bench_cross_entropy(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
     st = raw.stream
     results = []
     import oracle
-    for label, wt in (('unweighted', None), ('class-weighted', weight)):
+    import attorch_amd
+    kept = int((target != -100).sum())
+    iters = max(5, steps // 2)
+    # rows whose target is ignore_index are never read: T * kept / rows read, T written
+    read_bytes = tbytes * kept / rows_
+
+    def c_abi_step(wt, gdt, grad, loss_):
         def f():
             raw.check(lib.at_cross_entropy_fwd_bwd(logits.data_ptr(), tgt.data_ptr(),
-                                                   None if wt is None else wt.data_ptr(), loss.data_ptr(),
-                                                   dlogits.data_ptr(), ws.data_ptr(), wsb, rows_, feat, feat, feat,
-                                                   -100, dt, 0, dt, st()), 'ce')
-            raw.check(lib.at_cross_entropy_scale_grad(dlogits.data_ptr(), one.data_ptr(), rows_, feat, feat, dt, dt,
-                                                      st()), 'ce_scale')
-        ms = gpu_time_ms(f, max(5, steps // 2), warmup)
-        gbs = 2 * tbytes / ms / 1e6
+                                                   None if wt is None else wt.data_ptr(), loss_.data_ptr(),
+                                                   grad.data_ptr(), ws.data_ptr(), wsb, rows_, feat, feat, feat,
+                                                   -100, dt, 0, gdt, gdt, st()), 'ce')
+            # backward with an upstream gradient of one: the kernel reads the upstream value on
+            # the device and leaves the gradient the forward pass wrote as it is
+            raw.check(lib.at_cross_entropy_bwd(logits.data_ptr(), tgt.data_ptr(),
+                                               None if wt is None else wt.data_ptr(), one.data_ptr(),
+                                               ws.data_ptr(), grad.data_ptr(), rows_, feat, feat, feat, -100, 1,
+                                               dt, 0, dt, gdt, st()), 'ce_bwd')
+        return f
+
+    def module_times(wt, autocast):
+        crit = attorch_amd.CrossEntropyLoss(weight=wt)
+        xin = logits.clone().requires_grad_(True)
+
+        def fwd(_):
+            with torch.autocast('cuda', dtype=dtype, enabled=autocast):
+                return crit(xin, tgt)
+
+        def bwd(out, _):
+            xin.grad = None
+            out.backward()
+        return module_times_ms(fwd, bwd, iters, warmup)
+
+    for label, wt in (('unweighted', None), ('class-weighted', weight)):
+        ms = gpu_time_ms(c_abi_step(wt, dt, dlogits, loss), iters, warmup)
+        gbs = (read_bytes + tbytes) / ms / 1e6
         entry = {
             'workload': f'c3: CrossEntropyLoss fp16 fwd+bwd logits[{rows_},{feat}], 5% ignore_index, {label}',
             'metric': 'HBM GB/s', 'value': gbs, 'unit': 'GB/s', 'ms_fwd_bwd': ms,
+            'algorithmic_bytes': int(read_bytes + tbytes),
             'roofline': {'bound': 'hbm', 'achieved': gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
-                         'frac': gbs / PEAK_HBM_GBS, 'traffic': MEASURED_TRAFFIC_BYTES['c3_cross_entropy']},
+                         'frac': gbs / PEAK_HBM_GBS, **traffic_fields('c3_cross_entropy')},
+            'module_level': module_times(wt, False),
         }
         if with_cpu and wt is None:
             crow = 512
@@ -480,7 +654,31 @@ def bench_cross_entropy(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
             entry['cpu_baseline'] = {'value': 2 * crow * feat * 2 / sec / 1e9, 'unit': 'GB/s',
                                      'cores': torch.get_num_threads(), 'kind': 'port',
                                      'sample': f'first {crow} of {rows_} rows, oracle loss + gradient'}
+            lcg = lc.clone().requires_grad_(True)
+
+            def cpu_functional():
+                lcg.grad = None
+                torch.nn.functional.cross_entropy(lcg, tc, ignore_index=-100).backward()
+            entry['cpu_functional'] = functional_cpu_entry(
+                cpu_functional, 2 * crow * feat * 2 / 1e9, 'GB/s', f'first {crow} of {rows_} rows', dtype)
         results.append(entry)
+
+    # Under autocast the loss and the gradient of the fp16 logits are fp32 (the reference's
+    # custom_fwd(cast_inputs=float32) semantics): T read, 2T written, still one pass.
+    grad32 = torch.empty((rows_, feat), dtype=torch.float32, device='cuda')
+    loss32 = torch.empty((), dtype=torch.float32, device='cuda')
+    ms = gpu_time_ms(c_abi_step(None, raw._lib.dtype_id(torch.float32), grad32, loss32), iters, warmup)
+    gbs = (read_bytes + 2 * tbytes) / ms / 1e6
+    results.append({
+        'workload': f'c3 autocast: CrossEntropyLoss fp16 logits[{rows_},{feat}] -> fp32 loss and gradient, '
+                    f'5% ignore_index, unweighted',
+        'metric': 'HBM GB/s', 'value': gbs, 'unit': 'GB/s', 'ms_fwd_bwd': ms,
+        'algorithmic_bytes': int(read_bytes + 2 * tbytes),
+        'roofline': {'bound': 'hbm', 'achieved': gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                     'frac': gbs / PEAK_HBM_GBS, **traffic_fields('c3_cross_entropy_autocast')},
+        'module_level': module_times(None, True),
+    })
+    del grad32
 
     # The reference's alternative to the fused loss: LogSoftmax followed by NLLLoss
     # (weighted mean).  The NLL kernels gather one element per row forward and write the whole
@@ -509,7 +707,7 @@ def bench_cross_entropy(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
         'metric': 'HBM GB/s', 'value': gbs, 'unit': 'GB/s', 'ms_fwd': ms_f, 'ms_bwd': ms_b,
         'bwd_gbs': tbytes / ms_b / 1e6,
         'roofline': {'bound': 'hbm', 'achieved': gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
-                     'frac': gbs / PEAK_HBM_GBS, 'traffic': MEASURED_TRAFFIC_BYTES['c3_nll_loss']},
+                     'frac': gbs / PEAK_HBM_GBS, **traffic_fields('c3_nll_loss')},
     })
     return results
 
@@ -618,13 +816,13 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
         'workload': f'c5: Conv2d 3x3 s1 p1 bf16 fwd+bwd X[{n},{c},{h},{w_}] W[{c},{c},3,3]',
         'metric': 'conv TFLOP/s', 'value': conv_tf, 'unit': 'TFLOP/s', 'kernel_ms': {k_: t[k_] for k_ in t if 'conv' in k_},
         'roofline': {'bound': 'mfma', 'achieved': conv_tf, 'peak': PEAK_MFMA_16BIT_TFLOPS, 'unit': 'TFLOP/s',
-                     'frac': conv_tf / PEAK_MFMA_16BIT_TFLOPS, 'traffic': MEASURED_TRAFFIC_BYTES['c5_conv']},
+                     'frac': conv_tf / PEAK_MFMA_16BIT_TFLOPS, **traffic_fields('c5_conv')},
     }
     bn_entry = {
         'workload': f'c5: BatchNorm2d(train)+residual+ReLU bf16 fwd+bwd X[{n},{c},{h},{w_}]',
         'metric': 'HBM GB/s', 'value': bn_gbs, 'unit': 'GB/s', 'ms_fwd': t['bn_fwd'], 'ms_bwd': t['bn_bwd'],
         'roofline': {'bound': 'hbm', 'achieved': bn_gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
-                     'frac': bn_gbs / PEAK_HBM_GBS, 'traffic': MEASURED_TRAFFIC_BYTES['c5_batch_norm']},
+                     'frac': bn_gbs / PEAK_HBM_GBS, **traffic_fields('c5_batch_norm')},
         'buffer_rotation': f'{nsets} sets of 7 tensors (49 MiB each)',
     }
     # the block end to end through the modules (conv -> bn + residual + relu, fwd + bwd)
@@ -644,6 +842,26 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
         bn(conv(xin), rin).backward(dys[0])
 
     conv_entry['block_ms_fwd_bwd_modules'] = wall_time_ms(block, max(3, steps // 4), 2)
+
+    # each layer on its own through its module, inputs rotating as above
+    xins = [x.clone().requires_grad_(True) for x in xs]
+    rins = [r.clone().requires_grad_(True) for r in ress]
+
+    def bn_fwd_mod(i):
+        return bn(xins[i], rins[i])
+
+    def conv_fwd_mod(i):
+        return conv(xins[i])
+
+    def mod_bwd(out, i):
+        xins[i].grad = None
+        rins[i].grad = None
+        conv.weight.grad = None
+        bn.weight.grad = None
+        bn.bias.grad = None
+        out.backward(dys[i])
+    bn_entry['module_level'] = module_times_ms(bn_fwd_mod, mod_bwd, iters, warmup, nsets)
+    conv_entry['module_level'] = module_times_ms(conv_fwd_mod, mod_bwd, iters, warmup, nsets)
     if with_cpu:
         import oracle
         cn = 8
@@ -665,6 +883,23 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
         bn_entry['cpu_baseline'] = {'value': 9 * tbytes * cn / n / sec / 1e9, 'unit': 'GB/s',
                                     'cores': torch.get_num_threads(), 'kind': 'port',
                                     'sample': f'first {cn} of {n} images, oracle fwd+bwd'}
+        F = torch.nn.functional
+        xg, rg = xc.clone().requires_grad_(True), rc.clone().requires_grad_(True)
+        wg_, bw_, bb_ = (wc.clone().requires_grad_(True), bn_w.cpu().requires_grad_(True),
+                         bn_b.cpu().requires_grad_(True))
+        rm_c, rv_c = rm.cpu().to(dtype), rv.cpu().to(dtype)
+
+        def cpu_conv_functional():
+            xg.grad = wg_.grad = None
+            F.conv2d(xg, wg_, None, 1, 1).backward(dyc)
+
+        def cpu_bn_functional():
+            xg.grad = rg.grad = bw_.grad = bb_.grad = None
+            F.relu(F.batch_norm(xg, rm_c, rv_c, bw_, bb_, True, 0.1, 1e-5) + rg).backward(dyc)
+        conv_entry['cpu_functional'] = functional_cpu_entry(
+            cpu_conv_functional, 3 * gflop * cn / n / 1e3, 'TFLOP/s', f'first {cn} of {n} images', dtype)
+        bn_entry['cpu_functional'] = functional_cpu_entry(
+            cpu_bn_functional, 9 * tbytes * cn / n / 1e9, 'GB/s', f'first {cn} of {n} images', dtype)
     return [conv_entry, bn_entry]
 
 
@@ -707,6 +942,7 @@ def main() -> int:
                    'algorithmic_flop_per_step': 6 * 16384 * 4096 * 16384},
         'roofline': head['roofline'],
         'cpu_baseline': head.get('cpu_baseline'),
+        'cpu_functional': head.get('cpu_functional'),
         'frac_of_peak_step': head['frac_of_peak_step'],
         'kernel_ms': head['kernel_ms'], 'kernel_tflops': head['kernel_tflops'],
         'configs': extra,

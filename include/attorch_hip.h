@@ -146,10 +146,12 @@ int at_softmax_bwd(const void* dy, const void* y, void* dx, int64_t batch, int64
  * upstream gradient of 1:  dlogits = (softmax - onehot(target)) * w[target] / denom, with
  * denom = sum of w[target] over kept rows (or the kept-row count when weight is null).
  * Rows whose target equals ignore_index — or lies outside [0, feat) — contribute nothing and
- * get an all-zero gradient row. loss is one element of out_dtype; workspace needs
- * at_cross_entropy_workspace_bytes(batch) bytes; on return workspace[0] (fp32) holds denom.
- * dlogits may have the dtype of the logits or be fp32 (the reference's autocast policy returns
- * an fp32 loss and gradient for 16-bit logits, cross_entropy_loss_layer.py:59,108).
+ * get an all-zero gradient row. loss is one element of loss_dtype, dlogits has out_dtype;
+ * workspace needs at_cross_entropy_workspace_bytes(batch) bytes; on return workspace[0] (fp32)
+ * holds denom.  dlogits may have the dtype of the logits or be fp32 (the reference's autocast
+ * policy computes an fp32 loss and gradient for 16-bit logits, cross_entropy_loss_layer.py:59,108;
+ * autograd then rounds that gradient to the dtype of the logits, which out_dtype = logits_dtype
+ * with loss_dtype = fp32 produces in one step).
  * at_cross_entropy_bwd is the reference's backward kernel (cross_entropy_loss_kernels.py:96-172):
  * dlogits = output_grad * (softmax - onehot) * w[target] / denom, recomputed from the logits,
  * with output_grad read on the device as one element of grad_dtype (:155) and multiplied in
@@ -167,7 +169,7 @@ int at_cross_entropy_fwd_bwd(const void* logits, const int64_t* target, const vo
                              void* loss, void* dlogits, void* workspace, int64_t workspace_bytes,
                              int64_t batch, int64_t feat, int64_t logits_stride,
                              int64_t dlogits_stride, int64_t ignore_index, int logits_dtype,
-                             int weight_dtype, int out_dtype, at_stream_t stream);
+                             int weight_dtype, int out_dtype, int loss_dtype, at_stream_t stream);
 
 int at_cross_entropy_bwd(const void* logits, const int64_t* target, const void* weight,
                          const void* output_grad, const void* workspace, void* dlogits,
@@ -195,7 +197,7 @@ int at_cross_entropy_fwd_bwd_static(const void* logits, const int64_t* target,
                                     int64_t batch, int64_t feat, int64_t logits_stride,
                                     int64_t dlogits_stride, int64_t ignore_index,
                                     int logits_dtype, int weight_dtype, int out_dtype,
-                                    at_stream_t stream);
+                                    int loss_dtype, at_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * Negative log likelihood loss — replaces nll_loss_forward_kernel / nll_loss_backward_kernel,

@@ -66,7 +66,7 @@ def test_argument_errors_without_gpu() -> None:
     assert lib.at_act_bwd(p, p, p, None, None, 0, 4, 8, 8, 8, 8, 0, 0.0, 0, 0, 0, None) == -4
     assert lib.at_act_bwd(p, p, p, p, None, 0, 4, 8, 8, 8, 8, 4, 0.0, 0, 0, 0, None) == -5
     # missing / short workspace
-    assert lib.at_cross_entropy_fwd_bwd(p, p, None, p, None, None, 0, 4, 8, 8, 8, -100, 0, 0, 0, None) == -5
+    assert lib.at_cross_entropy_fwd_bwd(p, p, None, p, None, None, 0, 4, 8, 8, 8, -100, 0, 0, 0, 0, None) == -5
     assert lib.at_layer_norm_bwd(p, p, p, p, p, p, p, None, p, 16, 4, 8, 8, 8, 8, 0, 0, 0, 0, None) == -5
     assert lib.at_batch_norm_fwd(p, None, None, None, None, None, None, p, None, None, None, 0,
                                  4, 8, 1, 0.1, 1e-5, 0, 0.0, 0, 1, 0, 0, 0, None) == -5

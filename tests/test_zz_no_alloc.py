@@ -22,7 +22,8 @@ def run_pair(lib, rows, vocab, dtype, out_dtype, weighted, seed):
     target = target.cuda()
     weight = (0.5 + torch.rand(vocab, generator=gen)).cuda() if weighted else None
     stream = _lib.stream_of(x)
-    ids = (_lib.dtype_id(dtype), 0 if weight is None else _lib.dtype_id(weight.dtype), _lib.dtype_id(out_dtype))
+    ids = (_lib.dtype_id(dtype), 0 if weight is None else _lib.dtype_id(weight.dtype), _lib.dtype_id(out_dtype),
+           _lib.dtype_id(out_dtype))
 
     loss_a = torch.empty((), dtype=out_dtype, device='cuda')
     grad_a = torch.empty(rows, vocab, dtype=out_dtype, device='cuda')
@@ -64,7 +65,7 @@ def test_static_workspace_rejects_batches_beyond_its_limit() -> None:
     target = torch.zeros(rows, dtype=torch.int64, device='cuda')
     loss = torch.empty((), device='cuda')
     rc = lib.at_cross_entropy_fwd_bwd_static(x.data_ptr(), target.data_ptr(), None, loss.data_ptr(), None,
-                                             rows, vocab, vocab, vocab, -100, 0, 0, 0, _lib.stream_of(x))
+                                             rows, vocab, vocab, vocab, -100, 0, 0, 0, 0, _lib.stream_of(x))
     assert rc == -5   # AT_ERR_WORKSPACE
     with pytest.raises(RuntimeError, match='workspace'):
         _lib.check(rc, 'at_cross_entropy_fwd_bwd_static')
