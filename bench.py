@@ -38,20 +38,20 @@ PEAK_MFMA_FP32_TFLOPS = 157.3    # dense fp32 MFMA
 # the 256 MB Infinity Cache serves are included.  They belong to the kernel sources whose digest is
 # TRAFFIC_SOURCE_DIGEST: when the sources of the loaded library differ, `traffic` is reported as
 # null and the recorded figure moves to `traffic_recorded` (stale until the profile is redone).
-TRAFFIC_SOURCE_DIGEST = 'unset'
+TRAFFIC_SOURCE_DIGEST = '657b3fe26ba77a88'
 MEASURED_TRAFFIC_BYTES = {
-    'c4_linear_fwd': 4299419969,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.0 GiB read, 1.0 GiB written
-    'c2_layer_norm': 387435537,       # norm_fwd + norm_bwd + reduce_partials
-    'c2_rms_norm': 378436585,
-    'c2_softmax': 335720132,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
-    'c2_act_dropout': 336053007,      # act_dropout forward + backward
-    'c2_glu': 269037744,              # glu forward + backward
-    'c2_mse': 335722286,              # p_loss forward + backward
-    'c3_cross_entropy': 1610258526,   # ce_row_kernel (ignored rows are not read)
-    'c3_cross_entropy_autocast': None,
-    'c3_nll_loss': 827004360,         # nll forward (a gather) + the single-pass gradient write
-    'c5_conv': 687076692,             # 2 window kernels + weight gradient + 2 layout copies + weight reorders
-    'c5_batch_norm': 616867690,       # stats + apply + backward reduce + backward apply
+    'c4_linear_fwd': 4299194335,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.0 GiB read, 1.0 GiB written
+    'c2_layer_norm': 362345316,       # norm_fwd + norm_bwd + reduce_partials
+    'c2_rms_norm': 361815447,
+    'c2_softmax': 336103416,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
+    'c2_act_dropout': 336057469,      # act_dropout forward + backward
+    'c2_glu': 269044817,              # glu forward + backward
+    'c2_mse': 335730544,              # p_loss forward + backward
+    'c3_cross_entropy': 1717917526,   # ce_row_kernel (ignored rows are not read)
+    'c3_cross_entropy_autocast': 2450414716,
+    'c3_nll_loss': 827000369,         # nll forward (a gather) + the single-pass gradient write
+    'c5_conv': 687074860,             # 2 window kernels + weight gradient + 2 layout copies + weight reorders
+    'c5_batch_norm': 616984920,       # stats + apply + backward reduce + backward apply
 }
 
 
@@ -74,6 +74,7 @@ def kernel_source_digest() -> str:
 
 
 _DIGEST_MATCHES = None
+MODULE_TIMINGS = True
 
 
 def traffic_fields(key: str) -> Dict:
@@ -100,6 +101,9 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument('--configs', type=str, default='c1,c2,c3,c5',
                         help='secondary configs to measure besides the headline (c4); "none" skips them')
     parser.add_argument('--no-cpu', action='store_true', help='skip the CPU baselines')
+    parser.add_argument('--no-modules', action='store_true',
+                        help='skip the module-level (nn.Module + autograd, eager and HIP graph) timings; '
+                             'hardware-counter runs use this to profile the C-ABI launches only')
     parser.add_argument('--calibrate-copy', action='store_true',
                         help='also run a plain 256 MiB -> 256 MiB device copy, the known-size kernel that '
                              'hardware byte counters of a profiling run are scaled by')
@@ -145,6 +149,8 @@ def module_times_ms(forward: Callable[[int], torch.Tensor], backward: Callable[[
     forward(i) runs the layer on input set i and returns its output; backward(out, i)
     back-propagates from it.  Wall-clock over `iters` calls bracketed by device syncs.
     """
+    if not MODULE_TIMINGS:
+        return {}
     count = [0]
 
     def fwd_only():
@@ -323,6 +329,24 @@ def bench_linear(cfg: str, steps: int, warmup: int, with_cpu: bool) -> Dict:
                      **(traffic_fields('c4_linear_fwd') if cfg == 'c4' else {'traffic': None})},
         'frac_of_peak_step': flop / ms_step / 1e9 / peak,
     }
+    def mod_bwd(result, _):
+        xin.grad = None
+        layer.weight.grad = None
+        layer.bias.grad = None
+        result.backward(dyd)
+    out['module_level'] = module_times_ms(lambda _: layer(xin), mod_bwd, max(3, min(steps, 20)), warmup)
+    # torch's own GPU path for the same step (vendor BLAS + separate bias/activation kernels)
+    ref_layer = torch.nn.Linear(k, n, bias=True, device='cuda', dtype=dtype)
+    ref_act = torch.nn.GELU(approximate='tanh') if act == 'geluapprox' else torch.nn.ReLU()
+    xref = xd.clone().requires_grad_(True)
+
+    def ref_bwd(result, _):
+        xref.grad = None
+        ref_layer.weight.grad = None
+        ref_layer.bias.grad = None
+        result.backward(dyd)
+    out['torch_native'] = module_times_ms(lambda _: ref_act(ref_layer(xref)), ref_bwd, max(3, min(steps, 20)), warmup)
+    del ref_layer, xref
     if with_cpu:
         import oracle
         rows = min(m, 2048)
@@ -477,6 +501,13 @@ def bench_rows(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
     modules = {'LayerNorm': ln_mod, 'RMSNorm': rms_mod, 'Softmax': attorch_amd.Softmax(dim=-1),
                'LogSoftmax': attorch_amd.LogSoftmax(dim=-1), 'GELU(tanh)+Dropout(0.1) layer': act_mod}
 
+    ln_ref = torch.nn.LayerNorm(feat, dtype=dtype, device='cuda')
+    rms_ref = torch.nn.RMSNorm(feat, eps=1e-5, dtype=dtype, device='cuda')
+    natives = {'LayerNorm': ln_ref, 'RMSNorm': rms_ref, 'Softmax': torch.nn.Softmax(dim=-1),
+               'LogSoftmax': torch.nn.LogSoftmax(dim=-1),
+               'GELU(tanh)+Dropout(0.1) layer': torch.nn.Sequential(torch.nn.GELU(approximate='tanh'),
+                                                                    torch.nn.Dropout(0.1))}
+
     def module_level(mod):
         def fwd(i):
             return mod(xins[i])
@@ -521,6 +552,7 @@ def bench_rows(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
             'buffer_rotation': f'{nsets} sets of X/dY/Y/dX (64 MiB each)',
             'elementwise_reference': stream_ref,
             'module_level': module_level(modules[name]),
+            'torch_native': module_level(natives[name]),
         }
         if with_cpu:
             sec = cpu_time_s(cpu)
@@ -619,8 +651,8 @@ def bench_cross_entropy(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
                                                dt, 0, dt, gdt, st()), 'ce_bwd')
         return f
 
-    def module_times(wt, autocast):
-        crit = attorch_amd.CrossEntropyLoss(weight=wt)
+    def module_times(wt, autocast, native=False):
+        crit = (torch.nn if native else attorch_amd).CrossEntropyLoss(weight=wt)
         xin = logits.clone().requires_grad_(True)
 
         def fwd(_):
@@ -642,6 +674,7 @@ def bench_cross_entropy(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
             'roofline': {'bound': 'hbm', 'achieved': gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
                          'frac': gbs / PEAK_HBM_GBS, **traffic_fields('c3_cross_entropy')},
             'module_level': module_times(wt, False),
+            'torch_native': module_times(None if wt is None else wt.to(dtype), False, native=True),
         }
         if with_cpu and wt is None:
             crow = 512
@@ -677,6 +710,7 @@ def bench_cross_entropy(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
         'roofline': {'bound': 'hbm', 'achieved': gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
                      'frac': gbs / PEAK_HBM_GBS, **traffic_fields('c3_cross_entropy_autocast')},
         'module_level': module_times(None, True),
+        'torch_native': module_times(None, True, native=True),
     })
     del grad32
 
@@ -862,6 +896,20 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
         out.backward(dys[i])
     bn_entry['module_level'] = module_times_ms(bn_fwd_mod, mod_bwd, iters, warmup, nsets)
     conv_entry['module_level'] = module_times_ms(conv_fwd_mod, mod_bwd, iters, warmup, nsets)
+    # torch's own GPU path (MIOpen) for the same two layers
+    conv_ref = torch.nn.Conv2d(c, c, 3, padding=1, bias=False, device='cuda', dtype=dtype)
+    bn_ref = torch.nn.BatchNorm2d(c, device='cuda', dtype=dtype)
+
+    def ref_bwd(out, i):
+        xins[i].grad = None
+        rins[i].grad = None
+        conv_ref.weight.grad = None
+        bn_ref.weight.grad = None
+        bn_ref.bias.grad = None
+        out.backward(dys[i])
+    bn_entry['torch_native'] = module_times_ms(lambda i: torch.relu(bn_ref(xins[i]) + rins[i]), ref_bwd, iters,
+                                               warmup, nsets)
+    conv_entry['torch_native'] = module_times_ms(lambda i: conv_ref(xins[i]), ref_bwd, iters, warmup, nsets)
     if with_cpu:
         import oracle
         cn = 8
@@ -915,6 +963,8 @@ def main() -> int:
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
     torch.set_num_threads(os.cpu_count())
     with_cpu = not args.no_cpu
+    global MODULE_TIMINGS
+    MODULE_TIMINGS = not args.no_modules
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device='cuda').fill_(1)
         dst = torch.empty_like(src)
@@ -943,6 +993,8 @@ def main() -> int:
         'roofline': head['roofline'],
         'cpu_baseline': head.get('cpu_baseline'),
         'cpu_functional': head.get('cpu_functional'),
+        'module_level': head.get('module_level'),
+        'torch_native': head.get('torch_native'),
         'frac_of_peak_step': head['frac_of_peak_step'],
         'kernel_ms': head['kernel_ms'], 'kernel_tflops': head['kernel_tflops'],
         'configs': extra,

@@ -59,11 +59,11 @@ def test_conv2d(shape, out_dim, kernel, stride, padding, groups, bias, dtype) ->
     y = attorch_amd.Conv2dAutoGrad.apply(xd, wd, bd, *stride, *padding, groups)
     y.backward(dy.cuda())
     assert y.dtype is dtype
-    assert_close(y, y_ref, dtype, 'output', normalize=True)
-    assert_close(xd.grad, dx_ref, dtype, 'input_grad', normalize=True)
-    assert_close(wd.grad, dw_ref, dtype, 'weight_grad', normalize=True)
+    assert_close(y, y_ref, dtype, 'output')
+    assert_close(xd.grad, dx_ref, dtype, 'input_grad')
+    assert_close(wd.grad, dw_ref, dtype, 'weight_grad', batch_reduction=True)
     if bias:
-        assert_close(bd.grad, db_ref, dtype, 'bias_grad', normalize=True)
+        assert_close(bd.grad, db_ref, dtype, 'bias_grad', batch_reduction=True)
 
 
 def test_conv_modules_match_torch() -> None:
@@ -112,7 +112,7 @@ def test_conv_matrix_core_path_agrees_with_generic_kernel(dtype) -> None:
                                  *dims, dt, dt, dt, stream), 'fwd')
     _lib.check(lib.at_conv2d_fwd(_lib.ptr(x), _lib.ptr(wt), None, _lib.ptr(y_slow), None, 0,
                                  *dims, dt, dt, dt, stream), 'fwd')
-    assert_close(y_fast, y_slow.cpu(), dtype, 'output', normalize=True)
+    assert_close(y_fast, y_slow.cpu(), dtype, 'output')
     # the forward workspace starts with the channels-last input
     x_nhwc = ws_f[:x.numel() * 2].view(dtype).view(n, h, w, c)
     assert torch.equal(x_nhwc, x.permute(0, 2, 3, 1))
@@ -129,7 +129,7 @@ def test_conv_matrix_core_path_agrees_with_generic_kernel(dtype) -> None:
     _lib.check(lib.at_conv2d_bwd_input(_lib.ptr(dy), None, _lib.ptr(wt), _lib.ptr(dx_slow), None, 0,
                                        *dims, dt, stream), 'dx')
     assert torch.equal(dx_own, dx_shared)
-    assert_close(dx_own, dx_slow.cpu(), dtype, 'input_grad', normalize=True)
+    assert_close(dx_own, dx_slow.cpu(), dtype, 'input_grad')
 
     dw_own, dw_shared = torch.empty_like(wt), torch.empty_like(wt)
     _lib.check(lib.at_conv2d_bwd_weight(_lib.ptr(dy), None, _lib.ptr(x), None, _lib.ptr(dw_own), _lib.ptr(ws_w),
@@ -178,7 +178,7 @@ def test_conv_window_kernel_agrees_with_generic_kernel_at_size(n, c, h, w, o, pa
                                  *dims, dt, dt, dt, stream), 'fwd')
     _lib.check(lib.at_conv2d_fwd(_lib.ptr(x), _lib.ptr(wt), _lib.ptr(b), _lib.ptr(y_slow), None, 0,
                                  *dims, dt, dt, dt, stream), 'fwd')
-    assert_close(y_fast, y_slow.cpu(), dtype, 'output', normalize=True)
+    assert_close(y_fast, y_slow.cpu(), dtype, 'output')
     # weight gradient: the matrix-core path (all taps per workgroup for pad 1) against torch in fp32
     nb_w = lib.at_conv2d_bwd_weight_workspace_bytes(*dims, dt)
     ws_w = torch.empty(nb_w, dtype=torch.uint8, device='cuda')
@@ -186,7 +186,7 @@ def test_conv_window_kernel_agrees_with_generic_kernel_at_size(n, c, h, w, o, pa
     _lib.check(lib.at_conv2d_bwd_weight(_lib.ptr(dy), None, _lib.ptr(x), None, _lib.ptr(dw_fast), _lib.ptr(ws_w),
                                         nb_w, *dims, dt, stream), 'dw')
     dw_ref = torch.nn.grad.conv2d_weight(x.float(), wt.shape, dy.float(), stride=1, padding=pad, groups=groups)
-    assert_close(dw_fast, dw_ref.cpu(), dtype, 'weight_grad', normalize=True)
+    assert_close(dw_fast, dw_ref.cpu(), dtype, 'weight_grad', batch_reduction=True)
     nb_x = lib.at_conv2d_bwd_input_workspace_bytes(*dims, dt)
     if pad > k - 1:
         assert nb_x == 0                    # the input gradient as a convolution needs pad <= k - 1
@@ -198,7 +198,7 @@ def test_conv_window_kernel_agrees_with_generic_kernel_at_size(n, c, h, w, o, pa
                                        *dims, dt, stream), 'dx')
     _lib.check(lib.at_conv2d_bwd_input(_lib.ptr(dy), None, _lib.ptr(wt), _lib.ptr(dx_slow), None, 0,
                                        *dims, dt, stream), 'dx')
-    assert_close(dx_fast, dx_slow.cpu(), dtype, 'input_grad', normalize=True)
+    assert_close(dx_fast, dx_slow.cpu(), dtype, 'input_grad')
 
 
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
@@ -225,7 +225,7 @@ def test_conv_weight_gradient_all_taps_kernel(n, c, h, w, o, groups, dtype) -> N
     _lib.check(lib.at_conv2d_bwd_weight(_lib.ptr(dy), None, _lib.ptr(x), None, _lib.ptr(dw), _lib.ptr(ws), nb,
                                         *dims, dt, _lib.stream_of(x)), 'dw')
     ref = torch.nn.grad.conv2d_weight(x.float(), dw.shape, dy.float(), stride=1, padding=1, groups=groups)
-    assert_close(dw, ref.cpu(), dtype, 'weight_grad', normalize=True)
+    assert_close(dw, ref.cpu(), dtype, 'weight_grad', batch_reduction=True)
 
 
 BN_SHAPES = [(6, 5), (128, 1024), (2048, 768), (8, 960, 196), (2048, 64, 16), (2, 3, 224, 224),
@@ -269,10 +269,10 @@ def test_batch_norm_training(shape, dtype, affine, residual, act_func) -> None:
         assert_close(pre_act, pre_act_ref, dtype, 'pre_act')
     dx_ref, dw_ref, db_ref, dres_ref = oracle.batch_norm_backward(
         dy, x, saved[1], saved[2], w, affine, pre_act, name, param, compute=cd)
-    assert_close(xd.grad, dx_ref, dtype, 'input_grad', normalize=True)
+    assert_close(xd.grad, dx_ref, dtype, 'input_grad')
     if affine:
-        assert_close(wd.grad, dw_ref.to(dtype), dtype, 'weight_grad', normalize=True)
-        assert_close(bd.grad, db_ref.to(dtype), dtype, 'bias_grad', normalize=True)
+        assert_close(wd.grad, dw_ref.to(dtype), dtype, 'weight_grad', batch_reduction=True)
+        assert_close(bd.grad, db_ref.to(dtype), dtype, 'bias_grad', batch_reduction=True)
     if residual:
         assert_close(rd.grad, dres_ref, dtype, 'residual_grad')
 
@@ -304,9 +304,9 @@ def test_batch_norm_eval_backward_follows_the_reference(act_func, dtype) -> None
     assert_close(saved[1], running_mean, torch.float32, 'saved mean = running mean')
     dx_ref, dw_ref, db_ref, dres_ref = oracle.batch_norm_backward(
         dy, x, saved[1], saved[2], w, True, saved[4] if name is not None else None, name, param, compute=cd)
-    assert_close(xd.grad, dx_ref, dtype, 'input_grad', normalize=True)
-    assert_close(wd.grad, dw_ref.to(dtype), dtype, 'weight_grad', normalize=True)
-    assert_close(bd.grad, db_ref.to(dtype), dtype, 'bias_grad', normalize=True)
+    assert_close(xd.grad, dx_ref, dtype, 'input_grad')
+    assert_close(wd.grad, dw_ref.to(dtype), dtype, 'weight_grad', batch_reduction=True)
+    assert_close(bd.grad, db_ref.to(dtype), dtype, 'bias_grad', batch_reduction=True)
     assert_close(rd.grad, dres_ref, dtype, 'residual_grad')
 
 

@@ -30,9 +30,9 @@ def test_c1_linear_fp32_relu() -> None:
     y_ref, _ = oracle.linear_forward(x, w, b, 'relu', None, F32, compute=torch.float64)
     dx_ref, dw_ref, db_ref = oracle.linear_backward(dy, x, w, pre_act, 'relu', None, F32, compute=torch.float64)
     assert_close(y, y_ref, F32, 'output')
-    assert_close(xd.grad, dx_ref, F32, 'input_grad', normalize=True)
-    assert_close(wd.grad, dw_ref, F32, 'weight_grad', normalize=True)
-    assert_close(bd.grad, db_ref, F32, 'bias_grad', normalize=True)
+    assert_close(xd.grad, dx_ref, F32, 'input_grad')
+    assert_close(wd.grad, dw_ref, F32, 'weight_grad', batch_reduction=True)
+    assert_close(bd.grad, db_ref, F32, 'bias_grad', batch_reduction=True)
 
 
 def test_c2_norms_and_softmax_bf16() -> None:
@@ -46,8 +46,8 @@ def test_c2_norms_and_softmax_bf16() -> None:
     dx_ref, dw_ref, db_ref = oracle.layer_norm_backward(dy, x, mean, inv_std, w, BF16)
     assert_close(y, y_ref, BF16, 'layer_norm output')
     assert_close(xd.grad, dx_ref, BF16, 'layer_norm input_grad')
-    assert_close(wd.grad, dw_ref.to(BF16), BF16, 'layer_norm weight_grad', normalize=True)
-    assert_close(bd.grad, db_ref.to(BF16), BF16, 'layer_norm bias_grad', normalize=True)
+    assert_close(wd.grad, dw_ref.to(BF16), BF16, 'layer_norm weight_grad', batch_reduction=True)
+    assert_close(bd.grad, db_ref.to(BF16), BF16, 'layer_norm bias_grad', batch_reduction=True)
 
     xd, wd = x.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
     y = attorch_amd.RMSNormAutoGrad.apply(xd, wd, 1e-5)
@@ -56,7 +56,7 @@ def test_c2_norms_and_softmax_bf16() -> None:
     dx_ref, dw_ref = oracle.rms_norm_backward(dy, x, inv_rms, w)
     assert_close(y, y_ref, BF16, 'rms_norm output')
     assert_close(xd.grad, dx_ref, BF16, 'rms_norm input_grad')
-    assert_close(wd.grad, dw_ref.to(BF16), BF16, 'rms_norm weight_grad', normalize=True)
+    assert_close(wd.grad, dw_ref.to(BF16), BF16, 'rms_norm weight_grad', batch_reduction=True)
 
     for log in (False, True):
         xd = x.cuda().requires_grad_(True)
@@ -123,13 +123,13 @@ def test_c4_linear_bf16_gelu() -> None:
     assert_close(pre_act[rows.cuda()], pre_ref, BF16, 'pre_act rows')
     # backward of the sampled rows from the device's own pre-activation
     dx_ref, _, _ = oracle.linear_backward(dy[rows], x[rows], w, pre_act[rows.cuda()].cpu(), 'geluapprox', None, BF16)
-    assert_close(xd.grad[rows.cuda()], dx_ref, BF16, 'input_grad rows', normalize=True)
+    assert_close(xd.grad[rows.cuda()], dx_ref, BF16, 'input_grad rows')
     # weight gradient: a band of input features over the whole batch, and the bias gradient
     dz = (dy.float() * oracle.act_grad(pre_act.cpu().float(), 'geluapprox')).to(BF16)
     cols = torch.cat([torch.arange(0, 8), torch.arange(2048, 2056), torch.arange(k - 8, k)])
     dw_ref = (x[:, cols].float().T @ dz.float()).to(BF16)
-    assert_close(wd.grad[cols.cuda()], dw_ref, BF16, 'weight_grad rows', normalize=True)
-    assert_close(bd.grad, dz.float().sum(dim=0).to(BF16), BF16, 'bias_grad', normalize=True)
+    assert_close(wd.grad[cols.cuda()], dw_ref, BF16, 'weight_grad rows', batch_reduction=True)
+    assert_close(bd.grad, dz.float().sum(dim=0).to(BF16), BF16, 'bias_grad', batch_reduction=True)
 
 
 def test_c5_conv_bn_residual_relu_bf16() -> None:
@@ -142,17 +142,17 @@ def test_c5_conv_bn_residual_relu_bf16() -> None:
     conv_out.backward(dy.cuda())
     sub = slice(60, 64)
     assert_close(conv_out[sub], oracle.conv2d_forward(x[sub], wt, None, (1, 1), (1, 1), 1, BF16), BF16,
-                 'conv output slice', normalize=True)
+                 'conv output slice')
     dx_ref, dw_sub_ref, _ = oracle.conv2d_backward(dy[sub], x[sub], wt, (1, 1), (1, 1), 1, BF16)
-    assert_close(xd.grad[sub], dx_ref, BF16, 'conv input_grad slice', normalize=True)
+    assert_close(xd.grad[sub], dx_ref, BF16, 'conv input_grad slice')
     # weight gradient: the slice alone against the oracle, the full batch as the sum of its halves
     halves = []
     for part in (slice(0, 64), slice(64, 128), sub):
         xp, wp = x[part].cuda().requires_grad_(True), wt.cuda().requires_grad_(True)
         attorch_amd.Conv2dAutoGrad.apply(xp, wp, None, 1, 1, 1, 1, 1).backward(dy[part].cuda())
         halves.append(wp.grad.float())
-    assert_close(halves[2], dw_sub_ref, BF16, 'conv weight_grad slice', normalize=True)
-    assert_close(wd.grad.float(), halves[0] + halves[1], BF16, 'conv weight_grad additivity', normalize=True)
+    assert_close(halves[2], dw_sub_ref, BF16, 'conv weight_grad slice', batch_reduction=True)
+    assert_close(wd.grad.float(), halves[0] + halves[1], BF16, 'conv weight_grad additivity', batch_reduction=True)
 
     bn_w, bn_b = randn((c,), 5005, BF16, 0.1, 1.0), randn((c,), 5006, BF16, 0.1)
     rm, rv = torch.zeros(c), torch.ones(c)
@@ -170,7 +170,7 @@ def test_c5_conv_bn_residual_relu_bf16() -> None:
     assert_close(rvd, rv_ref, F32, 'running_var')
     dx_ref, dw_ref, db_ref, dres_ref = oracle.batch_norm_backward(dy, conv_cpu, saved[1], saved[2], bn_w, True, saved[4],
                                                                   'relu', None)
-    assert_close(cd.grad, dx_ref, BF16, 'batch_norm input_grad', normalize=True)
-    assert_close(wdv.grad, dw_ref.to(BF16), BF16, 'batch_norm weight_grad', normalize=True)
-    assert_close(bdv.grad, db_ref.to(BF16), BF16, 'batch_norm bias_grad', normalize=True)
+    assert_close(cd.grad, dx_ref, BF16, 'batch_norm input_grad')
+    assert_close(wdv.grad, dw_ref.to(BF16), BF16, 'batch_norm weight_grad', batch_reduction=True)
+    assert_close(bdv.grad, db_ref.to(BF16), BF16, 'batch_norm bias_grad', batch_reduction=True)
     assert_close(rd.grad, dres_ref, BF16, 'batch_norm residual_grad')

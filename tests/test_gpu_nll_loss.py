@@ -43,7 +43,7 @@ def test_nll_loss(shape, dtype, weighted, reduction) -> None:
     loss.backward(upstream.cuda())
     assert loss.dtype is dtype and loss.shape == loss_ref.shape
     # a sum over many entries grows with their number: compare on the scale of the result
-    assert_close(loss, loss_ref, dtype, 'loss', normalize=True)
+    assert_close(loss, loss_ref, dtype, 'loss')
     entries = target.numel()
     scale = entries if reduction == 'mean' else 1.0
     assert xd.grad.shape == x.shape and xd.grad.dtype is dtype

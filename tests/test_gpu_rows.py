@@ -45,9 +45,9 @@ def test_layer_norm(shape, dtype, affine, bias) -> None:
     # the reference's own test (tests/test_layer_norm_layer.py:109, rtol = atol = 1e-3).
     assert_close(xd.grad, dx_ref, dtype, 'input_grad', reference_tolerance=feat <= 4)
     if affine:
-        assert_close(wd.grad, dw_ref.to(dtype), dtype, 'weight_grad', normalize=True)
+        assert_close(wd.grad, dw_ref.to(dtype), dtype, 'weight_grad', batch_reduction=True)
     if bias:
-        assert_close(bd.grad, db_ref.to(dtype), dtype, 'bias_grad', normalize=True)
+        assert_close(bd.grad, db_ref.to(dtype), dtype, 'bias_grad', batch_reduction=True)
 
 
 @pytest.mark.parametrize('dtype', DTYPES)
@@ -72,7 +72,7 @@ def test_rms_norm(shape, dtype, affine, eps) -> None:
     # same conditioning remark as for LayerNorm (tests/test_rms_norm_layer.py:87-100 uses 1e-3)
     assert_close(xd.grad, dx_ref, dtype, 'input_grad', reference_tolerance=feat <= 4)
     if affine:
-        assert_close(wd.grad, dw_ref.to(dtype), dtype, 'weight_grad', normalize=True)
+        assert_close(wd.grad, dw_ref.to(dtype), dtype, 'weight_grad', batch_reduction=True)
 
 
 @pytest.mark.parametrize('dtype', DTYPES)
