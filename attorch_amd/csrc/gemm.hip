@@ -959,36 +959,69 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(SimpleArgs g) {
 
 // ------------------------------------------------------------------------------------------
 // fp32 operands, outputs too small to give every CU a 64x64 tile (a 512 x 256 layer): 32x32 output
-// tiles, four times as many workgroups, and the four waves of a workgroup share the contraction —
-// wave w multiplies k-steps w, w + 4, ... of every 64-wide k-tile — so the serial chain of MFMAs
-// per wave is a quarter as long; the four accumulators are added through LDS in a fixed order.
-// Tiles are fetched with 16-byte loads along the contiguous index of each operand, the next
-// k-tile travelling in registers while the current one is multiplied.
+// tiles, four times as many workgroups, and the eight waves of a workgroup share the contraction —
+// wave w multiplies k-steps w, w + 8, ... of every k-tile — so the serial chain of MFMAs per wave is
+// an eighth as long; the eight accumulators are added through LDS in a fixed order.
+// Such a launch lasts a few microseconds, most of them memory latency, so the loads run far ahead:
+// a ring of STAGES k-tiles travels in registers (the whole contraction of a 784-wide layer is
+// requested before the first multiply), and the LDS tiles are double-buffered, which leaves one
+// barrier per k-tile.  Tiles are fetched with 16-byte loads along the contiguous index of each
+// operand.
 // ------------------------------------------------------------------------------------------
-// TK (the k-tile) is 256 for long contractions: with so little arithmetic per byte an iteration
-// lasts about as long as its loads take to arrive, so fewer, larger iterations are faster.
-template <bool A_MC, bool B_KC, int TK>
-__global__ __launch_bounds__(256) void gemm_f32_split_kernel(GemmArgs g) {
+constexpr int kSplitWaves = 8, kSplitThreads = kSplitWaves * 64, kSplitStages = 4;
+
+// output_grad * act'(pre_act) for four elements.  Kept out of line: it is called from every stage
+// of an unrolled register ring, and the activation switch inlined at each call site makes a
+// kernel of a few microseconds spend them fetching instructions.
+__device__ __attribute__((noinline)) float4 pre_act_grad_vec(float4 g, float4 z, int act, float param) {
+  return make_float4(g.x * act_derivative(act, z.x, param), g.y * act_derivative(act, z.y, param),
+                     g.z * act_derivative(act, z.z, param), g.w * act_derivative(act, z.w, param));
+}
+
+// One 32x32 output tile of C = A B.  DZ names an operand that does not exist in memory: the
+// gradient of the pre-activation, output_grad * act'(pre_act), formed while its tile is staged
+// (DZ = 1: A, DZ = 2: B; `a` / `b` then point at output_grad and `p` at pre_act, both indexed
+// alike, row strides lda / ldb and ldp).  COLSUM (with DZ = 2) also sums the columns of the B
+// tiles this workgroup passes through LDS, i.e. the bias gradient of its 32 columns.
+struct SplitTile {
+  const float* a;
+  const float* b;
+  const float* p;
+  int64_t lda, ldb, ldp;
+  int M, N, K;     // extents of this product
+  int m0, n0;      // origin of the tile
+  int act;
+  float param;
+};
+
+template <int TK>
+struct SplitShape {
+  static constexpr int kPitchK = TK + 4, kPitchO = 32 + 4;
+  static constexpr int kTileFloats = 32 * kPitchK > TK * kPitchO ? 32 * kPitchK : TK * kPitchO;
+  static constexpr int kFoldFloats = kSplitWaves * 16 * 64;
+  static constexpr int kSmemFloats = 4 * kTileFloats > kFoldFloats ? 4 * kTileFloats : kFoldFloats;
+};
+
+// Returns the tile's accumulator (fragment layout of the 32x32 MFMA) in wave 0; the other waves
+// return garbage.  On return every wave has passed a barrier after its last use of smem except
+// wave 0's reads of the fold area, so wave 0 alone may go on using smem.
+template <bool A_MC, bool B_KC, int TK, int DZ, bool COLSUM>
+__device__ __forceinline__ f32x16 split_tile(const SplitTile& t, float* smem, float* colsum_out) {
   constexpr int TM = 32;
-  constexpr int NV = TK / 32;           // 16-byte vectors per lane, operand and k-tile
+  constexpr int NV = TK * 8 / kSplitThreads;   // 16-byte vectors per lane, operand and k-tile
+  static_assert(NV >= 1 && (TK / 2) % kSplitWaves == 0, "k-tile too small for the workgroup");
+  static_assert(!COLSUM || (DZ == 2 && !B_KC && TK % 16 == 0), "column sums are taken from a [k][n] tile");
   // LDS image of a tile: as in memory, rows padded by 4 floats (16-byte aligned rows, and the 32
   // lanes of a fragment read spread over the banks): [outer][TK + 4] for an operand whose rows
   // run along the contraction, [k][32 + 4] for the other layout.
-  constexpr int kPitchK = TK + 4, kPitchO = TM + 4;
-  constexpr int kTileFloats = TM * kPitchK > TK * kPitchO ? TM * kPitchK : TK * kPitchO;
-  __shared__ __align__(16) float smem[2 * kTileFloats > 4 * 64 * 16 ? 2 * kTileFloats : 4 * 64 * 16];
-  float* const sa = smem;
-  float* const sb = smem + kTileFloats;
-  const float* __restrict__ A = reinterpret_cast<const float*>(g.a);
-  const float* __restrict__ B = reinterpret_cast<const float*>(g.b);
-  const int nbn = (g.N + TM - 1) / TM;
-  const int m0 = (blockIdx.x / nbn) * TM, n0 = (blockIdx.x % nbn) * TM;
+  constexpr int kPitchK = SplitShape<TK>::kPitchK, kPitchO = SplitShape<TK>::kPitchO;
+  constexpr int kTileFloats = SplitShape<TK>::kTileFloats;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 
   // Each lane fetches NV 16-byte vectors per operand and k-tile: 4 consecutive k of one outer index
   // or 4 consecutive outer indices of one k, whichever is contiguous in memory.  Extents along the
   // vectors are multiples of 4 (host check), so a vector is inside or outside as a whole.
-  float4 ra[NV], rb[NV];
+  float4 ra[kSplitStages][NV], rb[kSplitStages][NV], rp[DZ ? kSplitStages : 1][NV];
   auto where = [&](bool outer_contig, int idx, int& o, int& k) {
     if (outer_contig) { k = idx >> 3; o = (idx & 7) * 4; } else { o = idx / (TK / 4); k = (idx % (TK / 4)) * 4; }
   };
@@ -996,27 +1029,27 @@ __global__ __launch_bounds__(256) void gemm_f32_split_kernel(GemmArgs g) {
     int o, k;
     where(outer_contig, idx, o, k);
     const int go = o0 + o, gk = k0 + k;
-    if (go >= o_lim || gk >= g.K) return make_float4(0.f, 0.f, 0.f, 0.f);
+    if (go >= o_lim || gk >= t.K) return make_float4(0.f, 0.f, 0.f, 0.f);
     return *reinterpret_cast<const float4*>(base + (outer_contig ? (int64_t)gk * ld + go : (int64_t)go * ld + gk));
   };
-  auto fetch = [&](int k0) {
+  auto fetch = [&](int st, int k0) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      ra[i] = fetch_one(A, g.lda, A_MC, m0, g.M, k0, threadIdx.x + i * 256);
-      rb[i] = fetch_one(B, g.ldb, !B_KC, n0, g.N, k0, threadIdx.x + i * 256);
+      ra[st][i] = fetch_one(t.a, t.lda, A_MC, t.m0, t.M, k0, threadIdx.x + i * kSplitThreads);
+      rb[st][i] = fetch_one(t.b, t.ldb, !B_KC, t.n0, t.N, k0, threadIdx.x + i * kSplitThreads);
+      if constexpr (DZ == 1) rp[st][i] = fetch_one(t.p, t.ldp, A_MC, t.m0, t.M, k0, threadIdx.x + i * kSplitThreads);
+      if constexpr (DZ == 2) rp[st][i] = fetch_one(t.p, t.ldp, !B_KC, t.n0, t.N, k0, threadIdx.x + i * kSplitThreads);
     }
+  };
+  auto pre_act_grad = [&](const float4& g, const float4& z) {   // zero where the fetch was outside
+    if (t.act == AT_ACT_RELU)
+      return make_float4(z.x <= 0.f ? 0.f : g.x, z.y <= 0.f ? 0.f : g.y, z.z <= 0.f ? 0.f : g.z, z.w <= 0.f ? 0.f : g.w);
+    return pre_act_grad_vec(g, z, t.act, t.param);
   };
   auto stage_one = [&](float* tile, bool outer_contig, const float4& v, int idx) {
     int o, k;
     where(outer_contig, idx, o, k);
     *reinterpret_cast<float4*>(tile + (outer_contig ? k * kPitchO + o : o * kPitchK + k)) = v;
-  };
-  auto stage = [&]() {
-#pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      stage_one(sa, A_MC, ra[i], threadIdx.x + i * 256);
-      stage_one(sb, !B_KC, rb[i], threadIdx.x + i * 256);
-    }
   };
   auto value = [&](const float* tile, bool outer_contig, int o, int k) {
     return tile[outer_contig ? k * kPitchO + o : o * kPitchK + k];
@@ -1025,33 +1058,149 @@ __global__ __launch_bounds__(256) void gemm_f32_split_kernel(GemmArgs g) {
   f32x16 acc;
 #pragma unroll
   for (int e = 0; e < 16; ++e) acc[e] = 0.f;
-  fetch(0);
-  for (int k0 = 0; k0 < g.K; k0 += TK) {
-    stage();
-    __syncthreads();
-    if (k0 + TK < g.K) fetch(k0 + TK);
+  float colsum = 0.f;   // COLSUM: column (threadIdx.x & 31), rows (threadIdx.x >> 5) + 16 j of every k-tile
 #pragma unroll
-    for (int q = 0; q < TK / 8; ++q) {
-      const int k = (q * 4 + wave) * 2 + (lane >> 5);   // k-step q * 4 + wave of this tile
-      // operands swapped so that a lane ends up with 4 consecutive n of one m
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(value(sb, !B_KC, lane & 31, k), value(sa, A_MC, lane & 31, k), acc, 0, 0, 0);
+  for (int st = 0; st < kSplitStages; ++st)
+    if (st * TK < t.K) fetch(st, st * TK);
+  // k-tile i sits in register stage i % STAGES and goes through LDS buffer i % 2.  The barrier of
+  // tile i is passed only after every wave has finished reading tile i - 1, so writing buffer
+  // (i + 1) % 2 after it cannot disturb a reader; one barrier per tile is enough.
+  for (int k_ring = 0; k_ring < t.K; k_ring += kSplitStages * TK) {
+#pragma unroll
+    for (int st = 0; st < kSplitStages; ++st) {
+      const int k0 = k_ring + st * TK;
+      if (k0 < t.K) {
+        float* const sa = smem + (st & 1) * 2 * kTileFloats;
+        float* const sb = sa + kTileFloats;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+          if constexpr (DZ == 1) ra[st][i] = pre_act_grad(ra[st][i], rp[st][i]);
+          if constexpr (DZ == 2) rb[st][i] = pre_act_grad(rb[st][i], rp[st][i]);
+          stage_one(sa, A_MC, ra[st][i], threadIdx.x + i * kSplitThreads);
+          stage_one(sb, !B_KC, rb[st][i], threadIdx.x + i * kSplitThreads);
+        }
+        __syncthreads();
+        if (k0 + kSplitStages * TK < t.K) fetch(st, k0 + kSplitStages * TK);
+#pragma unroll
+        for (int q = 0; q < TK / (2 * kSplitWaves); ++q) {
+          const int k = (q * kSplitWaves + wave) * 2 + (lane >> 5);   // k-step q * 8 + wave of this tile
+          // operands swapped so that a lane ends up with 4 consecutive n of one m
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(value(sb, !B_KC, lane & 31, k), value(sa, A_MC, lane & 31, k),
+                                                     acc, 0, 0, 0);
+        }
+        if constexpr (COLSUM) {   // rows beyond K were staged as zeros
+#pragma unroll
+          for (int j = 0; j < TK / 16; ++j) colsum += sb[((threadIdx.x >> 5) + 16 * j) * kPitchO + (threadIdx.x & 31)];
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  // the operand tiles are dead (barrier above): add the partial accumulators in wave order
+  float* fold = smem;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) fold[(r * kSplitWaves + wave) * 64 + lane] = acc[r];
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      float sum = fold[(r * kSplitWaves) * 64 + lane];
+#pragma unroll
+      for (int w = 1; w < kSplitWaves; ++w) sum += fold[(r * kSplitWaves + w) * 64 + lane];
+      acc[r] = sum;
+    }
+  }
+  if constexpr (COLSUM) {
+    // 16 row slices per column, added in slice order by the first 32 lanes of wave 1 (wave 0 is
+    // busy with the tile); the slices go through LDS behind the fold area's last reader
+    __syncthreads();
+    float* slices = smem;   // [16][32]
+    slices[(threadIdx.x >> 5) * 32 + (threadIdx.x & 31)] = colsum;
+    __syncthreads();
+    if (wave == 1 && lane < 32) {
+      float sum = slices[lane];
+#pragma unroll
+      for (int j = 1; j < 16; ++j) sum += slices[j * 32 + lane];
+      *colsum_out = sum;
     }
     __syncthreads();
   }
+  return acc;
+}
 
-  // the operand tiles are dead (barrier above): add the four partial accumulators in wave order
-  float* fold = smem;
-#pragma unroll
-  for (int r = 0; r < 16; ++r) fold[(r * 4 + wave) * 64 + lane] = acc[r];
-  __syncthreads();
-  if (wave != 0) return;
-#pragma unroll
-  for (int r = 0; r < 16; ++r)
-    acc[r] = (fold[(r * 4 + 0) * 64 + lane] + fold[(r * 4 + 1) * 64 + lane]) +
-             (fold[(r * 4 + 2) * 64 + lane] + fold[(r * 4 + 3) * 64 + lane]);
+template <bool A_MC, bool B_KC, int TK>
+__global__ __launch_bounds__(kSplitThreads) void gemm_f32_split_kernel(GemmArgs g) {
+  __shared__ __align__(16) float smem[SplitShape<TK>::kSmemFloats];
+  const int nbn = (g.N + 31) / 32;
+  const SplitTile t{reinterpret_cast<const float*>(g.a), reinterpret_cast<const float*>(g.b), nullptr,
+                    g.lda, g.ldb, 0, g.M, g.N, g.K, (int)(blockIdx.x / nbn) * 32, (int)(blockIdx.x % nbn) * 32,
+                    AT_ACT_NONE, 0.f};
+  const f32x16 acc = split_tile<A_MC, B_KC, TK, 0, false>(t, smem, nullptr);
+  if (threadIdx.x >= 64) return;
   __builtin_amdgcn_wave_barrier();
-  static_assert(32 * 36 <= 4 * 64 * 16, "the epilogue block fits");
-  wave_tile_epilogue<float>(acc, smem, g, m0, n0);
+  static_assert(32 * 36 <= SplitShape<TK>::kFoldFloats, "the epilogue block fits");
+  wave_tile_epilogue<float>(acc, smem, g, t.m0, t.n0);
+}
+
+// Backward pass of a small fp32 linear layer with an activation in one launch: the first
+// dx_tiles workgroups compute tiles of dX = dZ W^T, the others tiles of dW = X^T dZ, and the
+// dW workgroups of the first row block also write the bias gradient (column sums of dZ).
+// dZ = output_grad * act'(pre_act) is never stored: every workgroup forms the part it needs
+// while staging its tiles.  The contraction runs over out_feat for dX (k-tiles of TKX) and over
+// the batch for dW (k-tiles of TKW).
+struct SmallBwdArgs {
+  const float* output_grad;   // [batch, out_feat]
+  const float* pre_act;       // [batch, out_feat]
+  const float* input;         // [batch, in_feat]
+  const float* weight;        // [in_feat, out_feat]
+  float* input_grad;          // [batch, in_feat]
+  float* weight_grad;         // [in_feat, out_feat]
+  float* bias_grad;           // [out_feat] or null
+  int batch, in_feat, out_feat;
+  int64_t ld_g, ld_p, ld_x, ld_w, ld_dx, ld_dw;
+  int act;
+  float param;
+  int dx_tiles;
+};
+
+template <int TKX, int TKW>
+__global__ __launch_bounds__(kSplitThreads) void linear_bwd_small_kernel(SmallBwdArgs s) {
+  constexpr int kSmem = SplitShape<TKX>::kSmemFloats > SplitShape<TKW>::kSmemFloats ? SplitShape<TKX>::kSmemFloats
+                                                                                      : SplitShape<TKW>::kSmemFloats;
+  __shared__ __align__(16) float smem[kSmem];
+  GemmArgs g{};   // what the epilogue reads: plain stores of the tile
+  g.act = AT_ACT_NONE;
+  if ((int)blockIdx.x < s.dx_tiles) {
+    // dX[batch, in_feat]: A = dZ (rows along the contraction), B(k, n) = W[n, k] (likewise)
+    const int nbn = (s.in_feat + 31) / 32;
+    const SplitTile t{s.output_grad, s.weight, s.pre_act, s.ld_g, s.ld_w, s.ld_p, s.batch, s.in_feat, s.out_feat,
+                      (int)(blockIdx.x / nbn) * 32, (int)(blockIdx.x % nbn) * 32, s.act, s.param};
+    const f32x16 acc = split_tile<false, true, TKX, 1, false>(t, smem, nullptr);
+    if (threadIdx.x >= 64) return;
+    __builtin_amdgcn_wave_barrier();
+    g.c = s.input_grad; g.M = s.batch; g.N = s.in_feat; g.ldc = s.ld_dx;
+    wave_tile_epilogue<float>(acc, smem, g, t.m0, t.n0);
+  } else {
+    // dW[in_feat, out_feat]: A(m, k) = X[k, m], B = dZ[k, n], contraction over the batch
+    const int tile = (int)blockIdx.x - s.dx_tiles;
+    const int nbn = (s.out_feat + 31) / 32;
+    const SplitTile t{s.input, s.output_grad, s.pre_act, s.ld_x, s.ld_g, s.ld_p, s.in_feat, s.out_feat, s.batch,
+                      (tile / nbn) * 32, (tile % nbn) * 32, s.act, s.param};
+    f32x16 acc;
+    if (t.m0 == 0 && s.bias_grad) {
+      float column = 0.f;
+      acc = split_tile<true, false, TKW, 2, true>(t, smem, &column);
+      const int lane = threadIdx.x & 63;
+      if ((threadIdx.x >> 6) == 1 && lane < 32 && t.n0 + lane < s.out_feat) s.bias_grad[t.n0 + lane] = column;
+    } else {
+      acc = split_tile<true, false, TKW, 2, false>(t, smem, nullptr);
+    }
+    if (threadIdx.x >= 64) return;
+    __builtin_amdgcn_wave_barrier();
+    g.c = s.weight_grad; g.M = s.in_feat; g.N = s.out_feat; g.ldc = s.ld_dw;
+    wave_tile_epilogue<float>(acc, smem, g, t.m0, t.n0);
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1572,11 +1721,14 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
       const unsigned grid = (unsigned)(cdiv64(M, 32) * cdiv64(N, 32));
 #define AT_SPLIT_LAUNCH(TK)                                                                                              \
   {                                                                                                                      \
-    if (layout == kDx) hipLaunchKernelGGL((gemm_f32_split_kernel<false, true, TK>), dim3(grid), dim3(256), 0, stream, g);       \
-    else if (layout == kDw) hipLaunchKernelGGL((gemm_f32_split_kernel<true, false, TK>), dim3(grid), dim3(256), 0, stream, g);  \
-    else hipLaunchKernelGGL((gemm_f32_split_kernel<false, false, TK>), dim3(grid), dim3(256), 0, stream, g);                    \
+    if (layout == kDx)                                                                                                   \
+      hipLaunchKernelGGL((gemm_f32_split_kernel<false, true, TK>), dim3(grid), dim3(kSplitThreads), 0, stream, g);       \
+    else if (layout == kDw)                                                                                              \
+      hipLaunchKernelGGL((gemm_f32_split_kernel<true, false, TK>), dim3(grid), dim3(kSplitThreads), 0, stream, g);       \
+    else                                                                                                                 \
+      hipLaunchKernelGGL((gemm_f32_split_kernel<false, false, TK>), dim3(grid), dim3(kSplitThreads), 0, stream, g);      \
   }
-      if (K >= 512) AT_SPLIT_LAUNCH(256) else AT_SPLIT_LAUNCH(64)
+      if (K >= 512) AT_SPLIT_LAUNCH(128) else AT_SPLIT_LAUNCH(64)
 #undef AT_SPLIT_LAUNCH
       return launch_status();
     }
@@ -1648,6 +1800,63 @@ int at_linear_bwd_input(const void* pre_act_grad, const void* weight, void* inpu
   return run_gemm(kDx, pre_act_grad, weight, input_grad, nullptr, nullptr, batch, in_feat, out_feat,
                   grad_stride, weight_stride, input_grad_stride, 0, AT_ACT_NONE, 0.f, in_dtype, 0, out_dtype,
                   (hipStream_t)stream);
+}
+
+int at_linear_bwd_small_supported(int64_t batch, int64_t in_feat, int64_t out_feat, int dtype) {
+  if (dtype != AT_DTYPE_F32) return 0;
+  if (batch < 128 || in_feat < 32 || out_feat < 128) return 0;          // contractions of at least two k-tiles
+  if ((in_feat % 4) || (out_feat % 4)) return 0;                         // 16-byte vectors along the features
+  // small enough that neither product gives every CU a 64x64 tile (the same bound as the
+  // single products use for the 32x32 tiles)
+  const int64_t cus = device_cu_count();
+  if (cdiv64(batch, 64) * cdiv64(in_feat, 64) >= cus || cdiv64(in_feat, 64) * cdiv64(out_feat, 64) >= cus) return 0;
+  return 1;
+}
+
+int at_linear_bwd_small(const void* output_grad, const void* pre_act, const void* input, const void* weight,
+                        void* input_grad, void* weight_grad, void* bias_grad, int64_t batch, int64_t in_feat,
+                        int64_t out_feat, int64_t output_grad_stride, int64_t pre_act_stride, int64_t input_stride,
+                        int64_t weight_stride, int64_t input_grad_stride, int64_t weight_grad_stride, int act,
+                        float param, int dtype, at_stream_t stream) {
+  if (!output_grad || !input || !weight || !weight_grad) return AT_ERR_NULL;   // input_grad is optional
+  if (!act_valid(act)) return AT_ERR_ACT;
+  if (act != AT_ACT_NONE && !pre_act) return AT_ERR_NULL;
+  if (!at_linear_bwd_small_supported(batch, in_feat, out_feat, dtype)) return AT_ERR_UNSUPPORTED;
+  if (output_grad_stride < out_feat || (pre_act && pre_act_stride < out_feat) || input_stride < in_feat ||
+      weight_stride < out_feat || (input_grad && input_grad_stride < in_feat) || weight_grad_stride < out_feat)
+    return AT_ERR_DIM;
+  const int64_t strides[] = {output_grad_stride, pre_act ? pre_act_stride : 0, input_stride, weight_stride};
+  for (int64_t st : strides)
+    if (st % 4) return AT_ERR_ALIGN;
+  if (!aligned16(output_grad) || (pre_act && !aligned16(pre_act)) || !aligned16(input) || !aligned16(weight))
+    return AT_ERR_ALIGN;
+  const int64_t limit = (int64_t)1 << 31;
+  if (batch * output_grad_stride * 4 >= limit || batch * input_stride * 4 >= limit || in_feat * weight_stride * 4 >= limit)
+    return AT_ERR_UNSUPPORTED;
+  SmallBwdArgs s{};
+  s.output_grad = (const float*)output_grad;
+  // without an activation the derivative is 1 whatever it is evaluated at: any readable tensor of
+  // the gradient's shape serves as the second stream
+  s.pre_act = pre_act ? (const float*)pre_act : (const float*)output_grad;
+  s.input = (const float*)input;
+  s.weight = (const float*)weight;
+  s.input_grad = (float*)input_grad;
+  s.weight_grad = (float*)weight_grad;
+  s.bias_grad = (float*)bias_grad;
+  s.batch = (int)batch; s.in_feat = (int)in_feat; s.out_feat = (int)out_feat;
+  s.ld_g = output_grad_stride; s.ld_p = pre_act ? pre_act_stride : output_grad_stride;
+  s.ld_x = input_stride; s.ld_w = weight_stride; s.ld_dx = input_grad_stride; s.ld_dw = weight_grad_stride;
+  s.act = act; s.param = param;
+  s.dx_tiles = input_grad ? (int)(cdiv64(batch, 32) * cdiv64(in_feat, 32)) : 0;
+  const unsigned grid = (unsigned)(s.dx_tiles + cdiv64(in_feat, 32) * cdiv64(out_feat, 32));
+  // k-tiles of 128 for contractions of 512 and more, 64 below (the ring holds four of them)
+  const bool long_x = out_feat >= 512, long_w = batch >= 512;
+  hipStream_t hs = (hipStream_t)stream;
+  if (long_x && long_w) hipLaunchKernelGGL((linear_bwd_small_kernel<128, 128>), dim3(grid), dim3(kSplitThreads), 0, hs, s);
+  else if (long_x) hipLaunchKernelGGL((linear_bwd_small_kernel<128, 64>), dim3(grid), dim3(kSplitThreads), 0, hs, s);
+  else if (long_w) hipLaunchKernelGGL((linear_bwd_small_kernel<64, 128>), dim3(grid), dim3(kSplitThreads), 0, hs, s);
+  else hipLaunchKernelGGL((linear_bwd_small_kernel<64, 64>), dim3(grid), dim3(kSplitThreads), 0, hs, s);
+  return launch_status();
 }
 
 int64_t at_linear_bwd_weight_workspace_bytes(int64_t batch, int64_t in_feat, int64_t out_feat, int dtype) {

@@ -171,6 +171,35 @@ class LinearAutoGrad(torch.autograd.Function):
         _, out_feat_dim = weight.shape
         stream = _lib.stream_of(input)
 
+        if (weight.requires_grad and output_dtype is torch.float32
+                and output_grad.dtype is torch.float32 and flattened_input.dtype is torch.float32
+                and weight.dtype is torch.float32 and (pre_act is None or pre_act.dtype is torch.float32)
+                and lib.at_linear_bwd_small_supported(batch_dim, in_feat_dim, out_feat_dim,
+                                                      _lib.dtype_id(torch.float32))):
+            # small fp32 layer: activation gradient, both products and the bias sum in one launch
+            input_mm, weight_mm = _matrix(flattened_input), _matrix(weight)
+            pre_act_mm = None if ctx.act_func is None else _matrix(pre_act)
+            operands = [output_grad, input_mm, weight_mm] + ([] if pre_act_mm is None else [pre_act_mm])
+            if all(t.data_ptr() % 16 == 0 and _lib.row_stride(t) % 4 == 0 for t in operands):
+                input_grad = (torch.empty((batch_dim, in_feat_dim), dtype=output_dtype, device=device)
+                              if input.requires_grad else None)
+                weight_grad = torch.empty((in_feat_dim, out_feat_dim), dtype=output_dtype, device=device)
+                bias_grad = (torch.empty(out_feat_dim, dtype=output_dtype, device=device)
+                             if ctx.bias_requires_grad else None)
+                with torch.cuda.device_of(input):
+                    _lib.check(lib.at_linear_bwd_small(
+                        _lib.ptr(output_grad), _lib.ptr(pre_act_mm), _lib.ptr(input_mm), _lib.ptr(weight_mm),
+                        _lib.ptr(input_grad), _lib.ptr(weight_grad), _lib.ptr(bias_grad), batch_dim,
+                        in_feat_dim, out_feat_dim, _lib.row_stride(output_grad),
+                        0 if pre_act_mm is None else _lib.row_stride(pre_act_mm), _lib.row_stride(input_mm),
+                        _lib.row_stride(weight_mm), in_feat_dim, out_feat_dim,
+                        ctx.act if ctx.act_func is not None else 0,
+                        0.0 if ctx.param is None else ctx.param, _lib.dtype_id(torch.float32), stream),
+                        'at_linear_bwd_small')
+                if input_grad is not None:
+                    input_grad = input_grad.view_as(input)
+                return input_grad, weight_grad, bias_grad, None
+
         with torch.cuda.device_of(input):
             bias_grad = None
             if ctx.act_func is None:

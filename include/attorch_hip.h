@@ -321,6 +321,27 @@ int at_linear_bwd_weight(const void* input, const void* pre_act_grad, void* weig
                          int64_t grad_stride, int64_t weight_grad_stride, int in_dtype,
                          int out_dtype, at_stream_t stream);
 
+/* The whole backward pass of a small fp32 layer in one launch — act_func_backward
+ * (attorch/linear_layer.py:143-149 with act_kernels.py), the two products of :152-155 and the
+ * bias sum of :157: input_grad = dZ W^T, weight_grad = X^T dZ and, when bias_grad is non-null,
+ * bias_grad = column sums of dZ, with dZ = output_grad * act'(pre_act) formed on the fly and
+ * never stored (act = AT_ACT_NONE: dZ = output_grad, pre_act may be null; a null input_grad
+ * skips that product).  For layers whose
+ * gradients have too few tiles to fill the GPU, where launches cost more than arithmetic:
+ * at_linear_bwd_small_supported tells (1 / 0) whether a shape and dtype qualify (fp32, feature
+ * extents multiples of 4, both gradients smaller than one 64x64 tile per CU); other arguments
+ * return AT_ERR_UNSUPPORTED and the caller takes at_act_bwd + at_linear_bwd_input +
+ * at_linear_bwd_weight.  Results are summed in a fixed order. */
+int at_linear_bwd_small_supported(int64_t batch, int64_t in_feat, int64_t out_feat, int dtype);
+
+int at_linear_bwd_small(const void* output_grad, const void* pre_act, const void* input,
+                        const void* weight, void* input_grad, void* weight_grad, void* bias_grad,
+                        int64_t batch, int64_t in_feat, int64_t out_feat,
+                        int64_t output_grad_stride, int64_t pre_act_stride, int64_t input_stride,
+                        int64_t weight_stride, int64_t input_grad_stride,
+                        int64_t weight_grad_stride, int act, float param, int dtype,
+                        at_stream_t stream);
+
 int64_t at_act_bwd_workspace_bytes(int64_t rows, int64_t cols);
 
 int at_act_bwd(const void* output_grad, const void* input, void* input_grad, void* bias_grad,

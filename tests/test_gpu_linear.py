@@ -196,3 +196,77 @@ def test_linear_classifier_heads(shape, out_dim, act_func, dtype) -> None:
     """
     run_case(shape, out_dim, True, act_func, dtype)
     run_case(shape, out_dim, False, act_func, dtype)
+
+
+SMALL_BWD_CASES = [
+    # batch, in_feat, out_feat, act_func, bias, input needs a gradient
+    (512, 784, 256, 'relu', True, True),         # the MNIST-sized layer
+    (512, 784, 256, 'relu', True, False),        # first layer of a network: no input gradient
+    (128, 36, 128, 'gelu', False, True),
+    (200, 100, 132, None, True, True),           # no activation: dZ is the output gradient itself
+    (1000, 260, 512, 'leaky_relu_0.01', True, True),
+    (130, 1028, 640, 'geluapprox', True, True),
+]
+
+
+@pytest.mark.parametrize('batch, in_dim, out_dim, act_func, bias, input_grad', SMALL_BWD_CASES)
+def test_small_fp32_backward_in_one_launch(batch, in_dim, out_dim, act_func, bias, input_grad) -> None:
+    # shapes the one-launch backward serves: same results as the oracle, and as the three separate calls
+    from attorch_amd import _lib
+    lib = _lib.load()
+    dtype = torch.float32
+    assert lib.at_linear_bwd_small_supported(batch, in_dim, out_dim, _lib.dtype_id(dtype)) == 1
+    x = randn((batch, in_dim), 1, dtype)
+    w = randn((in_dim, out_dim), 2, dtype, in_dim ** -0.5)
+    b = randn((out_dim,), 3, dtype, 0.1) if bias else None
+    dy = randn((batch, out_dim), 4, dtype)
+    name, param = oracle.parse_act_func(act_func)
+    xd, wd = x.cuda().requires_grad_(input_grad), w.cuda().requires_grad_(True)
+    bd = b.cuda().requires_grad_(True) if bias else None
+    y = attorch_amd.LinearAutoGrad.apply(xd, wd, bd, act_func)
+    pre_act = y.grad_fn.saved_tensors[1]
+    pre_act = None if pre_act is None else pre_act.detach()
+    y.backward(dy.cuda())
+    dx_ref, dw_ref, db_ref = oracle.linear_backward(dy, x, w, None if pre_act is None else pre_act.cpu(), name, param,
+                                                    dtype, compute=torch.float64)
+    if input_grad:
+        assert_close(xd.grad, dx_ref, dtype, 'input_grad', dot_terms=out_dim, term_scale=in_dim ** -0.5)
+    else:
+        assert xd.grad is None
+    assert_close(wd.grad, dw_ref, dtype, 'weight_grad', batch_reduction=True)
+    if bias:
+        assert_close(bd.grad, db_ref, dtype, 'bias_grad', batch_reduction=True)
+
+    # the separate calls on the same operands
+    stream = _lib.stream_of(xd)
+    dyd, act = dy.cuda(), attorch_amd.act.act_id(name, param)
+    dz = dyd
+    if name is not None:
+        dz = torch.empty_like(dyd)
+        _lib.check(lib.at_act_bwd(dyd.data_ptr(), pre_act.data_ptr(), dz.data_ptr(), None, None, 0, batch, out_dim,
+                                  out_dim, out_dim, out_dim, act, 0.0 if param is None else param, 0, 0, 0, stream),
+                   'at_act_bwd')
+    dw_sep = torch.empty_like(wd)
+    _lib.check(lib.at_linear_bwd_weight(xd.data_ptr(), dz.data_ptr(), dw_sep.data_ptr(), None, 0, batch, in_dim,
+                                        out_dim, in_dim, out_dim, out_dim, 0, 0, stream), 'at_linear_bwd_weight')
+    assert_close(wd.grad, dw_sep.cpu(), dtype, 'weight_grad against the separate call', batch_reduction=True)
+    if input_grad:
+        dx_sep = torch.empty_like(xd)
+        _lib.check(lib.at_linear_bwd_input(dz.data_ptr(), wd.data_ptr(), dx_sep.data_ptr(), batch, in_dim, out_dim,
+                                           out_dim, out_dim, in_dim, 0, 0, stream), 'at_linear_bwd_input')
+        assert_close(xd.grad, dx_sep.cpu(), dtype, 'input_grad against the separate call', dot_terms=out_dim,
+                     term_scale=in_dim ** -0.5)
+
+
+def test_small_backward_declines_other_shapes() -> None:
+    from attorch_amd import _lib
+    lib = _lib.load()
+    f32, bf16 = _lib.dtype_id(torch.float32), _lib.dtype_id(torch.bfloat16)
+    assert lib.at_linear_bwd_small_supported(512, 784, 256, bf16) == 0       # fp32 only
+    assert lib.at_linear_bwd_small_supported(512, 783, 256, f32) == 0        # rows must allow 16-byte vectors
+    assert lib.at_linear_bwd_small_supported(16384, 4096, 4096, f32) == 0    # large layers take the tiled products
+    assert lib.at_linear_bwd_small_supported(64, 784, 256, f32) == 0
+    t = torch.zeros(4, device='cuda')
+    p = t.data_ptr()
+    assert lib.at_linear_bwd_small(p, p, p, p, p, p, None, 512, 783, 256, 256, 256, 783, 256, 783, 256, 4, 0.0, f32,
+                                   _lib.stream_of(t)) == -7                  # AT_ERR_UNSUPPORTED, nothing launched
