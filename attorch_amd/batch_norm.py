@@ -84,7 +84,11 @@ class BatchNormAutoGrad(torch.autograd.Function):
                          (add_pre_act and pre_act_add.requires_grad) or
                          (affine and weight.requires_grad) or
                          (affine and bias.requires_grad))
-        save_pre_act = requires_grad and (act_func is not None)
+        # relu, relu6 and hardtanh have the same derivative at the output as at the
+        # pre-activation (the flat pieces map to their end points), so the output serves in
+        # backward and the pre-activation is neither written nor kept
+        ctx.output_as_pre_act = act_func in ('relu', 'relu6', 'hardtanh')
+        save_pre_act = requires_grad and (act_func is not None) and not ctx.output_as_pre_act
 
         batch_dim, feat_dim, spatial_dim = _dims(input)
         input_k = input.contiguous()
@@ -120,7 +124,7 @@ class BatchNormAutoGrad(torch.autograd.Function):
         ctx.add_pre_act = add_pre_act
         if requires_grad:
             ctx.save_for_backward(input_k, mean, inv_std, weight_k,
-                                  pre_act if save_pre_act else None)
+                                  pre_act if save_pre_act else (output if ctx.output_as_pre_act else None))
 
         return output.view_as(input)
 

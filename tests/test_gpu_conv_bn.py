@@ -265,7 +265,12 @@ def test_batch_norm_training(shape, dtype, affine, residual, act_func) -> None:
     assert_close(rv, rv_ref, torch.float32, 'running_var')     # unbiased variance in the running stat
 
     pre_act = saved[4] if name is not None else None            # device's own pre-activation, see Linear test
-    if name is not None:
+    if name == 'relu':
+        # relu has the same derivative at its output as at its input, so the layer keeps the output
+        # in place of the pre-activation (and never writes the latter)
+        assert_close(pre_act, y_ref, dtype, 'output kept for backward')
+        assert torch.equal(pre_act > 0, pre_act_ref.to(dtype) > 0) or dtype is not torch.float32
+    elif name is not None:
         assert_close(pre_act, pre_act_ref, dtype, 'pre_act')
     dx_ref, dw_ref, db_ref, dres_ref = oracle.batch_norm_backward(
         dy, x, saved[1], saved[2], w, affine, pre_act, name, param, compute=cd)
