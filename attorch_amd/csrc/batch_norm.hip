@@ -51,28 +51,6 @@ __device__ __forceinline__ float block_sum(float v, float* smem) {
   return group_reduce(v, (int)blockDim.x, smem, SumOp(), 0.f);
 }
 
-// Enumerates the VEC-element chunks of channel c that belong to split p of P and calls
-// f(element_offset).  Planes with many chunks are walked plane by plane; small planes are
-// flattened so the lanes stay busy.
-template <int VEC, typename F>
-__device__ __forceinline__ void for_channel_chunks(int c, int p, int P, int64_t N, int C, int S, F&& f) {
-  const int sp = S / VEC;  // chunks per plane (S % VEC == 0 on the vector path, VEC == 1 otherwise)
-  if (sp >= kBnBlock) {
-    for (int64_t n = p; n < N; n += P) {
-      const int64_t base = (n * C + c) * (int64_t)S;
-      for (int i = threadIdx.x; i < sp; i += kBnBlock) f(base + (int64_t)i * VEC);
-    }
-  } else {
-    const int64_t planes = (N - p + P - 1) / P;  // planes n = p, p + P, ...
-    const int64_t total = planes * sp;
-    for (int64_t q = threadIdx.x; q < total; q += kBnBlock) {
-      const int64_t k = q / sp;
-      const int i = (int)(q - k * sp);
-      f(((p + k * P) * C + c) * (int64_t)S + (int64_t)i * VEC);
-    }
-  }
-}
-
 // Raw 16-byte (or narrower) image of VEC elements, widened on use: loads are issued into these
 // so that nothing has to wait before the next load is issued.
 template <typename T, int VEC>
@@ -87,29 +65,70 @@ struct RawVec {
   }
 };
 
+// The VEC-element chunks of channel c that split p of P owns (planes n = p, p + P, ..., flattened
+// so that the lanes stay busy whatever the plane size), U at a time per thread:
+// issue(u, element_offset) is called for the U chunks of a batch first — it should only start
+// loads — and use(u) afterwards for those of them that exist.  The loads of a batch are thus in
+// flight together; a chunk that does not exist is issued at the offset of the batch's first chunk
+// (which does), so that no load sits inside a branch.
+template <int VEC, int U, typename ISSUE, typename USE>
+__device__ __forceinline__ void for_channel_chunks_batched(int c, int p, int P, int64_t N, int C, int S,
+                                                           ISSUE&& issue, USE&& use) {
+  const uint32_t sp = (uint32_t)(S / VEC);
+  const int64_t planes = (N - p + P - 1) / P;   // planes n = p, p + P, ...
+  const int64_t total = planes * sp;
+  auto offset_of = [&](int64_t q) {
+    int64_t k;
+    uint32_t i;
+    if (total <= (int64_t)UINT32_MAX) {
+      const uint32_t q32 = (uint32_t)q, k32 = q32 / sp;
+      k = k32;
+      i = q32 - k32 * sp;
+    } else {
+      k = q / sp;
+      i = (uint32_t)(q - k * sp);
+    }
+    return ((p + k * P) * C + c) * (int64_t)S + (int64_t)i * VEC;
+  };
+  for (int64_t q0 = threadIdx.x; q0 < total; q0 += (int64_t)kBnBlock * U) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t q = q0 + (int64_t)u * kBnBlock;
+      issue(u, offset_of(q < total ? q : q0));
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (q0 + (int64_t)u * kBnBlock < total) use(u);
+  }
+}
+
 template <typename T, int VEC>
 __global__ __launch_bounds__(kBnBlock) void bn_stats_kernel(const T* __restrict__ x, float* __restrict__ part,
                                                            int64_t N, int C, int S, int P) {
   __shared__ Welford smem[kBnBlock / 64];
   const int c = blockIdx.x, p = blockIdx.y;
   Welford acc{0.f, 0.f, 0.f};
-  for_channel_chunks<VEC>(c, p, P, N, C, S, [&](int64_t off) {
-    float v[VEC];
-    load_f32<T, VEC>(x + off, v);
-    float s = 0.f;
+  constexpr int U = 4;
+  RawVec<T, VEC> raw[U];
+  for_channel_chunks_batched<VEC, U>(
+      c, p, P, N, C, S, [&](int u, int64_t off) { raw[u].load(x + off); },
+      [&](int u) {
+        float v[VEC];
+        raw[u].get(v);
+        float s = 0.f;
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) s += v[j];
-    const float m = s * (1.0f / VEC);
-    float m2 = 0.f;
+        for (int j = 0; j < VEC; ++j) s += v[j];
+        const float m = s * (1.0f / VEC);
+        float m2 = 0.f;
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) m2 += (v[j] - m) * (v[j] - m);
-    const float n = acc.n + VEC;
-    const float d = m - acc.mean;
-    const float f = __fdividef((float)VEC, n);
-    acc.m2 += m2 + d * d * acc.n * f;
-    acc.mean += d * f;
-    acc.n = n;
-  });
+        for (int j = 0; j < VEC; ++j) m2 += (v[j] - m) * (v[j] - m);
+        const float n = acc.n + VEC;
+        const float d = m - acc.mean;
+        const float f = __fdividef((float)VEC, n);
+        acc.m2 += m2 + d * d * acc.n * f;
+        acc.mean += d * f;
+        acc.n = n;
+      });
   const Welford r = wf_block_reduce(acc, smem);
   if (threadIdx.x == 0) {
     float* dst = part + ((int64_t)c * P + p) * 3;
@@ -249,26 +268,37 @@ __global__ __launch_bounds__(kBnBlock) void bn_bwd_reduce_kernel(
   const int c = blockIdx.x, p = blockIdx.y;
   const float mean = mean_in[c], inv_std = inv_std_in[c];
   float s1 = 0.f, s2 = 0.f;
-  for_channel_chunks<VEC>(c, p, P, N, C, S, [&](int64_t off) {
-    float g[VEC], xv[VEC];
-    load_f32<T, VEC>(dy + off, g);
-    load_f32<T, VEC>(x + off, xv);
-    if (ACT != AT_ACT_NONE) {
-      float z[VEC];
-      load_f32<T, VEC>(pre_act + off, z);
+  constexpr int U = 2;
+  RawVec<T, VEC> rg[U], rx[U], rz[ACT != AT_ACT_NONE ? U : 1];
+  int64_t offs[U];
+  for_channel_chunks_batched<VEC, U>(
+      c, p, P, N, C, S,
+      [&](int u, int64_t off) {
+        offs[u] = off;
+        rg[u].load(dy + off);
+        rx[u].load(x + off);
+        if constexpr (ACT != AT_ACT_NONE) rz[u].load(pre_act + off);
+      },
+      [&](int u) {
+        float g[VEC], xv[VEC];
+        rg[u].get(g);
+        rx[u].get(xv);
+        if constexpr (ACT != AT_ACT_NONE) {
+          float z[VEC];
+          rz[u].get(z);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) g[j] *= act_derivative(ACT, z[j], param);
-      store_f32<T, VEC>(g_out + off, g);
-      // the reference rounds pre_act_grad to the storage dtype before reducing it
+          for (int j = 0; j < VEC; ++j) g[j] *= act_derivative(ACT, z[j], param);
+          store_f32<T, VEC>(g_out + offs[u], g);
+          // the reference rounds pre_act_grad to the storage dtype before reducing it
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) g[j] = to_f32(from_f32<T>(g[j]));
-    }
+          for (int j = 0; j < VEC; ++j) g[j] = to_f32(from_f32<T>(g[j]));
+        }
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      s1 += g[j] * (xv[j] - mean) * inv_std;
-      s2 += g[j];
-    }
-  });
+        for (int j = 0; j < VEC; ++j) {
+          s1 += g[j] * (xv[j] - mean) * inv_std;
+          s2 += g[j];
+        }
+      });
   s1 = block_sum(s1, smem);
   s2 = block_sum(s2, smem);
   if (threadIdx.x == 0) {
