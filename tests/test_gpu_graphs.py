@@ -90,3 +90,46 @@ def test_captured_conv_block_replays_like_eager() -> None:
         torch.cuda.synchronize()
         for g, e in zip(got, expected):
             torch.testing.assert_close(g, e, rtol=0, atol=0)
+
+
+def test_captured_dropout_replays_the_captured_mask() -> None:
+    """
+    The dropout seed is drawn on the host when the layer is called and travels as a kernel
+    argument (as in the reference, attorch/act_layers.py:66), so a captured step keeps the mask it
+    was captured with: every replay drops the same elements, forward and backward alike.  (Eager
+    calls draw a new seed each time.)  Training under a graph with dropout therefore needs a
+    re-capture per step or dropout outside the graph; this test pins that behaviour.
+    """
+    layer = attorch_amd.GELU(approximate='tanh', drop_p=0.5)
+    static_x = torch.randn(64, 512, device='cuda', requires_grad=True)
+    upstream = torch.ones(64, 512, device='cuda')
+
+    def step():
+        y = layer(static_x)
+        (dx,) = torch.autograd.grad(y, static_x, upstream)
+        return y, dx
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_y, static_dx = step()
+
+    masks = []
+    for seed in range(3):
+        with torch.no_grad():
+            static_x.copy_(torch.randn(64, 512, device='cuda', generator=torch.Generator(device='cuda').manual_seed(seed))
+                           .abs() + 0.5)       # positive inputs: gelu(x) != 0, so a zero means "dropped"
+        graph.replay()
+        torch.cuda.synchronize()
+        dropped = static_y == 0
+        assert 0.4 < dropped.float().mean().item() < 0.6
+        assert torch.equal(dropped, static_dx == 0), 'forward and backward dropped different elements'
+        masks.append(dropped.clone())
+        eager_y, _ = step()                    # eager calls in between draw their own seeds
+        torch.cuda.synchronize()
+        assert not torch.equal(eager_y == 0, dropped)
+    assert torch.equal(masks[0], masks[1]) and torch.equal(masks[1], masks[2])
