@@ -66,6 +66,9 @@ __device__ __forceinline__ void lds_dma_16(const i32x4& rsrc, int byte_offset, c
 }
 
 __device__ __forceinline__ void lds_dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// Waits for all loads of the wave except the N issued last (the counter runs in issue order).
+template <int N>
+__device__ __forceinline__ void lds_dma_wait_newest() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
 // Fragment (32 rows x 16 k, 8 consecutive k per lane) of a tile laid out by lds_chunk_offset.
 __device__ __forceinline__ uint4 read_frag_kc(const char* tile, int row_base, int ks) {

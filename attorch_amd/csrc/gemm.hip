@@ -76,7 +76,9 @@ typedef __attribute__((address_space(3))) void lds_void_t;
 //    the row (lds_chunk_offset); fragments are plain 128-bit reads.
 //  * otherwise (memory [k][outer]): 64 k-rows x 512 bytes kept as loaded; every pair of rows
 //    is one contiguous KiB (one wave-wide load) followed by 64 bytes of padding, which
-//    spreads the 8 rows a transposing fragment read touches evenly over the banks.
+//    spreads the 8 rows a transposing fragment read touches evenly over the banks.  (Without the
+//    padding, k-row r keeping chunk x at position x ^ 2 (r & 3), the tiles are 2 KB smaller
+//    but the product that reads both operands this way is 2.7 % slower.)
 constexpr int kPairPitch = 1024 + 64;
 template <bool CONTRACT_CONTIG> constexpr int operand_tile_bytes() { return CONTRACT_CONTIG ? kTileBytes : 32 * kPairPitch; }
 
@@ -244,9 +246,16 @@ template <typename T, bool A_MC, bool B_KC, int ACT>
 __global__ __launch_bounds__(kBigThreads) void gemm_mfma16_kernel(GemmArgs g) {
   constexpr bool A_KC = !A_MC;
   constexpr int kATile = operand_tile_bytes<A_KC>(), kBTile = operand_tile_bytes<B_KC>();
-  constexpr int kStage = kATile + kBTile;
-  constexpr int kLds = 2 * kStage > kEpiBytes ? 2 * kStage : kEpiBytes;
-  __shared__ __attribute__((aligned(1024))) char lds[kLds];  // main loop: [stage][A|B]; epilogue: output tile
+  // When both operands are contraction-contiguous (32 KB tiles) the A tiles live in a ring of
+  // three stages and the B tiles in one of two — all of the CU's 160 KB: A's loads then run two
+  // k-tiles ahead of their use, B's one (see the main loop); that product gains 6 %.  The other
+  // layouts have padded tiles that do not fit a third stage (and the forward product, tried with
+  // unpadded tiles, gains under 1 % from it): two stages each.
+  constexpr int kAStages = (A_KC && B_KC) ? 3 : 2;
+  constexpr int kARing = kAStages * kATile;
+  constexpr int kLds = kARing + 2 * kBTile > kEpiBytes ? kARing + 2 * kBTile : kEpiBytes;
+  static_assert(kLds <= 160 * 1024, "the stages fill the LDS of a CU exactly");
+  __shared__ __attribute__((aligned(1024))) char lds[kLds];  // main loop: A ring | B ring; epilogue: output tile
   const T* __restrict__ A = reinterpret_cast<const T*>(g.a);
   const T* __restrict__ B = reinterpret_cast<const T*>(g.b);
 
@@ -286,36 +295,50 @@ __global__ __launch_bounds__(kBigThreads) void gemm_mfma16_kernel(GemmArgs g) {
   lb.init(B, g.ldb, n0, g.N, g.K);
   const int KT = (g.K + BK - 1) / BK;
 
-  auto load_frags = [&](const char* stage, int ks, uint4 (&af)[4], uint4 (&bf)[NJ]) {
+  auto load_frags = [&](const char* a_stage, const char* b_stage, int ks, uint4 (&af)[4], uint4 (&bf)[NJ]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) af[i] = read_frag<A_KC>(stage, wm * 128 + i * 32, ks);
+    for (int i = 0; i < 4; ++i) af[i] = read_frag<A_KC>(a_stage, wm * 128 + i * 32, ks);
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) bf[j] = read_frag<B_KC>(stage + kATile, wn * kBigWaveN + j * 32, ks);
+    for (int j = 0; j < NJ; ++j) bf[j] = read_frag<B_KC>(b_stage, wn * kBigWaveN + j * 32, ks);
   };
 
-  la.issue(0, lds);
-  lb.issue(0, lds + kATile);
+  char* const a_ring = lds;
+  char* const b_ring = lds + kARing;
+  la.issue(0, a_ring);
+  lb.issue(0, b_ring);
   lds_dma_wait_all();
   __syncthreads();
-  la.issue(1, lds + kStage);   // k-tile 1 travels while k-tile 0 is multiplied (zeros when there is none)
-  lb.issue(1, lds + kStage + kATile);
+  // k-tiles 1 (both operands) and 2 (A) travel while k-tile 0 is multiplied (zeros when there are
+  // none).  A's tile 2 is issued last: the in-order counter then lets it stay in flight across the
+  // first wait.
+  la.issue(1, a_ring + kATile);
+  lb.issue(1, b_ring + kBTile);
+  if (kAStages == 3) la.issue(2 < KT ? 2 : -1, a_ring + 2 * kATile);
   uint4 af[2][4], bf[2][NJ];
-  load_frags(lds, 0, af[0], bf[0]);
+  load_frags(a_ring, b_ring, 0, af[0], bf[0]);
 
   // One k-tile = four k-steps of 4 * NJ MFMAs per wave, the other instructions slotted between
   // them.  K-steps 0..2 multiply while the fragments of the following k-step are read.  Before
   // k-step 3 every fragment of the current stage is in registers, so the one barrier of the
-  // iteration both publishes k-tile kt+1 (issued a whole iteration earlier) and frees the
-  // current stage: k-step 3 multiplies while the loads of k-tile kt+2 are issued into it and the
-  // first fragments of k-tile kt+1 are read, so the MFMAs run on across the barrier.
+  // iteration both publishes k-tile kt+1 and frees the current stages: k-step 3 multiplies while
+  // B's k-tile kt+2 and then A's k-tile kt+3 are issued into them and the first fragments of
+  // k-tile kt+1 are read, so the MFMAs run on across the barrier.  The wait before the barrier
+  // leaves the newest kBigLoads loads of the wave (A's k-tile kt+2, issued last in the previous
+  // iteration) in flight: A's tiles have two iterations to arrive, B's one.
   // (sched_group_barrier masks: 0x8 MFMA, 0x2 VALU, 0x20 VMEM read, 0x100 LDS read.)
+  int a_slot = 0;   // kt % kAStages
   for (int kt = 0; kt < KT; ++kt) {
-    char* cur = lds + (kt & 1) * kStage;
-    char* nxt = lds + ((kt & 1) ^ 1) * kStage;
+    const int a_this = kAStages == 3 ? a_slot : (kt & 1);
+    const int a_next = kAStages == 3 ? (a_slot == 2 ? 0 : a_slot + 1) : (a_this ^ 1);
+    char* a_cur = a_ring + a_this * kATile;
+    char* a_nxt = a_ring + a_next * kATile;
+    char* b_cur = b_ring + (kt & 1) * kBTile;
+    char* b_nxt = b_ring + ((kt & 1) ^ 1) * kBTile;
+    a_slot = a_next;
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < BK / 16 - 1; ++ks) {
-      load_frags(cur, ks + 1, af[(ks + 1) & 1], bf[(ks + 1) & 1]);
+      load_frags(a_cur, b_cur, ks + 1, af[(ks + 1) & 1], bf[(ks + 1) & 1]);
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -329,20 +352,23 @@ __global__ __launch_bounds__(kBigThreads) void gemm_mfma16_kernel(GemmArgs g) {
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    lds_dma_wait_all();   // k-tile kt+1: this wave's part has landed
-    __syncthreads();      // ... and everybody's; nobody reads the current stage any more
+    // k-tile kt+1: this wave's part has landed
+    if (kAStages == 3) lds_dma_wait_newest<kBigLoads>(); else lds_dma_wait_all();
+    __syncthreads();                    // ... and everybody's; nobody reads the current stages any more
     // Past the last k-tile the loads are issued all the same, with offsets that are out of range:
     // they write zeros into a stage nobody reads, and the loop body has no branches.
     const int kt2 = kt + 2 < KT ? kt + 2 : -1;
-    load_frags(nxt, 0, af[0], bf[0]);
+    const int kt3 = kt + kAStages < KT ? kt + kAStages : -1;   // A's next tile: two or three ahead
+    load_frags(a_nxt, b_nxt, 0, af[0], bf[0]);
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
         // one global->LDS load behind each MFMA (2 * kBigLoads = 4 * NJ of either)
         const int t = i * NJ + j;
-        if (t < kBigLoads) la.issue_one(kt2, cur, t);
-        else lb.issue_one(kt2, cur + kATile, t - kBigLoads);
+        // with three A stages A's loads must be the wave's newest (they stay in flight over the wait)
+        if ((t < kBigLoads) == (kAStages == 3)) lb.issue_one(kt2, b_cur, t % kBigLoads);
+        else la.issue_one(kt3, a_cur, t % kBigLoads);
         acc[i][j] = Mfma16<T>::run(bf[1][j], af[1][i], acc[i][j]);
       }
 #pragma unroll
