@@ -57,6 +57,7 @@ PROTOTYPES = {
     'at_batch_norm_workspace_bytes': (L, [L]),
     'at_batch_norm_fwd': (I, [P, P, P, P, P, P, P, P, P, P, P, L, L, L, L, F, F, I, F, I, I, I, I, I, P]),
     'at_conv2d_fwd_workspace_bytes': (L, [L] * 14 + [I, I]),
+    'at_conv2d_fwd_leaves_nhwc': (I, [L] * 14 + [I, I]),
     'at_conv2d_fwd': (I, [P, P, P, P, P, L] + [L] * 14 + [I, I, I, P]),
     'at_conv2d_bwd_input_workspace_bytes': (L, [L] * 14 + [I]),
     'at_conv2d_bwd_input': (I, [P, P, P, P, P, L] + [L] * 14 + [I, P]),

@@ -127,8 +127,11 @@ class Conv2dAutoGrad(torch.autograd.Function):
         ctx.bias_requires_grad = False if bias is None else bias.requires_grad
         ctx.output_dtype = output_dtype
         # The matrix-core path leaves a channels-last copy of the input at the start of its
-        # workspace; the weight gradient reuses it instead of transposing the input again.
-        ctx.input_nhwc = workspace if requires_grad and weight.requires_grad else None
+        # workspace (unless it had to pad the channels); the weight gradient reuses it instead of
+        # transposing the input again.
+        keep = (requires_grad and weight.requires_grad and workspace is not None
+                and lib.at_conv2d_fwd_leaves_nhwc(*dims, dtype, dtype) == 1)
+        ctx.input_nhwc = workspace if keep else None
         if requires_grad:
             ctx.save_for_backward(input, weight)
 

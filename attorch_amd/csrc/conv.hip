@@ -511,6 +511,16 @@ int64_t at_conv2d_fwd_workspace_bytes(int64_t batch, int64_t in_feat, int64_t in
   return conv_igemm_fwd_workspace(problem_of(s, in_dtype));
 }
 
+int at_conv2d_fwd_leaves_nhwc(int64_t batch, int64_t in_feat, int64_t in_height, int64_t in_width, int64_t out_feat,
+                              int64_t out_height, int64_t out_width, int64_t kernel_height, int64_t kernel_width,
+                              int64_t stride_height, int64_t stride_width, int64_t padding_height,
+                              int64_t padding_width, int64_t groups, int in_dtype, int out_dtype) {
+  const ConvShape s = shape_of(batch, in_feat, in_height, in_width, out_feat, out_height, out_width, kernel_height,
+                               kernel_width, stride_height, stride_width, padding_height, padding_width, groups);
+  if (check_shape(s) || in_dtype != out_dtype) return 0;
+  return conv_igemm_fwd_leaves_nhwc(problem_of(s, in_dtype)) ? 1 : 0;
+}
+
 int at_conv2d_fwd(const void* input, const void* weight, const void* bias, void* output, void* workspace,
                   int64_t workspace_bytes, int64_t batch, int64_t in_feat, int64_t in_height, int64_t in_width,
                   int64_t out_feat, int64_t out_height, int64_t out_width, int64_t kernel_height,

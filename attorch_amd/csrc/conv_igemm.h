@@ -17,11 +17,17 @@ struct ConvProblem {
   int dtype;   // AT_DTYPE_F16 or AT_DTYPE_BF16 for every tensor
 };
 
-// True when the 16-bit implicit-GEMM kernels cover the problem (channel counts per group in
-// multiples of 64, 32-bit addressable tensors; the input gradient additionally needs stride 1).
+// True when the 16-bit implicit-GEMM kernels cover the problem: 32-bit addressable tensors;
+// contraction channels per group (input channels for the forward product, output channels for the
+// input gradient) in multiples of 64, or at least 16 (padded with zeros to the next multiple in
+// the channels-last copy); strides of the input gradient with sh * sw <= 4 (the gradient is
+// spread out by the strides); channel counts per group in multiples of 8 for the weight gradient.
 bool conv_igemm_supports_fwd(const ConvProblem& p);
 bool conv_igemm_supports_dx(const ConvProblem& p);
 bool conv_igemm_supports_dw(const ConvProblem& p);
+// True when the forward workspace afterwards begins with a plain [N][H][W][C] copy of the input
+// (no channel padding), which conv_igemm_dw accepts as x_nhwc.
+bool conv_igemm_fwd_leaves_nhwc(const ConvProblem& p);
 
 int64_t conv_igemm_fwd_workspace(const ConvProblem& p);
 int64_t conv_igemm_dx_workspace(const ConvProblem& p);
@@ -30,8 +36,9 @@ int64_t conv_igemm_dw_workspace(const ConvProblem& p);
 // Y = conv(X, W) + bias, all NCHW.
 int conv_igemm_fwd(const ConvProblem& p, const void* x, const void* w, const void* bias, int bias_dt,
                    void* y, void* workspace, hipStream_t stream);
-// dX = conv_transpose(dY, W), all NCHW (stride 1 only).  dy_nhwc: optional channels-last copy of
-// dY the caller already holds (saves the copy made here).
+// dX = conv_transpose(dY, W), all NCHW.  dy_nhwc: optional channels-last copy of dY the caller
+// already holds (saves the copy made here when the product can read it as it is: stride 1 and
+// output channels per group a multiple of 64).
 int conv_igemm_dx(const ConvProblem& p, const void* dy, const void* dy_nhwc, const void* w, void* dx,
                   void* workspace, hipStream_t stream);
 // dW[O][C/groups][KH][KW] = correlation of dY with X, all NCHW.  dy_nhwc / x_nhwc: optional

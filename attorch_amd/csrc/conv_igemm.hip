@@ -54,32 +54,56 @@ __device__ __forceinline__ int fast_div(int n, const FastDiv& f) {
 // ------------------------------------------------------------------------------------------
 // Layout changes.
 // ------------------------------------------------------------------------------------------
-// [N][C][HW] -> [N][HW][C] through a 64 x 64 LDS tile; 128-bit accesses on both sides when the
-// shapes allow (vec_in: HW % 8 == 0 and aligned source; vec_out: C % 8 == 0 and aligned target).
+// [N][C][HW] -> [N][HW'][C'] through a 64 x 64 LDS tile; 128-bit accesses on both sides when the
+// shapes allow (vec_in: HW % 8 == 0 and aligned source; the target rows are 16-byte aligned by
+// construction when vec_out is set).  The target may be wider than the source in two ways:
+//  * channels: every group of Cg source channels becomes Cgp >= Cg target channels (Cgp a
+//    multiple of 64 when it differs from Cg), the extra ones zero — the products below contract
+//    over whole 64-channel tiles;
+//  * pixels: source pixel (h, w) of a row of W lands at ((h * sh) * Wd + w * sw); the pixels in
+//    between are not written (the caller clears the target first when sh * sw > 1) — the input
+//    gradient of a strided layer is a stride-1 product over the gradient spread out like this.
+struct LayoutCopyArgs {
+  int C, HW;          // source channels and pixels per image
+  int Cg, Cgp;        // channels per group in the source and in the target
+  int W, Wd, sh, sw;  // source row length, target row length, pixel spreading
+  int HWd;            // target pixels per image
+  int vec_in, vec_out;
+};
+
 template <typename T>
 __global__ __launch_bounds__(256) void nchw_to_nhwc_kernel(const T* __restrict__ src, T* __restrict__ dst,
-                                                            int C, int HW, int vec_in, int vec_out) {
+                                                            LayoutCopyArgs a) {
   __shared__ uint32_t tile[64][33];   // [channel][pixel pair], padded
   const int n = blockIdx.z;
-  const int c0 = blockIdx.y * 64, p0 = blockIdx.x * 64;
-  const T* s = src + (int64_t)n * C * HW;
-  T* d = dst + (int64_t)n * HW * C;
+  const int p0 = blockIdx.x * 64;
+  // blockIdx.y counts 64-channel tiles of the target; without padding groups play no role
+  const bool padded = a.Cgp != a.Cg;
+  const int tiles_per_group = padded ? a.Cgp / 64 : 1;
+  const int grp = padded ? (int)blockIdx.y / tiles_per_group : 0;
+  const int in_group0 = padded ? ((int)blockIdx.y % tiles_per_group) * 64 : (int)blockIdx.y * 64;
+  const int src_c0 = grp * a.Cg + in_group0;                    // first source channel of the tile
+  const int src_c_end = padded ? grp * a.Cg + a.Cg : a.C;       // one past the last valid one
+  const int dst_c0 = blockIdx.y * 64;
+  const int Cd = padded ? (a.C / a.Cg) * a.Cgp : a.C;           // target channels
+  const T* s = src + (int64_t)n * a.C * a.HW;
+  T* d = dst + (int64_t)n * a.HWd * Cd;
   const int t = threadIdx.x;
 #pragma unroll
   for (int pass = 0; pass < 2; ++pass) {
     const int cl = pass * 32 + (t >> 3), pv = (t & 7) * 8;
-    const int c = c0 + cl, p = p0 + pv;
+    const int c = src_c0 + cl, p = p0 + pv;
     uint4 v = make_uint4(0, 0, 0, 0);
-    if (c < C) {
-      const T* q = s + (int64_t)c * HW + p;
-      if (vec_in && p + 8 <= HW) {
+    if (c < src_c_end) {
+      const T* q = s + (int64_t)c * a.HW + p;
+      if (a.vec_in && p + 8 <= a.HW) {
         v = *reinterpret_cast<const uint4*>(q);
       } else {
         union { uint4 raw; T e[8]; } u;
         u.raw = v;
 #pragma unroll
         for (int e = 0; e < 8; ++e)
-          if (p + e < HW) u.e[e] = q[e];
+          if (p + e < a.HW) u.e[e] = q[e];
         v = u.raw;
       }
     }
@@ -92,17 +116,22 @@ __global__ __launch_bounds__(256) void nchw_to_nhwc_kernel(const T* __restrict__
 #pragma unroll
   for (int pass = 0; pass < 2; ++pass) {
     const int pl = pass * 32 + (t >> 3), cv = (t & 7) * 8;
-    const int p = p0 + pl, c = c0 + cv;
-    if (p >= HW || c >= C) continue;
+    const int p = p0 + pl, c = dst_c0 + cv;
+    if (p >= a.HW || c >= Cd) continue;
     uint32_t w[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const uint32_t lo = tile[cv + 2 * e][pl >> 1], hi = tile[cv + 2 * e + 1][pl >> 1];
-      const int sh = (pl & 1) * 16;
-      w[e] = ((lo >> sh) & 0xffffu) | (((hi >> sh) & 0xffffu) << 16);
+      const int sft = (pl & 1) * 16;
+      w[e] = ((lo >> sft) & 0xffffu) | (((hi >> sft) & 0xffffu) << 16);
     }
-    T* q = d + (int64_t)p * C + c;
-    if (vec_out && c + 8 <= C) {
+    int pd = p;
+    if (a.sh != 1 || a.sw != 1) {
+      const int h = p / a.W;
+      pd = (h * a.sh) * a.Wd + (p - h * a.W) * a.sw;
+    }
+    T* q = d + (int64_t)pd * Cd + c;
+    if (a.vec_out && c + 8 <= Cd) {
       *reinterpret_cast<uint4*>(q) = make_uint4(w[0], w[1], w[2], w[3]);
     } else {
       union { uint32_t raw[4]; T e[8]; } u;
@@ -110,60 +139,69 @@ __global__ __launch_bounds__(256) void nchw_to_nhwc_kernel(const T* __restrict__
       for (int e = 0; e < 4; ++e) u.raw[e] = w[e];
 #pragma unroll
       for (int e = 0; e < 8; ++e)
-        if (c + e < C) q[e] = u.e[e];
+        if (c + e < Cd) q[e] = u.e[e];
     }
   }
 }
 
-// W[O][Cg][KH][KW] -> wt[rows][taps * cols]:
+// Clears `count16` 16-byte units (a kernel, not a memset: the calls may be captured in a HIP graph).
+__global__ __launch_bounds__(256) void conv_clear_kernel(uint4* __restrict__ dst, int64_t count16) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count16; i += stride)
+    dst[i] = make_uint4(0, 0, 0, 0);
+}
+
+// W[O][Cg][KH][KW] -> wt[rows][taps * colsp]; the columns of a tap are padded with zeros from
+// cols to colsp (the contraction channels per group as the products see them):
 //   forward  (flip = 0): wt[o][tap][c]              = W[o][c][tap]               (rows O,  cols Cg)
 //   dX       (flip = 1): wt[g*Cg + c][tap'][o in g] = W[g*Og + o][c][taps-1-tap'] (rows C, cols Og)
 template <typename T>
 __global__ void conv_weight_taps_kernel(const T* __restrict__ w, T* __restrict__ wt, int O, int Cg, int Og,
-                                        int taps, int flip, int64_t total) {
+                                        int taps, int flip, int colsp, int64_t total) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= total) return;
+  const int col = (int)(i % colsp);
+  const int tap = (int)((i / colsp) % taps);
+  const int row = (int)(i / ((int64_t)colsp * taps));
+  T v = from_f32<T>(0.f);
   if (!flip) {
-    const int c = (int)(i % Cg);
-    const int tap = (int)((i / Cg) % taps);
-    const int o = (int)(i / ((int64_t)Cg * taps));
-    wt[i] = w[((int64_t)o * Cg + c) * taps + tap];
-  } else {
-    const int ol = (int)(i % Og);
-    const int tap = (int)((i / Og) % taps);
-    const int row = (int)(i / ((int64_t)Og * taps));   // g * Cg + c
-    const int g = row / Cg, c = row - g * Cg;
-    wt[i] = w[(((int64_t)g * Og + ol) * Cg + c) * taps + (taps - 1 - tap)];
+    if (col < Cg) v = w[((int64_t)row * Cg + col) * taps + tap];
+  } else if (col < Og) {
+    const int g = row / Cg, c = row - g * Cg;   // row = g * Cg + c
+    v = w[(((int64_t)g * Og + col) * Cg + c) * taps + (taps - 1 - tap)];
   }
+  wt[i] = v;
 }
 
 // W[O][Cg][KH][KW] -> fragment-major copy of wt (as defined above) for the kernel that reads the
 // weights straight into registers: the 64 lanes x 16 bytes of one operand fragment (32 rows x 16 k)
 // are contiguous, ordered [group][row tile of 32][k / 16][lane]; rows past Og are zeros.
 // k = tap * Cg + c for the forward product (flip = 0); for the input gradient (flip = 1) the roles
-// of the channel counts are swapped and the taps mirrored.  Cg = contraction channels per group (a
-// multiple of 8), Og = rows per group.
+// of the channel counts are swapped and the taps mirrored.  Cg = contraction channels per group,
+// Cgp = the same padded to what the products contract over (a multiple of 16; channels from Cg on
+// are zeros), Og = rows per group.
 template <typename T>
-__global__ void conv_weight_frags_direct_kernel(const T* __restrict__ w, T* __restrict__ wf, int Cg, int Og, int taps,
-                                                int flip, int ntiles, int64_t total_chunks) {
+__global__ void conv_weight_frags_direct_kernel(const T* __restrict__ w, T* __restrict__ wf, int Cg, int Cgp, int Og,
+                                                int taps, int flip, int ntiles, int64_t total_chunks) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= total_chunks) return;
   const int lane = (int)(i & 63);
   const int64_t frag = i >> 6;
-  const int ksteps = taps * Cg / 16;
+  const int ksteps = taps * Cgp / 16;
   const int kstep = (int)(frag % ksteps);
   const int tile = (int)((frag / ksteps) % ntiles);
   const int grp = (int)(frag / ((int64_t)ksteps * ntiles));
   const int co = tile * 32 + (lane & 31);
   const int k0 = kstep * 16 + (lane >> 5) * 8;
-  const int tap = k0 / Cg, c = k0 - tap * Cg;
+  const int tap = k0 / Cgp, c = k0 - tap * Cgp;
   union { uint4 raw; T e[8]; } u;
   u.raw = make_uint4(0, 0, 0, 0);
   if (co < Og) {
 #pragma unroll
     for (int e = 0; e < 8; ++e)
-      u.e[e] = flip ? w[(((int64_t)grp * Cg + c + e) * Og + co) * taps + (taps - 1 - tap)]
-                    : w[(((int64_t)grp * Og + co) * Cg + c + e) * taps + tap];
+      if (c + e < Cg)
+        u.e[e] = flip ? w[(((int64_t)grp * Cg + c + e) * Og + co) * taps + (taps - 1 - tap)]
+                      : w[(((int64_t)grp * Og + co) * Cg + c + e) * taps + tap];
   }
   reinterpret_cast<uint4*>(wf)[i] = u.raw;
 }
@@ -903,25 +941,53 @@ inline bool sizes_ok(const ConvProblem& p) {
          p.N <= 65535;
 }
 
-int to_nhwc(const void* src, void* dst, int64_t N, int64_t C, int64_t HW, int dt, hipStream_t stream) {
-  const int vec_in = (HW % 8 == 0) && aligned16(src);
-  const int vec_out = (C % 8 == 0) && aligned16(dst);
-  const dim3 grid((unsigned)cdiv64(HW, 64), (unsigned)cdiv64(C, 64), (unsigned)N);
+inline int64_t pad64(int64_t v) { return (v + 63) / 64 * 64; }
+
+// Contraction channels per group: the products take whole 64-channel tiles, so other counts are
+// padded with zero channels in the channels-last copy and in the reordered weights.  From 16
+// channels on (at most four times the arithmetic) that still beats the kernels that gather.
+inline bool contract_ok(int64_t per_group) { return per_group % 64 == 0 || per_group >= 16; }
+
+// [N][C][H*W] -> [N][Hd*Wd][groups * Cgp]: channels of every group padded from C / groups to Cgp,
+// pixel (h, w) at (h * sh, w * sw) of an image of Hd x Wd = ((H-1) sh + 1) x ((W-1) sw + 1).
+int to_nhwc_ex(const void* src, void* dst, int64_t N, int64_t C, int64_t H, int64_t W, int64_t groups, int64_t Cgp,
+               int64_t sh, int64_t sw, int dt, hipStream_t stream) {
+  const int64_t Cg = C / groups, HW = H * W;
+  const bool padded = Cgp != Cg;
+  const int64_t Cd = padded ? groups * Cgp : C;
+  const int64_t Hd = (H - 1) * sh + 1, Wd = (W - 1) * sw + 1;
+  LayoutCopyArgs a{};
+  a.C = (int)C; a.HW = (int)HW; a.Cg = (int)Cg; a.Cgp = (int)Cgp;
+  a.W = (int)W; a.Wd = (int)Wd; a.sh = (int)sh; a.sw = (int)sw; a.HWd = (int)(Hd * Wd);
+  a.vec_in = (HW % 8 == 0) && aligned16(src);
+  a.vec_out = (Cd % 8 == 0) && aligned16(dst);
+  const dim3 grid((unsigned)cdiv64(HW, 64), (unsigned)(padded ? groups * (Cgp / 64) : cdiv64(C, 64)), (unsigned)N);
+  if (sh * sw > 1) {   // the pixels in between stay zero
+    const int64_t count16 = cdiv64(N * Hd * Wd * Cd * 2, 16);
+    int64_t blocks = cdiv64(count16, 256 * 4);
+    if (blocks > 65535) blocks = 65535;
+    hipLaunchKernelGGL(conv_clear_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (uint4*)dst, count16);
+  }
   return dispatch16(dt, [&](auto* tp) -> int {
     typedef std::remove_pointer_t<decltype(tp)> T;
-    hipLaunchKernelGGL((nchw_to_nhwc_kernel<T>), grid, dim3(256), 0, stream, (const T*)src, (T*)dst, (int)C,
-                       (int)HW, vec_in, vec_out);
+    hipLaunchKernelGGL((nchw_to_nhwc_kernel<T>), grid, dim3(256), 0, stream, (const T*)src, (T*)dst, a);
     return launch_status();
   });
 }
 
-int weight_taps(const void* w, void* wt, const ConvProblem& p, int flip, hipStream_t stream) {
-  const int64_t total = p.O * (p.C / p.groups) * p.KH * p.KW;
+int to_nhwc(const void* src, void* dst, int64_t N, int64_t C, int64_t HW, int dt, hipStream_t stream) {
+  return to_nhwc_ex(src, dst, N, C, 1, HW, 1, C, 1, 1, dt, stream);
+}
+
+// colsp: contraction channels per group as padded for the product
+int weight_taps(const void* w, void* wt, const ConvProblem& p, int flip, int64_t colsp, hipStream_t stream) {
+  const int64_t rows = flip ? p.C : p.O;
+  const int64_t total = rows * p.KH * p.KW * colsp;
   return dispatch16(p.dtype, [&](auto* tp) -> int {
     typedef std::remove_pointer_t<decltype(tp)> T;
     hipLaunchKernelGGL((conv_weight_taps_kernel<T>), dim3((unsigned)cdiv64(total, 256)), dim3(256), 0, stream,
                        (const T*)w, (T*)wt, (int)p.O, (int)(p.C / p.groups), (int)(p.O / p.groups),
-                       (int)(p.KH * p.KW), flip, total);
+                       (int)(p.KH * p.KW), flip, (int)colsp, total);
     return launch_status();
   });
 }
@@ -956,8 +1022,9 @@ int64_t halo_rows_needed(const IgemmArgs& g, int64_t n_img, int64_t OH, int KH) 
 }
 
 // One product out[(n,oh,ow), co] over channels-last `act`; see IgemmArgs for the meaning of the fields.
-int run_igemm(IgemmArgs g, const void* w, const ConvProblem& p, int flip, int64_t n_img, int64_t OH, int groups,
-              int dt, hipStream_t stream) {
+// cg_real: contraction channels per group in the weight tensor (g.Cg is that count padded to 64s).
+int run_igemm(IgemmArgs g, const void* w, const ConvProblem& p, int flip, int cg_real, int64_t n_img, int64_t OH,
+              int groups, int dt, hipStream_t stream) {
   g.OHW = (int)(OH * g.OW);
   g.M = (int)(n_img * g.OHW);
   g.K = g.KT * 64;
@@ -976,10 +1043,11 @@ int run_igemm(IgemmArgs g, const void* w, const ConvProblem& p, int flip, int64_
       const int ntiles = (g.Og + 31) / 32;
       const int64_t chunks = (int64_t)groups * ntiles * (g.K / 16) * 64;
       hipLaunchKernelGGL((conv_weight_frags_direct_kernel<T>), dim3((unsigned)cdiv64(chunks, 256)), dim3(256), 0,
-                         stream, (const T*)w, (T*)g.wf, g.Cg, g.Og, (int)(p.KH * p.KW), flip, ntiles, chunks);
+                         stream, (const T*)w, (T*)g.wf, cg_real, g.Cg, g.Og, (int)(p.KH * p.KW), flip, ntiles,
+                         chunks);
       hipLaunchKernelGGL((conv_igemm_halo_kernel<T>), grid, dim3(256), 0, stream, g);
     } else {
-      const int rc = weight_taps(w, const_cast<void*>(g.wt), p, flip, stream);
+      const int rc = weight_taps(w, const_cast<void*>(g.wt), p, flip, g.Cg, stream);
       if (rc) return rc;
       hipLaunchKernelGGL((conv_igemm_kernel<T>), grid, dim3(256), 0, stream, g);
     }
@@ -996,13 +1064,31 @@ inline int64_t frag_weight_bytes(int64_t groups, int64_t out_per_group, int64_t 
 }
 }  // namespace
 
+namespace {
+// sizes of the channels-last copies the products read
+inline int64_t fwd_act_bytes(const ConvProblem& p) { return p.N * p.H * p.W * p.groups * pad64(p.C / p.groups) * 2; }
+inline int64_t dx_rows(const ConvProblem& p) { return (p.OH - 1) * p.sh + 1; }
+inline int64_t dx_cols(const ConvProblem& p) { return (p.OW - 1) * p.sw + 1; }
+inline int64_t dx_act_bytes(const ConvProblem& p) {
+  return p.N * dx_rows(p) * dx_cols(p) * p.groups * pad64(p.O / p.groups) * 2;
+}
+}  // namespace
+
 bool conv_igemm_supports_fwd(const ConvProblem& p) {
-  return is16(p.dtype) && (p.C / p.groups) % 64 == 0 && sizes_ok(p) && p.N * p.OH * p.OW < kMaxBytes;
+  return is16(p.dtype) && contract_ok(p.C / p.groups) && sizes_ok(p) && fwd_act_bytes(p) < kMaxBytes &&
+         p.O * pad64(p.C / p.groups) * p.KH * p.KW * 2 < kMaxBytes && p.N * p.OH * p.OW < kMaxBytes;
 }
 
+// The input gradient of a strided layer is the stride-1 product over the output gradient spread
+// out by the strides (zeros in between): sh * sw times the arithmetic, so strides up to 2 x 2.
 bool conv_igemm_supports_dx(const ConvProblem& p) {
-  return is16(p.dtype) && (p.O / p.groups) % 64 == 0 && sizes_ok(p) && p.sh == 1 && p.sw == 1 &&
-         p.ph <= p.KH - 1 && p.pw <= p.KW - 1 && p.N * p.H * p.W < kMaxBytes;
+  return is16(p.dtype) && contract_ok(p.O / p.groups) && sizes_ok(p) && p.sh * p.sw <= 4 &&
+         p.ph <= p.KH - 1 && p.pw <= p.KW - 1 && dx_act_bytes(p) < kMaxBytes &&
+         p.C * pad64(p.O / p.groups) * p.KH * p.KW * 2 < kMaxBytes && p.N * p.H * p.W < kMaxBytes;
+}
+
+bool conv_igemm_fwd_leaves_nhwc(const ConvProblem& p) {
+  return conv_igemm_supports_fwd(p) && (p.C / p.groups) % 64 == 0;
 }
 
 bool conv_igemm_supports_dw(const ConvProblem& p) {
@@ -1012,14 +1098,16 @@ bool conv_igemm_supports_dw(const ConvProblem& p) {
 
 int64_t conv_igemm_fwd_workspace(const ConvProblem& p) {
   if (!conv_igemm_supports_fwd(p)) return 0;
-  return round256(p.N * p.C * p.H * p.W * 2) + round256(p.O * (p.C / p.groups) * p.KH * p.KW * 2) +
-         round256(frag_weight_bytes(p.groups, p.O / p.groups, (p.C / p.groups) * p.KH * p.KW));
+  const int64_t cgp = pad64(p.C / p.groups);
+  return round256(fwd_act_bytes(p)) + round256(p.O * cgp * p.KH * p.KW * 2) +
+         round256(frag_weight_bytes(p.groups, p.O / p.groups, cgp * p.KH * p.KW));
 }
 
 int64_t conv_igemm_dx_workspace(const ConvProblem& p) {
   if (!conv_igemm_supports_dx(p)) return 0;
-  return round256(p.N * p.O * p.OH * p.OW * 2) + round256(p.O * (p.C / p.groups) * p.KH * p.KW * 2) +
-         round256(frag_weight_bytes(p.groups, p.C / p.groups, (p.O / p.groups) * p.KH * p.KW));
+  const int64_t ogp = pad64(p.O / p.groups);
+  return round256(dx_act_bytes(p)) + round256(p.C * ogp * p.KH * p.KW * 2) +
+         round256(frag_weight_bytes(p.groups, p.C / p.groups, ogp * p.KH * p.KW));
 }
 
 namespace {
@@ -1044,19 +1132,20 @@ int64_t conv_igemm_dw_workspace(const ConvProblem& p) {
 int conv_igemm_fwd(const ConvProblem& p, const void* x, const void* w, const void* bias, int bias_dt,
                    void* y, void* workspace, hipStream_t stream) {
   char* ws = static_cast<char*>(workspace);
+  const int64_t cg = p.C / p.groups, cgp = pad64(cg);
   void* xh = ws;
-  void* wt = ws + round256(p.N * p.C * p.H * p.W * 2);
-  int rc = to_nhwc(x, xh, p.N, p.C, p.H * p.W, p.dtype, stream);
+  void* wt = ws + round256(fwd_act_bytes(p));
+  int rc = to_nhwc_ex(x, xh, p.N, p.C, p.H, p.W, p.groups, cgp, 1, 1, p.dtype, stream);
   if (rc) return rc;
   IgemmArgs g{};
   g.act = xh; g.wt = wt; g.out = y; g.bias = bias; g.bias_dt = bias_dt;
-  g.wf = static_cast<char*>(wt) + round256(p.O * (p.C / p.groups) * p.KH * p.KW * 2);
-  g.IH = (int)p.H; g.IW = (int)p.W; g.Ctot = (int)p.C; g.Cg = (int)(p.C / p.groups); g.Og = (int)(p.O / p.groups);
+  g.wf = static_cast<char*>(wt) + round256(p.O * cgp * p.KH * p.KW * 2);
+  g.IH = (int)p.H; g.IW = (int)p.W; g.Ctot = (int)(p.groups * cgp); g.Cg = (int)cgp; g.Og = (int)(p.O / p.groups);
   g.KW = (int)p.KW; g.OW = (int)p.OW; g.sh = (int)p.sh; g.sw = (int)p.sw; g.ph = (int)p.ph; g.pw = (int)p.pw;
   g.KT = (int)(p.KH * p.KW * (g.Cg / 64));
-  g.act_bytes = p.N * p.C * p.H * p.W * 2;
-  g.wt_bytes = p.O * g.Cg * p.KH * p.KW * 2;
-  return run_igemm(g, w, p, 0, p.N, p.OH, (int)p.groups, p.dtype, stream);
+  g.act_bytes = fwd_act_bytes(p);
+  g.wt_bytes = p.O * cgp * p.KH * p.KW * 2;
+  return run_igemm(g, w, p, 0, (int)cg, p.N, p.OH, (int)p.groups, p.dtype, stream);
 }
 
 int conv_nchw_to_nhwc(const void* src, void* dst, int64_t N, int64_t C, int64_t HW, int dtype,
@@ -1069,24 +1158,27 @@ int conv_nchw_to_nhwc(const void* src, void* dst, int64_t N, int64_t C, int64_t 
 int conv_igemm_dx(const ConvProblem& p, const void* dy, const void* dy_nhwc, const void* w, void* dx,
                   void* workspace, hipStream_t stream) {
   char* ws = static_cast<char*>(workspace);
-  const void* dyh = dy_nhwc;
-  void* wt = ws + round256(p.N * p.O * p.OH * p.OW * 2);
+  const int64_t og = p.O / p.groups, ogp = pad64(og);
+  // the caller's channels-last copy serves only when the product reads dY as it is
+  const void* dyh = (ogp == og && p.sh == 1 && p.sw == 1) ? dy_nhwc : nullptr;
+  void* wt = ws + round256(dx_act_bytes(p));
   int rc = AT_OK;
   if (!dyh) {
-    rc = to_nhwc(dy, ws, p.N, p.O, p.OH * p.OW, p.dtype, stream);
+    rc = to_nhwc_ex(dy, ws, p.N, p.O, p.OH, p.OW, p.groups, ogp, p.sh, p.sw, p.dtype, stream);
     dyh = ws;
   }
   if (rc) return rc;
   // dX[n, c, ih, iw] = sum_{taps', o} dY[n, ih + kh' - (KH-1-ph), iw + kw' - (KW-1-pw), o] * W[o, c, mirrored tap]
   IgemmArgs g{};
   g.act = dyh; g.wt = wt; g.out = dx; g.bias = nullptr; g.bias_dt = 0;
-  g.wf = static_cast<char*>(wt) + round256(p.O * (p.C / p.groups) * p.KH * p.KW * 2);
-  g.IH = (int)p.OH; g.IW = (int)p.OW; g.Ctot = (int)p.O; g.Cg = (int)(p.O / p.groups); g.Og = (int)(p.C / p.groups);
+  g.wf = static_cast<char*>(wt) + round256(p.C * ogp * p.KH * p.KW * 2);
+  g.IH = (int)dx_rows(p); g.IW = (int)dx_cols(p); g.Ctot = (int)(p.groups * ogp); g.Cg = (int)ogp;
+  g.Og = (int)(p.C / p.groups);
   g.KW = (int)p.KW; g.OW = (int)p.W; g.sh = 1; g.sw = 1; g.ph = (int)(p.KH - 1 - p.ph); g.pw = (int)(p.KW - 1 - p.pw);
   g.KT = (int)(p.KH * p.KW * (g.Cg / 64));
-  g.act_bytes = p.N * p.O * p.OH * p.OW * 2;
-  g.wt_bytes = p.O * (p.C / p.groups) * p.KH * p.KW * 2;
-  return run_igemm(g, w, p, 1, p.N, p.H, (int)p.groups, p.dtype, stream);
+  g.act_bytes = dx_act_bytes(p);
+  g.wt_bytes = p.C * ogp * p.KH * p.KW * 2;
+  return run_igemm(g, w, p, 1, (int)og, p.N, p.H, (int)p.groups, p.dtype, stream);
 }
 
 int conv_igemm_dw(const ConvProblem& p, const void* dy, const void* dy_nhwc, const void* x, const void* x_nhwc,

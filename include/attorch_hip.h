@@ -402,13 +402,18 @@ int at_batch_norm_bwd(const void* output_grad, const void* pre_act, const void* 
  * [out_feat, in_feat / groups, kernel_height, kernel_width], output
  * [batch, out_feat, out_height, out_width] with out = (in + 2*padding - kernel) / stride + 1
  * (conv_layer.py:18-36), which the call checks.  bias nullable.
- *   Workspace: 16-bit tensors with channel counts per group in multiples of 64 run on the
- *   matrix cores from channels-last copies kept in caller-provided workspace; each
+ *   Workspace: 16-bit tensors run on the matrix cores from channels-last copies kept in
+ *   caller-provided workspace when the contraction channels per group (input channels for
+ *   forward, output channels for bwd_input) are a multiple of 64 or at least 16 (the copy is
+ *   then padded with zero channels to the next multiple), for bwd_input with
+ *   stride_height * stride_width <= 4 (the gradient is spread out by the strides first) and for
+ *   bwd_weight with channel counts per group in multiples of 8; each
  *   at_conv2d_*_workspace_bytes(...) returns the bytes that path wants for the given shape
  *   (0: no such path).  forward and bwd_input fall back to the generic kernel when the
  *   workspace is null or smaller; bwd_weight always needs its workspace (split-K partials).
  *   Channels-last copies can be shared between calls: at_conv2d_fwd leaves the copy of the
- *   input ([batch, height, width, feat]) at the start of its workspace, at_nchw_to_nhwc makes
+ *   input ([batch, height, width, feat]) at the start of its workspace when
+ *   at_conv2d_fwd_leaves_nhwc(...) returns 1 (no channel padding was needed), at_nchw_to_nhwc makes
  *   one of any 16-bit NCHW tensor, and the backward entry points take such copies through
  *   their nullable *_nhwc arguments instead of making their own (matrix-core path only).
  *   at_channel_sum: out[feat] = sum over batch and space of a [batch, feat, spatial] tensor.
@@ -420,6 +425,12 @@ int64_t at_conv2d_fwd_workspace_bytes(int64_t batch, int64_t in_feat, int64_t in
                                       int64_t stride_width, int64_t padding_height,
                                       int64_t padding_width, int64_t groups, int in_dtype,
                                       int out_dtype);
+
+int at_conv2d_fwd_leaves_nhwc(int64_t batch, int64_t in_feat, int64_t in_height, int64_t in_width,
+                              int64_t out_feat, int64_t out_height, int64_t out_width,
+                              int64_t kernel_height, int64_t kernel_width, int64_t stride_height,
+                              int64_t stride_width, int64_t padding_height,
+                              int64_t padding_width, int64_t groups, int in_dtype, int out_dtype);
 
 int at_conv2d_fwd(const void* input, const void* weight, const void* bias, void* output,
                   void* workspace, int64_t workspace_bytes, int64_t batch, int64_t in_feat,

@@ -31,6 +31,14 @@ CONV_CASES = [
     ((2, 128, 9, 8), 64, (1, 1), (1, 1), (0, 0), 1),
     ((1, 64, 12, 10), 64, (5, 3), (1, 1), (2, 0), 1),
     ((5, 64, 20, 24), 64, (3, 3), (1, 1), (1, 1), 1),
+    # contraction channels per group that are not multiples of 64 (padded with zero channels in the
+    # channels-last copy) and strided layers, whose input gradient runs over the spread-out gradient
+    ((2, 32, 14, 14), 64, (3, 3), (1, 1), (1, 1), 1),
+    ((2, 96, 9, 11), 80, (3, 3), (1, 1), (1, 1), 1),
+    ((2, 96, 12, 12), 96, (3, 3), (2, 2), (1, 1), 2),
+    ((3, 64, 15, 17), 128, (3, 3), (2, 2), (1, 1), 1),
+    ((2, 128, 10, 10), 64, (1, 1), (2, 2), (0, 0), 1),
+    ((2, 16, 8, 9), 16, (3, 3), (1, 2), (1, 1), 1),
     # thin groups take the direct kernels: depthwise with a channel multiplier and more taps than
     # one accumulation pass holds, a pooling-shaped depthwise layer, a three-channel stem (input
     # gradient only), and few output channels without groups
@@ -334,3 +342,27 @@ def test_batch_norm_modules_train_then_eval(track_running_stats) -> None:
     ours1d = attorch_amd.BatchNorm1d(12)
     torch.testing.assert_close(ours1d(x.flatten(2)), torch.nn.BatchNorm1d(12, device='cuda')(x.flatten(2)),
                                rtol=1e-4, atol=1e-5)
+
+
+def test_matrix_core_path_covers_padded_channels_and_strided_input_gradients() -> None:
+    # which shapes get the 16-bit matrix-core path (a non-zero workspace request is how it shows)
+    from attorch_amd import _lib
+    lib = _lib.load()
+    bf16 = _lib.dtype_id(torch.bfloat16)
+
+    def dims(shape, out_dim, kernel, stride, padding, groups):
+        n, c, h, w = shape
+        oh = (h + 2 * padding[0] - kernel[0]) // stride[0] + 1
+        ow = (w + 2 * padding[1] - kernel[1]) // stride[1] + 1
+        return (n, c, h, w, out_dim, oh, ow, *kernel, *stride, *padding, groups)
+
+    for case in (((2, 32, 14, 14), 64, (3, 3), (1, 1), (1, 1), 1), ((2, 96, 12, 12), 96, (3, 3), (2, 2), (1, 1), 2),
+                 ((3, 64, 15, 17), 128, (3, 3), (2, 2), (1, 1), 1), ((2, 16, 8, 9), 16, (3, 3), (1, 2), (1, 1), 1)):
+        d = dims(*case)
+        assert lib.at_conv2d_fwd_workspace_bytes(*d, bf16, bf16) > 0, case
+        assert lib.at_conv2d_bwd_input_workspace_bytes(*d, bf16) > 0, case
+    # fewer than 16 contraction channels per group, or strides beyond 2 x 2, stay on the other kernels
+    d = dims((2, 8, 8, 8), 64, (3, 3), (1, 1), (1, 1), 1)
+    assert lib.at_conv2d_fwd_workspace_bytes(*d, bf16, bf16) == 0
+    d = dims((2, 64, 16, 16), 64, (3, 3), (3, 2), (1, 1), 1)
+    assert lib.at_conv2d_bwd_input_workspace_bytes(*d, bf16) == 0

@@ -90,14 +90,24 @@ def test_argument_errors_without_gpu() -> None:
     # inconsistent convolution geometry
     dims = [1, 4, 8, 8, 4, 9, 9, 3, 3, 1, 1, 1, 1, 1]
     assert lib.at_conv2d_fwd(p, p, None, p, None, 0, *dims, 0, 0, 0, None) == -2
-    # workspace queries: the matrix-core convolution path wants 16-bit tensors and channel
-    # counts per group in multiples of 64; anything else asks for no forward workspace
+    # workspace queries: the matrix-core convolution path wants 16-bit tensors and at least 16
+    # contraction channels per group (padded to multiples of 64 in its channels-last copy);
+    # anything else asks for no forward workspace
     good = [2, 64, 8, 8, 128, 8, 8, 3, 3, 1, 1, 1, 1, 1]
     assert lib.at_conv2d_fwd_workspace_bytes(*good, 2, 2) >= 2 * 64 * 8 * 8 * 2 + 128 * 64 * 9 * 2
     assert lib.at_conv2d_fwd_workspace_bytes(*good, 0, 0) == 0
     assert lib.at_conv2d_fwd_workspace_bytes(*dims, 2, 2) == 0
+    assert lib.at_conv2d_fwd_leaves_nhwc(*good, 2, 2) == 1
+    thin = list(good); thin[1] = 32                       # 32 input channels: copy padded to 64, not reusable
+    assert lib.at_conv2d_fwd_workspace_bytes(*thin, 2, 2) >= 2 * 64 * 8 * 8 * 2 + 128 * 64 * 9 * 2
+    assert lib.at_conv2d_fwd_leaves_nhwc(*thin, 2, 2) == 0
+    thin[1] = 8
+    assert lib.at_conv2d_fwd_workspace_bytes(*thin, 2, 2) == 0
     assert lib.at_conv2d_bwd_input_workspace_bytes(*good, 1) > 0
+    # strided input gradient: the output gradient is spread over (OH-1)*2+1 = 7 rows and columns
     strided = list(good); strided[5] = strided[6] = 4; strided[9] = strided[10] = 2
+    assert lib.at_conv2d_bwd_input_workspace_bytes(*strided, 1) >= 2 * 7 * 7 * 128 * 2 + 64 * 128 * 9 * 2
+    strided[5] = strided[6] = 3; strided[9] = strided[10] = 3   # 3 x 3 strides: nine times the arithmetic, no
     assert lib.at_conv2d_bwd_input_workspace_bytes(*strided, 1) == 0
     assert lib.at_conv2d_bwd_weight_workspace_bytes(*good, 0) > 0
     # weight gradient of the linear layer: slices of the batch only for 16-bit tensors, a long
