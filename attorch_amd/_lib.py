@@ -58,6 +58,10 @@ PROTOTYPES = {
     'at_batch_norm_fwd': (I, [P, P, P, P, P, P, P, P, P, P, P, L, L, L, L, F, F, I, F, I, I, I, I, I, P]),
     'at_conv2d_fwd_workspace_bytes': (L, [L] * 14 + [I, I]),
     'at_conv2d_fwd_leaves_nhwc': (I, [L] * 14 + [I, I]),
+    'at_conv2d_nhwc_workspace_bytes': (L, [I] + [L] * 14 + [I]),
+    'at_conv2d_fwd_nhwc': (I, [P, P, P, P, P, L] + [L] * 14 + [I, I, P]),
+    'at_conv2d_bwd_input_nhwc': (I, [P, P, P, P, L] + [L] * 14 + [I, P]),
+    'at_conv2d_bwd_weight_nhwc': (I, [P, P, P, P, L] + [L] * 14 + [I, P]),
     'at_conv2d_fwd': (I, [P, P, P, P, P, L] + [L] * 14 + [I, I, I, P]),
     'at_conv2d_bwd_input_workspace_bytes': (L, [L] * 14 + [I]),
     'at_conv2d_bwd_input': (I, [P, P, P, P, P, L] + [L] * 14 + [I, P]),

@@ -102,16 +102,43 @@ class Conv2dAutoGrad(torch.autograd.Function):
         output_dtype = get_output_dtype(input.dtype, autocast='fp16')
         # Under autocast the operands are rounded to the low-precision dtype first
         # (conv_kernels.py:191-193).
-        input_k = input.to(output_dtype).contiguous()
         weight_k = weight.to(output_dtype).contiguous()
         bias_k = None if bias is None else bias.to(output_dtype).contiguous()
-        output = torch.empty((batch_dim, out_feat_dim, out_height, out_width),
-                             device=input.device, dtype=output_dtype)
         dims = (batch_dim, in_feat_dim, in_height, in_width, out_feat_dim, out_height, out_width,
                 kernel_height, kernel_width, stride_height, stride_width,
                 padding_height, padding_width, groups)
 
         dtype = _lib.dtype_id(output_dtype)
+        requires_grad = (input.requires_grad or
+                         weight.requires_grad or
+                         (bias is not None and bias.requires_grad))
+        ctx.dims = dims
+        ctx.bias_requires_grad = False if bias is None else bias.requires_grad
+        ctx.output_dtype = output_dtype
+        ctx.input_nhwc = None
+
+        # Tensors that are channels-last in memory (torch.channels_last) are what the matrix-core
+        # kernels read and write: no layout copies, and the output is channels-last too.
+        ctx.channels_last = (input.dtype is output_dtype and not input.is_contiguous()
+                             and input.is_contiguous(memory_format=torch.channels_last)
+                             and lib.at_conv2d_nhwc_workspace_bytes(0, *dims, dtype) > 0)
+        if ctx.channels_last:
+            output = torch.empty((batch_dim, out_feat_dim, out_height, out_width), device=input.device,
+                                 dtype=output_dtype, memory_format=torch.channels_last)
+            with torch.cuda.device_of(input):
+                workspace, workspace_bytes = _workspace(
+                    lib.at_conv2d_nhwc_workspace_bytes(0, *dims, dtype), input.device)
+                _lib.check(lib.at_conv2d_fwd_nhwc(
+                    _lib.ptr(input), _lib.ptr(weight_k), _lib.ptr(bias_k), _lib.ptr(output),
+                    _lib.ptr(workspace), workspace_bytes, *dims, dtype, dtype,
+                    _lib.stream_of(input)), 'at_conv2d_fwd_nhwc')
+            if requires_grad:
+                ctx.save_for_backward(input, weight)
+            return output
+
+        input_k = input.to(output_dtype).contiguous()
+        output = torch.empty((batch_dim, out_feat_dim, out_height, out_width),
+                             device=input.device, dtype=output_dtype)
         with torch.cuda.device_of(input):
             workspace, workspace_bytes = _workspace(
                 lib.at_conv2d_fwd_workspace_bytes(*dims, dtype, dtype), input.device)
@@ -120,12 +147,6 @@ class Conv2dAutoGrad(torch.autograd.Function):
                 _lib.ptr(workspace), workspace_bytes, *dims, dtype, dtype, dtype,
                 _lib.stream_of(input)), 'at_conv2d_fwd')
 
-        requires_grad = (input.requires_grad or
-                         weight.requires_grad or
-                         (bias is not None and bias.requires_grad))
-        ctx.dims = dims
-        ctx.bias_requires_grad = False if bias is None else bias.requires_grad
-        ctx.output_dtype = output_dtype
         # The matrix-core path leaves a channels-last copy of the input at the start of its
         # workspace (unless it had to pad the channels); the weight gradient reuses it instead of
         # transposing the input again.
@@ -154,6 +175,76 @@ class Conv2dAutoGrad(torch.autograd.Function):
         dims = ctx.dims
         (batch_dim, in_feat_dim, _, _, out_feat_dim, out_height, out_width,
          kernel_height, kernel_width, _, _, _, _, groups) = dims
+        stream = _lib.stream_of(input)
+        dtype = _lib.dtype_id(output_dtype)
+
+        input_grad = weight_grad = bias_grad = None
+        if ctx.channels_last:
+            # channels-last gradients in and out; a product this path does not cover is left to
+            # the channels-first code below
+            grad_last = output_grad.to(output_dtype).contiguous(memory_format=torch.channels_last)
+            need_input = input.requires_grad
+            need_weight = weight.requires_grad
+            with torch.cuda.device_of(input):
+                n_bytes = lib.at_conv2d_nhwc_workspace_bytes(1, *dims, dtype) if need_input else 0
+                if n_bytes > 0:
+                    weight_k = weight.to(output_dtype).contiguous()
+                    input_grad = torch.empty(input.shape, dtype=output_dtype, device=device,
+                                             memory_format=torch.channels_last)
+                    workspace, workspace_bytes = _workspace(n_bytes, device)
+                    _lib.check(lib.at_conv2d_bwd_input_nhwc(
+                        _lib.ptr(grad_last), _lib.ptr(weight_k), _lib.ptr(input_grad),
+                        _lib.ptr(workspace), workspace_bytes, *dims, dtype, stream),
+                        'at_conv2d_bwd_input_nhwc')
+                    need_input = False
+                n_bytes = lib.at_conv2d_nhwc_workspace_bytes(2, *dims, dtype) if need_weight else 0
+                if n_bytes > 0:
+                    weight_grad = torch.empty(weight.shape, dtype=output_dtype, device=device)
+                    workspace, workspace_bytes = _workspace(n_bytes, device)
+                    _lib.check(lib.at_conv2d_bwd_weight_nhwc(
+                        _lib.ptr(grad_last), _lib.ptr(input), _lib.ptr(weight_grad),
+                        _lib.ptr(workspace), workspace_bytes, *dims, dtype, stream),
+                        'at_conv2d_bwd_weight_nhwc')
+                    need_weight = False
+                if ctx.bias_requires_grad:
+                    # the bias gradient: column sums of the [batch * height * width, out_feat] matrix
+                    rows = batch_dim * out_height * out_width
+                    bias_grad = torch.empty(out_feat_dim, dtype=output_dtype, device=device)
+                    workspace, workspace_bytes = _workspace(
+                        lib.at_colsum_workspace_bytes(rows, out_feat_dim), device)
+                    _lib.check(lib.at_colsum(
+                        _lib.ptr(grad_last), _lib.ptr(bias_grad), _lib.ptr(workspace), workspace_bytes,
+                        rows, out_feat_dim, out_feat_dim, dtype, dtype, stream), 'at_colsum')
+            if not (need_input or need_weight):
+                return input_grad, weight_grad, bias_grad, None, None, None, None, None
+            rest = Conv2dAutoGrad._backward_channels_first(
+                ctx, input, weight, output_grad, need_input, need_weight, False)
+            return (input_grad if input_grad is not None else rest[0],
+                    weight_grad if weight_grad is not None else rest[1], bias_grad,
+                    None, None, None, None, None)
+        return Conv2dAutoGrad._backward_channels_first(
+            ctx, input, weight, output_grad, input.requires_grad, weight.requires_grad,
+            ctx.bias_requires_grad)
+
+    @staticmethod
+    def _backward_channels_first(
+        ctx: Any,
+        input: Tensor,
+        weight: Tensor,
+        output_grad: Tensor,
+        need_input: bool,
+        need_weight: bool,
+        need_bias: bool,
+        ) -> Tuple[Optional[Tensor], ...]:
+        """
+        The three gradients from contiguous [batch, feat, height, width] tensors.
+        """
+        lib = _lib.load()
+        output_dtype = ctx.output_dtype
+        device = input.device
+        dims = ctx.dims
+        (batch_dim, in_feat_dim, _, _, out_feat_dim, out_height, out_width,
+         kernel_height, kernel_width, _, _, _, _, groups) = dims
         output_grad = output_grad.to(output_dtype).contiguous()
         stream = _lib.stream_of(input)
         dtype = _lib.dtype_id(output_dtype)
@@ -161,15 +252,15 @@ class Conv2dAutoGrad(torch.autograd.Function):
         input_grad = weight_grad = bias_grad = None
         with torch.cuda.device_of(input):
             input_workspace_bytes = (lib.at_conv2d_bwd_input_workspace_bytes(*dims, dtype)
-                                     if input.requires_grad else 0)
+                                     if need_input else 0)
             # one channels-last copy of the output gradient serves both products
             output_grad_nhwc = None
-            if input_workspace_bytes > 0 and weight.requires_grad:
+            if input_workspace_bytes > 0 and need_weight:
                 output_grad_nhwc = torch.empty_like(output_grad)
                 _lib.check(lib.at_nchw_to_nhwc(
                     _lib.ptr(output_grad), _lib.ptr(output_grad_nhwc), batch_dim, out_feat_dim,
                     out_height * out_width, dtype, stream), 'at_nchw_to_nhwc')
-            if input.requires_grad:
+            if need_input:
                 weight_k = weight.to(output_dtype).contiguous()
                 input_grad = torch.empty(input.shape, dtype=output_dtype, device=device)
                 workspace, workspace_bytes = _workspace(input_workspace_bytes, device)
@@ -177,7 +268,7 @@ class Conv2dAutoGrad(torch.autograd.Function):
                     _lib.ptr(output_grad), _lib.ptr(output_grad_nhwc), _lib.ptr(weight_k),
                     _lib.ptr(input_grad), _lib.ptr(workspace), workspace_bytes, *dims, dtype,
                     stream), 'at_conv2d_bwd_input')
-            if weight.requires_grad:
+            if need_weight:
                 input_k = input.to(output_dtype).contiguous()
                 weight_grad = torch.empty(weight.shape, dtype=output_dtype, device=device)
                 workspace, workspace_bytes = _workspace(
@@ -187,7 +278,7 @@ class Conv2dAutoGrad(torch.autograd.Function):
                     _lib.ptr(ctx.input_nhwc), _lib.ptr(weight_grad),
                     _lib.ptr(workspace), workspace_bytes, *dims, dtype, stream),
                     'at_conv2d_bwd_weight')
-            if ctx.bias_requires_grad:
+            if need_bias:
                 bias_grad = torch.empty(out_feat_dim, dtype=output_dtype, device=device)
                 _lib.check(lib.at_channel_sum(
                     _lib.ptr(output_grad), _lib.ptr(bias_grad), batch_dim, out_feat_dim,

@@ -691,6 +691,75 @@ int at_conv2d_bwd_weight(const void* output_grad, const void* output_grad_nhwc, 
   });
 }
 
+// ---- channels-last tensors ([batch, height, width, feat]) in and out, 16-bit matrix-core path only ----
+int64_t at_conv2d_nhwc_workspace_bytes(int pass, int64_t batch, int64_t in_feat, int64_t in_height, int64_t in_width, int64_t out_feat,
+    int64_t out_height, int64_t out_width, int64_t kernel_height, int64_t kernel_width, int64_t stride_height,
+    int64_t stride_width, int64_t padding_height, int64_t padding_width, int64_t groups, int dtype) {
+  const ConvShape s = shape_of(batch, in_feat, in_height, in_width, out_feat, out_height, out_width, kernel_height,
+                               kernel_width, stride_height, stride_width, padding_height, padding_width, groups);
+  if (check_shape(s)) return 0;
+  const ConvProblem p = problem_of(s, dtype);
+  if (pass == 0) return conv_igemm_fwd_last_workspace(p);
+  if (pass == 1) return conv_igemm_dx_last_workspace(p);
+  if (pass == 2) return conv_igemm_dw_workspace(p);
+  return 0;
+}
+
+int at_conv2d_fwd_nhwc(const void* input, const void* weight, const void* bias, void* output, void* workspace,
+                       int64_t workspace_bytes, int64_t batch, int64_t in_feat, int64_t in_height, int64_t in_width, int64_t out_feat,
+    int64_t out_height, int64_t out_width, int64_t kernel_height, int64_t kernel_width, int64_t stride_height,
+    int64_t stride_width, int64_t padding_height, int64_t padding_width, int64_t groups, int dtype, int bias_dtype, at_stream_t stream) {
+  if (!input || !weight || !output) return AT_ERR_NULL;
+  if (!dtype_valid(dtype) || (bias && !dtype_valid(bias_dtype))) return AT_ERR_DTYPE;
+  const ConvShape s = shape_of(batch, in_feat, in_height, in_width, out_feat, out_height, out_width, kernel_height,
+                               kernel_width, stride_height, stride_width, padding_height, padding_width, groups);
+  int rc = check_shape(s);
+  if (rc) return rc;
+  const ConvProblem p = problem_of(s, dtype);
+  const int64_t need = conv_igemm_fwd_last_workspace(p);
+  if (need <= 0) return AT_ERR_UNSUPPORTED;
+  if (!workspace || workspace_bytes < need) return AT_ERR_WORKSPACE;
+  if (!aligned16(workspace) || !aligned16(input) || !aligned16(output)) return AT_ERR_ALIGN;
+  return conv_igemm_fwd_last(p, input, weight, bias, bias_dtype, output, workspace, (hipStream_t)stream);
+}
+
+int at_conv2d_bwd_input_nhwc(const void* output_grad, const void* weight, void* input_grad, void* workspace,
+                             int64_t workspace_bytes, int64_t batch, int64_t in_feat, int64_t in_height, int64_t in_width, int64_t out_feat,
+    int64_t out_height, int64_t out_width, int64_t kernel_height, int64_t kernel_width, int64_t stride_height,
+    int64_t stride_width, int64_t padding_height, int64_t padding_width, int64_t groups, int dtype, at_stream_t stream) {
+  if (!output_grad || !weight || !input_grad) return AT_ERR_NULL;
+  if (!dtype_valid(dtype)) return AT_ERR_DTYPE;
+  const ConvShape s = shape_of(batch, in_feat, in_height, in_width, out_feat, out_height, out_width, kernel_height,
+                               kernel_width, stride_height, stride_width, padding_height, padding_width, groups);
+  int rc = check_shape(s);
+  if (rc) return rc;
+  const ConvProblem p = problem_of(s, dtype);
+  const int64_t need = conv_igemm_dx_last_workspace(p);
+  if (need <= 0) return AT_ERR_UNSUPPORTED;
+  if (!workspace || workspace_bytes < need) return AT_ERR_WORKSPACE;
+  if (!aligned16(workspace) || !aligned16(output_grad) || !aligned16(input_grad)) return AT_ERR_ALIGN;
+  return conv_igemm_dx_last(p, output_grad, weight, input_grad, workspace, (hipStream_t)stream);
+}
+
+int at_conv2d_bwd_weight_nhwc(const void* output_grad, const void* input, void* weight_grad, void* workspace,
+                              int64_t workspace_bytes, int64_t batch, int64_t in_feat, int64_t in_height, int64_t in_width, int64_t out_feat,
+    int64_t out_height, int64_t out_width, int64_t kernel_height, int64_t kernel_width, int64_t stride_height,
+    int64_t stride_width, int64_t padding_height, int64_t padding_width, int64_t groups, int dtype, at_stream_t stream) {
+  if (!output_grad || !input || !weight_grad) return AT_ERR_NULL;
+  if (!dtype_valid(dtype)) return AT_ERR_DTYPE;
+  const ConvShape s = shape_of(batch, in_feat, in_height, in_width, out_feat, out_height, out_width, kernel_height,
+                               kernel_width, stride_height, stride_width, padding_height, padding_width, groups);
+  int rc = check_shape(s);
+  if (rc) return rc;
+  const ConvProblem p = problem_of(s, dtype);
+  const int64_t need = conv_igemm_dw_workspace(p);
+  if (need <= 0) return AT_ERR_UNSUPPORTED;
+  if (!workspace || workspace_bytes < need) return AT_ERR_WORKSPACE;
+  if (!aligned16(workspace) || !aligned16(output_grad) || !aligned16(input)) return AT_ERR_ALIGN;
+  // both operands are already channels-last: the channels-first arguments are not read
+  return conv_igemm_dw(p, nullptr, output_grad, nullptr, input, weight_grad, workspace, (hipStream_t)stream);
+}
+
 int at_nchw_to_nhwc(const void* src, void* dst, int64_t batch, int64_t feat, int64_t spatial, int dtype,
                     at_stream_t stream) {
   if (!src || !dst) return AT_ERR_NULL;

@@ -45,6 +45,18 @@ int conv_igemm_dx(const ConvProblem& p, const void* dy, const void* dy_nhwc, con
 // channels-last copies the caller already holds.
 int conv_igemm_dw(const ConvProblem& p, const void* dy, const void* dy_nhwc, const void* x, const void* x_nhwc,
                   void* dw, void* workspace, hipStream_t stream);
+// The same products on channels-last tensors ([N][H][W][C]) in and out: no layout copies, the
+// workspace holds the reordered weights only.  Input channels per group (forward) / output
+// channels per group (input gradient, stride 1 only) in multiples of 64.  The weight gradient of
+// channels-last tensors is conv_igemm_dw with both *_nhwc arguments given.
+bool conv_igemm_supports_fwd_last(const ConvProblem& p);
+bool conv_igemm_supports_dx_last(const ConvProblem& p);
+int64_t conv_igemm_fwd_last_workspace(const ConvProblem& p);
+int64_t conv_igemm_dx_last_workspace(const ConvProblem& p);
+int conv_igemm_fwd_last(const ConvProblem& p, const void* x_last, const void* w, const void* bias, int bias_dt,
+                        void* y_last, void* workspace, hipStream_t stream);
+int conv_igemm_dx_last(const ConvProblem& p, const void* dy_last, const void* w, void* dx_last, void* workspace,
+                       hipStream_t stream);
 // [N][C][HW] -> [N][HW][C] for a 16-bit dtype.
 int conv_nchw_to_nhwc(const void* src, void* dst, int64_t N, int64_t C, int64_t HW, int dtype,
                       hipStream_t stream);

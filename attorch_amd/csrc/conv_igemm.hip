@@ -226,12 +226,110 @@ struct IgemmArgs {
   int KT;             // K / 64
   int tiles_per_tap;  // Cg / 64
   int nbn;            // column tiles per group
-  int vec_store;      // OHW % 8 == 0 and 16-byte aligned output
+  int vec_store;      // 16-byte stores: OHW % 8 == 0 (channels-first) or Og and the channel total % 8 == 0, aligned output
+  int out_last;       // the output is channels-last, [N][OH][OW][groups * Og]
   int64_t act_bytes, wt_bytes;
   FastDiv div_ohw, div_ow;
 };
 
-template <typename T>
+// Epilogue of the forward / input-gradient kernels: the 128 x 64 tile goes through LDS (dead after
+// the main loop; the caller has synchronised) and leaves in 16-byte pieces.
+//   Channels-first output: a lane holds, for tile t and register r, pixel wm*64 + t*32 + (r/4)*8 +
+//   (lane/32)*4 + r%4 of output channel wn*32 + lane%32; the tile is laid down as
+//   [channel][pixel] and leaves as runs of 8 pixels of one channel (NCHW rows).
+//   Channels-last output (MFMA operands the other way round): a lane holds channel wn*32 +
+//   (r/4)*8 + (lane/32)*4 + r%4 of pixel wm*64 + t*32 + lane%32; the tile is laid down as
+//   [pixel][channel] and leaves as 8 channels of one pixel — consecutive pixels are consecutive
+//   rows of groups * Og channels, so no division is needed to place them.
+constexpr int kCEpiPitchLast = CBN * 2 + 16;   // bytes per pixel row of the channels-last epilogue tile
+template <typename T, bool OUT_LAST>
+__device__ __forceinline__ void igemm_epilogue(const f32x16 (&acc)[2], char* lds, const IgemmArgs& g, int grp, int m0,
+                                               int n0, int wm, int wn) {
+  const int lane = threadIdx.x & 63;
+  T* __restrict__ out = reinterpret_cast<T*>(g.out);
+  const int Otot = g.Og * (int)gridDim.z;
+  if (OUT_LAST) {
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {
+      const int ch = wn * 32 + rg * 8 + (lane >> 5) * 4;
+      float bv4[4] = {0.f, 0.f, 0.f, 0.f};
+      if (g.bias) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (n0 + ch + e < g.Og) bv4[e] = load_scalar_f32(g.bias, g.bias_dt, grp * g.Og + n0 + ch + e);
+      }
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = acc[t][rg * 4 + e] + bv4[e];
+        const int pix = wm * 64 + t * 32 + (lane & 31);
+        store_f32<T, 4>(reinterpret_cast<T*>(lds + pix * kCEpiPitchLast) + ch, v);
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int id = threadIdx.x + 256 * s;
+      const int pix = id >> 3, ch = (id & 7) * 8;
+      const int co = n0 + ch, m = m0 + pix;
+      if (co >= g.Og || m >= g.M) continue;
+      const uint4 v = *reinterpret_cast<const uint4*>(lds + pix * kCEpiPitchLast + ch * 2);
+      T* dst = out + (int64_t)m * Otot + grp * g.Og + co;
+      if (g.vec_store) {
+        *reinterpret_cast<uint4*>(dst) = v;
+      } else {
+        union { uint4 raw; T e[8]; } u;
+        u.raw = v;
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (co + e < g.Og) dst[e] = u.e[e];
+      }
+    }
+    return;
+  }
+  const int col = wn * 32 + (lane & 31);
+  float bv = 0.f;
+  if (g.bias && n0 + col < g.Og) bv = load_scalar_f32(g.bias, g.bias_dt, grp * g.Og + n0 + col);
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = acc[t][rg * 4 + e] + bv;
+      const int pix = wm * 64 + t * 32 + rg * 8 + (lane >> 5) * 4;
+      store_f32<T, 4>(reinterpret_cast<T*>(lds + col * kCEpiPitch) + pix, v);
+    }
+  __syncthreads();
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    const int id = threadIdx.x + 256 * s;
+    const int col2 = id >> 4, pc = id & 15;
+    const int co = n0 + col2, m = m0 + pc * 8;
+    if (co >= g.Og || m >= g.M) continue;
+    const uint4 v = *reinterpret_cast<const uint4*>(lds + col2 * kCEpiPitch + pc * 16);
+    if (g.vec_store) {
+      const int n = fast_div(m, g.div_ohw);
+      const int p = m - n * g.OHW;
+      *reinterpret_cast<uint4*>(out + ((int64_t)n * Otot + grp * g.Og + co) * g.OHW + p) = v;
+    } else {
+      union { uint4 raw; T e[8]; } u;
+      u.raw = v;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int mm = m + e;
+        if (mm < g.M) {
+          const int n = fast_div(mm, g.div_ohw);
+          const int p = mm - n * g.OHW;
+          out[((int64_t)n * Otot + grp * g.Og + co) * g.OHW + p] = u.e[e];
+        }
+      }
+    }
+  }
+}
+
+template <typename T, bool OUT_LAST>
 __global__ __launch_bounds__(256) void conv_igemm_kernel(IgemmArgs g) {
   __shared__ __attribute__((aligned(1024))) char lds[2 * kCStage];
   const int grp = blockIdx.z;
@@ -316,59 +414,16 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(IgemmArgs g) {
       const uint4 a0 = read_frag_kc(cur, wm * 64, ks);
       const uint4 a1 = read_frag_kc(cur, wm * 64 + 32, ks);
       const uint4 b = read_frag_kc(cur + kCATile, wn * 32, ks);
-      acc[0] = Mfma16<T>::run(a0, b, acc[0]);
-      acc[1] = Mfma16<T>::run(a1, b, acc[1]);
+      // which operand goes first decides what a lane ends up with: four consecutive pixels of
+      // one channel (channels-first output) or four consecutive channels of one pixel
+      acc[0] = OUT_LAST ? Mfma16<T>::run(b, a0, acc[0]) : Mfma16<T>::run(a0, b, acc[0]);
+      acc[1] = OUT_LAST ? Mfma16<T>::run(b, a1, acc[1]) : Mfma16<T>::run(a1, b, acc[1]);
     }
     lds_dma_wait_all();   // this wave's part of the next stage has landed
     __syncthreads();      // ... and everybody else's; the current stage may be overwritten
   }
 
-  // ---- epilogue: lane holds, for tile t and register r, pixel wm*64 + t*32 + (r/4)*8 +
-  // (lane/32)*4 + r%4 of output channel wn*32 + lane%32; the tile goes through LDS as
-  // [channel][pixel] and leaves as runs of 8 pixels of one channel (NCHW rows) ----
-  T* __restrict__ out = reinterpret_cast<T*>(g.out);
-  {
-    const int col = wn * 32 + (lane & 31);
-    float bv = 0.f;
-    if (g.bias && n0 + col < g.Og) bv = load_scalar_f32(g.bias, g.bias_dt, grp * g.Og + n0 + col);
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        float v[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = acc[t][rg * 4 + e] + bv;
-        const int pix = wm * 64 + t * 32 + rg * 8 + (lane >> 5) * 4;
-        store_f32<T, 4>(reinterpret_cast<T*>(lds + col * kCEpiPitch) + pix, v);
-      }
-  }
-  __syncthreads();
-  const int Otot = g.Og * (int)gridDim.z;
-#pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    const int id = threadIdx.x + 256 * s;
-    const int col = id >> 4, pc = id & 15;
-    const int co = n0 + col, m = m0 + pc * 8;
-    if (co >= g.Og || m >= g.M) continue;
-    const uint4 v = *reinterpret_cast<const uint4*>(lds + col * kCEpiPitch + pc * 16);
-    if (g.vec_store) {
-      const int n = fast_div(m, g.div_ohw);
-      const int p = m - n * g.OHW;
-      *reinterpret_cast<uint4*>(out + ((int64_t)n * Otot + grp * g.Og + co) * g.OHW + p) = v;
-    } else {
-      union { uint4 raw; T e[8]; } u;
-      u.raw = v;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int mm = m + e;
-        if (mm < g.M) {
-          const int n = fast_div(mm, g.div_ohw);
-          const int p = mm - n * g.OHW;
-          out[((int64_t)n * Otot + grp * g.Og + co) * g.OHW + p] = u.e[e];
-        }
-      }
-    }
-  }
+  igemm_epilogue<T, OUT_LAST>(acc, lds, g, grp, m0, n0, wm, wn);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -383,7 +438,7 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(IgemmArgs g) {
 constexpr int kHaloRows = 288;                       // input pixels a tile may span
 constexpr int kHaloBytes = (kHaloRows + 1) * 128;    // + the zero row
 
-template <typename T>
+template <typename T, bool OUT_LAST>
 __global__ __launch_bounds__(256) void conv_igemm_halo_kernel(IgemmArgs g) {
   __shared__ __attribute__((aligned(1024))) char lds[kHaloBytes];
   const int grp = blockIdx.z;
@@ -488,8 +543,8 @@ __global__ __launch_bounds__(256) void conv_igemm_halo_kernel(IgemmArgs g) {
         const int chunk = ks * 2 + (lane >> 5);
         const uint4 a0 = *reinterpret_cast<const uint4*>(lds + rowaddr[0] + ((chunk ^ swz[0]) << 4));
         const uint4 a1 = *reinterpret_cast<const uint4*>(lds + rowaddr[1] + ((chunk ^ swz[1]) << 4));
-        acc[0] = Mfma16<T>::run(a0, bw[ks], acc[0]);
-        acc[1] = Mfma16<T>::run(a1, bw[ks], acc[1]);
+        acc[0] = OUT_LAST ? Mfma16<T>::run(bw[ks], a0, acc[0]) : Mfma16<T>::run(a0, bw[ks], acc[0]);
+        acc[1] = OUT_LAST ? Mfma16<T>::run(bw[ks], a1, acc[1]) : Mfma16<T>::run(a1, bw[ks], acc[1]);
       }
       if (++kw == g.KW) {
         kw = 0;
@@ -508,50 +563,7 @@ __global__ __launch_bounds__(256) void conv_igemm_halo_kernel(IgemmArgs g) {
     }
   }
   __syncthreads();   // the window is dead: LDS becomes the output tile
-
-  T* __restrict__ out = reinterpret_cast<T*>(g.out);
-  {
-    const int col = wn * 32 + (lane & 31);
-    float bv = 0.f;
-    if (g.bias && n0 + col < g.Og) bv = load_scalar_f32(g.bias, g.bias_dt, grp * g.Og + n0 + col);
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        float v[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = acc[t][rg * 4 + e] + bv;
-        const int pix = wm * 64 + t * 32 + rg * 8 + (lane >> 5) * 4;
-        store_f32<T, 4>(reinterpret_cast<T*>(lds + col * kCEpiPitch) + pix, v);
-      }
-  }
-  __syncthreads();
-  const int Otot = g.Og * (int)gridDim.z;
-#pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    const int id = threadIdx.x + 256 * s;
-    const int col = id >> 4, pc = id & 15;
-    const int oc = n0 + col, m = m0 + pc * 8;
-    if (oc >= g.Og || m >= g.M) continue;
-    const uint4 v = *reinterpret_cast<const uint4*>(lds + col * kCEpiPitch + pc * 16);
-    if (g.vec_store) {
-      const int n = fast_div(m, g.div_ohw);
-      const int p = m - n * g.OHW;
-      *reinterpret_cast<uint4*>(out + ((int64_t)n * Otot + grp * g.Og + oc) * g.OHW + p) = v;
-    } else {
-      union { uint4 raw; T e[8]; } u;
-      u.raw = v;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int mm = m + e;
-        if (mm < g.M) {
-          const int n = fast_div(mm, g.div_ohw);
-          const int p = mm - n * g.OHW;
-          out[((int64_t)n * Otot + grp * g.Og + oc) * g.OHW + p] = u.e[e];
-        }
-      }
-    }
-  }
+  igemm_epilogue<T, OUT_LAST>(acc, lds, g, grp, m0, n0, wm, wn);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1030,7 +1042,7 @@ int run_igemm(IgemmArgs g, const void* w, const ConvProblem& p, int flip, int cg
   g.K = g.KT * 64;
   g.tiles_per_tap = g.Cg / 64;
   g.nbn = (int)cdiv64(g.Og, CBN);
-  g.vec_store = (g.OHW % 8 == 0) && aligned16(g.out);
+  g.vec_store = g.out_last ? (g.Og % 8 == 0) && aligned16(g.out) : (g.OHW % 8 == 0) && aligned16(g.out);
   g.div_ohw = make_fastdiv(g.OHW);
   g.div_ow = make_fastdiv(g.OW);
   const dim3 grid((unsigned)(cdiv64(g.M, CBM) * g.nbn), 1, (unsigned)groups);
@@ -1045,11 +1057,13 @@ int run_igemm(IgemmArgs g, const void* w, const ConvProblem& p, int flip, int cg
       hipLaunchKernelGGL((conv_weight_frags_direct_kernel<T>), dim3((unsigned)cdiv64(chunks, 256)), dim3(256), 0,
                          stream, (const T*)w, (T*)g.wf, cg_real, g.Cg, g.Og, (int)(p.KH * p.KW), flip, ntiles,
                          chunks);
-      hipLaunchKernelGGL((conv_igemm_halo_kernel<T>), grid, dim3(256), 0, stream, g);
+      if (g.out_last) hipLaunchKernelGGL((conv_igemm_halo_kernel<T, true>), grid, dim3(256), 0, stream, g);
+      else hipLaunchKernelGGL((conv_igemm_halo_kernel<T, false>), grid, dim3(256), 0, stream, g);
     } else {
       const int rc = weight_taps(w, const_cast<void*>(g.wt), p, flip, g.Cg, stream);
       if (rc) return rc;
-      hipLaunchKernelGGL((conv_igemm_kernel<T>), grid, dim3(256), 0, stream, g);
+      if (g.out_last) hipLaunchKernelGGL((conv_igemm_kernel<T, true>), grid, dim3(256), 0, stream, g);
+      else hipLaunchKernelGGL((conv_igemm_kernel<T, false>), grid, dim3(256), 0, stream, g);
     }
     return launch_status();
   });
@@ -1146,6 +1160,62 @@ int conv_igemm_fwd(const ConvProblem& p, const void* x, const void* w, const voi
   g.act_bytes = fwd_act_bytes(p);
   g.wt_bytes = p.O * cgp * p.KH * p.KW * 2;
   return run_igemm(g, w, p, 0, (int)cg, p.N, p.OH, (int)p.groups, p.dtype, stream);
+}
+
+// ---- channels-last tensors in and out: no copies, the workspace holds the reordered weights only ----
+bool conv_igemm_supports_fwd_last(const ConvProblem& p) {
+  return is16(p.dtype) && (p.C / p.groups) % 64 == 0 && sizes_ok(p) && p.N * p.OH * p.OW < kMaxBytes;
+}
+
+bool conv_igemm_supports_dx_last(const ConvProblem& p) {
+  return is16(p.dtype) && (p.O / p.groups) % 64 == 0 && sizes_ok(p) && p.sh == 1 && p.sw == 1 &&
+         p.ph <= p.KH - 1 && p.pw <= p.KW - 1 && p.N * p.H * p.W < kMaxBytes;
+}
+
+namespace {
+inline int64_t last_weight_workspace(const ConvProblem& p, int64_t rows_per_group, int64_t contract_per_group) {
+  const int64_t taps = p.KH * p.KW;
+  return round256(p.groups * rows_per_group * contract_per_group * taps * 2) +
+         round256(frag_weight_bytes(p.groups, rows_per_group, contract_per_group * taps));
+}
+}  // namespace
+
+int64_t conv_igemm_fwd_last_workspace(const ConvProblem& p) {
+  return conv_igemm_supports_fwd_last(p) ? last_weight_workspace(p, p.O / p.groups, p.C / p.groups) : 0;
+}
+
+int64_t conv_igemm_dx_last_workspace(const ConvProblem& p) {
+  return conv_igemm_supports_dx_last(p) ? last_weight_workspace(p, p.C / p.groups, p.O / p.groups) : 0;
+}
+
+int conv_igemm_fwd_last(const ConvProblem& p, const void* x_last, const void* w, const void* bias, int bias_dt,
+                        void* y_last, void* workspace, hipStream_t stream) {
+  char* wt = static_cast<char*>(workspace);
+  const int64_t cg = p.C / p.groups;
+  IgemmArgs g{};
+  g.act = x_last; g.wt = wt; g.out = y_last; g.bias = bias; g.bias_dt = bias_dt; g.out_last = 1;
+  g.wf = wt + round256(p.O * cg * p.KH * p.KW * 2);
+  g.IH = (int)p.H; g.IW = (int)p.W; g.Ctot = (int)p.C; g.Cg = (int)cg; g.Og = (int)(p.O / p.groups);
+  g.KW = (int)p.KW; g.OW = (int)p.OW; g.sh = (int)p.sh; g.sw = (int)p.sw; g.ph = (int)p.ph; g.pw = (int)p.pw;
+  g.KT = (int)(p.KH * p.KW * (g.Cg / 64));
+  g.act_bytes = p.N * p.C * p.H * p.W * 2;
+  g.wt_bytes = p.O * cg * p.KH * p.KW * 2;
+  return run_igemm(g, w, p, 0, (int)cg, p.N, p.OH, (int)p.groups, p.dtype, stream);
+}
+
+int conv_igemm_dx_last(const ConvProblem& p, const void* dy_last, const void* w, void* dx_last, void* workspace,
+                       hipStream_t stream) {
+  char* wt = static_cast<char*>(workspace);
+  const int64_t og = p.O / p.groups;
+  IgemmArgs g{};
+  g.act = dy_last; g.wt = wt; g.out = dx_last; g.bias = nullptr; g.bias_dt = 0; g.out_last = 1;
+  g.wf = wt + round256(p.C * og * p.KH * p.KW * 2);
+  g.IH = (int)p.OH; g.IW = (int)p.OW; g.Ctot = (int)p.O; g.Cg = (int)og; g.Og = (int)(p.C / p.groups);
+  g.KW = (int)p.KW; g.OW = (int)p.W; g.sh = 1; g.sw = 1; g.ph = (int)(p.KH - 1 - p.ph); g.pw = (int)(p.KW - 1 - p.pw);
+  g.KT = (int)(p.KH * p.KW * (g.Cg / 64));
+  g.act_bytes = p.N * p.O * p.OH * p.OW * 2;
+  g.wt_bytes = p.C * og * p.KH * p.KW * 2;
+  return run_igemm(g, w, p, 1, (int)og, p.N, p.H, (int)p.groups, p.dtype, stream);
 }
 
 int conv_nchw_to_nhwc(const void* src, void* dst, int64_t N, int64_t C, int64_t HW, int dtype,

@@ -50,6 +50,7 @@ MEASURED_TRAFFIC_BYTES = {
     'c3_cross_entropy': 1717917526,   # ce_row_kernel (ignored rows are not read)
     'c3_cross_entropy_autocast': 2450414716,
     'c3_nll_loss': 827000369,         # nll forward (a gather) + the single-pass gradient write
+    'c5_conv_channels_last': None,     # the two window kernels + weight gradient + weight reorders, no copies
     'c5_conv': 687074860,             # 2 window kernels + weight gradient + 2 layout copies + weight reorders
     'c5_batch_norm': 616984920,       # stats + apply + backward reduce + backward apply
 }
@@ -863,6 +864,42 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
                      'frac': bn_gbs / PEAK_HBM_GBS, **traffic_fields('c5_batch_norm')},
         'buffer_rotation': f'{nsets} sets of 6 tensors (49 MiB each)',
     }
+    # The same three products on tensors that are channels-last in memory (torch.channels_last): the
+    # layout the kernels work in, so the two layout copies disappear.
+    last = torch.channels_last
+    xl = [x.contiguous(memory_format=last) for x in xs]
+    dyl = [d.contiguous(memory_format=last) for d in dys]
+    yl = [torch.empty_like(xl[0]) for _ in range(nsets)]
+    dxl = [torch.empty_like(xl[0]) for _ in range(nsets)]
+    lws = [lib.at_conv2d_nhwc_workspace_bytes(k_, *dims, dt) for k_ in range(3)]
+    lwork = torch.empty(max(*lws, 16), dtype=torch.uint8, device='cuda')
+
+    def last_f():
+        i = nxt()
+        raw.check(lib.at_conv2d_fwd_nhwc(xl[i].data_ptr(), wt.data_ptr(), None, yl[i].data_ptr(), lwork.data_ptr(),
+                                         lws[0], *dims, dt, dt, st()), 'conv_fwd_nhwc')
+
+    def last_dx():
+        i = nxt()
+        raw.check(lib.at_conv2d_bwd_input_nhwc(dyl[i].data_ptr(), wt.data_ptr(), dxl[i].data_ptr(), lwork.data_ptr(),
+                                               lws[1], *dims, dt, st()), 'conv_dx_nhwc')
+
+    def last_dw():
+        i = nxt()
+        raw.check(lib.at_conv2d_bwd_weight_nhwc(dyl[i].data_ptr(), xl[i].data_ptr(), dwt.data_ptr(),
+                                                lwork.data_ptr(), lws[2], *dims, dt, st()), 'conv_dw_nhwc')
+    tl = {k_: gpu_time_ms(f, iters, warmup) for k_, f in (('conv_fwd', last_f), ('conv_bwd_input', last_dx),
+                                                         ('conv_bwd_weight', last_dw))}
+    last_ms = sum(tl.values())
+    last_tf = 3 * gflop / last_ms
+    conv_last_entry = {
+        'workload': f'c5 with channels-last tensors: Conv2d 3x3 s1 p1 bf16 fwd+bwd X[{n},{c},{h},{w_}] '
+                    f'W[{c},{c},3,3], memory format torch.channels_last',
+        'metric': 'conv TFLOP/s', 'value': last_tf, 'unit': 'TFLOP/s', 'kernel_ms': tl,
+        'roofline': {'bound': 'mfma', 'achieved': last_tf, 'peak': PEAK_MFMA_16BIT_TFLOPS, 'unit': 'TFLOP/s',
+                     'frac': last_tf / PEAK_MFMA_16BIT_TFLOPS, **traffic_fields('c5_conv_channels_last')},
+    }
+
     # the block end to end through the modules (conv -> bn + residual + relu, fwd + bwd)
     conv = attorch_amd.Conv2d(c, c, 3, padding=1, bias=False, dtype=dtype)
     bn = attorch_amd.BatchNorm2d(c, act_func='relu', dtype=dtype)
@@ -914,6 +951,21 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
     bn_entry['torch_native'] = module_times_ms(lambda i: torch.relu(bn_ref(xins[i]) + rins[i]), ref_bwd, iters,
                                                warmup, nsets)
     conv_entry['torch_native'] = module_times_ms(lambda i: conv_ref(xins[i]), ref_bwd, iters, warmup, nsets)
+    xlins = [x.detach().clone(memory_format=last).requires_grad_(True) for x in xs]
+
+    def last_bwd(out, i):
+        xlins[i].grad = None
+        conv.weight.grad = None
+        out.backward(dyl[i])
+    conv_last_entry['module_level'] = module_times_ms(lambda i: conv(xlins[i]), last_bwd, iters, warmup, nsets)
+    conv_ref_last = conv_ref.to(memory_format=last)
+
+    def ref_last_bwd(out, i):
+        xlins[i].grad = None
+        conv_ref_last.weight.grad = None
+        out.backward(dyl[i])
+    conv_last_entry['torch_native'] = module_times_ms(lambda i: conv_ref_last(xlins[i]), ref_last_bwd, iters, warmup,
+                                                      nsets)
     if with_cpu:
         import oracle
         cn = 8
@@ -952,7 +1004,7 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
             cpu_conv_functional, 3 * gflop * cn / n / 1e3, 'TFLOP/s', f'first {cn} of {n} images', dtype)
         bn_entry['cpu_functional'] = functional_cpu_entry(
             cpu_bn_functional, 8 * tbytes * cn / n / 1e9, 'GB/s', f'first {cn} of {n} images', dtype)
-    return [conv_entry, bn_entry]
+    return [conv_entry, conv_last_entry, bn_entry]
 
 
 def main() -> int:

@@ -472,6 +472,43 @@ int at_conv2d_bwd_weight(const void* output_grad, const void* output_grad_nhwc,
                          int64_t stride_height, int64_t stride_width, int64_t padding_height,
                          int64_t padding_width, int64_t groups, int dtype, at_stream_t stream);
 
+/* The same three products for tensors that are channels-last in memory ([batch, height, width,
+ * feat], what torch.channels_last gives a [batch, feat, height, width] tensor) — the layout the
+ * matrix-core kernels work in, so nothing is copied: input and output of every call are
+ * channels-last, the weight ([out_feat, in_feat / groups, kh, kw]) and its gradient are not.
+ * The reference's kernels take any strides (attorch/conv_layer.py:102-116 passes them on), so
+ * such tensors are within its interface.  16-bit tensors only; forward needs in_feat / groups,
+ * bwd_input out_feat / groups in multiples of 64 (and stride 1), bwd_weight both in multiples
+ * of 8.  at_conv2d_nhwc_workspace_bytes(pass, ...) (pass 0 forward, 1 bwd_input, 2 bwd_weight)
+ * returns the workspace the call needs, 0 when this path does not cover the shape (the calls
+ * then return AT_ERR_UNSUPPORTED and the caller converts to channels-first). */
+int64_t at_conv2d_nhwc_workspace_bytes(int pass, int64_t batch, int64_t in_feat, int64_t in_height,
+                                       int64_t in_width, int64_t out_feat, int64_t out_height, int64_t out_width,
+                                       int64_t kernel_height, int64_t kernel_width, int64_t stride_height,
+                                       int64_t stride_width, int64_t padding_height, int64_t padding_width,
+                                       int64_t groups, int dtype);
+
+int at_conv2d_fwd_nhwc(const void* input, const void* weight, const void* bias, void* output,
+                       void* workspace, int64_t workspace_bytes, int64_t batch, int64_t in_feat, int64_t in_height,
+                       int64_t in_width, int64_t out_feat, int64_t out_height, int64_t out_width,
+                       int64_t kernel_height, int64_t kernel_width, int64_t stride_height,
+                       int64_t stride_width, int64_t padding_height, int64_t padding_width,
+                       int64_t groups, int dtype, int bias_dtype, at_stream_t stream);
+
+int at_conv2d_bwd_input_nhwc(const void* output_grad, const void* weight, void* input_grad,
+                             void* workspace, int64_t workspace_bytes, int64_t batch, int64_t in_feat, int64_t in_height,
+                             int64_t in_width, int64_t out_feat, int64_t out_height, int64_t out_width,
+                             int64_t kernel_height, int64_t kernel_width, int64_t stride_height,
+                             int64_t stride_width, int64_t padding_height, int64_t padding_width,
+                             int64_t groups, int dtype, at_stream_t stream);
+
+int at_conv2d_bwd_weight_nhwc(const void* output_grad, const void* input, void* weight_grad,
+                              void* workspace, int64_t workspace_bytes, int64_t batch, int64_t in_feat, int64_t in_height,
+                              int64_t in_width, int64_t out_feat, int64_t out_height, int64_t out_width,
+                              int64_t kernel_height, int64_t kernel_width, int64_t stride_height,
+                              int64_t stride_width, int64_t padding_height, int64_t padding_width,
+                              int64_t groups, int dtype, at_stream_t stream);
+
 int at_nchw_to_nhwc(const void* src, void* dst, int64_t batch, int64_t feat, int64_t spatial,
                     int dtype, at_stream_t stream);
 

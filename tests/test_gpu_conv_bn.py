@@ -366,3 +366,62 @@ def test_matrix_core_path_covers_padded_channels_and_strided_input_gradients() -
     assert lib.at_conv2d_fwd_workspace_bytes(*d, bf16, bf16) == 0
     d = dims((2, 64, 16, 16), 64, (3, 3), (3, 2), (1, 1), 1)
     assert lib.at_conv2d_bwd_input_workspace_bytes(*d, bf16) == 0
+
+
+CHANNELS_LAST_CASES = [
+    # shape, out_dim, kernel, stride, padding, groups
+    ((4, 64, 28, 28), 64, (3, 3), (1, 1), (1, 1), 1),      # every product stays channels-last
+    ((3, 64, 7, 9), 96, (3, 3), (1, 1), (1, 1), 1),        # partial tiles; 96 output channels: dX falls back
+    ((2, 128, 10, 12), 128, (3, 3), (2, 2), (1, 1), 2),    # groups, strided: dX falls back
+    ((2, 128, 9, 8), 64, (1, 1), (1, 1), (0, 0), 1),
+    ((1, 64, 12, 10), 64, (5, 3), (1, 1), (2, 0), 1),
+    ((2, 32, 14, 14), 64, (3, 3), (1, 1), (1, 1), 1),      # 32 input channels: the forward product falls back
+]
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('shape, out_dim, kernel, stride, padding, groups', CHANNELS_LAST_CASES)
+@pytest.mark.parametrize('bias', [False, True])
+def test_conv2d_channels_last(shape, out_dim, kernel, stride, padding, groups, bias, dtype) -> None:
+    # tensors in torch.channels_last memory format: same values as the oracle, and the layout is kept
+    fan_in = shape[1] // groups * kernel[0] * kernel[1]
+    x = randn(shape, 1, dtype)
+    w = randn((out_dim, shape[1] // groups, *kernel), 2, dtype, fan_in ** -0.5)
+    b = randn((out_dim,), 3, dtype) if bias else None
+    cd = compute_dtype(dtype)
+    y_ref = oracle.conv2d_forward(x, w, b, stride, padding, groups, dtype, compute=cd)
+    dy = randn(y_ref.shape, 4, dtype)
+    dx_ref, dw_ref, db_ref = oracle.conv2d_backward(dy, x, w, stride, padding, groups, dtype, compute=cd)
+
+    xd = x.cuda().contiguous(memory_format=torch.channels_last).requires_grad_(True)
+    wd = w.cuda().requires_grad_(True)
+    bd = b.cuda().requires_grad_(True) if bias else None
+    y = attorch_amd.Conv2dAutoGrad.apply(xd, wd, bd, *stride, *padding, groups)
+    y.backward(dy.cuda().contiguous(memory_format=torch.channels_last))
+    assert y.dtype is dtype and y.shape == y_ref.shape
+    if shape[1] // groups % 64 == 0:
+        assert y.is_contiguous(memory_format=torch.channels_last)
+    assert_close(y, y_ref, dtype, 'output')
+    assert_close(xd.grad, dx_ref, dtype, 'input_grad')
+    assert_close(wd.grad, dw_ref, dtype, 'weight_grad', batch_reduction=True)
+    if bias:
+        assert_close(bd.grad, db_ref, dtype, 'bias_grad', batch_reduction=True)
+
+
+def test_conv2d_channels_last_matches_channels_first_bitwise() -> None:
+    # the same kernels run on both layouts: identical results for the block of BASELINE config 5
+    dtype = torch.bfloat16
+    x = randn((8, 64, 56, 56), 1, dtype).cuda()
+    w = randn((64, 64, 3, 3), 2, dtype, 576 ** -0.5).cuda()
+    dy = randn((8, 64, 56, 56), 3, dtype).cuda()
+    results = []
+    for fmt in (torch.contiguous_format, torch.channels_last):
+        xd = x.detach().clone(memory_format=fmt).requires_grad_(True)
+        wd = w.clone().requires_grad_(True)
+        y = attorch_amd.Conv2dAutoGrad.apply(xd, wd, None, 1, 1, 1, 1, 1)
+        y.backward(dy.contiguous(memory_format=fmt))
+        results.append((y.detach(), xd.grad, wd.grad))
+    assert results[1][0].is_contiguous(memory_format=torch.channels_last)
+    assert results[1][1].is_contiguous(memory_format=torch.channels_last)
+    for first, last in zip(*results):
+        assert torch.equal(first, last)
