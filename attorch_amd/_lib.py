@@ -56,6 +56,9 @@ PROTOTYPES = {
     'at_colsum': (I, [P, P, P, L, L, L, L, I, I, P]),
     'at_batch_norm_workspace_bytes': (L, [L]),
     'at_batch_norm_fwd': (I, [P, P, P, P, P, P, P, P, P, P, P, L, L, L, L, F, F, I, F, I, I, I, I, I, P]),
+    'at_batch_norm_nhwc_supported': (I, [L, I]),
+    'at_batch_norm_fwd_nhwc': (I, [P, P, P, P, P, P, P, P, P, P, P, L, L, L, L, F, F, I, F, I, I, I, I, I, P]),
+    'at_batch_norm_bwd_nhwc': (I, [P, P, P, P, P, P, P, P, P, P, P, L, L, L, L, I, F, I, I, P]),
     'at_conv2d_fwd_workspace_bytes': (L, [L] * 14 + [I, I]),
     'at_conv2d_fwd_leaves_nhwc': (I, [L] * 14 + [I, I]),
     'at_conv2d_nhwc_workspace_bytes': (L, [I] + [L] * 14 + [I]),

@@ -91,8 +91,18 @@ class BatchNormAutoGrad(torch.autograd.Function):
         save_pre_act = requires_grad and (act_func is not None) and not ctx.output_as_pre_act
 
         batch_dim, feat_dim, spatial_dim = _dims(input)
-        input_k = input.contiguous()
-        residual_k = pre_act_add.to(input.dtype).contiguous() if add_pre_act else None
+        # Channels-last 4D tensors (torch.channels_last) are processed and returned in that layout.
+        layout = torch.contiguous_format
+        if (input.dim() == 4 and not input.is_contiguous()
+                and input.is_contiguous(memory_format=torch.channels_last)
+                and lib.at_batch_norm_nhwc_supported(feat_dim, _lib.dtype_id(input.dtype))):
+            layout = torch.channels_last
+        ctx.layout = layout
+        forward_entry = (lib.at_batch_norm_fwd_nhwc if layout is torch.channels_last
+                         else lib.at_batch_norm_fwd)
+        input_k = input.contiguous(memory_format=layout)
+        residual_k = (pre_act_add.to(input.dtype).contiguous(memory_format=layout)
+                      if add_pre_act else None)
         output = torch.empty_like(input_k)
         pre_act = torch.empty_like(input_k) if save_pre_act else None
         if requires_grad:
@@ -108,7 +118,7 @@ class BatchNormAutoGrad(torch.autograd.Function):
         workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=input.device)
 
         with torch.cuda.device_of(input):
-            _lib.check(lib.at_batch_norm_fwd(
+            _lib.check(forward_entry(
                 _lib.ptr(input_k), _lib.ptr(weight_k), _lib.ptr(bias_k), _lib.ptr(mean),
                 _lib.ptr(inv_std), _lib.ptr(residual_k), _lib.ptr(pre_act), _lib.ptr(output),
                 _lib.ptr(running_mean) if use_running else None,
@@ -143,7 +153,9 @@ class BatchNormAutoGrad(torch.autograd.Function):
         batch_dim, feat_dim, spatial_dim = _dims(input)
         device = input.device
 
-        output_grad_k = output_grad.to(input.dtype).contiguous()
+        output_grad_k = output_grad.to(input.dtype).contiguous(memory_format=ctx.layout)
+        backward_entry = (lib.at_batch_norm_bwd_nhwc if ctx.layout is torch.channels_last
+                          else lib.at_batch_norm_bwd)
         input_grad = torch.empty_like(input)
         pre_act_grad = torch.empty_like(input) if ctx.act_func is not None else None
         if ctx.affine:
@@ -155,7 +167,7 @@ class BatchNormAutoGrad(torch.autograd.Function):
         workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=device)
 
         with torch.cuda.device_of(input):
-            _lib.check(lib.at_batch_norm_bwd(
+            _lib.check(backward_entry(
                 _lib.ptr(output_grad_k), _lib.ptr(pre_act), _lib.ptr(input), _lib.ptr(mean),
                 _lib.ptr(inv_std), _lib.ptr(weight), _lib.ptr(input_grad), _lib.ptr(pre_act_grad),
                 _lib.ptr(weight_grad), _lib.ptr(bias_grad), _lib.ptr(workspace), workspace_bytes,

@@ -426,6 +426,384 @@ inline void apply_grid(int64_t planes, int S, int vec, dim3* grid) {
 
 constexpr int kMaxSplits = 1024;
 
+// ------------------------------------------------------------------------------------------
+// Channels-last tensors: a [rows = N * S][C] matrix, statistics per column.
+// A row is C / VEC 16-byte chunks (at most 256 of them); lane t of a 256-lane workgroup owns chunk
+// t % chunks_per_row of the rows (t / chunks_per_row) + k * rows_per_step it is given, so its VEC
+// channels never change and their parameters live in registers.  Every pass reads whole rows,
+// fully coalesced.  Passes: partial statistics per (row slice, channel) -> one wave per channel
+// merges them (same arithmetic as the channels-first path) and leaves mean / inv_std (forward) or
+// the three coefficients of the input gradient (backward) in the workspace -> elementwise pass.
+// ------------------------------------------------------------------------------------------
+struct LastRows {
+  int64_t rows;
+  int C;
+  int chunks_per_row;   // C / VEC
+  int rows_per_step;    // 256 / chunks_per_row
+  int64_t rows_per_block;
+};
+
+template <int VEC>
+__device__ __forceinline__ bool last_lane(const LastRows& g, int& chunk, int& row_in_step) {
+  chunk = threadIdx.x % g.chunks_per_row;
+  row_in_step = threadIdx.x / g.chunks_per_row;
+  return row_in_step < g.rows_per_step;
+}
+
+// Rows r0 + row_in_step + k * rows_per_step (< r1) of this lane's chunk, U at a time: issue(u, offset)
+// for all of a batch first (rows that do not exist are issued at the batch's first row), then
+// use(u) for those that exist.
+template <int VEC, int U, typename ISSUE, typename USE>
+__device__ __forceinline__ void for_rows_batched(const LastRows& g, int64_t r0, int64_t r1, int chunk,
+                                                 int row_in_step, ISSUE&& issue, USE&& use) {
+  for (int64_t r = r0 + row_in_step; r < r1; r += (int64_t)g.rows_per_step * U) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t ru = r + (int64_t)u * g.rows_per_step;
+      issue(u, (ru < r1 ? ru : r) * g.C + (int64_t)chunk * VEC);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (r + (int64_t)u * g.rows_per_step < r1) use(u);
+  }
+}
+
+// part[(c * P + p) * 3 + {0, 1, 2}] = (count, mean, M2) of channel c over row slice p.
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBnBlock) void bn_last_stats_kernel(const T* __restrict__ x, float* __restrict__ part,
+                                                                LastRows g, int P) {
+  __shared__ float sm[kBnBlock * (2 * VEC + 1)];
+  int chunk, row_in_step;
+  const bool active = last_lane<VEC>(g, chunk, row_in_step);
+  const int p = blockIdx.x;
+  const int64_t r0 = p * g.rows_per_block;
+  const int64_t r1 = r0 + g.rows_per_block < g.rows ? r0 + g.rows_per_block : g.rows;
+  float n = 0.f, mean[VEC], m2[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) mean[j] = m2[j] = 0.f;
+  if (active) {
+    constexpr int U = 8;
+    RawVec<T, VEC> raw[U];
+    for_rows_batched<VEC, U>(
+        g, r0, r1, chunk, row_in_step, [&](int u, int64_t off) { raw[u].load(x + off); },
+        [&](int u) {
+          float v[VEC];
+          raw[u].get(v);
+          n += 1.f;
+          const float inv_n = __fdividef(1.f, n);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) {
+            const float d = v[j] - mean[j];
+            mean[j] += d * inv_n;
+            m2[j] += d * (v[j] - mean[j]);
+          }
+        });
+  }
+  // lanes of one chunk, one per row of a step: merged pairwise through LDS, row r taking in row
+  // r + s for s = the largest power of two below the row count, then half of it, ... (a fixed tree)
+  float* mine = sm + threadIdx.x * (2 * VEC + 1);
+  int s = 1;
+  while (s * 2 < g.rows_per_step) s *= 2;
+  for (; s > 0; s >>= 1) {
+    mine[0] = n;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      mine[1 + j] = mean[j];
+      mine[1 + VEC + j] = m2[j];
+    }
+    __syncthreads();
+    if (active && row_in_step < s && row_in_step + s < g.rows_per_step) {
+      const float* other = sm + ((row_in_step + s) * g.chunks_per_row + chunk) * (2 * VEC + 1);
+      const float nb = other[0];
+      const float nn = n + nb;
+      if (nn > 0.f) {
+        const float f = nb / nn;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float d = other[1 + j] - mean[j];
+          m2[j] += other[1 + VEC + j] + d * d * n * f;
+          mean[j] += d * f;
+        }
+      }
+      n = nn;
+    }
+    __syncthreads();
+  }
+  if (active && row_in_step == 0) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      float* dst = part + ((int64_t)(chunk * VEC + j) * P + p) * 3;
+      dst[0] = n; dst[1] = mean[j]; dst[2] = m2[j];
+    }
+  }
+}
+
+// The per-channel values of a pass, staged once per workgroup: value v of channel c at sm[v * C + c].
+// f(c, out) computes the NV values of channel c.  Returns after a barrier.
+template <int NV, typename F>
+__device__ __forceinline__ void stage_channel_values(float* sm, int C, F&& f) {
+  for (int c = threadIdx.x; c < C; c += kBnBlock) {
+    float out[NV];
+    f(c, out);
+#pragma unroll
+    for (int v = 0; v < NV; ++v) sm[v * C + c] = out[v];
+  }
+  __syncthreads();
+}
+constexpr int kLastMaxC = kBnBlock * 8;   // channels of a row: at most 256 chunks of 8
+
+// One wave per channel: merges the partial statistics (or takes the running ones), leaves
+// stat[c] = mean, stat[C + c] = inv_std in the workspace, writes the optional outputs and
+// updates the running statistics.
+__global__ __launch_bounds__(64) void bn_last_finalize_kernel(
+    const float* __restrict__ part, int P, float* __restrict__ stat, float* __restrict__ mean_out,
+    float* __restrict__ inv_std_out, void* __restrict__ running_mean, void* __restrict__ running_var, int rdt,
+    int update_running, float momentum, float eps, int C) {
+  __shared__ float smem[4];
+  const int c = blockIdx.x;
+  float mean, var, count;
+  channel_stats(part, P, c, running_mean, running_var, rdt, smem, mean, var, count);
+  if (threadIdx.x != 0) return;
+  const float inv_std = rsqrtf(var + eps);
+  stat[c] = mean;
+  stat[C + c] = inv_std;
+  if (mean_out) mean_out[c] = mean;
+  if (inv_std_out) inv_std_out[c] = inv_std;
+  if (update_running) {
+    const float rm = load_scalar_f32(running_mean, rdt, c), rv = load_scalar_f32(running_var, rdt, c);
+    store_scalar_f32(running_mean, rdt, c, (1.f - momentum) * rm + momentum * mean);
+    store_scalar_f32(running_var, rdt, c, (1.f - momentum) * rv + momentum * var * count / (count - 1.f));
+  }
+}
+
+// y = act(w * (x - mean) * inv_std + b (+ residual)), rows in slices of rows_per_block.
+template <typename T, int VEC, int ACT>
+__global__ __launch_bounds__(kBnBlock) void bn_last_apply_kernel(
+    const T* __restrict__ x, const T* __restrict__ res, T* __restrict__ pre_act, T* __restrict__ y,
+    const float* __restrict__ stat, const void* __restrict__ w, const void* __restrict__ b, int wdt, LastRows g,
+    float param) {
+  __shared__ float sm[2 * kLastMaxC];
+  stage_channel_values<2>(sm, g.C, [&](int c, float (&out)[2]) {
+    const float wt = w ? load_scalar_f32(w, wdt, c) : 1.f;
+    const float bs = b ? load_scalar_f32(b, wdt, c) : 0.f;
+    out[0] = wt * stat[g.C + c];
+    out[1] = bs - stat[c] * out[0];
+  });
+  int chunk, row_in_step;
+  if (!last_lane<VEC>(g, chunk, row_in_step)) return;
+  float scale[VEC], shift[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    scale[j] = sm[chunk * VEC + j];
+    shift[j] = sm[g.C + chunk * VEC + j];
+  }
+  const int64_t r0 = blockIdx.x * g.rows_per_block;
+  const int64_t r1 = r0 + g.rows_per_block < g.rows ? r0 + g.rows_per_block : g.rows;
+  constexpr int U = 4;
+  RawVec<T, VEC> xin[U], rin[U];
+  int64_t offs[U];
+  for_rows_batched<VEC, U>(
+      g, r0, r1, chunk, row_in_step,
+      [&](int u, int64_t off) {
+        offs[u] = off;
+        xin[u].load(x + off);
+        if (res) rin[u].load(res + off);   // uniform
+      },
+      [&](int u) {
+        float v[VEC];
+        xin[u].get(v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = fmaf(v[j], scale[j], shift[j]);
+        if (res) {
+          float r[VEC];
+          rin[u].get(r);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) v[j] += r[j];
+        }
+        if (ACT != AT_ACT_NONE) {
+          if (pre_act) store_f32<T, VEC>(pre_act + offs[u], v);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) v[j] = act_forward(ACT, v[j], param);
+        }
+        store_f32<T, VEC>(y + offs[u], v);
+      });
+}
+
+// part[(c * P + p) * 2 + {0, 1}] = (sum g x_hat, sum g) of channel c over row slice p, with
+// g = dy * act'(pre_act), which is also written to g_out when an activation is fused.
+template <typename T, int VEC, int ACT>
+__global__ __launch_bounds__(kBnBlock) void bn_last_bwd_reduce_kernel(
+    const T* __restrict__ dy, const T* __restrict__ pre_act, const T* __restrict__ x, T* __restrict__ g_out,
+    const float* __restrict__ mean_in, const float* __restrict__ inv_std_in, float* __restrict__ part, LastRows g,
+    int P, float param) {
+  __shared__ float sm[kBnBlock * 2 * VEC];
+  int chunk, row_in_step;
+  const bool active = last_lane<VEC>(g, chunk, row_in_step);
+  const int p = blockIdx.x;
+  const int64_t r0 = p * g.rows_per_block;
+  const int64_t r1 = r0 + g.rows_per_block < g.rows ? r0 + g.rows_per_block : g.rows;
+  float s1[VEC], s2[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) s1[j] = s2[j] = 0.f;
+  if (active) {
+    float mean[VEC], inv_std[VEC];
+    if (((reinterpret_cast<uintptr_t>(mean_in) | reinterpret_cast<uintptr_t>(inv_std_in)) & 15) == 0) {
+      load_f32<float, VEC>(mean_in + chunk * VEC, mean);
+      load_f32<float, VEC>(inv_std_in + chunk * VEC, inv_std);
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        mean[j] = mean_in[chunk * VEC + j];
+        inv_std[j] = inv_std_in[chunk * VEC + j];
+      }
+    }
+    constexpr int U = 4;
+    RawVec<T, VEC> rg[U], rx[U], rz[ACT != AT_ACT_NONE ? U : 1];
+    int64_t offs[U];
+    for_rows_batched<VEC, U>(
+        g, r0, r1, chunk, row_in_step,
+        [&](int u, int64_t off) {
+          offs[u] = off;
+          rg[u].load(dy + off);
+          rx[u].load(x + off);
+          if constexpr (ACT != AT_ACT_NONE) rz[u].load(pre_act + off);
+        },
+        [&](int u) {
+          float gv[VEC], xv[VEC];
+          rg[u].get(gv);
+          rx[u].get(xv);
+          if constexpr (ACT != AT_ACT_NONE) {
+            float z[VEC];
+            rz[u].get(z);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) gv[j] *= act_derivative(ACT, z[j], param);
+            store_f32<T, VEC>(g_out + offs[u], gv);
+            // the reference rounds pre_act_grad to the storage dtype before reducing it
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) gv[j] = to_f32(from_f32<T>(gv[j]));
+          }
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) {
+            s1[j] += gv[j] * (xv[j] - mean[j]) * inv_std[j];
+            s2[j] += gv[j];
+          }
+        });
+  }
+  float* mine = sm + threadIdx.x * 2 * VEC;
+  int s = 1;
+  while (s * 2 < g.rows_per_step) s *= 2;
+  for (; s > 0; s >>= 1) {   // the same fixed tree as in the statistics pass
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      mine[j] = s1[j];
+      mine[VEC + j] = s2[j];
+    }
+    __syncthreads();
+    if (active && row_in_step < s && row_in_step + s < g.rows_per_step) {
+      const float* other = sm + ((row_in_step + s) * g.chunks_per_row + chunk) * 2 * VEC;
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        s1[j] += other[j];
+        s2[j] += other[VEC + j];
+      }
+    }
+    __syncthreads();
+  }
+  if (active && row_in_step == 0) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      float* dst = part + ((int64_t)(chunk * VEC + j) * P + p) * 2;
+      dst[0] = s1[j]; dst[1] = s2[j];
+    }
+  }
+}
+
+// One wave per channel: sums the partial pairs, writes the weight and bias gradients and leaves
+// the coefficients of input_grad = a * g - (b1 * (x - mean) + b2) in the workspace:
+// coef[c] = a = inv_std * w, coef[C + c] = b1, coef[2C + c] = b2, coef[3C + c] = mean.
+__global__ __launch_bounds__(64) void bn_last_bwd_finalize_kernel(
+    const float* __restrict__ part, int P, float count, const float* __restrict__ mean_in,
+    const float* __restrict__ inv_std_in, const void* __restrict__ w, int wdt, float* __restrict__ coef,
+    float* __restrict__ weight_grad, float* __restrict__ bias_grad, int C) {
+  const int c = blockIdx.x;
+  float s1 = 0.f, s2 = 0.f;
+  for (int p = threadIdx.x; p < P; p += 64) {
+    s1 += part[((int64_t)c * P + p) * 2];
+    s2 += part[((int64_t)c * P + p) * 2 + 1];
+  }
+  s1 = wave_reduce(s1, 64, SumOp());
+  s2 = wave_reduce(s2, 64, SumOp());
+  if (threadIdx.x != 0) return;
+  if (weight_grad) weight_grad[c] = s1;
+  if (bias_grad) bias_grad[c] = s2;
+  const float inv_std = inv_std_in[c];
+  const float wt = w ? load_scalar_f32(w, wdt, c) : 1.f;
+  const float t1 = s1 * wt / count, t2 = s2 * wt / count;
+  coef[c] = inv_std * wt;
+  coef[C + c] = inv_std * t1 * inv_std;
+  coef[2 * C + c] = inv_std * t2;
+  coef[3 * C + c] = mean_in[c];
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBnBlock) void bn_last_bwd_apply_kernel(const T* __restrict__ gin, const T* __restrict__ x,
+                                                                    T* __restrict__ dx, const float* __restrict__ coef,
+                                                                    LastRows g) {
+  int chunk, row_in_step;
+  if (!last_lane<VEC>(g, chunk, row_in_step)) return;
+  float a[VEC], b1[VEC], b2[VEC], mean[VEC];
+  {
+    // 16-byte loads: the coefficient arrays are laid out by channel and chunk * VEC is a multiple of 4
+    float tmp[4][VEC];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) load_f32<float, VEC>(coef + (int64_t)v * g.C + chunk * VEC, tmp[v]);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) { a[j] = tmp[0][j]; b1[j] = tmp[1][j]; b2[j] = tmp[2][j]; mean[j] = tmp[3][j]; }
+  }
+  const int64_t r0 = blockIdx.x * g.rows_per_block;
+  const int64_t r1 = r0 + g.rows_per_block < g.rows ? r0 + g.rows_per_block : g.rows;
+  constexpr int U = 4;
+  RawVec<T, VEC> rg[U], rx[U];
+  int64_t offs[U];
+  for_rows_batched<VEC, U>(
+      g, r0, r1, chunk, row_in_step,
+      [&](int u, int64_t off) {
+        offs[u] = off;
+        rg[u].load(gin + off);
+        rx[u].load(x + off);
+      },
+      [&](int u) {
+        float gv[VEC], xv[VEC];
+        rg[u].get(gv);
+        rx[u].get(xv);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) gv[j] = a[j] * gv[j] - (b1[j] * (xv[j] - mean[j]) + b2[j]);
+        store_f32<T, VEC>(dx + offs[u], gv);
+      });
+}
+
+// Geometry of the channels-last passes, or false when the layout does not fit them.
+inline bool last_rows(int64_t rows, int64_t feat, int dtype, int64_t chunks_per_block, int64_t max_blocks, LastRows* g,
+                      int* blocks) {
+  const int vec = 16 / dtype_size(dtype);
+  if (feat % vec != 0 || feat / vec > kBnBlock) return false;
+  g->rows = rows;
+  g->C = (int)feat;
+  g->chunks_per_row = (int)(feat / vec);
+  g->rows_per_step = kBnBlock / g->chunks_per_row;
+  // rows per block: whole steps, about chunks_per_block 16-byte chunks per lane
+  int64_t steps = chunks_per_block;
+  int64_t per_block = steps * g->rows_per_step;
+  int64_t nb = cdiv64(rows, per_block);
+  if (nb > max_blocks) {
+    per_block = cdiv64(cdiv64(rows, max_blocks), g->rows_per_step) * g->rows_per_step;
+    nb = cdiv64(rows, per_block);
+  }
+  g->rows_per_block = per_block;
+  *blocks = (int)nb;
+  return true;
+}
+
 }  // namespace
 }  // namespace at_hip
 
@@ -545,6 +923,99 @@ int at_batch_norm_bwd(const void* output_grad, const void* pre_act, const void* 
       hipLaunchKernelGGL((bn_bwd_apply_kernel<T, 1>), grid, dim3(kBnBlock), 0, stream, (const T*)g_for_apply,
                          (const T*)input, (T*)input_grad, mean, inv_std, part, P, count, weight_grad, bias_grad,
                          weight, param_dtype, C, S, planes);
+    return launch_status();
+  });
+}
+
+int at_batch_norm_nhwc_supported(int64_t feat, int dtype) {
+  if (!dtype_valid(dtype) || feat <= 0) return 0;
+  const int vec = 16 / dtype_size(dtype);
+  return feat % vec == 0 && feat / vec <= kBnBlock ? 1 : 0;
+}
+
+int at_batch_norm_fwd_nhwc(const void* input, const void* weight, const void* bias, float* mean, float* inv_std,
+                           const void* pre_act_add, void* pre_act, void* output, void* running_mean,
+                           void* running_var, void* workspace, int64_t workspace_bytes, int64_t batch,
+                           int64_t feat, int64_t spatial, float momentum, float eps, int act, float param,
+                           int track_running_stats, int is_train, int dtype, int param_dtype, int running_dtype,
+                           at_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (!input || !output) return AT_ERR_NULL;
+  if (!dtype_valid(dtype) || ((weight || bias) && !dtype_valid(param_dtype)) ||
+      ((running_mean || running_var) && !dtype_valid(running_dtype)))
+    return AT_ERR_DTYPE;
+  if (!act_valid(act)) return AT_ERR_ACT;
+  if (batch <= 0 || feat <= 0 || spatial <= 0 || feat > INT32_MAX || spatial > INT32_MAX) return AT_ERR_DIM;
+  const bool batch_stats = is_train || !track_running_stats;
+  if (!batch_stats && (!running_mean || !running_var)) return AT_ERR_NULL;
+  if (!workspace || workspace_bytes < at_batch_norm_workspace_bytes(feat)) return AT_ERR_WORKSPACE;
+  if (!at_batch_norm_nhwc_supported(feat, dtype)) return AT_ERR_UNSUPPORTED;
+  if (!aligned16(input) || !aligned16(output) || (pre_act_add && !aligned16(pre_act_add)) ||
+      (pre_act && !aligned16(pre_act)))
+    return AT_ERR_ALIGN;
+  if (!(weight && bias)) weight = bias = nullptr;  // affine only with both (batch_norm_layer.py:116)
+  if (pre_act == output) pre_act = nullptr;
+
+  float* part = (float*)workspace;
+  const int C = (int)feat;
+  float* stat = part + (int64_t)C * kMaxSplits * 3;   // mean[C], inv_std[C]
+  const int64_t rows = batch * spatial;
+  LastRows gs, ga;
+  int P = 0, blocks = 0;
+  if (!last_rows(rows, feat, dtype, 16, 512, &gs, &P) || !last_rows(rows, feat, dtype, 8, 65535, &ga, &blocks))
+    return AT_ERR_UNSUPPORTED;
+  return dispatch_dtype(dtype, [&](auto* tp) -> int {
+    typedef std::remove_pointer_t<decltype(tp)> T;
+    constexpr int VEC = 16 / (int)sizeof(T);
+    if (batch_stats)
+      hipLaunchKernelGGL((bn_last_stats_kernel<T, VEC>), dim3(P), dim3(kBnBlock), 0, stream, (const T*)input, part, gs,
+                         P);
+    const int update = batch_stats && track_running_stats && is_train && running_mean && running_var;
+    hipLaunchKernelGGL(bn_last_finalize_kernel, dim3(C), dim3(64), 0, stream, batch_stats ? part : nullptr, P, stat,
+                       mean, inv_std, running_mean, running_var, running_dtype, update, momentum, eps, C);
+    AT_BN_ACT_SWITCH(act, hipLaunchKernelGGL((bn_last_apply_kernel<T, VEC, ACT>), dim3(blocks), dim3(kBnBlock), 0,
+                                             stream, (const T*)input, (const T*)pre_act_add, (T*)pre_act, (T*)output,
+                                             stat, weight, bias, param_dtype, ga, param));
+    return launch_status();
+  });
+}
+
+int at_batch_norm_bwd_nhwc(const void* output_grad, const void* pre_act, const void* input, const float* mean,
+                           const float* inv_std, const void* weight, void* input_grad, void* pre_act_grad,
+                           float* weight_grad, float* bias_grad, void* workspace, int64_t workspace_bytes,
+                           int64_t batch, int64_t feat, int64_t spatial, int act, float param, int dtype,
+                           int param_dtype, at_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (!output_grad || !input || !mean || !inv_std || !input_grad) return AT_ERR_NULL;
+  if (!dtype_valid(dtype) || (weight && !dtype_valid(param_dtype))) return AT_ERR_DTYPE;
+  if (!act_valid(act)) return AT_ERR_ACT;
+  if (act != AT_ACT_NONE && (!pre_act || !pre_act_grad)) return AT_ERR_NULL;
+  if (batch <= 0 || feat <= 0 || spatial <= 0 || feat > INT32_MAX || spatial > INT32_MAX) return AT_ERR_DIM;
+  if (!workspace || workspace_bytes < at_batch_norm_workspace_bytes(feat)) return AT_ERR_WORKSPACE;
+  if (!at_batch_norm_nhwc_supported(feat, dtype)) return AT_ERR_UNSUPPORTED;
+  if (!aligned16(output_grad) || !aligned16(input) || !aligned16(input_grad) || (pre_act && !aligned16(pre_act)) ||
+      (pre_act_grad && !aligned16(pre_act_grad)))
+    return AT_ERR_ALIGN;
+
+  float* part = (float*)workspace;
+  const int C = (int)feat;
+  float* coef = part + (int64_t)C * kMaxSplits * 3;   // 4 floats per channel
+  const int64_t rows = batch * spatial;
+  LastRows gs, ga;
+  int P = 0, blocks = 0;
+  if (!last_rows(rows, feat, dtype, 16, 512, &gs, &P) || !last_rows(rows, feat, dtype, 8, 65535, &ga, &blocks))
+    return AT_ERR_UNSUPPORTED;
+  const void* g_for_apply = act != AT_ACT_NONE ? pre_act_grad : output_grad;
+  return dispatch_dtype(dtype, [&](auto* tp) -> int {
+    typedef std::remove_pointer_t<decltype(tp)> T;
+    constexpr int VEC = 16 / (int)sizeof(T);
+    AT_BN_ACT_SWITCH(act, hipLaunchKernelGGL((bn_last_bwd_reduce_kernel<T, VEC, ACT>), dim3(P), dim3(kBnBlock), 0,
+                                             stream, (const T*)output_grad, (const T*)pre_act, (const T*)input,
+                                             (T*)pre_act_grad, mean, inv_std, part, gs, P, param));
+    hipLaunchKernelGGL(bn_last_bwd_finalize_kernel, dim3(C), dim3(64), 0, stream, part, P, (float)rows, mean, inv_std,
+                       weight, param_dtype, coef, weight_grad, bias_grad, C);
+    hipLaunchKernelGGL((bn_last_bwd_apply_kernel<T, VEC>), dim3(blocks), dim3(kBnBlock), 0, stream,
+                       (const T*)g_for_apply, (const T*)input, (T*)input_grad, coef, ga);
     return launch_status();
   });
 }

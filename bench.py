@@ -52,6 +52,7 @@ MEASURED_TRAFFIC_BYTES = {
     'c3_nll_loss': 827000369,         # nll forward (a gather) + the single-pass gradient write
     'c5_conv_channels_last': None,     # the two window kernels + weight gradient + weight reorders, no copies
     'c5_conv': 687074860,             # 2 window kernels + weight gradient + 2 layout copies + weight reorders
+    'c5_batch_norm_channels_last': None,
     'c5_batch_norm': 616984920,       # stats + apply + backward reduce + backward apply
 }
 
@@ -900,6 +901,36 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
                      'frac': last_tf / PEAK_MFMA_16BIT_TFLOPS, **traffic_fields('c5_conv_channels_last')},
     }
 
+    # BatchNorm on the same channels-last tensors
+    rl = [r.contiguous(memory_format=last) for r in ress]
+    bn_yl = [torch.empty_like(xl[0]) for _ in range(nsets)]
+    dzl = [torch.empty_like(xl[0]) for _ in range(nsets)]
+
+    def bn_last_f():
+        i = nxt()
+        raw.check(lib.at_batch_norm_fwd_nhwc(xl[i].data_ptr(), bn_w.data_ptr(), bn_b.data_ptr(), mean.data_ptr(),
+                                             rstd.data_ptr(), rl[i].data_ptr(), None, bn_yl[i].data_ptr(),
+                                             rm.data_ptr(), rv.data_ptr(), bn_ws.data_ptr(), bn_wsb, n, c, h * w_,
+                                             0.1, 1e-5, 4, 0.0, 1, 1, dt, dt, 0, st()), 'bn_fwd_nhwc')
+
+    def bn_last_b():
+        i = nxt()
+        raw.check(lib.at_batch_norm_bwd_nhwc(dyl[i].data_ptr(), bn_yl[i].data_ptr(), xl[i].data_ptr(),
+                                             mean.data_ptr(), rstd.data_ptr(), bn_w.data_ptr(), dxl[i].data_ptr(),
+                                             dzl[i].data_ptr(), wg.data_ptr(), bg.data_ptr(), bn_ws.data_ptr(),
+                                             bn_wsb, n, c, h * w_, 4, 0.0, dt, dt, st()), 'bn_bwd_nhwc')
+    for i in range(nsets):
+        counter[0] = i - 1
+        bn_last_f()
+    tbl = {k_: gpu_time_ms(f, iters, warmup) for k_, f in (('bn_fwd', bn_last_f), ('bn_bwd', bn_last_b))}
+    bn_last_gbs = 8 * n * c * h * w_ * 2 / (tbl['bn_fwd'] + tbl['bn_bwd']) / 1e6
+    bn_last_entry = {
+        'workload': f'c5 with channels-last tensors: BatchNorm2d(train)+residual+ReLU bf16 fwd+bwd X[{n},{c},{h},{w_}]',
+        'metric': 'HBM GB/s', 'value': bn_last_gbs, 'unit': 'GB/s', 'ms_fwd': tbl['bn_fwd'], 'ms_bwd': tbl['bn_bwd'],
+        'roofline': {'bound': 'hbm', 'achieved': bn_last_gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                     'frac': bn_last_gbs / PEAK_HBM_GBS, **traffic_fields('c5_batch_norm_channels_last')},
+    }
+
     # the block end to end through the modules (conv -> bn + residual + relu, fwd + bwd)
     conv = attorch_amd.Conv2d(c, c, 3, padding=1, bias=False, dtype=dtype)
     bn = attorch_amd.BatchNorm2d(c, act_func='relu', dtype=dtype)
@@ -917,6 +948,17 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
         bn(conv(xin), rin).backward(dys[0])
 
     conv_entry['block_ms_fwd_bwd_modules'] = wall_time_ms(block, max(3, steps // 4), 2)
+    xin_l = xs[0].detach().clone(memory_format=last).requires_grad_(True)
+    rin_l = ress[0].detach().clone(memory_format=last).requires_grad_(True)
+
+    def block_last():
+        xin_l.grad = None
+        rin_l.grad = None
+        conv.weight.grad = None
+        bn.weight.grad = None
+        bn.bias.grad = None
+        bn(conv(xin_l), rin_l).backward(dyl[0])
+    conv_last_entry['block_ms_fwd_bwd_modules'] = wall_time_ms(block_last, max(3, steps // 4), 2)
 
     # each layer on its own through its module, inputs rotating as above
     xins = [x.clone().requires_grad_(True) for x in xs]
@@ -1004,7 +1046,7 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
             cpu_conv_functional, 3 * gflop * cn / n / 1e3, 'TFLOP/s', f'first {cn} of {n} images', dtype)
         bn_entry['cpu_functional'] = functional_cpu_entry(
             cpu_bn_functional, 8 * tbytes * cn / n / 1e9, 'GB/s', f'first {cn} of {n} images', dtype)
-    return [conv_entry, conv_last_entry, bn_entry]
+    return [conv_entry, conv_last_entry, bn_entry, bn_last_entry]
 
 
 def main() -> int:

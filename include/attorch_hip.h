@@ -393,6 +393,30 @@ int at_batch_norm_bwd(const void* output_grad, const void* pre_act, const void* 
                       int64_t spatial, int act, float param, int dtype, int param_dtype,
                       at_stream_t stream);
 
+/* The same two calls for tensors that are channels-last in memory ([batch, spatial..., feat], a
+ * [batch * spatial, feat] matrix with statistics per column): same arguments, meanings and
+ * workspace.  The reference reads its input through strides (batch_norm_layer.py:130-157), so
+ * such tensors are within its interface.  Covered when feat is a multiple of the 16-byte vector
+ * (8 for 16-bit, 4 for fp32 tensors) of at most 256 vectors — at_batch_norm_nhwc_supported
+ * tells; otherwise the calls return AT_ERR_UNSUPPORTED and the caller converts to
+ * channels-first. */
+int at_batch_norm_nhwc_supported(int64_t feat, int dtype);
+
+int at_batch_norm_fwd_nhwc(const void* input, const void* weight, const void* bias, float* mean,
+                           float* inv_std, const void* pre_act_add, void* pre_act, void* output,
+                           void* running_mean, void* running_var, void* workspace,
+                           int64_t workspace_bytes, int64_t batch, int64_t feat, int64_t spatial,
+                           float momentum, float eps, int act, float param,
+                           int track_running_stats, int is_train, int dtype, int param_dtype,
+                           int running_dtype, at_stream_t stream);
+
+int at_batch_norm_bwd_nhwc(const void* output_grad, const void* pre_act, const void* input,
+                           const float* mean, const float* inv_std, const void* weight,
+                           void* input_grad, void* pre_act_grad, float* weight_grad,
+                           float* bias_grad, void* workspace, int64_t workspace_bytes,
+                           int64_t batch, int64_t feat, int64_t spatial, int act, float param,
+                           int dtype, int param_dtype, at_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * Conv2d (NCHW, zero padding, stride, groups, no dilation) — replaces conv2d_forward_kernel,
  * attorch/conv_kernels.py:68-207 (launched from attorch/conv_layer.py:102-112), the bias add

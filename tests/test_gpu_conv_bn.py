@@ -425,3 +425,78 @@ def test_conv2d_channels_last_matches_channels_first_bitwise() -> None:
     assert results[1][1].is_contiguous(memory_format=torch.channels_last)
     for first, last in zip(*results):
         assert torch.equal(first, last)
+
+
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('shape', [(4, 64, 7, 7), (2, 96, 5, 6), (3, 8, 4, 4), (5, 24, 3, 5), (2, 2048, 2, 3)])
+@pytest.mark.parametrize('affine, residual, act_func', [(True, True, 'relu'), (False, False, None),
+                                                        (True, False, 'silu'), (True, True, 'leaky_relu_0.01')])
+def test_batch_norm_channels_last(shape, dtype, affine, residual, act_func) -> None:
+    # torch.channels_last tensors: a [batch * height * width, feat] matrix with statistics per column
+    feat = shape[1]
+    x = randn(shape, 1, dtype)
+    w = randn((feat,), 2, dtype) if affine else None
+    b = randn((feat,), 3, dtype) if affine else None
+    res = randn(shape, 4, dtype) if residual else None
+    dy = randn(shape, 5, dtype)
+    running_mean = randn((feat,), 6)
+    running_var = randn((feat,), 7).abs() + 0.5
+    cd = compute_dtype(dtype)
+    name, param = oracle.parse_act_func(act_func)
+    y_ref, pre_act_ref, mean, inv_std, rm_ref, rv_ref = oracle.batch_norm_forward(
+        x, True, w, b, running_mean, running_var, 0.2, 1e-5, True, res, name, param, compute=cd)
+
+    last = torch.channels_last
+    xd = x.cuda().contiguous(memory_format=last).requires_grad_(True)
+    wd = w.cuda().requires_grad_(True) if affine else None
+    bd = b.cuda().requires_grad_(True) if affine else None
+    rd = res.cuda().contiguous(memory_format=last).requires_grad_(True) if residual else None
+    rm, rv = running_mean.cuda(), running_var.cuda()
+    y = attorch_amd.BatchNormAutoGrad.apply(xd, True, wd, bd, rm, rv, 0.2, 1e-5, True, rd, act_func)
+    saved = [None if t is None else t.detach().cpu() for t in y.grad_fn.saved_tensors]
+    y.backward(dy.cuda().contiguous(memory_format=last))
+    vec = 4 if dtype is torch.float32 else 8
+    supported = feat % vec == 0 and feat // vec <= 256     # otherwise the layer converts to channels-first
+    if supported:
+        assert y.is_contiguous(memory_format=last) and xd.grad.is_contiguous(memory_format=last)
+    assert_close(y, y_ref, dtype, 'output')
+    assert_close(rm, rm_ref, torch.float32, 'running_mean')
+    assert_close(rv, rv_ref, torch.float32, 'running_var')
+    assert_close(saved[1], mean, torch.float32, 'mean')
+    pre_act = saved[4] if name is not None else None
+    dx_ref, dw_ref, db_ref, dres_ref = oracle.batch_norm_backward(
+        dy, x, saved[1], saved[2], w, affine, pre_act, name, param, compute=cd)
+    assert_close(xd.grad, dx_ref, dtype, 'input_grad')
+    if affine:
+        assert_close(wd.grad, dw_ref.to(dtype), dtype, 'weight_grad', batch_reduction=True)
+        assert_close(bd.grad, db_ref.to(dtype), dtype, 'bias_grad', batch_reduction=True)
+    if residual:
+        assert_close(rd.grad, dres_ref, dtype, 'residual_grad')
+
+
+def test_batch_norm_channels_last_eval_and_block() -> None:
+    # evaluation mode on running statistics, and conv -> batch norm staying channels-last end to end
+    dtype = torch.bfloat16
+    last = torch.channels_last
+    x = randn((4, 64, 14, 14), 1, dtype).cuda()
+    conv = attorch_amd.Conv2d(64, 64, 3, padding=1, bias=False, dtype=dtype)
+    bn = attorch_amd.BatchNorm2d(64, act_func='relu', dtype=dtype)
+    results = []
+    for fmt in (torch.contiguous_format, last):
+        xin = x.detach().clone(memory_format=fmt).requires_grad_(True)
+        bn.train()
+        bn.running_mean.zero_(), bn.running_var.fill_(1.0)
+        out = bn(conv(xin), xin)
+        out.float().square().mean().backward()
+        bn.eval()
+        with torch.no_grad():
+            out_eval = bn(conv(xin), xin)
+        results.append((out.detach(), xin.grad, out_eval, conv.weight.grad.clone(), bn.weight.grad.clone()))
+        conv.weight.grad = None
+        bn.weight.grad = bn.bias.grad = None
+        if fmt is last:
+            assert out.is_contiguous(memory_format=last) and xin.grad.is_contiguous(memory_format=last)
+            assert out_eval.is_contiguous(memory_format=last)
+    names = ('output', 'input_grad', 'eval output', 'conv weight_grad', 'bn weight_grad')
+    for name, first, second in zip(names, *results):
+        assert_close(second, first.cpu(), dtype, name, batch_reduction='weight_grad' in name)
