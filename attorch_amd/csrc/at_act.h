@@ -39,7 +39,13 @@ __device__ __forceinline__ float act_forward(int act, float x, float p) {
     case AT_ACT_RELU: return fmaxf(0.f, x);
     case AT_ACT_GELU: return 0.5f * (1.f + act_erf(0.707106781f * x)) * x;
     // 0.5 * (1 + tanh(u)) = sigmoid(2u)
-    case AT_ACT_GELUAPPROX: return x * act_sigmoid(1.5957691216f * x * (1.f + 0.044715f * x * x));
+    case AT_ACT_GELUAPPROX: {
+      // x * sigmoid(2u) with 2u = 1.5957691216 x (1 + 0.044715 x^2), as x / (1 + 2^(-2u log2 e)):
+      // the constants folded into one polynomial in front of the exponential (5 plain operations
+      // and 2 transcendental ones per element; the epilogue of the large GEMM is bound by them)
+      constexpr float k1 = -1.5957691216f * 1.4426950409f, k3 = k1 * 0.044715f;
+      return x * act_rcp(1.f + __builtin_amdgcn_exp2f(x * fmaf(k3, x * x, k1)));
+    }
     case AT_ACT_SILU: return x * act_sigmoid(x);
     case AT_ACT_RELU6: return fminf(fmaxf(0.f, x), 6.f);
     case AT_ACT_HARDSIGMOID: return fmaxf(0.f, fminf(1.f, x / 6.f + 0.5f));
