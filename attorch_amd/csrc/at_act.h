@@ -76,9 +76,14 @@ __device__ __forceinline__ float act_derivative(int act, float x, float p) {
       return 0.39894228f * __expf(-0.5f * x * x) * x + cdf;
     }
     case AT_ACT_GELUAPPROX: {
-      // with s = sigmoid(2u): 0.5 * (1 + tanh u) = s and 0.5 * (1 - tanh^2 u) = 2 s (1 - s)
-      const float sg = act_sigmoid(1.5957691216f * x * (1.f + 0.044715f * x * x));
-      return sg + x * 2.f * sg * (1.f - sg) * 0.7978845608f * (1.f + 3.f * 0.044715f * x * x);
+      // with s = sigmoid(2u), 2u = 1.5957691216 x (1 + 0.044715 x^2): 0.5 (1 + tanh u) = s and
+      // 0.5 (1 - tanh^2 u) = 2 s (1 - s), so the derivative is s + x s (1 - s) d(2u)/dx with
+      // d(2u)/dx = 1.5957691216 (1 + 3 * 0.044715 x^2); constants folded as in the forward form
+      constexpr float k1 = -1.5957691216f * 1.4426950409f, k3 = k1 * 0.044715f;
+      constexpr float c1 = 1.5957691216f, c3 = 1.5957691216f * 3.f * 0.044715f;
+      const float x2 = x * x;
+      const float sg = act_rcp(1.f + __builtin_amdgcn_exp2f(x * fmaf(k3, x2, k1)));
+      return fmaf(fmaf(-sg, sg, sg), x * fmaf(c3, x2, c1), sg);
     }
     case AT_ACT_SILU: { const float s = act_sigmoid(x); return s * (x * (1.f - s) + 1.f); }
     case AT_ACT_RELU6: return (0.f < x && x < 6.f) ? 1.f : 0.f;
