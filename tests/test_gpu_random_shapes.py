@@ -67,7 +67,10 @@ def _linear_case(rng: random.Random, index: int) -> None:
 def _conv_case(rng: random.Random, index: int) -> None:
     dtype = rng.choice(DTYPES)
     groups = rng.choice([1, 1, 1, 2, 3])
-    in_per_group, out_per_group = rng.choice([1, 3, 8, 64, 72, 128]), rng.choice([1, 2, 24, 32, 64, 96])
+    # odd cases: thin and unaligned channel counts; even cases: counts the matrix-core path pads or takes as they are
+    in_choices, out_choices = (([1, 3, 8, 64, 72, 128], [1, 2, 24, 32, 64, 96]) if index % 2 else
+                               ([16, 32, 48, 64, 96, 128], [16, 32, 64, 80, 128, 192]))
+    in_per_group, out_per_group = rng.choice(in_choices), rng.choice(out_choices)
     kernel = rng.choice([(1, 1), (3, 3), (3, 3), (5, 5), (3, 1), (2, 4), (7, 7)])
     stride = rng.choice([(1, 1), (1, 1), (2, 2), (1, 2)])
     padding = (rng.choice([0, 1, 2, 3]), rng.choice([0, 1, 2, 3]))
@@ -76,18 +79,24 @@ def _conv_case(rng: random.Random, index: int) -> None:
     if height + 2 * padding[0] < kernel[0] or width + 2 * padding[1] < kernel[1]:
         return
     bias = rng.random() < 0.5
+    channels_last = rng.random() < 0.5      # tensors in torch.channels_last memory format
     what = (f'conv case {index}: [{batch}, {in_per_group * groups}, {height}, {width}] -> {out_per_group * groups} '
-            f'k{kernel} s{stride} p{padding} g{groups} {dtype} bias={bias}')
+            f'k{kernel} s{stride} p{padding} g{groups} {dtype} bias={bias} channels_last={channels_last}')
     torch.manual_seed(index)
     layer = attorch_amd.Conv2d(in_per_group * groups, out_per_group * groups, kernel, stride=stride,
                                padding=padding, groups=groups, bias=bias, device='cuda', dtype=dtype)
-    x = torch.randn(batch, in_per_group * groups, height, width, device='cuda', dtype=dtype, requires_grad=True)
-    xr = x.detach().double().requires_grad_(True)
+    x = torch.randn(batch, in_per_group * groups, height, width, device='cuda', dtype=dtype)
+    if channels_last:
+        x = x.contiguous(memory_format=torch.channels_last)
+    x.requires_grad_(True)
+    xr = x.detach().double().contiguous().requires_grad_(True)
     wr = layer.weight.detach().double().requires_grad_(True)
     br = layer.bias.detach().double().requires_grad_(True) if bias else None
     y = layer(x)
     yr = F.conv2d(xr, wr, br, stride, padding, 1, groups)
-    dy = torch.randn_like(y)
+    dy = torch.randn(y.shape, device='cuda', dtype=dtype)
+    if channels_last:
+        dy = dy.contiguous(memory_format=torch.channels_last)
     y.backward(dy)
     yr.backward(dy.double())
     assert_close(y, yr, dtype, what + ' output')
@@ -167,7 +176,7 @@ def test_linear_random_shapes(chunk) -> None:
         _linear_case(rng, index)
 
 
-@pytest.mark.parametrize('chunk', range(3))
+@pytest.mark.parametrize('chunk', range(4))
 def test_conv_random_shapes(chunk) -> None:
     rng = random.Random(2000 + chunk)
     for index in range(chunk * 25, chunk * 25 + 25):
