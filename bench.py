@@ -38,22 +38,22 @@ PEAK_MFMA_FP32_TFLOPS = 157.3    # dense fp32 MFMA
 # the 256 MB Infinity Cache serves are included.  They belong to the kernel sources whose digest is
 # TRAFFIC_SOURCE_DIGEST: when the sources of the loaded library differ, `traffic` is reported as
 # null and the recorded figure moves to `traffic_recorded` (stale until the profile is redone).
-TRAFFIC_SOURCE_DIGEST = '34f927a731c9e228'
+TRAFFIC_SOURCE_DIGEST = 'f20f7a01bc9c05ae'
 MEASURED_TRAFFIC_BYTES = {
-    'c4_linear_fwd': 4297497242,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.0 GiB read, 1.0 GiB written
-    'c2_layer_norm': 362343427,       # norm_fwd + norm_bwd + reduce_partials
-    'c2_rms_norm': 361810204,
-    'c2_softmax': 336099889,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
-    'c2_act_dropout': 336053176,      # act_dropout forward + backward
-    'c2_glu': 269042474,              # glu forward + backward
-    'c2_mse': 335727343,              # p_loss forward + backward
-    'c3_cross_entropy': 1717874654,   # ce_row_kernel (ignored rows are not read)
-    'c3_cross_entropy_autocast': 2450230471,
-    'c3_nll_loss': 827000325,         # nll forward (a gather) + the single-pass gradient write
-    'c5_conv_channels_last': 481286789,     # the two window kernels + weight gradient + weight reorders, no copies
-    'c5_conv': 687132079,             # 2 window kernels + weight gradient + 2 layout copies + weight reorders
-    'c5_batch_norm_channels_last': 568570444,
-    'c5_batch_norm': 565697471,       # stats + apply + backward reduce + backward apply
+    'c4_linear_fwd': 4323178300,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.0 GiB read, 1.0 GiB written
+    'c2_layer_norm': 362342145,       # norm_fwd + norm_bwd + reduce_partials
+    'c2_rms_norm': 361810010,
+    'c2_softmax': 336099504,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
+    'c2_act_dropout': 336029242,      # act_dropout forward + backward
+    'c2_glu': 269052007,              # glu forward + backward
+    'c2_mse': 335726831,              # p_loss forward + backward
+    'c3_cross_entropy': 1717793978,   # ce_row_kernel (ignored rows are not read)
+    'c3_cross_entropy_autocast': 2450222083,
+    'c3_nll_loss': 827001726,         # nll forward (a gather) + the single-pass gradient write
+    'c5_conv_channels_last': 481278590,     # the two window kernels + weight gradient + weight reorders, no copies
+    'c5_conv': 687127779,             # 2 window kernels + weight gradient + 2 layout copies + weight reorders
+    'c5_batch_norm_channels_last': 568579129,
+    'c5_batch_norm': 565707084,       # stats + apply + backward reduce + backward apply
 }
 
 
