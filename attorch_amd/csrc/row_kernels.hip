@@ -683,7 +683,7 @@ __global__ __launch_bounds__(MAXB) void softmax_fwd_kernel(
   // With few enough elements per lane the exponentials of the second sweep (the shifted logits for
   // log-softmax) stay in registers as fp32 and the third sweep is one multiplication per element;
   // otherwise the third sweep computes them again from the cached row.
-  constexpr bool KEEP = ITERS * VEC <= (MAXB <= 256 ? 32 : 16);
+  constexpr bool KEEP = ITERS * VEC <= (MAXB <= 256 ? 64 : 16);
   constexpr float kLog2e = 1.4426950408889634f, kLn2 = 0.6931471805599453f;
   __shared__ float slots[2][16];
   int parity = 0;
