@@ -110,6 +110,28 @@ def test_argument_errors_without_gpu() -> None:
     strided[5] = strided[6] = 3; strided[9] = strided[10] = 3   # 3 x 3 strides: nine times the arithmetic, no
     assert lib.at_conv2d_bwd_input_workspace_bytes(*strided, 1) == 0
     assert lib.at_conv2d_bwd_weight_workspace_bytes(*good, 0) > 0
+    # channels-last entry points: covered shapes ask for a workspace (reordered weights only), others
+    # for none, and the calls say "unsupported" / "workspace" before touching the device
+    assert 0 < lib.at_conv2d_nhwc_workspace_bytes(0, *good, 2) < lib.at_conv2d_fwd_workspace_bytes(*good, 2, 2)
+    assert lib.at_conv2d_nhwc_workspace_bytes(1, *good, 2) > 0
+    assert lib.at_conv2d_nhwc_workspace_bytes(2, *good, 2) > 0
+    assert lib.at_conv2d_nhwc_workspace_bytes(0, *thin[:1], 32, *thin[2:], 2) == 0   # 32 input channels
+    assert lib.at_conv2d_nhwc_workspace_bytes(0, *good, 0) == 0                       # fp32
+    assert lib.at_conv2d_fwd_nhwc(p, p, None, p, None, 0, *good, 2, 0, None) == -5
+    assert lib.at_conv2d_fwd_nhwc(p, p, None, p, p, 1 << 30, *good, 0, 0, None) == -7
+    assert lib.at_conv2d_bwd_input_nhwc(None, p, p, p, 1 << 30, *good, 2, None) == -1
+    assert lib.at_conv2d_bwd_weight_nhwc(p, p, p, None, 0, *good, 2, None) == -5
+    assert lib.at_batch_norm_nhwc_supported(64, 2) == 1 and lib.at_batch_norm_nhwc_supported(1024, 0) == 1
+    assert lib.at_batch_norm_nhwc_supported(7, 2) == 0 and lib.at_batch_norm_nhwc_supported(4096, 2) == 0
+    assert lib.at_batch_norm_fwd_nhwc(p, None, None, None, None, None, None, p, None, None, p, 1 << 30, 4, 7, 9,
+                                      0.1, 1e-5, 0, 0.0, 0, 1, 2, 0, 0, None) == -7
+    assert lib.at_batch_norm_bwd_nhwc(p, None, p, None, p, None, p, None, None, None, p, 1 << 30, 4, 64, 9, 0, 0.0,
+                                      2, 0, None) == -1
+    # one-launch backward of a small fp32 layer: argument errors before anything else
+    assert lib.at_linear_bwd_small(None, p, p, p, p, p, None, 512, 784, 256, 256, 256, 784, 256, 784, 256, 4, 0.0, 0,
+                                   None) == -1
+    assert lib.at_linear_bwd_small(p, None, p, p, p, p, None, 512, 784, 256, 256, 256, 784, 256, 784, 256, 4, 0.0, 0,
+                                   None) == -1     # an activation needs its pre-activation
     # weight gradient of the linear layer: slices of the batch only for 16-bit tensors, a long
     # batch and a weight matrix that is small next to the GPU
     assert lib.at_linear_bwd_weight_workspace_bytes(16384, 256, 256, 2) >= 2 * 256 * 256 * 4
