@@ -259,12 +259,15 @@ __global__ __launch_bounds__(kBigThreads) void gemm_mfma16_kernel(GemmArgs g) {
   const T* __restrict__ A = reinterpret_cast<const T*>(g.a);
   const T* __restrict__ B = reinterpret_cast<const T*>(g.b);
 
-  // ---- workgroup -> output tile, XCD aware ----
+  // ---- workgroup -> output tiles, XCD aware.  The grid may be smaller than the number of tiles
+  // (a multiple of 8 workgroups, so that a workgroup's tiles all carry its XCD number): a
+  // workgroup then takes tiles blockIdx.x, blockIdx.x + gridDim.x, ... one after the other ----
   const int nbm = (g.M + BM - 1) / BM, nbn = (g.N + BN - 1) / BN;
   const int total = nbm * nbn;
+  for (int tile_id = blockIdx.x; tile_id < total; tile_id += gridDim.x) {
   int logical;
   {
-    const int bid = blockIdx.x, xcd = bid & 7, idx = bid >> 3;
+    const int bid = tile_id, xcd = bid & 7, idx = bid >> 3;
     const int q = total >> 3, rem = total & 7;
     logical = xcd * q + (xcd < rem ? xcd : rem) + idx;
   }
@@ -381,6 +384,8 @@ __global__ __launch_bounds__(kBigThreads) void gemm_mfma16_kernel(GemmArgs g) {
   lds_dma_wait_all();   // the zero-fill loads past the end: the epilogue reuses the stages
 
   big_tile_epilogue<T, ACT>(acc, lds, g, m0, n0);
+  __syncthreads();      // the epilogue's readers of LDS are done before the next tile's loads land
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1664,7 +1669,9 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
 
   if (fast) {
     GemmArgs g{a, b, c, pre_act, bias, (int)M, (int)N, (int)K, lda, ldb, ldc, ldp, act, param, bias_dt, nullptr, 0, 0};
-    const unsigned grid = (unsigned)big_tiles;
+    // one workgroup per CU at a time (LDS): a grid of that many walks the tiles itself
+    const int64_t resident = (int64_t)device_cu_count() / 8 * 8;
+    const unsigned grid = (unsigned)(big_tiles > resident && resident > 0 ? resident : big_tiles);
     return dispatch_dtype(in_dt, [&](auto* tp) -> int {
       typedef std::remove_pointer_t<decltype(tp)> T;
       if constexpr (std::is_same<T, float>::value) {
