@@ -242,18 +242,24 @@ struct IgemmArgs {
 //   [pixel][channel] and leaves as 8 channels of one pixel — consecutive pixels are consecutive
 //   rows of groups * Og channels, so no division is needed to place them.
 constexpr int kCEpiPitchLast = CBN * 2 + 16;   // bytes per pixel row of the channels-last epilogue tile
+
+// First half: accumulators (+ bias) into the LDS tile, barrier, and this thread's four 16-byte
+// pieces back into registers.  `bias_tile`, when given, holds the 64 bias values of the tile's
+// channels as floats in LDS (a workgroup that walks over many tiles loads them once).
 template <typename T, bool OUT_LAST>
-__device__ __forceinline__ void igemm_epilogue(const f32x16 (&acc)[2], char* lds, const IgemmArgs& g, int grp, int m0,
-                                               int n0, int wm, int wn) {
-  const int lane = threadIdx.x & 63;
-  T* __restrict__ out = reinterpret_cast<T*>(g.out);
-  const int Otot = g.Og * (int)gridDim.z;
+__device__ __forceinline__ void igemm_epilogue_stage(const f32x16 (&acc)[2], char* lds, const IgemmArgs& g, int grp,
+                                                     int n0, int wm, int wn, int tid, const float* bias_tile,
+                                                     uint4 (&piece)[4]) {
+  const int lane = tid & 63;
   if (OUT_LAST) {
 #pragma unroll
     for (int rg = 0; rg < 4; ++rg) {
       const int ch = wn * 32 + rg * 8 + (lane >> 5) * 4;
       float bv4[4] = {0.f, 0.f, 0.f, 0.f};
-      if (g.bias) {
+      if (bias_tile) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) bv4[e] = bias_tile[ch + e];
+      } else if (g.bias) {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
           if (n0 + ch + e < g.Og) bv4[e] = load_scalar_f32(g.bias, g.bias_dt, grp * g.Og + n0 + ch + e);
@@ -270,27 +276,16 @@ __device__ __forceinline__ void igemm_epilogue(const f32x16 (&acc)[2], char* lds
     __syncthreads();
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      const int id = threadIdx.x + 256 * s;
+      const int id = tid + 256 * s;
       const int pix = id >> 3, ch = (id & 7) * 8;
-      const int co = n0 + ch, m = m0 + pix;
-      if (co >= g.Og || m >= g.M) continue;
-      const uint4 v = *reinterpret_cast<const uint4*>(lds + pix * kCEpiPitchLast + ch * 2);
-      T* dst = out + (int64_t)m * Otot + grp * g.Og + co;
-      if (g.vec_store) {
-        *reinterpret_cast<uint4*>(dst) = v;
-      } else {
-        union { uint4 raw; T e[8]; } u;
-        u.raw = v;
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (co + e < g.Og) dst[e] = u.e[e];
-      }
+      piece[s] = *reinterpret_cast<const uint4*>(lds + pix * kCEpiPitchLast + ch * 2);
     }
     return;
   }
   const int col = wn * 32 + (lane & 31);
   float bv = 0.f;
-  if (g.bias && n0 + col < g.Og) bv = load_scalar_f32(g.bias, g.bias_dt, grp * g.Og + n0 + col);
+  if (bias_tile) bv = bias_tile[col];
+  else if (g.bias && n0 + col < g.Og) bv = load_scalar_f32(g.bias, g.bias_dt, grp * g.Og + n0 + col);
 #pragma unroll
   for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -304,18 +299,51 @@ __device__ __forceinline__ void igemm_epilogue(const f32x16 (&acc)[2], char* lds
   __syncthreads();
 #pragma unroll
   for (int s = 0; s < 4; ++s) {
-    const int id = threadIdx.x + 256 * s;
+    const int id = tid + 256 * s;
+    const int col2 = id >> 4, pc = id & 15;
+    piece[s] = *reinterpret_cast<const uint4*>(lds + col2 * kCEpiPitch + pc * 16);
+  }
+}
+
+// Second half: the four pieces out to memory.
+template <typename T, bool OUT_LAST>
+__device__ __forceinline__ void igemm_epilogue_store(const uint4 (&piece)[4], const IgemmArgs& g, int grp, int m0,
+                                                     int n0, int tid) {
+  T* __restrict__ out = reinterpret_cast<T*>(g.out);
+  const int Otot = g.Og * (int)gridDim.z;
+  if (OUT_LAST) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int id = tid + 256 * s;
+      const int pix = id >> 3, ch = (id & 7) * 8;
+      const int co = n0 + ch, m = m0 + pix;
+      if (co >= g.Og || m >= g.M) continue;
+      T* dst = out + (int64_t)m * Otot + grp * g.Og + co;
+      if (g.vec_store) {
+        *reinterpret_cast<uint4*>(dst) = piece[s];
+      } else {
+        union { uint4 raw; T e[8]; } u;
+        u.raw = piece[s];
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (co + e < g.Og) dst[e] = u.e[e];
+      }
+    }
+    return;
+  }
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    const int id = tid + 256 * s;
     const int col2 = id >> 4, pc = id & 15;
     const int co = n0 + col2, m = m0 + pc * 8;
     if (co >= g.Og || m >= g.M) continue;
-    const uint4 v = *reinterpret_cast<const uint4*>(lds + col2 * kCEpiPitch + pc * 16);
     if (g.vec_store) {
       const int n = fast_div(m, g.div_ohw);
       const int p = m - n * g.OHW;
-      *reinterpret_cast<uint4*>(out + ((int64_t)n * Otot + grp * g.Og + co) * g.OHW + p) = v;
+      *reinterpret_cast<uint4*>(out + ((int64_t)n * Otot + grp * g.Og + co) * g.OHW + p) = piece[s];
     } else {
       union { uint4 raw; T e[8]; } u;
-      u.raw = v;
+      u.raw = piece[s];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int mm = m + e;
@@ -327,6 +355,14 @@ __device__ __forceinline__ void igemm_epilogue(const f32x16 (&acc)[2], char* lds
       }
     }
   }
+}
+
+template <typename T, bool OUT_LAST>
+__device__ __forceinline__ void igemm_epilogue(const f32x16 (&acc)[2], char* lds, const IgemmArgs& g, int grp, int m0,
+                                               int n0, int wm, int wn, int tid) {
+  uint4 piece[4];
+  igemm_epilogue_stage<T, OUT_LAST>(acc, lds, g, grp, n0, wm, wn, tid, nullptr, piece);
+  igemm_epilogue_store<T, OUT_LAST>(piece, g, grp, m0, n0, tid);
 }
 
 template <typename T, bool OUT_LAST>
@@ -423,7 +459,7 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(IgemmArgs g) {
     __syncthreads();      // ... and everybody else's; the current stage may be overwritten
   }
 
-  igemm_epilogue<T, OUT_LAST>(acc, lds, g, grp, m0, n0, wm, wn);
+  igemm_epilogue<T, OUT_LAST>(acc, lds, g, grp, m0, n0, wm, wn, threadIdx.x);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -501,7 +537,10 @@ __global__ __launch_bounds__(256) void conv_igemm_halo_kernel(IgemmArgs g) {
 #pragma unroll
     for (int i = 0; i < kHaloRows / 32; ++i) {
       const int row = (wave + 4 * i) * 8 + (lane >> 3);
-      const int chunk = (lane & 7) ^ (row & 7);   // window rows are read at any offset: swizzle by row % 8 only
+      // A fragment read takes 16 consecutive window rows (128 bytes each) starting anywhere: with
+      // the chunk index XORed with (row / 2) % 8 those rows occupy the 16 different 16-byte
+      // columns of the banks, whatever the first row is.
+      const int chunk = (lane & 7) ^ ((row >> 1) & 7);
       const int off = ((q_lo + row) * g.Ctot + grp * g.Cg + cc * 64 + chunk * 8) * 2;   // negative: out of range
       doff[i] = row < rows ? off : kOobOffset;
     }
@@ -536,7 +575,7 @@ __global__ __launch_bounds__(256) void conv_igemm_halo_kernel(IgemmArgs g) {
         const bool ok = (unsigned)ih < (unsigned)g.IH && (unsigned)iw < (unsigned)g.IW;
         const int row = ok ? f_row[t] + kh * g.IW + kw : kHaloRows;
         rowaddr[t] = row * 128;
-        swz[t] = row & 7;
+        swz[t] = (row >> 1) & 7;
       }
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
@@ -563,7 +602,180 @@ __global__ __launch_bounds__(256) void conv_igemm_halo_kernel(IgemmArgs g) {
     }
   }
   __syncthreads();   // the window is dead: LDS becomes the output tile
-  igemm_epilogue<T, OUT_LAST>(acc, lds, g, grp, m0, n0, wm, wn);
+  igemm_epilogue<T, OUT_LAST>(acc, lds, g, grp, m0, n0, wm, wn, threadIdx.x);
+}
+
+// ------------------------------------------------------------------------------------------
+// Forward / input-gradient kernel, input window in LDS and the weights resident in registers.
+// ------------------------------------------------------------------------------------------
+// With 64 contraction channels per group and TAPS taps, the weights a wave multiplies by (32
+// output channels x K = 64 TAPS) are TAPS * 16 registers per lane: 144 for a 3x3 filter.  A
+// workgroup then fetches them once and walks over many tiles of 128 output pixels: the window of
+// the next tile travels into the second of two LDS buffers while the current one is multiplied
+// (fragments of every tap read at shifted rows, as in the kernel above), and the buffer just
+// multiplied from serves as the staging area of the epilogue.  Two workgroups share a CU (two
+// waves per SIMD, 256 registers each).  The tiles of the grid are dealt out in eight contiguous
+// ranges, one per XCD (workgroup b runs on XCD b % 8), so that the input rows two neighbouring
+// tiles share are fetched into one L2 only.
+constexpr int kStatWin = (kHaloRows + 1) * 128;    // window + the zero row
+
+template <typename T, bool OUT_LAST, int TAPS>
+__global__ __launch_bounds__(256, 2) void conv_igemm_stationary_kernel(IgemmArgs g, int tiles_m) {
+  __shared__ __attribute__((aligned(1024))) char lds[2 * kStatWin + CBN * 4];
+  float* const bias_tile = reinterpret_cast<float*>(lds + 2 * kStatWin);   // the tile's bias values, if any
+  const int grp = blockIdx.z;
+  const int n0 = blockIdx.y * CBN;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int KH = TAPS / g.KW;
+
+  const int xcd = blockIdx.x & 7, per_xcd = gridDim.x >> 3;   // the grid is a multiple of 8 wide
+  const int t_end = (int)(((int64_t)(xcd + 1) * tiles_m) >> 3);
+  int tile = (int)(((int64_t)xcd * tiles_m) >> 3) + (blockIdx.x >> 3);
+  if (tile >= t_end) return;
+
+  // q of (tap 0,0) for an output pixel
+  auto q_of = [&](int m, int& ih0, int& iw0) -> int {
+    const int n = fast_div(m, g.div_ohw);
+    const int p = m - n * g.OHW;
+    const int oh = fast_div(p, g.div_ow);
+    const int ow = p - oh * g.OW;
+    ih0 = oh * g.sh - g.ph;
+    iw0 = ow * g.sw - g.pw;
+    return (n * g.IH + ih0) * g.IW + iw0;
+  };
+  const i32x4 ra = make_buffer_rsrc(g.act, g.act_bytes);
+  // Starts the loads of tile t's window into `win` (offsets first, then the loads back to back;
+  // rows past the window read zeros).
+  auto issue_window = [&](int t, char* win) {
+    // the lane's part of the offsets is recomputed per tile on purpose (the empty asm hides that
+    // it never changes): kept across the main loop it would take the registers the fragment
+    // prefetch needs
+    int lane_v = lane;
+    asm volatile("" : "+v"(lane_v));
+    int d0, d1;
+    const int m0 = t * CBM;
+    const int m_last = m0 + CBM - 1 < g.M ? m0 + CBM - 1 : g.M - 1;
+    const int q_lo = q_of(m0, d0, d1);
+    const int rows = q_of(m_last, d0, d1) + (KH - 1) * g.IW + g.KW - q_lo;   // <= kHaloRows (host check)
+    int doff[kHaloRows / 32];
+#pragma unroll
+    for (int i = 0; i < kHaloRows / 32; ++i) {
+      const int row = (wave + 4 * i) * 8 + (lane_v >> 3);
+      const int chunk = (lane_v & 7) ^ ((row >> 1) & 7);   // as in the kernel above
+      const int off = ((q_lo + row) * g.Ctot + grp * g.Cg + chunk * 8) * 2;   // negative: out of range
+      doff[i] = row < rows ? off : kOobOffset;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < kHaloRows / 32; ++i) lds_dma_16(ra, doff[i], win + (wave + 4 * i) * 1024);
+  };
+
+  if (threadIdx.x < 64)   // the zero rows of both buffers
+    reinterpret_cast<uint32_t*>(lds + (threadIdx.x >> 5) * kStatWin + kHaloRows * 128)[threadIdx.x & 31] = 0u;
+  issue_window(tile, lds);
+  if (g.bias && threadIdx.x < CBN)
+    bias_tile[threadIdx.x] =
+        n0 + (int)threadIdx.x < g.Og ? load_scalar_f32(g.bias, g.bias_dt, grp * g.Og + n0 + threadIdx.x) : 0.f;
+
+  // this wave's weights: fragment-major, one fragment = 64 lanes x 16 bytes, K / 16 fragments per
+  // tile of 32 output channels
+  const int ntiles32 = (g.Og + 31) >> 5;
+  const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(
+      g.wf, 0, (int)((int64_t)gridDim.z * ntiles32 * g.K * 64), 0x00020000);
+  const int wrow = ((grp * ntiles32 + (n0 >> 5) + wn) * (g.K >> 4)) * 1024 + lane * 16;
+  uint4 wreg[TAPS * 4];
+#pragma unroll
+  for (int i = 0; i < TAPS * 4; ++i)
+    wreg[i] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rw, wrow, i * 1024, 0));
+
+  lds_dma_wait_all();
+  __syncthreads();
+  // The window of the next tile is always on its way while a tile is worked on: it is requested
+  // as soon as the buffer it goes into has been emptied by the epilogue of the tile before, and
+  // waited for only after the next epilogue's LDS work, a whole tile later.
+  if (tile + per_xcd < t_end) issue_window(tile + per_xcd, lds + kStatWin);
+  int buf = 0;
+  for (; tile < t_end; tile += per_xcd) {
+    char* const win = lds + buf * kStatWin;
+
+    const int m0 = tile * CBM;
+    int d0, d1;
+    const int q_lo = q_of(m0, d0, d1);
+    int f_ih0[2], f_iw0[2], f_row[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int m = m0 + wm * 64 + t * 32 + (lane & 31);
+      if (m < g.M) {
+        f_row[t] = q_of(m, f_ih0[t], f_iw0[t]) - q_lo;
+      } else {
+        f_ih0[t] = -(1 << 24);
+        f_iw0[t] = 0;
+        f_row[t] = 0;
+      }
+    }
+    f32x16 acc[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[t][e] = 0.f;
+
+    // Fragment address of k-step 0 of a tap: row * 128 + ((lane / 32) ^ (row / 2)) % 8 * 16; k-step ks
+    // sits at that address with ks XORed into bits 5-6 (the chunk swizzle is an XOR as well).
+    // The fragments are fetched two k-steps ahead of the MFMAs that use them.
+    int kh = 0, kw = 0;
+    auto tap_address = [&](int t) -> int {
+      const int ih = f_ih0[t] + kh, iw = f_iw0[t] + kw;
+      const bool ok = (unsigned)ih < (unsigned)g.IH && (unsigned)iw < (unsigned)g.IW;
+      const int row = ok ? f_row[t] + kh * g.IW + kw : kHaloRows;
+      return row * 128 + ((((lane >> 5) ^ (row >> 1)) & 7) << 4);
+    };
+    auto next_tap = [&]() {
+      if (++kw == g.KW) {
+        kw = 0;
+        ++kh;
+      }
+    };
+    constexpr int kSteps = TAPS * 4, kAhead = 2;
+    uint4 af[kAhead + 1][2];
+    int abase[2] = {tap_address(0), tap_address(1)};
+    auto fetch = [&](int step) {
+      if (step > 0 && (step & 3) == 0) {
+        next_tap();
+        abase[0] = tap_address(0);
+        abase[1] = tap_address(1);
+      }
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+        af[step % (kAhead + 1)][t] = *reinterpret_cast<const uint4*>(win + (abase[t] ^ ((step & 3) << 5)));
+    };
+#pragma unroll
+    for (int st = 0; st < kAhead; ++st) fetch(st);
+#pragma unroll
+    for (int st = 0; st < kSteps; ++st) {
+      __builtin_amdgcn_sched_barrier(0);   // a k-step's address arithmetic stays in its k-step
+      if (st + kAhead < kSteps) fetch(st + kAhead);
+      const uint4 bw = wreg[st];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+        acc[t] = OUT_LAST ? Mfma16<T>::run(bw, af[st % (kAhead + 1)][t], acc[t])
+                          : Mfma16<T>::run(af[st % (kAhead + 1)][t], bw, acc[t]);
+    }
+    __syncthreads();      // nobody reads the current window any more: it becomes the output tile
+    {
+      // as for the window offsets: what the epilogue derives from the thread index is recomputed per tile
+      int tid = threadIdx.x;
+      asm volatile("" : "+v"(tid));
+      uint4 piece[4];
+      igemm_epilogue_stage<T, OUT_LAST>(acc, win, g, grp, n0, tid >> 7, (tid >> 6) & 1, tid, g.bias ? bias_tile : nullptr,
+                                        piece);
+      lds_dma_wait_all();   // this wave's part of the next window (requested a tile ago) has landed
+      __syncthreads();      // ... and everybody's; the output tile has been read: its buffer is free
+      if (tile + 2 * per_xcd < t_end) issue_window(tile + 2 * per_xcd, win);
+      igemm_epilogue_store<T, OUT_LAST>(piece, g, grp, m0, n0, tid);
+    }
+    buf ^= 1;
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1051,14 +1263,28 @@ int run_igemm(IgemmArgs g, const void* w, const ConvProblem& p, int flip, int cg
   const bool resident = window > 0 && window <= kHaloRows;
   return dispatch16(dt, [&](auto* tp) -> int {
     typedef std::remove_pointer_t<decltype(tp)> T;
+    // weights in registers: 3x3-sized filters over 64 channels, enough tiles for every resident
+    // workgroup (two per CU) to walk over several
+    const int64_t tiles_m = cdiv64(g.M, CBM);
+    const int stat_grid = device_cu_count() * 2 / 8 * 8;
+    const bool stationary = resident && g.tiles_per_tap == 1 && g.KT == 9 && stat_grid >= 8 && tiles_m >= 4 * stat_grid;
     if (resident) {
       const int ntiles = (g.Og + 31) / 32;
       const int64_t chunks = (int64_t)groups * ntiles * (g.K / 16) * 64;
       hipLaunchKernelGGL((conv_weight_frags_direct_kernel<T>), dim3((unsigned)cdiv64(chunks, 256)), dim3(256), 0,
                          stream, (const T*)w, (T*)g.wf, cg_real, g.Cg, g.Og, (int)(p.KH * p.KW), flip, ntiles,
                          chunks);
-      if (g.out_last) hipLaunchKernelGGL((conv_igemm_halo_kernel<T, true>), grid, dim3(256), 0, stream, g);
-      else hipLaunchKernelGGL((conv_igemm_halo_kernel<T, false>), grid, dim3(256), 0, stream, g);
+      if (stationary) {
+        const dim3 sgrid((unsigned)stat_grid, (unsigned)g.nbn, (unsigned)groups);
+        if (g.out_last)
+          hipLaunchKernelGGL((conv_igemm_stationary_kernel<T, true, 9>), sgrid, dim3(256), 0, stream, g, (int)tiles_m);
+        else
+          hipLaunchKernelGGL((conv_igemm_stationary_kernel<T, false, 9>), sgrid, dim3(256), 0, stream, g, (int)tiles_m);
+      } else if (g.out_last) {
+        hipLaunchKernelGGL((conv_igemm_halo_kernel<T, true>), grid, dim3(256), 0, stream, g);
+      } else {
+        hipLaunchKernelGGL((conv_igemm_halo_kernel<T, false>), grid, dim3(256), 0, stream, g);
+      }
     } else {
       const int rc = weight_taps(w, const_cast<void*>(g.wt), p, flip, g.Cg, stream);
       if (rc) return rc;

@@ -159,6 +159,11 @@ def test_conv_matrix_core_path_agrees_with_generic_kernel(dtype) -> None:
     (41, 64, 56, 56, 64, 2, 1, False),     # padding wider than the filter reach (forward only)
     (96, 64, 23, 23, 64, 1, 1, False),     # two output rows per k-tile of the weight gradient, odd row count
     (128, 128, 7, 7, 192, 1, 1, True),     # whole 7x7 images per k-tile, several channel tiles
+    # more than 8 tiles per CU: the kernel that keeps the 3x3 x 64-channel weights in registers and walks over tiles
+    (88, 64, 56, 56, 64, 1, 1, True),
+    (90, 64, 55, 55, 128, 1, 1, True),     # last tile partly empty, two channel tiles
+    (96, 128, 56, 56, 128, 1, 2, False),   # two groups
+    (100, 64, 57, 57, 40, 1, 1, True),     # element stores, channel tile partly empty
 ])
 def test_conv_window_kernel_agrees_with_generic_kernel_at_size(n, c, h, w, o, pad, groups, bias, dtype) -> None:
     """
@@ -425,6 +430,27 @@ def test_conv2d_channels_last_matches_channels_first_bitwise() -> None:
     assert results[1][1].is_contiguous(memory_format=torch.channels_last)
     for first, last in zip(*results):
         assert torch.equal(first, last)
+
+
+@pytest.mark.parametrize('shape, out_dim, bias', [((88, 64, 56, 56), 64, True), ((90, 64, 55, 55), 40, False)])
+def test_conv2d_weights_resident_kernel_same_on_both_layouts(shape, out_dim, bias) -> None:
+    # batch sizes at which a workgroup walks over several tiles with the weights in registers
+    dtype = torch.bfloat16
+    x = randn(shape, 1, dtype).cuda()
+    w = randn((out_dim, shape[1], 3, 3), 2, dtype, 576 ** -0.5).cuda()
+    b = randn((out_dim,), 4, dtype).cuda() if bias else None
+    dy = randn((shape[0], out_dim, shape[2], shape[3]), 3, dtype).cuda()
+    results = []
+    for fmt in (torch.contiguous_format, torch.channels_last):
+        xd = x.detach().clone(memory_format=fmt).requires_grad_(True)
+        wd = w.clone().requires_grad_(True)
+        y = attorch_amd.Conv2dAutoGrad.apply(xd, wd, b, 1, 1, 1, 1, 1)
+        y.backward(dy.contiguous(memory_format=fmt))
+        results.append((y.detach(), xd.grad, wd.grad))
+    for first, last in zip(*results):
+        assert torch.equal(first, last)
+    ref = torch.nn.functional.conv2d(x.float(), w.float(), None if b is None else b.float(), 1, 1)
+    assert_close(results[1][0], ref.cpu(), dtype, 'output')
 
 
 @pytest.mark.parametrize('dtype', DTYPES)
