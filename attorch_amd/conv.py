@@ -280,9 +280,20 @@ class Conv2dAutoGrad(torch.autograd.Function):
                     'at_conv2d_bwd_weight')
             if need_bias:
                 bias_grad = torch.empty(out_feat_dim, dtype=output_dtype, device=device)
-                _lib.check(lib.at_channel_sum(
-                    _lib.ptr(output_grad), _lib.ptr(bias_grad), batch_dim, out_feat_dim,
-                    out_height * out_width, dtype, dtype, stream), 'at_channel_sum')
+                if output_grad_nhwc is not None:
+                    # the channels-last copy is a [batch * height * width, out_feat] matrix:
+                    # its column sums use the whole GPU whatever the channel count
+                    rows = batch_dim * out_height * out_width
+                    workspace, workspace_bytes = _workspace(
+                        lib.at_colsum_workspace_bytes(rows, out_feat_dim), device)
+                    _lib.check(lib.at_colsum(
+                        _lib.ptr(output_grad_nhwc), _lib.ptr(bias_grad), _lib.ptr(workspace),
+                        workspace_bytes, rows, out_feat_dim, out_feat_dim, dtype, dtype,
+                        stream), 'at_colsum')
+                else:
+                    _lib.check(lib.at_channel_sum(
+                        _lib.ptr(output_grad), _lib.ptr(bias_grad), batch_dim, out_feat_dim,
+                        out_height * out_width, dtype, dtype, stream), 'at_channel_sum')
 
         return input_grad, weight_grad, bias_grad, None, None, None, None, None
 

@@ -418,18 +418,50 @@ __global__ __launch_bounds__(256) void conv_direct_dw_kernel(ConvArgs g) {
   }
 }
 
-// Per-channel sum over batch and space of a [N, C, S] tensor (bias gradient).
-template <typename T>
-__global__ __launch_bounds__(256) void channel_sum_kernel(const T* __restrict__ x, void* __restrict__ out,
-                                                         int out_dt, int64_t N, int C, int64_t S) {
-  __shared__ float smem[16];
+// Per-channel sum over batch and space of a [N, C, S] tensor (bias gradient): one workgroup of
+// 1024 lanes per channel.  VEC: the planes are whole 16-byte vectors (S a multiple of the vector
+// length, aligned base): a lane then reads vectors, four of them in flight at a time, and walks
+// the planes in the order (image, vector); otherwise element by element.  The order of the sum is
+// fixed by the launch shape, so the result is the same run to run.
+constexpr int kChannelSumBlock = 1024;
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kChannelSumBlock) void channel_sum_kernel(const T* __restrict__ x, void* __restrict__ out,
+                                                                      int out_dt, int64_t N, int C, int64_t S) {
+  __shared__ float smem[kChannelSumBlock / kWave];
   const int c = blockIdx.x;
   float s = 0.f;
-  for (int64_t n = 0; n < N; ++n) {
-    const T* plane = x + (n * C + c) * S;
-    for (int64_t i = threadIdx.x; i < S; i += 256) s += to_f32(plane[i]);
+  if (VEC) {
+    constexpr int kPer = 16 / sizeof(T), kUnroll = 4;
+    const int64_t vec_per_plane = S / kPer, total = N * vec_per_plane;
+    float part[kUnroll] = {0.f, 0.f, 0.f, 0.f};
+    for (int64_t v0 = threadIdx.x; v0 < total; v0 += (int64_t)kUnroll * kChannelSumBlock) {
+      uint4 raw[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int64_t v = v0 + (int64_t)u * kChannelSumBlock;
+        // 32-bit division whenever the vector count allows it (64-bit division is a long routine)
+        const int64_t n = total <= INT32_MAX ? (int64_t)((uint32_t)v / (uint32_t)vec_per_plane) : v / vec_per_plane;
+        const int64_t i = v - n * vec_per_plane;
+        raw[u] = v < total ? reinterpret_cast<const uint4*>(x + (n * C + c) * S)[i] : make_uint4(0, 0, 0, 0);
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        float f[kPer];
+        unpack16<T>(raw[u], f);
+        float t = 0.f;
+#pragma unroll
+        for (int e = 0; e < kPer; ++e) t += f[e];
+        part[u] += t;
+      }
+    }
+    s = (part[0] + part[1]) + (part[2] + part[3]);
+  } else {
+    for (int64_t n = 0; n < N; ++n) {
+      const T* plane = x + (n * C + c) * S;
+      for (int64_t i = threadIdx.x; i < S; i += kChannelSumBlock) s += to_f32(plane[i]);
+    }
   }
-  s = group_reduce(s, 256, smem, SumOp(), 0.f);
+  s = group_reduce(s, kChannelSumBlock, smem, SumOp(), 0.f);
   if (threadIdx.x == 0) store_scalar_f32(out, out_dt, c, s);
 }
 
@@ -773,8 +805,12 @@ int at_channel_sum(const void* x, void* out, int64_t batch, int64_t feat, int64_
   if (batch <= 0 || feat <= 0 || spatial <= 0 || feat > INT32_MAX) return AT_ERR_DIM;
   return dispatch_dtype(x_dtype, [&](auto* tp) -> int {
     typedef std::remove_pointer_t<decltype(tp)> T;
-    hipLaunchKernelGGL((channel_sum_kernel<T>), dim3((unsigned)feat), dim3(256), 0, (hipStream_t)stream,
-                       (const T*)x, out, out_dtype, batch, (int)feat, spatial);
+    if (spatial % (16 / (int64_t)sizeof(T)) == 0 && aligned16(x))
+      hipLaunchKernelGGL((channel_sum_kernel<T, true>), dim3((unsigned)feat), dim3(kChannelSumBlock), 0,
+                         (hipStream_t)stream, (const T*)x, out, out_dtype, batch, (int)feat, spatial);
+    else
+      hipLaunchKernelGGL((channel_sum_kernel<T, false>), dim3((unsigned)feat), dim3(kChannelSumBlock), 0,
+                         (hipStream_t)stream, (const T*)x, out, out_dtype, batch, (int)feat, spatial);
     return launch_status();
   });
 }

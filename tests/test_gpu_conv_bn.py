@@ -432,6 +432,21 @@ def test_conv2d_channels_last_matches_channels_first_bitwise() -> None:
         assert torch.equal(first, last)
 
 
+@pytest.mark.parametrize('dtype', DTYPES)
+@pytest.mark.parametrize('batch, feat, spatial', [(5, 7, 64), (3, 5, 63), (130, 3, 1000), (1, 1, 8), (2, 9, 1)])
+def test_channel_sum(batch, feat, spatial, dtype) -> None:
+    # the bias gradient of a channels-first tensor, output_grad.sum((0, 2, 3)) (conv_layer.py:162):
+    # planes that are whole 16-byte vectors and planes that are not
+    from attorch_amd import _lib
+    lib = _lib.load()
+    x = randn((batch, feat, spatial), 5, dtype).cuda()
+    out = torch.empty(feat, dtype=dtype, device='cuda')
+    dt = _lib.dtype_id(dtype)
+    _lib.check(lib.at_channel_sum(_lib.ptr(x), _lib.ptr(out), batch, feat, spatial, dt, dt, _lib.stream_of(x)),
+               'at_channel_sum')
+    assert_close(out, x.double().sum((0, 2)).cpu(), dtype, 'channel sum', batch_reduction=True)
+
+
 @pytest.mark.parametrize('shape, out_dim, bias', [((88, 64, 56, 56), 64, True), ((90, 64, 55, 55), 40, False)])
 def test_conv2d_weights_resident_kernel_same_on_both_layouts(shape, out_dim, bias) -> None:
     # batch sizes at which a workgroup walks over several tiles with the weights in registers
