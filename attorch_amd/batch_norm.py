@@ -98,7 +98,12 @@ class BatchNormAutoGrad(torch.autograd.Function):
                 and lib.at_batch_norm_nhwc_supported(feat_dim, _lib.dtype_id(input.dtype))):
             layout = torch.channels_last
         ctx.layout = layout
-        forward_entry = (lib.at_batch_norm_fwd_nhwc if layout is torch.channels_last
+        # Without spatial extent ([batch, feat] inputs) the contiguous tensor already is a matrix
+        # of rows of features: the same kernels as for channels-last tensors apply, and read it
+        # along its rows instead of one feature at a time.
+        ctx.rows_of_features = layout is torch.channels_last or (
+            spatial_dim == 1 and bool(lib.at_batch_norm_nhwc_supported(feat_dim, _lib.dtype_id(input.dtype))))
+        forward_entry = (lib.at_batch_norm_fwd_nhwc if ctx.rows_of_features
                          else lib.at_batch_norm_fwd)
         input_k = input.contiguous(memory_format=layout)
         residual_k = (pre_act_add.to(input.dtype).contiguous(memory_format=layout)
@@ -154,7 +159,7 @@ class BatchNormAutoGrad(torch.autograd.Function):
         device = input.device
 
         output_grad_k = output_grad.to(input.dtype).contiguous(memory_format=ctx.layout)
-        backward_entry = (lib.at_batch_norm_bwd_nhwc if ctx.layout is torch.channels_last
+        backward_entry = (lib.at_batch_norm_bwd_nhwc if ctx.rows_of_features
                           else lib.at_batch_norm_bwd)
         input_grad = torch.empty_like(input)
         pre_act_grad = torch.empty_like(input) if ctx.act_func is not None else None

@@ -241,7 +241,7 @@ def test_conv_weight_gradient_all_taps_kernel(n, c, h, w, o, groups, dtype) -> N
     assert_close(dw, ref.cpu(), dtype, 'weight_grad', batch_reduction=True)
 
 
-BN_SHAPES = [(6, 5), (128, 1024), (2048, 768), (8, 960, 196), (2048, 64, 16), (2, 3, 224, 224),
+BN_SHAPES = [(6, 5), (128, 1024), (2048, 768), (300, 2048), (77, 40, 1), (8, 960, 196), (2048, 64, 16), (2, 3, 224, 224),
              (16, 64, 56, 56), (32, 128, 7, 7), (3, 7, 3, 5)]
 
 
