@@ -135,7 +135,33 @@ def stream_of(tensor: Tensor) -> int:
     """
     Raw hipStream_t of the current PyTorch stream on the tensor's device.
     """
-    return torch.cuda.current_stream(tensor.device).cuda_stream
+    # the raw handle straight from the C extension: torch.cuda.current_stream() builds a Stream
+    # object first, several microseconds of a call that is made once per launch
+    return torch._C._cuda_getCurrentRawStream(tensor.get_device())
+
+
+class _NoGuard:
+    """
+    Stand-in for a device guard when the wanted device is already the current one.
+    """
+    def __enter__(self) -> None:
+        return None
+
+    def __exit__(self, *exc: object) -> bool:
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def device_guard(tensor: Tensor):
+    """
+    Context manager that makes the tensor's device the current one for the launches inside it;
+    free of cost in the usual case that it already is.
+    """
+    if tensor.get_device() == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device_of(tensor)
 
 
 def require_gpu(tensor: Tensor, what: str) -> None:

@@ -23,7 +23,7 @@ from .act import act_id, parse_act_func
 def _launch_forward(input: Tensor, act: int, param: float, drop_p: float, seed: int) -> Tensor:
     flattened_input = input.contiguous().view(-1)
     output = torch.empty_like(flattened_input)
-    with torch.cuda.device_of(input):
+    with _lib.device_guard(input):
         _lib.check(_lib.load().at_act_dropout_fwd(
             _lib.ptr(flattened_input), _lib.ptr(output), flattened_input.numel(), act, param,
             drop_p, seed, _lib.dtype_id(input.dtype), _lib.stream_of(input)),
@@ -38,7 +38,7 @@ def _launch_backward(output_grad: Tensor, input: Optional[Tensor], act: int, par
     flattened_grad = output_grad.to(reference.dtype).contiguous().view(-1)
     flattened_input = None if input is None else input.contiguous().view(-1)
     input_grad = torch.empty_like(flattened_grad)
-    with torch.cuda.device_of(output_grad):
+    with _lib.device_guard(output_grad):
         _lib.check(_lib.load().at_act_dropout_bwd(
             _lib.ptr(flattened_grad), _lib.ptr(flattened_input), _lib.ptr(input_grad),
             flattened_grad.numel(), act, param, drop_p, seed, _lib.dtype_id(reference.dtype),

@@ -122,7 +122,7 @@ class BatchNormAutoGrad(torch.autograd.Function):
         workspace_bytes = lib.at_batch_norm_workspace_bytes(feat_dim)
         workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=input.device)
 
-        with torch.cuda.device_of(input):
+        with _lib.device_guard(input):
             _lib.check(forward_entry(
                 _lib.ptr(input_k), _lib.ptr(weight_k), _lib.ptr(bias_k), _lib.ptr(mean),
                 _lib.ptr(inv_std), _lib.ptr(residual_k), _lib.ptr(pre_act), _lib.ptr(output),
@@ -171,7 +171,7 @@ class BatchNormAutoGrad(torch.autograd.Function):
         workspace_bytes = lib.at_batch_norm_workspace_bytes(feat_dim)
         workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=device)
 
-        with torch.cuda.device_of(input):
+        with _lib.device_guard(input):
             _lib.check(backward_entry(
                 _lib.ptr(output_grad_k), _lib.ptr(pre_act), _lib.ptr(input), _lib.ptr(mean),
                 _lib.ptr(inv_std), _lib.ptr(weight), _lib.ptr(input_grad), _lib.ptr(pre_act_grad),

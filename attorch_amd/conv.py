@@ -125,7 +125,7 @@ class Conv2dAutoGrad(torch.autograd.Function):
         if ctx.channels_last:
             output = torch.empty((batch_dim, out_feat_dim, out_height, out_width), device=input.device,
                                  dtype=output_dtype, memory_format=torch.channels_last)
-            with torch.cuda.device_of(input):
+            with _lib.device_guard(input):
                 workspace, workspace_bytes = _workspace(
                     lib.at_conv2d_nhwc_workspace_bytes(0, *dims, dtype), input.device)
                 _lib.check(lib.at_conv2d_fwd_nhwc(
@@ -139,7 +139,7 @@ class Conv2dAutoGrad(torch.autograd.Function):
         input_k = input.to(output_dtype).contiguous()
         output = torch.empty((batch_dim, out_feat_dim, out_height, out_width),
                              device=input.device, dtype=output_dtype)
-        with torch.cuda.device_of(input):
+        with _lib.device_guard(input):
             workspace, workspace_bytes = _workspace(
                 lib.at_conv2d_fwd_workspace_bytes(*dims, dtype, dtype), input.device)
             _lib.check(lib.at_conv2d_fwd(
@@ -185,7 +185,7 @@ class Conv2dAutoGrad(torch.autograd.Function):
             grad_last = output_grad.to(output_dtype).contiguous(memory_format=torch.channels_last)
             need_input = input.requires_grad
             need_weight = weight.requires_grad
-            with torch.cuda.device_of(input):
+            with _lib.device_guard(input):
                 n_bytes = lib.at_conv2d_nhwc_workspace_bytes(1, *dims, dtype) if need_input else 0
                 if n_bytes > 0:
                     weight_k = weight.to(output_dtype).contiguous()
@@ -250,7 +250,7 @@ class Conv2dAutoGrad(torch.autograd.Function):
         dtype = _lib.dtype_id(output_dtype)
 
         input_grad = weight_grad = bias_grad = None
-        with torch.cuda.device_of(input):
+        with _lib.device_guard(input):
             input_workspace_bytes = (lib.at_conv2d_bwd_input_workspace_bytes(*dims, dtype)
                                      if need_input else 0)
             # one channels-last copy of the output gradient serves both products

@@ -73,7 +73,7 @@ class CrossEntropyLossAutoGrad(torch.autograd.Function):
         workspace_bytes = lib.at_cross_entropy_workspace_bytes(batch_dim)
         workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=input.device)
 
-        with torch.cuda.device_of(input):
+        with _lib.device_guard(input):
             _lib.check(lib.at_cross_entropy_fwd_bwd(
                 _lib.ptr(logits), _lib.ptr(target_k), _lib.ptr(weight_k), _lib.ptr(output),
                 _lib.ptr(input_grad), _lib.ptr(workspace), workspace_bytes, batch_dim, feat_dim,
@@ -129,7 +129,7 @@ class CrossEntropyLossAutoGrad(torch.autograd.Function):
         else:
             input_grad, holds_unit_grad = torch.empty_like(unit_grad), 0
 
-        with torch.cuda.device_of(logits):
+        with _lib.device_guard(logits):
             _lib.check(lib.at_cross_entropy_bwd(
                 _lib.ptr(logits), _lib.ptr(target_k), _lib.ptr(weight_k), _lib.ptr(output_grad),
                 _lib.ptr(workspace), _lib.ptr(input_grad), batch_dim, feat_dim,

@@ -69,7 +69,7 @@ class GLUAutoGrad(torch.autograd.Function):
         out_shape = list(input.shape)
         out_shape[dim] //= 2
         output = torch.empty(out_shape, dtype=input.dtype, device=input.device)
-        with torch.cuda.device_of(input):
+        with _lib.device_guard(input):
             _lib.check(lib.at_glu_fwd(_lib.ptr(input_k), _lib.ptr(output), outer, half, act,
                                       0.0 if param is None else param, _lib.dtype_id(input.dtype),
                                       _lib.stream_of(input)), 'at_glu_fwd')
@@ -95,7 +95,7 @@ class GLUAutoGrad(torch.autograd.Function):
         outer, half = ctx.geometry
         output_grad = output_grad.contiguous()
         input_grad = torch.empty_like(input_k)
-        with torch.cuda.device_of(input_k):
+        with _lib.device_guard(input_k):
             _lib.check(lib.at_glu_bwd(_lib.ptr(output_grad), _lib.ptr(input_k), _lib.ptr(input_grad),
                                       outer, half, ctx.act, 0.0 if ctx.param is None else ctx.param,
                                       _lib.dtype_id(input_k.dtype), _lib.stream_of(input_k)), 'at_glu_bwd')

@@ -132,7 +132,7 @@ class LinearAutoGrad(torch.autograd.Function):
         output = torch.empty((batch_dim, out_feat_dim), device=input.device, dtype=output_dtype)
         pre_act = torch.empty_like(output) if save_pre_act else output
 
-        with torch.cuda.device_of(input):
+        with _lib.device_guard(input):
             _lib.check(lib.at_linear_fwd(
                 _lib.ptr(input_k), _lib.ptr(weight_k), _lib.ptr(bias_k), _lib.ptr(pre_act),
                 _lib.ptr(output), batch_dim, contract_dim, out_feat_dim, _lib.row_stride(input_k),
@@ -186,7 +186,7 @@ class LinearAutoGrad(torch.autograd.Function):
                 weight_grad = torch.empty((in_feat_dim, out_feat_dim), dtype=output_dtype, device=device)
                 bias_grad = (torch.empty(out_feat_dim, dtype=output_dtype, device=device)
                              if ctx.bias_requires_grad else None)
-                with torch.cuda.device_of(input):
+                with _lib.device_guard(input):
                     _lib.check(lib.at_linear_bwd_small(
                         _lib.ptr(output_grad), _lib.ptr(pre_act_mm), _lib.ptr(input_mm), _lib.ptr(weight_mm),
                         _lib.ptr(input_grad), _lib.ptr(weight_grad), _lib.ptr(bias_grad), batch_dim,
@@ -200,7 +200,7 @@ class LinearAutoGrad(torch.autograd.Function):
                     input_grad = input_grad.view_as(input)
                 return input_grad, weight_grad, bias_grad, None
 
-        with torch.cuda.device_of(input):
+        with _lib.device_guard(input):
             bias_grad = None
             if ctx.act_func is None:
                 pre_act_grad = output_grad

@@ -78,7 +78,7 @@ class NLLLossAutoGrad(torch.autograd.Function):
             if reduction != 'none':
                 workspace_bytes = lib.at_nll_loss_workspace_bytes(batch_dim, spatial_dim)
                 workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=device)
-            with torch.cuda.device_of(input):
+            with _lib.device_guard(input):
                 _lib.check(lib.at_nll_loss_fwd(
                     _lib.ptr(input_k), _lib.ptr(target_k), _lib.ptr(weight_k), _lib.ptr(output),
                     _lib.ptr(sum_weights), _lib.ptr(workspace), workspace_bytes or 0, batch_dim,
@@ -110,7 +110,7 @@ class NLLLossAutoGrad(torch.autograd.Function):
         input_grad = torch.empty(ctx.input_shape, dtype=ctx.output_dtype, device=target_k.device)
         if input_grad.numel() > 0:
             output_grad = output_grad.contiguous()
-            with torch.cuda.device_of(target_k):
+            with _lib.device_guard(target_k):
                 _lib.check(lib.at_nll_loss_bwd(
                     _lib.ptr(output_grad), _lib.ptr(target_k), _lib.ptr(weight_k), _lib.ptr(sum_weights),
                     _lib.ptr(input_grad), batch_dim, feat_dim, ctx.spatial_dim,

@@ -80,7 +80,7 @@ class LayerNormAutoGrad(torch.autograd.Function):
         if add_bias and bias_k.dtype != weight_k.dtype:
             bias_k = bias_k.to(weight_k.dtype)
 
-        with torch.cuda.device_of(input):
+        with _lib.device_guard(input):
             _lib.check(lib.at_layer_norm_fwd(
                 _lib.ptr(flattened_input), _lib.ptr(weight_k), _lib.ptr(bias_k),
                 _lib.ptr(mean), _lib.ptr(inv_std), _lib.ptr(output),
@@ -128,7 +128,7 @@ class LayerNormAutoGrad(torch.autograd.Function):
             workspace = torch.empty(workspace_bytes, device=device, dtype=torch.uint8)
         weight_k = _param_for_kernel(weight, flattened_input) if scale_by_weight else None
 
-        with torch.cuda.device_of(flattened_input):
+        with _lib.device_guard(flattened_input):
             _lib.check(lib.at_layer_norm_bwd(
                 _lib.ptr(flattened_output_grad), _lib.ptr(flattened_input),
                 _lib.ptr(mean), _lib.ptr(inv_std), _lib.ptr(weight_k),
@@ -219,7 +219,7 @@ class RMSNormAutoGrad(torch.autograd.Function):
                    if requires_grad else None)
         weight_k = _param_for_kernel(weight, flattened_input)
 
-        with torch.cuda.device_of(input):
+        with _lib.device_guard(input):
             _lib.check(lib.at_rms_norm_fwd(
                 _lib.ptr(flattened_input), _lib.ptr(weight_k), _lib.ptr(inv_rms), _lib.ptr(output),
                 batch_dim, feat_dim, _lib.row_stride(flattened_input), _lib.row_stride(output), eps,
@@ -261,7 +261,7 @@ class RMSNormAutoGrad(torch.autograd.Function):
             workspace = torch.empty(workspace_bytes, device=device, dtype=torch.uint8)
         weight_k = _param_for_kernel(weight, flattened_input)
 
-        with torch.cuda.device_of(flattened_input):
+        with _lib.device_guard(flattened_input):
             _lib.check(lib.at_rms_norm_bwd(
                 _lib.ptr(flattened_output_grad), _lib.ptr(flattened_input), _lib.ptr(inv_rms),
                 _lib.ptr(weight_k), _lib.ptr(input_grad), _lib.ptr(weight_grad),

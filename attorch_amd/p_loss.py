@@ -63,7 +63,7 @@ class PLossAutoGrad(torch.autograd.Function):
             if reduction != 'none':
                 workspace_bytes = lib.at_p_loss_workspace_bytes(size)
                 workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=device)
-            with torch.cuda.device_of(input):
+            with _lib.device_guard(input):
                 _lib.check(lib.at_p_loss_fwd(
                     _lib.ptr(input_k), _lib.ptr(target_k), _lib.ptr(output), _lib.ptr(workspace),
                     workspace_bytes or 0, size, p_loss, REDUCTIONS[reduction], param,
@@ -96,7 +96,7 @@ class PLossAutoGrad(torch.autograd.Function):
         target_grad = torch.empty_like(target_k, dtype=ctx.output_dtype) if needs_target else None
         if size > 0:
             output_grad = output_grad.contiguous()
-            with torch.cuda.device_of(input_k):
+            with _lib.device_guard(input_k):
                 _lib.check(lib.at_p_loss_bwd(
                     _lib.ptr(output_grad), _lib.ptr(input_k), _lib.ptr(target_k), _lib.ptr(input_grad),
                     _lib.ptr(target_grad), size, ctx.p_loss, REDUCTIONS[ctx.reduction], ctx.param,

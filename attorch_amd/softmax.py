@@ -46,7 +46,7 @@ class SoftmaxAutoGrad(torch.autograd.Function):
         output_dtype = get_output_dtype(input.dtype, autocast='fp32')
         output = torch.empty((batch_dim, feat_dim), device=input.device, dtype=output_dtype)
 
-        with torch.cuda.device_of(input):
+        with _lib.device_guard(input):
             _lib.check(lib.at_softmax_fwd(
                 _lib.ptr(flattened_input), _lib.ptr(output), batch_dim, feat_dim,
                 _lib.row_stride(flattened_input), _lib.row_stride(output), int(neg), int(log),
@@ -75,7 +75,7 @@ class SoftmaxAutoGrad(torch.autograd.Function):
         batch_dim, feat_dim = output.shape
         input_grad = torch.empty_like(output)
 
-        with torch.cuda.device_of(output):
+        with _lib.device_guard(output):
             _lib.check(lib.at_softmax_bwd(
                 _lib.ptr(flattened_output_grad), _lib.ptr(output), _lib.ptr(input_grad),
                 batch_dim, feat_dim, _lib.row_stride(flattened_output_grad), _lib.row_stride(output),
