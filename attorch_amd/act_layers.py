@@ -14,9 +14,10 @@ from typing import Any, Optional, Tuple
 import torch
 from torch import Tensor
 from torch import nn
-from torch.amp import custom_bwd, custom_fwd
+from torch.amp import custom_fwd
 
 from . import _lib
+from .utils import custom_bwd
 from .act import act_id, parse_act_func
 
 
@@ -92,7 +93,7 @@ class ActFuncAutoGrad(torch.autograd.Function):
         return _launch_forward(input, ctx.act, ctx.param, ctx.drop_p, ctx.seed)
 
     @staticmethod
-    @custom_bwd(device_type='cuda')
+    @custom_bwd
     def backward(
         ctx: Any,
         output_grad: Tensor,
@@ -155,7 +156,7 @@ class DropoutAutoGrad(torch.autograd.Function):
         return _launch_forward(input, 0, 0.0, ctx.drop_p, ctx.seed)
 
     @staticmethod
-    @custom_bwd(device_type='cuda')
+    @custom_bwd
     def backward(
         ctx: Any,
         output_grad: Tensor,

@@ -13,9 +13,10 @@ from typing import Any, Optional, Tuple
 import torch
 from torch import Tensor
 from torch import nn
-from torch.amp import custom_bwd, custom_fwd
+from torch.amp import custom_fwd
 
 from . import _lib
+from .utils import custom_bwd
 from .act import act_id, parse_act_func
 
 
@@ -144,7 +145,7 @@ class BatchNormAutoGrad(torch.autograd.Function):
         return output.view_as(input)
 
     @staticmethod
-    @custom_bwd(device_type='cuda')
+    @custom_bwd
     def backward(
         ctx: Any,
         output_grad: Tensor,

@@ -11,10 +11,10 @@ from typing import Any, Optional, Tuple
 import torch
 from torch import Tensor
 from torch import nn
-from torch.amp import custom_bwd, custom_fwd
+from torch.amp import custom_fwd
 
 from . import _lib
-from .utils import get_output_dtype
+from .utils import custom_bwd, get_output_dtype
 
 
 def _param_for_kernel(param: Optional[Tensor], input: Tensor) -> Optional[Tensor]:
@@ -234,7 +234,7 @@ class RMSNormAutoGrad(torch.autograd.Function):
         return output.view_as(input)
 
     @staticmethod
-    @custom_bwd(device_type='cuda')
+    @custom_bwd
     def backward(
         ctx: Any,
         output_grad: Tensor,

@@ -2,6 +2,7 @@
 Mixed-precision dtype policy shared by the layers.
 """
 
+import functools
 from typing import Optional
 
 import torch
@@ -43,3 +44,25 @@ def get_output_dtype(
         return torch.float32
     raise RuntimeError(f'Autocast type {autocast} is invalid. '
                        'Options are None, fp16, and fp32')
+
+
+def custom_bwd(bwd):
+    """
+    Runs ``backward`` in the autocast state its ``forward`` (decorated with
+    ``torch.amp.custom_fwd(device_type='cuda')``) ran in, like
+    ``torch.amp.custom_bwd(device_type='cuda')`` as the reference uses it
+    (e.g. attorch/act_layers.py:83).  torch's decorator builds and enters an autocast context
+    on every call; the autograd thread almost always is in that state already (no autocast in
+    either pass), and then this one calls ``backward`` directly.
+    """
+    @functools.wraps(bwd)
+    def decorate_bwd(ctx, *args, **kwargs):
+        enabled = ctx._fwd_used_autocast
+        if torch.is_autocast_enabled('cuda') == enabled and (
+                not enabled or torch.get_autocast_dtype('cuda') == ctx._dtype):
+            return bwd(ctx, *args, **kwargs)
+        with torch.autocast(device_type='cuda', enabled=enabled, dtype=ctx._dtype):
+            return bwd(ctx, *args, **kwargs)
+
+    return decorate_bwd
+
