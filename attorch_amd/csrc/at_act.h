@@ -109,4 +109,22 @@ __device__ __forceinline__ float act_derivative(int act, float x, float p) {
   }
 }
 
+// Runs the statement(s) with `ACT` a compile-time constant equal to the runtime id: inside, calls
+// of act_forward(ACT, ...) / act_derivative(ACT, ...) fold to the one formula, so a loop over many
+// elements pays for the choice once instead of once per element.
+#define AT_ACT_DISPATCH(ACT_VALUE, ...)                                                               \
+  switch (ACT_VALUE) {                                                                                \
+    case 0: { constexpr int ACT = 0; __VA_ARGS__; break; }   case 1: { constexpr int ACT = 1; __VA_ARGS__; break; }   \
+    case 2: { constexpr int ACT = 2; __VA_ARGS__; break; }   case 3: { constexpr int ACT = 3; __VA_ARGS__; break; }   \
+    case 4: { constexpr int ACT = 4; __VA_ARGS__; break; }   case 5: { constexpr int ACT = 5; __VA_ARGS__; break; }   \
+    case 6: { constexpr int ACT = 6; __VA_ARGS__; break; }   case 7: { constexpr int ACT = 7; __VA_ARGS__; break; }   \
+    case 8: { constexpr int ACT = 8; __VA_ARGS__; break; }   case 9: { constexpr int ACT = 9; __VA_ARGS__; break; }   \
+    case 10: { constexpr int ACT = 10; __VA_ARGS__; break; } case 11: { constexpr int ACT = 11; __VA_ARGS__; break; } \
+    case 12: { constexpr int ACT = 12; __VA_ARGS__; break; } case 13: { constexpr int ACT = 13; __VA_ARGS__; break; } \
+    case 14: { constexpr int ACT = 14; __VA_ARGS__; break; } case 15: { constexpr int ACT = 15; __VA_ARGS__; break; } \
+    case 16: { constexpr int ACT = 16; __VA_ARGS__; break; } case 17: { constexpr int ACT = 17; __VA_ARGS__; break; } \
+    case 18: { constexpr int ACT = 18; __VA_ARGS__; break; } case 19: { constexpr int ACT = 19; __VA_ARGS__; break; } \
+    case 20: { constexpr int ACT = 20; __VA_ARGS__; break; } default: { constexpr int ACT = 21; __VA_ARGS__; break; } \
+  }
+
 }  // namespace at_hip

@@ -1454,13 +1454,22 @@ __global__ __launch_bounds__(256) void act_bwd_kernel(
         }
       }
     }
+    // the derivative's formula is chosen once per row block, not once per element
+    auto derive = [&](auto act_c) {
+      constexpr int ACT = decltype(act_c)::value;
+#pragma unroll
+      for (int u = 0; u < ROWS; ++u)
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) zz[u][j] = act_derivative(ACT, zz[u][j], param);
+    };
+    AT_ACT_DISPATCH(act, derive(std::integral_constant<int, ACT>()));
 #pragma unroll
     for (int u = 0; u < ROWS; ++u) {
       const int64_t r = rb + u;
       if (r < r1) {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
-          d[u][j] = to_f32(from_f32<TZ>(d[u][j] * act_derivative(act, zz[u][j], param)));  // summed as stored
+          d[u][j] = to_f32(from_f32<TZ>(d[u][j] * zz[u][j]));  // summed as stored
           sum[j] += d[u][j];
         }
         if (VEC_OK) store_f32<TZ, VEC>(dz + r * dzs + c, d[u]);
@@ -1476,6 +1485,90 @@ __global__ __launch_bounds__(256) void act_bwd_kernel(
 #pragma unroll
     for (int j = 0; j < VEC; ++j)
       if (c + j < N) part[(int64_t)blockIdx.y * N + c + j] = sum[j];
+  }
+}
+
+// The same pass for whole 16-byte vectors, shaped for bandwidth: a workgroup is 32 column lanes (8
+// columns each) times 8 row lanes of kActTileRows / 8 rows each, i.e. one tile of 32 rows x 256
+// columns per step, and as a rule one step per workgroup (grid = (N / 256, row slices of 32
+// rows)).  Many short-lived workgroups keep more bytes in flight than few long-lived ones: in a
+// loop the next loads queue behind the acknowledgement of the wave's own stores.  The column
+// sums of the 8 row lanes are folded through LDS in a fixed order.
+constexpr int kActTileRows = 32, kActTileCols = 256;
+template <typename TDY, typename TZ>
+__global__ __launch_bounds__(256) void act_bwd_tile_kernel(
+    const TDY* __restrict__ dy, const TZ* __restrict__ z, TZ* __restrict__ dz, float* __restrict__ part,
+    int64_t M, int N, int64_t dys, int64_t zs, int64_t dzs, int act, float param, int64_t rows_per_slice) {
+  constexpr int VEC = 8, ROWS = kActTileRows / 8;
+  constexpr int ND = (int)sizeof(TDY) * VEC / 16, NZ = (int)sizeof(TZ) * VEC / 16;   // 16-byte vectors per row
+  __shared__ float fold[8][32][VEC + 1];
+  const int cx = threadIdx.x & 31, ry = threadIdx.x >> 5;
+  const int c = (blockIdx.x * 32 + cx) * VEC;
+  const bool in_cols = c < N;
+  const int cc = in_cols ? c : 0;   // lanes past the last column work on column 0 and drop the result
+  const int64_t r0 = (int64_t)blockIdx.y * rows_per_slice;
+  const int64_t r1 = r0 + rows_per_slice < M ? r0 + rows_per_slice : M;
+  float sum[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) sum[j] = 0.f;
+  for (int64_t rb = r0 + ry * ROWS; rb < r1; rb += kActTileRows) {
+    uint4 rd[ROWS][ND], rz[ROWS][NZ];
+#pragma unroll
+    for (int u = 0; u < ROWS; ++u) {
+      const int64_t r = rb + u < r1 ? rb + u : r1 - 1;   // past the slice: its last row again, not used
+#pragma unroll
+      for (int q = 0; q < ND; ++q) rd[u][q] = reinterpret_cast<const uint4*>(dy + r * dys + cc)[q];
+#pragma unroll
+      for (int q = 0; q < NZ; ++q) rz[u][q] = reinterpret_cast<const uint4*>(z + r * zs + cc)[q];
+    }
+    float d[ROWS][VEC], zz[ROWS][VEC];
+#pragma unroll
+    for (int u = 0; u < ROWS; ++u) {
+      union { uint4 raw[ND]; TDY e[VEC]; } ud;
+      union { uint4 raw[NZ]; TZ e[VEC]; } uz;
+#pragma unroll
+      for (int q = 0; q < ND; ++q) ud.raw[q] = rd[u][q];
+#pragma unroll
+      for (int q = 0; q < NZ; ++q) uz.raw[q] = rz[u][q];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        d[u][j] = to_f32(ud.e[j]);
+        zz[u][j] = to_f32(uz.e[j]);
+      }
+    }
+    auto derive = [&](auto act_c) {
+      constexpr int ACT = decltype(act_c)::value;
+#pragma unroll
+      for (int u = 0; u < ROWS; ++u)
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) zz[u][j] = act_derivative(ACT, zz[u][j], param);
+    };
+    AT_ACT_DISPATCH(act, derive(std::integral_constant<int, ACT>()));
+#pragma unroll
+    for (int u = 0; u < ROWS; ++u) {
+      const int64_t r = rb + u;
+      if (r < r1 && in_cols) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          d[u][j] = to_f32(from_f32<TZ>(d[u][j] * zz[u][j]));  // summed as stored
+          sum[j] += d[u][j];
+        }
+        store_f32<TZ, VEC>(dz + r * dzs + c, d[u]);
+      }
+    }
+  }
+  if (part) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) fold[ry][cx][j] = sum[j];
+    __syncthreads();
+    // lane (cx, j') sums column cx * 8 + j' over the 8 row lanes, always in the same order
+    const int col = threadIdx.x;   // 0 .. 255: column of the tile
+    const int fx = col >> 3, fj = col & 7;
+    float t = 0.f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) t += fold[k][fx][fj];
+    const int64_t gc = (int64_t)blockIdx.x * kActTileCols + col;
+    if (gc < N) part[(int64_t)blockIdx.y * N + gc] = t;
   }
 }
 
@@ -1933,6 +2026,31 @@ int at_act_bwd(const void* output_grad, const void* input, void* input_grad, voi
   const bool vec_ok = cols % 8 == 0 && aligned16(output_grad) && aligned16(input) && aligned16(input_grad) &&
                       (output_grad_stride * gs) % 16 == 0 && (input_stride * is) % 16 == 0 &&
                       (input_grad_stride * is) % 16 == 0;
+  float* part = bias_grad ? (float*)workspace : nullptr;
+  if (vec_ok) {
+    // tiles of 32 rows x 256 columns, one per workgroup unless the partial buffer would outgrow
+    // its slices (then a workgroup walks down several tiles)
+    const unsigned gx = (unsigned)cdiv64(cols, kActTileCols);
+    int64_t slices = cdiv64(rows, kActTileRows);
+    const int64_t max_slices = bias_grad ? kActBwdMaxSlices : 65535;
+    if (slices > max_slices) slices = max_slices;
+    int64_t rows_per_slice = cdiv64(cdiv64(rows, slices), kActTileRows) * kActTileRows;
+    slices = cdiv64(rows, rows_per_slice);
+    int rc = dispatch_dtype(grad_dtype, [&](auto* tg) -> int {
+      typedef std::remove_pointer_t<decltype(tg)> TG;
+      return dispatch_dtype(input_dtype, [&](auto* tz) -> int {
+        typedef std::remove_pointer_t<decltype(tz)> TZ;
+        hipLaunchKernelGGL((act_bwd_tile_kernel<TG, TZ>), dim3(gx, (unsigned)slices), dim3(256), 0,
+                           (hipStream_t)stream, (const TG*)output_grad, (const TZ*)input, (TZ*)input_grad, part, rows,
+                           (int)cols, output_grad_stride, input_stride, input_grad_stride, act, param, rows_per_slice);
+        return launch_status();
+      });
+    });
+    if (rc || !bias_grad) return rc;
+    hipLaunchKernelGGL(colsum_final_kernel, dim3((unsigned)cdiv64(cols, kColsumFinalCols)), dim3(256), 0,
+                       (hipStream_t)stream, (const float*)workspace, bias_grad, bias_grad_dtype, (int)slices, (int)cols);
+    return launch_status();
+  }
   // enough workgroups to fill the chip, few enough row slices to keep the partial buffer small
   const unsigned gx = (unsigned)cdiv64(cols, 256 * 8);
   int64_t slices = cdiv64((int64_t)device_cu_count() * 16, gx);
@@ -1940,7 +2058,6 @@ int at_act_bwd(const void* output_grad, const void* input, void* input_grad, voi
   if (slices > rows) slices = rows;
   const int64_t rows_per_slice = cdiv64(rows, slices);
   slices = cdiv64(rows, rows_per_slice);
-  float* part = bias_grad ? (float*)workspace : nullptr;
   int rc = dispatch_dtype(grad_dtype, [&](auto* tg) -> int {
     typedef std::remove_pointer_t<decltype(tg)> TG;
     return dispatch_dtype(input_dtype, [&](auto* tz) -> int {
