@@ -30,17 +30,16 @@ __global__ __launch_bounds__(256) void glu_kernel(const T* __restrict__ input, c
     load_f32<T, VEC>(x1p + half, x2);
     if (!BACKWARD) {
       float y[VEC];
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) y[j] = x1[j] * act_forward(act, x2[j], param);
+      // the activation's formula is chosen once per vector, not once per element
+      AT_ACT_DISPATCH(act, _Pragma("unroll") for (int j = 0; j < VEC; ++j) y[j] = x1[j] * act_forward(ACT, x2[j], param));
       store_f32<T, VEC>(out + o * half + l, y);
     } else {
       float dy[VEC], d1[VEC], d2[VEC];
       load_f32<T, VEC>(output_grad + o * half + l, dy);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        d1[j] = dy[j] * act_forward(act, x2[j], param);
-        d2[j] = dy[j] * x1[j] * act_derivative(act, x2[j], param);
-      }
+      AT_ACT_DISPATCH(act, _Pragma("unroll") for (int j = 0; j < VEC; ++j) {
+        d1[j] = dy[j] * act_forward(ACT, x2[j], param);
+        d2[j] = dy[j] * x1[j] * act_derivative(ACT, x2[j], param);
+      });
       T* g1 = out + (o * 2) * half + l;
       store_f32<T, VEC>(g1, d1);
       store_f32<T, VEC>(g1 + half, d2);
@@ -60,7 +59,9 @@ int launch(const void* input, const void* output_grad, void* out, int64_t outer,
   const bool vector = half % vec == 0 && aligned16(input) && aligned16(out) && (!BACKWARD || aligned16(output_grad));
   const int64_t items = outer * (vector ? half / vec : half);
   int64_t blocks = cdiv64(items, 256);
-  const int64_t cap = (int64_t)device_cu_count() * 16;
+  // as a rule one vector per lane and one step per workgroup: short-lived waves keep more bytes
+  // in flight than a capped grid whose lanes loop (their next loads queue behind their own stores)
+  const int64_t cap = (int64_t)1 << 22;
   if (blocks > cap) blocks = cap;
   const bool small = outer * half * 2 + 16 < ((int64_t)1 << 31);
   auto go = [&](auto* tp, auto idx, auto vflag) -> int {

@@ -230,7 +230,9 @@ int at_nll_loss_bwd(const void* output_grad, const int64_t* target, const void* 
   const int64_t total = batch * feat * spatial;
   const int64_t n_vec = cdiv64(total, 16 / dtype_size(out_dtype));
   int64_t blocks = cdiv64(n_vec, kNllBlock);
-  const int64_t cap = (int64_t)device_cu_count() * 16;
+  // as a rule one step per workgroup: short-lived waves keep more bytes in flight than a capped
+  // grid whose lanes loop (their next loads queue behind their own stores)
+  const int64_t cap = (int64_t)1 << 22;
   if (blocks > cap) blocks = cap;
   const float inv_count = 1.0f / (float)(batch * spatial);
   const bool vector_ok = aligned16(input_grad);
