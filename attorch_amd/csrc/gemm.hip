@@ -1164,14 +1164,40 @@ template <bool A_MC, bool B_KC, int TK>
 __global__ __launch_bounds__(kSplitThreads) void gemm_f32_split_kernel(GemmArgs g) {
   __shared__ __align__(16) float smem[SplitShape<TK>::kSmemFloats];
   const int nbn = (g.N + 31) / 32;
-  const SplitTile t{reinterpret_cast<const float*>(g.a), reinterpret_cast<const float*>(g.b), nullptr,
-                    g.lda, g.ldb, 0, g.M, g.N, g.K, (int)(blockIdx.x / nbn) * 32, (int)(blockIdx.x % nbn) * 32,
+  // g.partial (weight-gradient layout only: both operands stored [k][row]): workgroup row y of
+  // the grid contracts k-tiles [y * kt_per_split, (y + 1) * kt_per_split) and leaves its tile in
+  // partial[y] for gemm_split_finish_kernel
+  const int k_begin = g.partial ? (int)blockIdx.y * g.kt_per_split * TK : 0;
+  const int k_len = g.partial ? (g.K - k_begin < g.kt_per_split * TK ? g.K - k_begin : g.kt_per_split * TK) : g.K;
+  const SplitTile t{reinterpret_cast<const float*>(g.a) + (int64_t)k_begin * g.lda,
+                    reinterpret_cast<const float*>(g.b) + (int64_t)k_begin * g.ldb, nullptr,
+                    g.lda, g.ldb, 0, g.M, g.N, k_len, (int)(blockIdx.x / nbn) * 32, (int)(blockIdx.x % nbn) * 32,
                     AT_ACT_NONE, 0.f};
   const f32x16 acc = split_tile<A_MC, B_KC, TK, 0, false>(t, smem, nullptr);
   if (threadIdx.x >= 64) return;
   __builtin_amdgcn_wave_barrier();
   static_assert(32 * 36 <= SplitShape<TK>::kFoldFloats, "the epilogue block fits");
-  wave_tile_epilogue<float>(acc, smem, g, t.m0, t.n0);
+  if (g.partial) {
+    GemmArgs to_partial = g;
+    to_partial.c = g.partial + (int64_t)blockIdx.y * g.M * g.ldw;
+    to_partial.ldc = g.ldw;
+    wave_tile_epilogue<float>(acc, smem, to_partial, t.m0, t.n0);
+  } else {
+    wave_tile_epilogue<float>(acc, smem, g, t.m0, t.n0);
+  }
+}
+
+// Slices of the batch for a small fp32 weight gradient (few 32x32 tiles, a long contraction):
+// enough to give every CU two workgroups, each slice at least 8 k-tiles of 128 long.  1 = none.
+inline int dw_split_count_f32(int64_t M, int64_t N, int64_t K) {
+  const int64_t tiles = cdiv64(M, 32) * cdiv64(N, 32);
+  const int64_t want = (int64_t)device_cu_count() * 2 / tiles;
+  const int64_t kt = K / 128;
+  int64_t splits = want < kt / 8 ? want : kt / 8;
+  if (splits > 64) splits = 64;
+  if (splits < 2) return 1;
+  const int64_t per = cdiv64(cdiv64(K, 128), splits);
+  return (int)cdiv64(cdiv64(K, 128), per);   // no empty slice
 }
 
 // Backward pass of a small fp32 linear layer with an activation in one launch: the first
@@ -1845,6 +1871,21 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
     // outputs with fewer 64x64 tiles than CUs: 32x32 tiles, the contraction shared by the waves
     if (cdiv64(M, 64) * cdiv64(N, 64) < device_cu_count() && K >= 128 && (M % 4) == 0 && (N % 4) == 0) {
       const unsigned grid = (unsigned)(cdiv64(M, 32) * cdiv64(N, 32));
+      if (layout == kDw && workspace && K >= 512) {
+        const int splits = dw_split_count_f32(M, N, K);
+        const int64_t pitch = dw_partial_pitch(N);
+        if (splits > 1 && workspace_bytes >= (int64_t)splits * M * pitch * 4) {
+          g.partial = (float*)workspace;
+          g.kt_per_split = (int)cdiv64(cdiv64(K, 128), splits);
+          g.ldw = (int)pitch;
+          hipLaunchKernelGGL((gemm_f32_split_kernel<true, false, 128>), dim3(grid, (unsigned)splits), dim3(kSplitThreads),
+                             0, stream, g);
+          const int64_t items = M * (pitch / 8);
+          hipLaunchKernelGGL((gemm_split_finish_kernel<float>), dim3((unsigned)cdiv64(items, 256)), dim3(256), 0, stream,
+                             (const float*)workspace, (float*)c, (int)M, (int)N, (int)pitch, ldc, splits);
+          return launch_status();
+        }
+      }
 #define AT_SPLIT_LAUNCH(TK)                                                                                              \
   {                                                                                                                      \
     if (layout == kDx)                                                                                                   \
@@ -1988,6 +2029,14 @@ int at_linear_bwd_small(const void* output_grad, const void* pre_act, const void
 int64_t at_linear_bwd_weight_workspace_bytes(int64_t batch, int64_t in_feat, int64_t out_feat, int dtype) {
   if (batch <= 0 || in_feat <= 0 || out_feat <= 0 || !dtype_valid(dtype)) return 0;
   if (out_feat <= kSkinnyCols) return skinny_dw_workspace_bytes(batch, in_feat);
+  if (dtype == AT_DTYPE_F32) {
+    // the condition under which run_gemm takes the 32x32-tile kernel, and its slices of the batch
+    if (cdiv64(in_feat, 64) * cdiv64(out_feat, 64) >= device_cu_count() || batch < 512 || in_feat % 4 || out_feat % 4 ||
+        in_feat < 32 || out_feat < 32)
+      return 0;
+    const int splits = dw_split_count_f32(in_feat, out_feat, batch);
+    return splits > 1 ? (int64_t)splits * in_feat * dw_partial_pitch(out_feat) * 4 : 0;
+  }
   if (dtype != AT_DTYPE_F16 && dtype != AT_DTYPE_BF16) return 0;
   if (in_feat < 64 || out_feat < 64 || in_feat * out_feat < (int64_t)MT * MT) return 0;
   if (!prefer_mid_tiles(in_feat, out_feat)) return 0;

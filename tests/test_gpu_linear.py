@@ -150,6 +150,31 @@ def test_weight_grad_split_agrees_with_one_piece(batch, in_dim, out_dim, dtype) 
     torch.testing.assert_close(dw.double().cpu(), results[0], rtol=0, atol=0)
 
 
+@pytest.mark.parametrize('batch, in_dim, out_dim', [(32768, 256, 256), (5000, 100, 96), (8192, 64, 384), (2048, 32, 36)])
+def test_fp32_weight_grad_slices_of_the_batch(batch, in_dim, out_dim) -> None:
+    """
+    C ABI: a small fp32 weight gradient with a long batch is computed in slices of the batch when
+    the caller passes the workspace (fixed-order sum of fp32 partial tiles); with and without it
+    the result is the float64 product to fp32 accumulation error.
+    """
+    from attorch_amd import _lib
+    lib = _lib.load()
+    x = randn((batch, in_dim), 1).cuda()
+    dz = randn((batch, out_dim), 2).cuda()
+    stream = _lib.stream_of(x)
+    workspace_bytes = lib.at_linear_bwd_weight_workspace_bytes(batch, in_dim, out_dim, 0)
+    assert workspace_bytes > 0
+    expected = x.double().cpu().T @ dz.double().cpu()
+    for use_workspace in (False, True):
+        dw = torch.full((in_dim, out_dim), float('nan'), device='cuda')
+        workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device='cuda') if use_workspace else None
+        _lib.check(lib.at_linear_bwd_weight(
+            _lib.ptr(x), _lib.ptr(dz), _lib.ptr(dw), _lib.ptr(workspace), workspace_bytes if use_workspace else 0,
+            batch, in_dim, out_dim, in_dim, out_dim, out_dim, 0, 0, stream), 'at_linear_bwd_weight')
+        assert_close(dw, expected, torch.float32, f'weight_grad, workspace={use_workspace}', batch_reduction=True,
+                     dot_terms=batch)
+
+
 @pytest.mark.parametrize('dtype', DTYPES)
 def test_extent_one_dimensions_with_arbitrary_strides(dtype) -> None:
     """
