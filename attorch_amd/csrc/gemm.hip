@@ -230,11 +230,27 @@ __device__ __forceinline__ void big_tile_epilogue(f32x16 (&acc)[4][kBigNJ], char
       if (rows16) {
         *reinterpret_cast<uint4*>(out) = v;
       } else {
-        union { uint4 raw; T e[8]; } u;
-        u.raw = v;
+        // Rows that do not start on 16-byte boundaries (an odd row stride) or a tile that sticks
+        // out over the last column: the row segment is still written as whole 16-byte vectors
+        // wherever memory allows — lane j takes the j-th aligned vector inside the segment and
+        // gathers its 8 elements from LDS — and only the few elements before the first and after
+        // the last aligned vector go out one by one.
+        const int j = threadIdx.x & 31;
+        const int ncols = g.N - n0 < BN ? g.N - n0 : BN;
+        T* seg = dst + (int64_t)m * ldd + n0;
+        const T* src = reinterpret_cast<const T*>(lds + ml * kEpiPitch);
+        const int head = (int)(((16 - (reinterpret_cast<uintptr_t>(seg) & 15)) & 15) >> 1);   // elements before the first boundary
+        const int first = head < ncols ? head : ncols;
+        const int nfull = (ncols - first) >> 3;
+        if (j < nfull) {
+          union { uint4 raw; T e[8]; } u;
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (n0 + cseg + e < g.N) out[e] = u.e[e];
+          for (int e = 0; e < 8; ++e) u.e[e] = src[first + j * 8 + e];
+          *reinterpret_cast<uint4*>(seg + first + j * 8) = u.raw;
+        }
+        if (j < first) seg[j] = src[j];
+        const int tail0 = first + nfull * 8;
+        if (tail0 + j < ncols && j < 8) seg[tail0 + j] = src[tail0 + j];
       }
     }
   }

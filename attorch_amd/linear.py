@@ -123,14 +123,27 @@ class LinearAutoGrad(torch.autograd.Function):
         if bias_k is not None and output_dtype != input.dtype:
             bias_k = bias_k.to(output_dtype)
         contract_dim = in_feat_dim
+        ctx.padded_weight = None
         if _pad_features(batch_dim, in_feat_dim, out_feat_dim, compute_dtype):
             # zeros along the contraction add nothing; padded output columns are never stored
             contract_dim = _round_up8(in_feat_dim)
             input_k = _zero_pad(input_k, batch_dim, contract_dim)
             weight_k = _zero_pad(weight_k, contract_dim, _round_up8(out_feat_dim))
+            if input.requires_grad:
+                # the input gradient multiplies by the same padded copy: keep it instead of
+                # padding the weight a second time
+                ctx.padded_weight = weight_k
 
         output = torch.empty((batch_dim, out_feat_dim), device=input.device, dtype=output_dtype)
-        pre_act = torch.empty_like(output) if save_pre_act else output
+        if save_pre_act and ctx.padded_weight is not None and out_feat_dim % 8:
+            # the saved pre-activation gets rows that start on 16-byte boundaries (row stride
+            # rounded up, the spare columns zero): the kernels then write and later read it in
+            # whole vectors
+            padded = torch.empty((batch_dim, _round_up8(out_feat_dim)), device=input.device, dtype=output_dtype)
+            padded[:, out_feat_dim:].zero_()
+            pre_act = padded[:, :out_feat_dim]
+        else:
+            pre_act = torch.empty_like(output) if save_pre_act else output
 
         with _lib.device_guard(input):
             _lib.check(lib.at_linear_fwd(
@@ -202,8 +215,31 @@ class LinearAutoGrad(torch.autograd.Function):
 
         with _lib.device_guard(input):
             bias_grad = None
+            padded_cols = _round_up8(out_feat_dim)
             if ctx.act_func is None:
                 pre_act_grad = output_grad
+            elif (pre_act.stride(0) == padded_cols and padded_cols != out_feat_dim
+                  and output_grad.dtype is pre_act.dtype):
+                # rows of the saved pre-activation are padded to whole vectors (see forward): one
+                # zero-padded copy of the output gradient lets the activation gradient run on whole
+                # vectors too, and its result is the padded operand both products need
+                output_grad_p = _zero_pad(output_grad, batch_dim, padded_cols)
+                pre_act_grad_p = torch.empty((batch_dim, padded_cols), dtype=pre_act.dtype, device=device)
+                bias_grad_p = workspace = None
+                workspace_bytes = 0
+                if ctx.bias_requires_grad:
+                    bias_grad_p = torch.empty(padded_cols, dtype=pre_act.dtype, device=device)
+                    workspace_bytes = lib.at_act_bwd_workspace_bytes(batch_dim, padded_cols)
+                    workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=device)
+                _lib.check(lib.at_act_bwd(
+                    _lib.ptr(output_grad_p), _lib.ptr(pre_act), _lib.ptr(pre_act_grad_p),
+                    _lib.ptr(bias_grad_p), _lib.ptr(workspace), workspace_bytes,
+                    batch_dim, padded_cols, padded_cols, padded_cols, padded_cols, ctx.act,
+                    0.0 if ctx.param is None else ctx.param, _lib.dtype_id(pre_act.dtype),
+                    _lib.dtype_id(pre_act.dtype), _lib.dtype_id(pre_act.dtype), stream), 'at_act_bwd')
+                pre_act_grad = pre_act_grad_p[:, :out_feat_dim]
+                if bias_grad_p is not None:
+                    bias_grad = bias_grad_p[:out_feat_dim].clone()
             else:
                 pre_act_grad = torch.empty((batch_dim, out_feat_dim), dtype=pre_act.dtype,
                                            device=device)
@@ -229,12 +265,19 @@ class LinearAutoGrad(torch.autograd.Function):
             contract_dim = out_feat_dim
             if pad:
                 contract_dim = _round_up8(out_feat_dim)
-                grad_mm = _zero_pad(grad_mm, batch_dim, contract_dim)
+                if grad_mm.stride(0) == contract_dim and grad_mm.shape[1] != contract_dim:
+                    # a view of a buffer whose rows are padded with zeros already
+                    grad_mm = grad_mm.as_strided((batch_dim, contract_dim), (contract_dim, 1))
+                else:
+                    grad_mm = _zero_pad(grad_mm, batch_dim, contract_dim)
             input_grad = weight_grad = None
             if input.requires_grad:
-                weight_mm = _matrix(weight.to(output_dtype))
-                if pad:
-                    weight_mm = _zero_pad(weight_mm, in_feat_dim, contract_dim)
+                if pad and ctx.padded_weight is not None and ctx.padded_weight.dtype is output_dtype:
+                    weight_mm = ctx.padded_weight
+                else:
+                    weight_mm = _matrix(weight.to(output_dtype))
+                    if pad:
+                        weight_mm = _zero_pad(weight_mm, in_feat_dim, contract_dim)
                 input_grad = torch.empty((batch_dim, in_feat_dim), dtype=output_dtype, device=device)
                 _lib.check(lib.at_linear_bwd_input(
                     _lib.ptr(grad_mm), _lib.ptr(weight_mm), _lib.ptr(input_grad), batch_dim,

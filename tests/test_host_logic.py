@@ -132,10 +132,12 @@ def test_argument_errors_without_gpu() -> None:
                                    None) == -1
     assert lib.at_linear_bwd_small(p, None, p, p, p, p, None, 512, 784, 256, 256, 256, 784, 256, 784, 256, 4, 0.0, 0,
                                    None) == -1     # an activation needs its pre-activation
-    # weight gradient of the linear layer: slices of the batch only for 16-bit tensors, a long
-    # batch and a weight matrix that is small next to the GPU
+    # weight gradient of the linear layer: slices of the batch for a long batch and a weight
+    # matrix that is small next to the GPU
     assert lib.at_linear_bwd_weight_workspace_bytes(16384, 256, 256, 2) >= 2 * 256 * 256 * 4
-    assert lib.at_linear_bwd_weight_workspace_bytes(16384, 256, 256, 0) == 0
+    assert lib.at_linear_bwd_weight_workspace_bytes(16384, 256, 256, 0) >= 2 * 256 * 256 * 4
+    assert lib.at_linear_bwd_weight_workspace_bytes(512, 256, 256, 0) == 0
+    assert lib.at_linear_bwd_weight_workspace_bytes(16384, 4096, 4096, 0) == 0
     assert lib.at_linear_bwd_weight_workspace_bytes(64, 256, 256, 2) == 0
     assert lib.at_linear_bwd_weight_workspace_bytes(16384, 8192, 8192, 2) == 0
     assert lib.at_linear_bwd_weight(None, p, p, None, 0, 4, 8, 8, 8, 8, 8, 0, 0, None) == -1
