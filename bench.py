@@ -38,22 +38,22 @@ PEAK_MFMA_FP32_TFLOPS = 157.3    # dense fp32 MFMA
 # the 256 MB Infinity Cache serves are included.  They belong to the kernel sources whose digest is
 # TRAFFIC_SOURCE_DIGEST: when the sources of the loaded library differ, `traffic` is reported as
 # null and the recorded figure moves to `traffic_recorded` (stale until the profile is redone).
-TRAFFIC_SOURCE_DIGEST = 'fe9baa43d82379cd'
+TRAFFIC_SOURCE_DIGEST = '06fbb0d30cdfd740'
 MEASURED_TRAFFIC_BYTES = {
-    'c4_linear_fwd': 4460356697,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.0 GiB read, 1.0 GiB written
-    'c2_layer_norm': 362354506,       # norm_fwd + norm_bwd + reduce_partials
-    'c2_rms_norm': 361818420,
-    'c2_softmax': 336104804,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
-    'c2_act_dropout': 336035692,      # act_dropout forward + backward
-    'c2_glu': 269058606,              # glu forward + backward
-    'c2_mse': 335737106,              # p_loss forward + backward
-    'c3_cross_entropy': 1718021568,   # ce_row_kernel (ignored rows are not read)
-    'c3_cross_entropy_autocast': 2450300586,
-    'c3_nll_loss': 826986631,         # nll forward (a gather) + the single-pass gradient write
-    'c5_conv_channels_last': 481402106,     # the two window kernels + weight gradient + weight reorders, no copies
-    'c5_conv': 687269000,             # 2 window kernels + weight gradient + 2 layout copies + weight reorders
-    'c5_batch_norm_channels_last': 568594843,
-    'c5_batch_norm': 565712634,       # stats + apply + backward reduce + backward apply
+    'c4_linear_fwd': 4517018597,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.0 GiB read, 1.0 GiB written
+    'c2_layer_norm': 362345481,       # norm_fwd + norm_bwd + reduce_partials
+    'c2_rms_norm': 361807943,
+    'c2_softmax': 336095690,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
+    'c2_act_dropout': 335784954,      # act_dropout forward + backward
+    'c2_glu': 268580569,              # glu forward + backward
+    'c2_mse': 335721710,              # p_loss forward + backward
+    'c3_cross_entropy': 1717963287,   # ce_row_kernel (ignored rows are not read)
+    'c3_cross_entropy_autocast': 2450455893,
+    'c3_nll_loss': 826879974,         # nll forward (a gather) + the single-pass gradient write
+    'c5_conv_channels_last': 389735315,     # the two weights-in-registers kernels + weight gradient + weight reorders, no copies
+    'c5_conv': 595389513,             # the same + 2 layout copies
+    'c5_batch_norm_channels_last': 568572906,
+    'c5_batch_norm': 565690725,       # stats + apply + backward reduce + backward apply
 }
 
 
