@@ -197,3 +197,38 @@ def test_host_tensors_raise_instead_of_faulting() -> None:
         torch.autograd.grad(y, x, torch.ones(8, 16))       # upstream gradient on the host
     with pytest.raises(RuntimeError, match='there is no CPU path'):
         attorch_amd.Softmax(dim=-1)(torch.zeros(2, 3))
+
+
+def test_custom_bwd_restores_the_forward_autocast_state() -> None:
+    """
+    utils.custom_bwd must behave like torch.amp.custom_bwd(device_type='cuda'): backward sees the
+    autocast state (and dtype) its forward ran in, whatever the state of the calling thread.
+    """
+    from torch.amp import custom_fwd
+    from attorch_amd.utils import custom_bwd
+    seen = []
+
+    class Probe(torch.autograd.Function):
+        @staticmethod
+        @custom_fwd(device_type='cuda')
+        def forward(ctx, x):
+            return x * 2
+
+        @staticmethod
+        @custom_bwd
+        def backward(ctx, g):
+            seen.append((torch.is_autocast_enabled('cuda'), torch.get_autocast_dtype('cuda')))
+            return g * 2
+
+    x = torch.ones(3, requires_grad=True, device='cuda')
+    Probe.apply(x).sum().backward()                       # no autocast anywhere
+    with torch.autocast('cuda', dtype=torch.bfloat16):
+        y = Probe.apply(x)
+    y.sum().backward()                                    # forward under autocast, backward outside
+    y = Probe.apply(x)
+    with torch.autocast('cuda', dtype=torch.float16):
+        y.sum().backward()                                # forward outside, backward called inside
+    assert seen[0][0] is False
+    assert seen[1] == (True, torch.bfloat16)
+    assert seen[2][0] is False
+    assert not torch.is_autocast_enabled('cuda')
