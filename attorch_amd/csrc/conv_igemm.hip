@@ -1123,22 +1123,42 @@ __global__ __launch_bounds__(kRowsWaves * 64) void conv_dw_rows_kernel(DwRowsArg
 template <typename T>
 __global__ __launch_bounds__(256) void conv_dw_finish_kernel(const float* __restrict__ part, T* __restrict__ dw,
                                                               int splits, int Cg, int taps, int64_t total) {
-  __shared__ float sm[4][64];
-  const int col = threadIdx.x & 63, slice = threadIdx.x >> 6;
-  const int64_t i = (int64_t)blockIdx.x * 64 + col;   // index into a partial: (o, tap, c)
-  float s = 0.f;
+  // 16 lanes of 4 consecutive partial elements each (one 16-byte load per split) times 16 slice
+  // lanes that stride the splits, 8 loads in flight per lane; the 16 slice sums are folded
+  // through LDS in a fixed order.  total % 4 == 0 (the contraction channels are padded to 64).
+  __shared__ float4 sm[16][16];
+  const int col = threadIdx.x & 15, slice = threadIdx.x >> 4;
+  const int64_t i = ((int64_t)blockIdx.x * 16 + col) * 4;   // index into a partial: (o, tap, c)
+  float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
   if (i < total) {
-#pragma unroll 4
-    for (int sp = slice; sp < splits; sp += 4) s += part[(int64_t)sp * total + i];
+    const float* src = part + i;
+    for (int sp0 = slice; sp0 < splits; sp0 += 16 * 8) {
+      float4 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int sp = sp0 + 16 * u;
+        v[u] = *reinterpret_cast<const float4*>(src + (int64_t)(sp < splits ? sp : sp0) * total);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (sp0 + 16 * u < splits) {
+          s.x += v[u].x; s.y += v[u].y; s.z += v[u].z; s.w += v[u].w;
+        }
+    }
   }
   sm[slice][col] = s;
   __syncthreads();
-  if (slice == 0 && i < total) {
-    s = (sm[0][col] + sm[1][col]) + (sm[2][col] + sm[3][col]);
-    const int c = (int)(i % Cg);
-    const int tap = (int)((i / Cg) % taps);
-    const int64_t o = i / ((int64_t)Cg * taps);
-    dw[(o * Cg + c) * taps + tap] = from_f32<T>(s);
+  if (slice < 4 && i < total) {
+    // lane (col, e = slice) finishes element i + e
+    const int e = slice;
+    float t = 0.f;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) t += reinterpret_cast<const float*>(&sm[k][col])[e];
+    const int64_t idx = i + e;
+    const int c = (int)(idx % Cg);
+    const int tap = (int)((idx / Cg) % taps);
+    const int64_t o = idx / ((int64_t)Cg * taps);
+    dw[(o * Cg + c) * taps + tap] = from_f32<T>(t);
   }
 }
 
