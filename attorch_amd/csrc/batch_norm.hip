@@ -437,7 +437,8 @@ constexpr int kMaxSplits = 1024;
 // ------------------------------------------------------------------------------------------
 struct LastRows {
   int64_t rows;
-  int C;
+  int C;                // channels the workgroups cover (a slab of the row when the row is wider)
+  int64_t stride;       // elements from one row to the next
   int chunks_per_row;   // C / VEC
   int rows_per_step;    // 256 / chunks_per_row
   int64_t rows_per_block;
@@ -460,7 +461,7 @@ __device__ __forceinline__ void for_rows_batched(const LastRows& g, int64_t r0, 
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int64_t ru = r + (int64_t)u * g.rows_per_step;
-      issue(u, (ru < r1 ? ru : r) * g.C + (int64_t)chunk * VEC);
+      issue(u, (ru < r1 ? ru : r) * g.stride + (int64_t)chunk * VEC);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -783,12 +784,13 @@ __global__ __launch_bounds__(kBnBlock) void bn_last_bwd_apply_kernel(const T* __
 }
 
 // Geometry of the channels-last passes, or false when the layout does not fit them.
-inline bool last_rows(int64_t rows, int64_t feat, int dtype, int64_t chunks_per_block, int64_t max_blocks, LastRows* g,
-                      int* blocks) {
+inline bool last_rows(int64_t rows, int64_t feat, int64_t stride, int dtype, int64_t chunks_per_block,
+                      int64_t max_blocks, LastRows* g, int* blocks) {
   const int vec = 16 / dtype_size(dtype);
   if (feat % vec != 0 || feat / vec > kBnBlock) return false;
   g->rows = rows;
   g->C = (int)feat;
+  g->stride = stride;
   g->chunks_per_row = (int)(feat / vec);
   g->rows_per_step = kBnBlock / g->chunks_per_row;
   // rows per block: whole steps, about chunks_per_block 16-byte chunks per lane
@@ -803,6 +805,14 @@ inline bool last_rows(int64_t rows, int64_t feat, int dtype, int64_t chunks_per_
   *blocks = (int)nb;
   return true;
 }
+
+// p + elems elements (null stays null): the column slab of a tensor or of a parameter vector
+inline const void* slab_of(const void* p, int64_t elems, int dt) {
+  return p ? (const char*)p + elems * dtype_size(dt) : nullptr;
+}
+inline void* slab_of_mut(void* p, int64_t elems, int dt) { return p ? (char*)p + elems * dtype_size(dt) : nullptr; }
+inline float* slab_of_f32(float* p, int64_t elems) { return p ? p + elems : nullptr; }
+inline const float* slab_of_f32c(const float* p, int64_t elems) { return p ? p + elems : nullptr; }
 
 }  // namespace
 }  // namespace at_hip
@@ -929,9 +939,10 @@ int at_batch_norm_bwd(const void* output_grad, const void* pre_act, const void* 
 
 int at_batch_norm_nhwc_supported(int64_t feat, int dtype) {
   if (!dtype_valid(dtype) || feat <= 0) return 0;
-  const int vec = 16 / dtype_size(dtype);
-  return feat % vec == 0 && feat / vec <= kBnBlock ? 1 : 0;
+  // rows wider than one workgroup's 256 chunks of 16 bytes are processed in column slabs
+  return feat % (16 / dtype_size(dtype)) == 0 ? 1 : 0;
 }
+
 
 int at_batch_norm_fwd_nhwc(const void* input, const void* weight, const void* bias, float* mean, float* inv_std,
                            const void* pre_act_add, void* pre_act, void* output, void* running_mean,
@@ -957,27 +968,41 @@ int at_batch_norm_fwd_nhwc(const void* input, const void* weight, const void* bi
   if (pre_act == output) pre_act = nullptr;
 
   float* part = (float*)workspace;
-  const int C = (int)feat;
-  float* stat = part + (int64_t)C * kMaxSplits * 3;   // mean[C], inv_std[C]
   const int64_t rows = batch * spatial;
-  LastRows gs, ga;
-  int P = 0, blocks = 0;
-  if (!last_rows(rows, feat, dtype, 16, 512, &gs, &P) || !last_rows(rows, feat, dtype, 8, 65535, &ga, &blocks))
-    return AT_ERR_UNSUPPORTED;
-  return dispatch_dtype(dtype, [&](auto* tp) -> int {
-    typedef std::remove_pointer_t<decltype(tp)> T;
-    constexpr int VEC = 16 / (int)sizeof(T);
-    if (batch_stats)
-      hipLaunchKernelGGL((bn_last_stats_kernel<T, VEC>), dim3(P), dim3(kBnBlock), 0, stream, (const T*)input, part, gs,
-                         P);
-    const int update = batch_stats && track_running_stats && is_train && running_mean && running_var;
-    hipLaunchKernelGGL(bn_last_finalize_kernel, dim3(C), dim3(64), 0, stream, batch_stats ? part : nullptr, P, stat,
-                       mean, inv_std, running_mean, running_var, running_dtype, update, momentum, eps, C);
-    AT_BN_ACT_SWITCH(act, hipLaunchKernelGGL((bn_last_apply_kernel<T, VEC, ACT>), dim3(blocks), dim3(kBnBlock), 0,
-                                             stream, (const T*)input, (const T*)pre_act_add, (T*)pre_act, (T*)output,
-                                             stat, weight, bias, param_dtype, ga, param));
-    return launch_status();
-  });
+  const int64_t slab = (int64_t)(16 / dtype_size(dtype)) * kBnBlock;   // channels one workgroup row covers
+  for (int64_t c0 = 0; c0 < feat; c0 += slab) {
+    const int C = (int)(feat - c0 < slab ? feat - c0 : slab);
+    float* stat = part + (int64_t)C * kMaxSplits * 3;   // mean[C], inv_std[C]
+    LastRows gs, ga;
+    int P = 0, blocks = 0;
+    if (!last_rows(rows, C, feat, dtype, 16, 512, &gs, &P) || !last_rows(rows, C, feat, dtype, 8, 65535, &ga, &blocks))
+      return AT_ERR_UNSUPPORTED;
+    const void* x = slab_of(input, c0, dtype);
+    const void* res = slab_of(pre_act_add, c0, dtype);
+    void* pre = slab_of_mut(pre_act, c0, dtype);
+    void* y = slab_of_mut(output, c0, dtype);
+    const void* w = slab_of(weight, c0, param_dtype);
+    const void* b = slab_of(bias, c0, param_dtype);
+    void* rm = slab_of_mut(running_mean, c0, running_dtype);
+    void* rv = slab_of_mut(running_var, c0, running_dtype);
+    float* mean_c = slab_of_f32(mean, c0);
+    float* inv_std_c = slab_of_f32(inv_std, c0);
+    const int rc = dispatch_dtype(dtype, [&](auto* tp) -> int {
+      typedef std::remove_pointer_t<decltype(tp)> T;
+      constexpr int VEC = 16 / (int)sizeof(T);
+      if (batch_stats)
+        hipLaunchKernelGGL((bn_last_stats_kernel<T, VEC>), dim3(P), dim3(kBnBlock), 0, stream, (const T*)x, part, gs, P);
+      const int update = batch_stats && track_running_stats && is_train && running_mean && running_var;
+      hipLaunchKernelGGL(bn_last_finalize_kernel, dim3(C), dim3(64), 0, stream, batch_stats ? part : nullptr, P, stat,
+                         mean_c, inv_std_c, rm, rv, running_dtype, update, momentum, eps, C);
+      AT_BN_ACT_SWITCH(act, hipLaunchKernelGGL((bn_last_apply_kernel<T, VEC, ACT>), dim3(blocks), dim3(kBnBlock), 0,
+                                               stream, (const T*)x, (const T*)res, (T*)pre, (T*)y, stat, w, b,
+                                               param_dtype, ga, param));
+      return launch_status();
+    });
+    if (rc) return rc;
+  }
+  return AT_OK;
 }
 
 int at_batch_norm_bwd_nhwc(const void* output_grad, const void* pre_act, const void* input, const float* mean,
@@ -998,26 +1023,41 @@ int at_batch_norm_bwd_nhwc(const void* output_grad, const void* pre_act, const v
     return AT_ERR_ALIGN;
 
   float* part = (float*)workspace;
-  const int C = (int)feat;
-  float* coef = part + (int64_t)C * kMaxSplits * 3;   // 4 floats per channel
   const int64_t rows = batch * spatial;
-  LastRows gs, ga;
-  int P = 0, blocks = 0;
-  if (!last_rows(rows, feat, dtype, 16, 512, &gs, &P) || !last_rows(rows, feat, dtype, 8, 65535, &ga, &blocks))
-    return AT_ERR_UNSUPPORTED;
-  const void* g_for_apply = act != AT_ACT_NONE ? pre_act_grad : output_grad;
-  return dispatch_dtype(dtype, [&](auto* tp) -> int {
-    typedef std::remove_pointer_t<decltype(tp)> T;
-    constexpr int VEC = 16 / (int)sizeof(T);
-    AT_BN_ACT_SWITCH(act, hipLaunchKernelGGL((bn_last_bwd_reduce_kernel<T, VEC, ACT>), dim3(P), dim3(kBnBlock), 0,
-                                             stream, (const T*)output_grad, (const T*)pre_act, (const T*)input,
-                                             (T*)pre_act_grad, mean, inv_std, part, gs, P, param));
-    hipLaunchKernelGGL(bn_last_bwd_finalize_kernel, dim3(C), dim3(64), 0, stream, part, P, (float)rows, mean, inv_std,
-                       weight, param_dtype, coef, weight_grad, bias_grad, C);
-    hipLaunchKernelGGL((bn_last_bwd_apply_kernel<T, VEC>), dim3(blocks), dim3(kBnBlock), 0, stream,
-                       (const T*)g_for_apply, (const T*)input, (T*)input_grad, coef, ga);
-    return launch_status();
-  });
+  const int64_t slab = (int64_t)(16 / dtype_size(dtype)) * kBnBlock;
+  for (int64_t c0 = 0; c0 < feat; c0 += slab) {
+    const int C = (int)(feat - c0 < slab ? feat - c0 : slab);
+    float* coef = part + (int64_t)C * kMaxSplits * 3;   // 4 floats per channel
+    LastRows gs, ga;
+    int P = 0, blocks = 0;
+    if (!last_rows(rows, C, feat, dtype, 16, 512, &gs, &P) || !last_rows(rows, C, feat, dtype, 8, 65535, &ga, &blocks))
+      return AT_ERR_UNSUPPORTED;
+    const void* dy = slab_of(output_grad, c0, dtype);
+    const void* pre = slab_of(pre_act, c0, dtype);
+    const void* x = slab_of(input, c0, dtype);
+    void* dx = slab_of_mut(input_grad, c0, dtype);
+    void* dpre = slab_of_mut(pre_act_grad, c0, dtype);
+    const void* w = slab_of(weight, c0, param_dtype);
+    const float* mean_c = slab_of_f32c(mean, c0);
+    const float* inv_std_c = slab_of_f32c(inv_std, c0);
+    float* wg = slab_of_f32(weight_grad, c0);
+    float* bg = slab_of_f32(bias_grad, c0);
+    const void* g_for_apply = act != AT_ACT_NONE ? dpre : dy;
+    const int rc = dispatch_dtype(dtype, [&](auto* tp) -> int {
+      typedef std::remove_pointer_t<decltype(tp)> T;
+      constexpr int VEC = 16 / (int)sizeof(T);
+      AT_BN_ACT_SWITCH(act, hipLaunchKernelGGL((bn_last_bwd_reduce_kernel<T, VEC, ACT>), dim3(P), dim3(kBnBlock), 0,
+                                               stream, (const T*)dy, (const T*)pre, (const T*)x, (T*)dpre, mean_c,
+                                               inv_std_c, part, gs, P, param));
+      hipLaunchKernelGGL(bn_last_bwd_finalize_kernel, dim3(C), dim3(64), 0, stream, part, P, (float)rows, mean_c,
+                         inv_std_c, w, param_dtype, coef, wg, bg, C);
+      hipLaunchKernelGGL((bn_last_bwd_apply_kernel<T, VEC>), dim3(blocks), dim3(kBnBlock), 0, stream,
+                         (const T*)g_for_apply, (const T*)x, (T*)dx, coef, ga);
+      return launch_status();
+    });
+    if (rc) return rc;
+  }
+  return AT_OK;
 }
 
 }  // extern "C"

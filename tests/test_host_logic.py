@@ -122,7 +122,7 @@ def test_argument_errors_without_gpu() -> None:
     assert lib.at_conv2d_bwd_input_nhwc(None, p, p, p, 1 << 30, *good, 2, None) == -1
     assert lib.at_conv2d_bwd_weight_nhwc(p, p, p, None, 0, *good, 2, None) == -5
     assert lib.at_batch_norm_nhwc_supported(64, 2) == 1 and lib.at_batch_norm_nhwc_supported(1024, 0) == 1
-    assert lib.at_batch_norm_nhwc_supported(7, 2) == 0 and lib.at_batch_norm_nhwc_supported(4096, 2) == 0
+    assert lib.at_batch_norm_nhwc_supported(7, 2) == 0 and lib.at_batch_norm_nhwc_supported(4096, 2) == 1   # wide rows: column slabs
     assert lib.at_batch_norm_fwd_nhwc(p, None, None, None, None, None, None, p, None, None, p, 1 << 30, 4, 7, 9,
                                       0.1, 1e-5, 0, 0.0, 0, 1, 2, 0, 0, None) == -7
     assert lib.at_batch_norm_bwd_nhwc(p, None, p, None, p, None, p, None, None, None, p, 1 << 30, 4, 64, 9, 0, 0.0,
