@@ -397,9 +397,10 @@ int at_batch_norm_bwd(const void* output_grad, const void* pre_act, const void* 
  * [batch * spatial, feat] matrix with statistics per column): same arguments, meanings and
  * workspace.  The reference reads its input through strides (batch_norm_layer.py:130-157), so
  * such tensors are within its interface.  Covered when feat is a multiple of the 16-byte vector
- * (8 for 16-bit, 4 for fp32 tensors) of at most 256 vectors — at_batch_norm_nhwc_supported
- * tells; otherwise the calls return AT_ERR_UNSUPPORTED and the caller converts to
- * channels-first. */
+ * (8 for 16-bit, 4 for fp32 tensors) — at_batch_norm_nhwc_supported tells; rows wider than 256
+ * vectors are processed in column slabs.  Otherwise the calls return AT_ERR_UNSUPPORTED and the
+ * caller converts to channels-first.  With spatial = 1 these are the calls for [batch, feat]
+ * inputs. */
 int at_batch_norm_nhwc_supported(int64_t feat, int dtype);
 
 int at_batch_norm_fwd_nhwc(const void* input, const void* weight, const void* bias, float* mean,
