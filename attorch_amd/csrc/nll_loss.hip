@@ -114,49 +114,64 @@ __global__ __launch_bounds__(kNllBlock) void nll_bwd_kernel(
   }
 }
 
-// spatial == 1 (a [batch, feat] matrix): a 16-byte vector of the flat gradient lies in one row
-// or straddles two, and holds at most one non-zero per row, at flat position row * feat +
-// target[row].  No per-element index arithmetic; IDX is 32-bit when the tensor allows it.
-template <typename TG, typename TO, typename IDX>
+// spatial == 1 (a [batch, feat] matrix): the gradient is zero except at flat position
+// row * feat + target[row] of every row.  A workgroup owns one 16 KB piece of the flat gradient:
+// it clears the piece in LDS, the rows that overlap it (found with two divisions per workgroup,
+// not one per vector) drop their value into it, and the piece leaves as whole 16-byte vectors.
+// Every byte of the gradient is written exactly once (no memset, no second launch), and the
+// per-vector work is a few instructions, so the pass runs at the speed of a plain fill.
+constexpr int kNllTileBytes = 16384;
+template <typename TG, typename TO>
 __global__ __launch_bounds__(kNllBlock) void nll_bwd_rows_kernel(
     const TG* __restrict__ output_grad, const int64_t* __restrict__ target, const void* __restrict__ weight, int wdt,
-    const float* __restrict__ sum_weights, TO* __restrict__ input_grad, IDX batch, IDX feat, int reduction,
+    const float* __restrict__ sum_weights, TO* __restrict__ input_grad, int64_t batch, int64_t feat, int reduction,
     float inv_count) {
   constexpr int VEC = 16 / (int)sizeof(TO);
-  const IDX total = batch * feat;
+  constexpr int kTileElems = kNllTileBytes / (int)sizeof(TO);
+  constexpr int kVecPerLane = kNllTileBytes / 16 / kNllBlock;
+  __shared__ __attribute__((aligned(16))) TO tile[kTileElems];
+  const int64_t total = batch * feat;
   float scale = -1.f;
   if (reduction == AT_REDUCTION_MEAN) scale = weight ? -1.f / sum_weights[0] : -inv_count;
   if (reduction != AT_REDUCTION_NONE) scale *= to_f32(output_grad[0]);
-  const IDX n_vec = (total + VEC - 1) / VEC;
-  const IDX stride = (IDX)gridDim.x * kNllBlock;
-  for (IDX v = (IDX)blockIdx.x * kNllBlock + threadIdx.x; v < n_vec; v += stride) {
-    const IDX f0 = v * VEC;
-    const IDX row = f0 / feat;
-    float g[VEC];
+  for (int64_t e0 = (int64_t)blockIdx.x * kTileElems; e0 < total; e0 += (int64_t)gridDim.x * kTileElems) {
+    const int64_t e1 = e0 + kTileElems < total ? e0 + kTileElems : total;
+    // 32-bit division whenever the tensor allows it
+    int64_t row_lo, row_hi;
+    if (total <= (int64_t)UINT32_MAX) {
+      row_lo = (uint32_t)e0 / (uint32_t)feat;
+      row_hi = (uint32_t)(e1 - 1) / (uint32_t)feat;
+    } else {
+      row_lo = e0 / feat;
+      row_hi = (e1 - 1) / feat;
+    }
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) g[j] = 0.f;
-#pragma unroll
-    for (int k = 0; k < 2; ++k) {
-      const IDX r = row + k;
-      if (r >= batch || r * feat >= f0 + VEC) break;   // the second row only when the vector reaches it
+    for (int i = 0; i < kVecPerLane; ++i)
+      reinterpret_cast<uint4*>(tile)[threadIdx.x + i * kNllBlock] = make_uint4(0u, 0u, 0u, 0u);
+    __syncthreads();
+    for (int64_t r = row_lo + threadIdx.x; r <= row_hi; r += kNllBlock) {
       const int64_t t = target[r];
-      if (t < 0 || t >= (int64_t)feat) continue;
-      const IDX pos = r * feat + (IDX)t;
-      if (pos < f0 || pos >= f0 + VEC) continue;
+      if (t < 0 || t >= feat) continue;
+      const int64_t pos = r * feat + t;
+      if (pos < e0 || pos >= e1) continue;
       float coef = scale;
       if (reduction == AT_REDUCTION_NONE) coef *= to_f32(output_grad[r]);
       if (weight) coef *= load_scalar_f32(weight, wdt, t);
-      const int d = (int)(pos - f0);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) g[j] = j == d ? coef : g[j];
+      tile[pos - e0] = from_f32<TO>(coef);
     }
-    if (f0 + VEC <= total) {
-      store_f32<TO, VEC>(input_grad + f0, g);
-    } else {
+    __syncthreads();
 #pragma unroll
-      for (int j = 0; j < VEC; ++j)
-        if (f0 + j < total) input_grad[f0 + j] = from_f32<TO>(g[j]);
+    for (int i = 0; i < kVecPerLane; ++i) {
+      const int v = threadIdx.x + i * kNllBlock;
+      const int64_t f0 = e0 + (int64_t)v * VEC;
+      if (f0 + VEC <= total) {
+        reinterpret_cast<uint4*>(input_grad + e0)[v] = reinterpret_cast<const uint4*>(tile)[v];
+      } else {
+        for (int j = 0; j < VEC; ++j)
+          if (f0 + j < total) input_grad[f0 + j] = tile[v * VEC + j];
+      }
     }
+    __syncthreads();   // the piece has left before the next one is cleared
   }
 }
 
@@ -240,16 +255,12 @@ int at_nll_loss_bwd(const void* output_grad, const int64_t* target, const void* 
     typedef std::remove_pointer_t<decltype(gp)> TG;
     return dispatch_dtype(out_dtype, [&](auto* op) -> int {
       typedef std::remove_pointer_t<decltype(op)> TO;
-      constexpr int VEC = 16 / (int)sizeof(TO);
-      if (spatial == 1 && feat >= VEC && vector_ok) {
-        if (total + VEC < ((int64_t)1 << 31))
-          hipLaunchKernelGGL((nll_bwd_rows_kernel<TG, TO, uint32_t>), dim3((unsigned)blocks), dim3(kNllBlock), 0,
-                             stream, (const TG*)output_grad, target, weight, weight_dtype, sum_weights,
-                             (TO*)input_grad, (uint32_t)batch, (uint32_t)feat, reduction, inv_count);
-        else
-          hipLaunchKernelGGL((nll_bwd_rows_kernel<TG, TO, int64_t>), dim3((unsigned)blocks), dim3(kNllBlock), 0,
-                             stream, (const TG*)output_grad, target, weight, weight_dtype, sum_weights,
-                             (TO*)input_grad, batch, feat, reduction, inv_count);
+      if (spatial == 1 && vector_ok) {
+        int64_t tiles = cdiv64(total * (int64_t)sizeof(TO), kNllTileBytes);
+        if (tiles > cap) tiles = cap;
+        hipLaunchKernelGGL((nll_bwd_rows_kernel<TG, TO>), dim3((unsigned)tiles), dim3(kNllBlock), 0, stream,
+                           (const TG*)output_grad, target, weight, weight_dtype, sum_weights, (TO*)input_grad, batch,
+                           feat, reduction, inv_count);
         return launch_status();
       }
       hipLaunchKernelGGL((nll_bwd_kernel<TG, TO>), dim3((unsigned)blocks), dim3(kNllBlock), 0, stream,
