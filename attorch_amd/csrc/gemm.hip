@@ -67,7 +67,6 @@ constexpr int kBigWaveN = BN / (kBigWaves / 2);    // columns per wave
 constexpr int kBigNJ = kBigWaveN / 32;             // 32-column MFMA tiles per wave
 constexpr int kTileBytes = BM * BK * 2;  // one operand tile, 32 KiB
 constexpr int kEpiPitch = BN * 2 + 16;   // bytes per row of the epilogue tile in LDS (padded against bank conflicts)
-constexpr int kEpiBytes = BM * kEpiPitch;
 
 typedef __attribute__((address_space(3))) void lds_void_t;
 
@@ -90,9 +89,11 @@ struct OperandLoader {
   int k_step;     // bytes per k-tile
   int k_lane;     // k of this lane inside a k-tile (contract-contiguous layout only)
   int K;
+  int tid;        // threadIdx.x, or a copy of it that the compiler cannot see through (see the caller)
 
-  __device__ __forceinline__ void init(const T* base, int64_t ld, int outer0, int outer_total, int K_) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __device__ __forceinline__ void init(const T* base, int64_t ld, int outer0, int outer_total, int K_, int tid_) {
+    tid = tid_;
+    const int lane = tid & 63, wave = tid >> 6;
     K = K_;
     if (CONTRACT_CONTIG) {
       rsrc = make_buffer_rsrc(base, ((int64_t)(outer_total - 1) * ld + K_) * 2);   // the last row ends at its last element
@@ -125,7 +126,7 @@ struct OperandLoader {
   // Load i (0 .. kBigLoads-1) of this lane for k-tile `kt`; kt < 0 gives an offset that is out of
   // range (the load writes zeros).
   __device__ __forceinline__ void issue_one(int kt, char* tile, int i) const {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = tid & 63, wave = tid >> 6;
     {
       const int q = wave * kBigLoads + i;
       int off;
@@ -170,90 +171,121 @@ __device__ __forceinline__ uint4 read_frag(const char* tile, int outer_base, int
 }
 
 // Epilogue of the 256x256 kernels: bias, optional pre-activation copy and activation, out through LDS.
-template <typename T, int ACT>
-__device__ __forceinline__ void big_tile_epilogue(f32x16 (&acc)[4][kBigNJ], char* lds, const GemmArgs& g, int m0,
-                                                  int n0) {
+// The tile leaves in four chunks of 64 rows through a staging area of 33 KB that does not touch the
+// first stage of either operand, so that `prefetch_next` — called once all waves are done with the
+// main loop's buffers — can already request the first k-tile of the workgroup's next output
+// tile: it lands while this tile is written out, and the next tile starts without waiting for its
+// first loads or, on this architecture's single in-order memory counter, for this tile's stores.
+// Returns the number of global stores each lane issued after `prefetch_next` when that number is
+// the same for every lane (a full tile with 16-byte aligned rows), -1 otherwise.
+constexpr int kEpiRows = 64;                                   // rows per chunk
+constexpr int kEpiStageBytes = kEpiRows * kEpiPitch;           // 33 792
+constexpr int kEpiBiasBytes = BN * 4;                          // the tile's bias values as floats, behind the chunk
+constexpr int kEpiSweeps = kEpiRows / (kBigThreads / 32);      // 16-byte stores per lane and chunk
+template <typename T, int ACT, typename Prefetch>
+__device__ __forceinline__ int big_tile_epilogue(f32x16 (&acc)[4][kBigNJ], char* stage, const GemmArgs& g, int m0,
+                                                 int n0, Prefetch&& prefetch_next) {
   constexpr int NJ = kBigNJ;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // a thread index the compiler takes for a new value: what the epilogue derives from it is worked
+  // out here and not kept in registers across the main loop
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));
+  const int lane = tid & 63, wave = tid >> 6;
   const int wm = wave / (kBigWaves / 2), wn = wave % (kBigWaves / 2);
   const int frag_row = lane & 31, frag_half = lane >> 5;
   // A lane holds, for tile (i, j) and register group rg, C[m][n .. n+3] with
   //   m = wm*128 + i*32 + lane%32,  n = wn*kBigWaveN + j*32 + rg*8 + (lane/32)*4   (tile-local).
   // Storing that straight to memory touches 32 rows per instruction with 16 bytes each; instead
-  // the finished tile goes through LDS (free after the main loop) and leaves as whole rows:
-  // 32 lanes x 16 bytes = one 512-byte row segment per half-wave.
+  // the rows go through LDS and leave whole: 32 lanes x 16 bytes = one 512-byte row segment per
+  // half-wave.  Chunk c holds rows 64 c .. 64 c + 63: row tiles 2 (c % 2), 2 (c % 2) + 1 of the
+  // four waves with wm = c / 2.
   T* __restrict__ C = reinterpret_cast<T*>(g.c);
   T* __restrict__ P = reinterpret_cast<T*>(g.pre_act);
   const bool rows16 = ((g.ldc & 7) == 0) && aligned16_dev(C) && (n0 + BN <= g.N) &&
                       (!P || (((g.ldp & 7) == 0) && aligned16_dev(P)));
+  const bool exact = rows16 && m0 + BM <= g.M;
+  float* const bias_tile = reinterpret_cast<float*>(stage + kEpiStageBytes);
+  // the bias of the tile's columns goes to LDS before anything else: a global load further down
+  // would make the compiler wait for every store issued before it
+  float bias_value = 0.f;
+  if (g.bias && tid < BN && n0 + (int)tid < g.N)
+    bias_value = load_scalar_f32(g.bias, g.bias_dt, n0 + tid);
+  __syncthreads();              // every wave is done with the main loop's reads of LDS
+  if (tid < BN) bias_tile[tid] = bias_value;
+  // a use of the loaded value on every path: the compiler's wait for it comes here, not as a wait
+  // for everything in flight somewhere behind the request below
+  asm volatile("" ::"v"(bias_value));
+  prefetch_next();
   constexpr int n_out = ACT != AT_ACT_NONE ? 2 : 1;
+  int outputs = 0;
 #pragma unroll
   for (int pass = 0; pass < n_out; ++pass) {
     const bool is_pre = (n_out == 2 && pass == 0);
     T* __restrict__ dst = is_pre ? P : C;
     const int64_t ldd = is_pre ? g.ldp : g.ldc;
     if (is_pre && !P) continue;   // uniform
-    __syncthreads();              // previous readers of LDS (main loop or previous pass) are done
+    ++outputs;
 #pragma unroll
-    for (int j = 0; j < NJ; ++j)
+    for (int c = 0; c < BM / kEpiRows; ++c) {
+      __syncthreads();            // previous readers of the staging area are done (and the bias is in place)
+      if (wm == (c >> 1)) {
 #pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        const int nl = wn * kBigWaveN + j * 32 + rg * 8 + frag_half * 4;
-        float bv[4] = {0.f, 0.f, 0.f, 0.f};
-        if (g.bias) {
+        for (int j = 0; j < NJ; ++j)
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (n0 + nl + e < g.N) bv[e] = load_scalar_f32(g.bias, g.bias_dt, n0 + nl + e);
-        }
+          for (int rg = 0; rg < 4; ++rg) {
+            const int nl = wn * kBigWaveN + j * 32 + rg * 8 + frag_half * 4;
+            const float4 bv = *reinterpret_cast<const float4*>(bias_tile + nl);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          float v[4];
+            for (int ii = 0; ii < 2; ++ii) {
+              const int i = (c & 1) * 2 + ii;
+              float v[4] = {acc[i][j][rg * 4 + 0] + bv.x, acc[i][j][rg * 4 + 1] + bv.y, acc[i][j][rg * 4 + 2] + bv.z,
+                            acc[i][j][rg * 4 + 3] + bv.w};
+              if (ACT != AT_ACT_NONE && !is_pre) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            v[e] = acc[i][j][rg * 4 + e] + bv[e];
-            if (ACT != AT_ACT_NONE && !is_pre) v[e] = act_forward(ACT, v[e], g.param);
+                for (int e = 0; e < 4; ++e) v[e] = act_forward(ACT, v[e], g.param);
+              }
+              store_f32<T, 4>(reinterpret_cast<T*>(stage + (ii * 32 + frag_row) * kEpiPitch) + nl, v);
+            }
           }
-          const int ml = wm * 128 + i * 32 + frag_row;
-          store_f32<T, 4>(reinterpret_cast<T*>(lds + ml * kEpiPitch) + nl, v);
-        }
       }
-    __syncthreads();
-    // 2 rows per wave and sweep, 32 lanes x 16 bytes per row
-    const int rsub = threadIdx.x >> 5, cseg = (threadIdx.x & 31) * 8;
-#pragma unroll 4
-    for (int r0 = 0; r0 < BM; r0 += kBigThreads / 32) {
-      const int ml = r0 + rsub;
-      const int m = m0 + ml;
-      if (m >= g.M) continue;
-      const uint4 v = *reinterpret_cast<const uint4*>(lds + ml * kEpiPitch + cseg * 2);
-      T* out = dst + (int64_t)m * ldd + n0 + cseg;
-      if (rows16) {
-        *reinterpret_cast<uint4*>(out) = v;
-      } else {
-        // Rows that do not start on 16-byte boundaries (an odd row stride) or a tile that sticks
-        // out over the last column: the row segment is still written as whole 16-byte vectors
-        // wherever memory allows — lane j takes the j-th aligned vector inside the segment and
-        // gathers its 8 elements from LDS — and only the few elements before the first and after
-        // the last aligned vector go out one by one.
-        const int j = threadIdx.x & 31;
-        const int ncols = g.N - n0 < BN ? g.N - n0 : BN;
-        T* seg = dst + (int64_t)m * ldd + n0;
-        const T* src = reinterpret_cast<const T*>(lds + ml * kEpiPitch);
-        const int head = (int)(((16 - (reinterpret_cast<uintptr_t>(seg) & 15)) & 15) >> 1);   // elements before the first boundary
-        const int first = head < ncols ? head : ncols;
-        const int nfull = (ncols - first) >> 3;
-        if (j < nfull) {
-          union { uint4 raw; T e[8]; } u;
+      __syncthreads();
+      // 2 rows per wave and sweep, 32 lanes x 16 bytes per row
+      const int rsub = tid >> 5, cseg = (tid & 31) * 8;
 #pragma unroll
-          for (int e = 0; e < 8; ++e) u.e[e] = src[first + j * 8 + e];
-          *reinterpret_cast<uint4*>(seg + first + j * 8) = u.raw;
+      for (int r0 = 0; r0 < kEpiRows; r0 += kBigThreads / 32) {
+        const int ml = r0 + rsub;
+        const int m = m0 + c * kEpiRows + ml;
+        if (m >= g.M) continue;
+        if (rows16) {
+          const uint4 v = *reinterpret_cast<const uint4*>(stage + ml * kEpiPitch + cseg * 2);
+          *reinterpret_cast<uint4*>(dst + (int64_t)m * ldd + n0 + cseg) = v;
+        } else {
+          // Rows that do not start on 16-byte boundaries (an odd row stride) or a tile that sticks
+          // out over the last column: the row segment is still written as whole 16-byte vectors
+          // wherever memory allows — lane j takes the j-th aligned vector inside the segment and
+          // gathers its 8 elements from LDS — and only the few elements before the first and after
+          // the last aligned vector go out one by one.
+          const int j = tid & 31;
+          const int ncols = g.N - n0 < BN ? g.N - n0 : BN;
+          T* seg = dst + (int64_t)m * ldd + n0;
+          const T* src = reinterpret_cast<const T*>(stage + ml * kEpiPitch);
+          const int head = (int)(((16 - (reinterpret_cast<uintptr_t>(seg) & 15)) & 15) >> 1);   // elements before the first boundary
+          const int first = head < ncols ? head : ncols;
+          const int nfull = (ncols - first) >> 3;
+          if (j < nfull) {
+            union { uint4 raw; T e[8]; } u;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) u.e[e] = src[first + j * 8 + e];
+            *reinterpret_cast<uint4*>(seg + first + j * 8) = u.raw;
+          }
+          if (j < first) seg[j] = src[j];
+          const int tail0 = first + nfull * 8;
+          if (tail0 + j < ncols && j < 8) seg[tail0 + j] = src[tail0 + j];
         }
-        if (j < first) seg[j] = src[j];
-        const int tail0 = first + nfull * 8;
-        if (tail0 + j < ncols && j < 8) seg[tail0 + j] = src[tail0 + j];
       }
     }
   }
+  return exact ? outputs * (BM / kEpiRows) * kEpiSweeps : -1;
 }
 
 // ACT is the compile-time activation id of the epilogue (the act switch must fold away: the
@@ -269,9 +301,14 @@ __global__ __launch_bounds__(kBigThreads) void gemm_mfma16_kernel(GemmArgs g) {
   // unpadded tiles, gains under 1 % from it): two stages each.
   constexpr int kAStages = (A_KC && B_KC) ? 3 : 2;
   constexpr int kARing = kAStages * kATile;
-  constexpr int kLds = kARing + 2 * kBTile > kEpiBytes ? kARing + 2 * kBTile : kEpiBytes;
+  constexpr int kLds = kARing + 2 * kBTile;
   static_assert(kLds <= 160 * 1024, "the stages fill the LDS of a CU exactly");
-  __shared__ __attribute__((aligned(1024))) char lds[kLds];  // main loop: A ring | B ring; epilogue: output tile
+  // The epilogue's staging area lies behind the first stage of A where A's later stages hold it,
+  // else in B's second stage: the first stage of either operand stays free for the next tile.
+  constexpr int kEpiNeed = kEpiStageBytes + kEpiBiasBytes;
+  constexpr int kEpiOff = (kAStages - 1) * kATile >= kEpiNeed ? kATile : kARing + kBTile;
+  static_assert(kEpiOff == kATile || kBTile >= kEpiNeed, "the staging area fits behind the first stages");
+  __shared__ __attribute__((aligned(1024))) char lds[kLds];  // A ring | B ring; the epilogue stages chunks of the output at kEpiOff
   const T* __restrict__ A = reinterpret_cast<const T*>(g.a);
   const T* __restrict__ B = reinterpret_cast<const T*>(g.b);
 
@@ -280,25 +317,31 @@ __global__ __launch_bounds__(kBigThreads) void gemm_mfma16_kernel(GemmArgs g) {
   // workgroup then takes tiles blockIdx.x, blockIdx.x + gridDim.x, ... one after the other ----
   const int nbm = (g.M + BM - 1) / BM, nbn = (g.N + BN - 1) / BN;
   const int total = nbm * nbn;
-  for (int tile_id = blockIdx.x; tile_id < total; tile_id += gridDim.x) {
-  int logical;
-  {
-    const int bid = tile_id, xcd = bid & 7, idx = bid >> 3;
+  auto tile_origin = [&](int bid, int& m0_, int& n0_) {
+    const int xcd = bid & 7, idx = bid >> 3;
     const int q = total >> 3, rem = total & 7;
-    logical = xcd * q + (xcd < rem ? xcd : rem) + idx;
-  }
-  constexpr int GROUP = 8;
-  const int per_group = GROUP * nbn;
-  const int first_m = (logical / per_group) * GROUP;
-  const int gsz = nbm - first_m < GROUP ? nbm - first_m : GROUP;
-  const int in_group = logical % per_group;
-  const int m0 = (first_m + in_group % gsz) * BM;
-  const int n0 = (in_group / gsz) * BN;
+    const int logical = xcd * q + (xcd < rem ? xcd : rem) + idx;
+    constexpr int GROUP = 8;
+    const int per_group = GROUP * nbn;
+    const int first_m = (logical / per_group) * GROUP;
+    const int gsz = nbm - first_m < GROUP ? nbm - first_m : GROUP;
+    const int in_group = logical % per_group;
+    m0_ = (first_m + in_group % gsz) * BM;
+    n0_ = (in_group / gsz) * BN;
+  };
+  char* const a_ring = lds;
+  char* const b_ring = lds + kARing;
+  // k-tile 0 of a tile after the workgroup's first is requested from inside the epilogue of the
+  // tile before it; `stores_behind` is what that epilogue issued after the request (-1: unknown)
+  bool requested = false;
+  int stores_behind = -1;
+  for (int tile_id = blockIdx.x; tile_id < total; tile_id += gridDim.x) {
+  int m0, n0;
+  tile_origin(tile_id, m0, n0);
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wave = threadIdx.x >> 6;
   constexpr int NJ = kBigNJ;
   const int wm = wave / (kBigWaves / 2), wn = wave % (kBigWaves / 2);
-  const int frag_row = lane & 31, frag_half = lane >> 5;
 
   f32x16 acc[4][NJ];
 #pragma unroll
@@ -310,8 +353,10 @@ __global__ __launch_bounds__(kBigThreads) void gemm_mfma16_kernel(GemmArgs g) {
 
   OperandLoader<T, A_KC> la;
   OperandLoader<T, B_KC> lb;
-  la.init(A, g.lda, m0, g.M, g.K);
-  lb.init(B, g.ldb, n0, g.N, g.K);
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));   // keeps the lane's offsets from being hoisted out of the tile loop and held across the epilogue
+  la.init(A, g.lda, m0, g.M, g.K, tid);
+  lb.init(B, g.ldb, n0, g.N, g.K, tid);
   const int KT = (g.K + BK - 1) / BK;
 
   auto load_frags = [&](const char* a_stage, const char* b_stage, int ks, uint4 (&af)[4], uint4 (&bf)[NJ]) {
@@ -321,12 +366,16 @@ __global__ __launch_bounds__(kBigThreads) void gemm_mfma16_kernel(GemmArgs g) {
     for (int j = 0; j < NJ; ++j) bf[j] = read_frag<B_KC>(b_stage, wn * kBigWaveN + j * 32, ks);
   };
 
-  char* const a_ring = lds;
-  char* const b_ring = lds + kARing;
-  la.issue(0, a_ring);
-  lb.issue(0, b_ring);
-  lds_dma_wait_all();
-  __syncthreads();
+  if (!requested) {
+    la.issue(0, a_ring);
+    lb.issue(0, b_ring);
+  }
+  // The memory counter runs in issue order and counts stores too: leaving exactly the stores of
+  // the last epilogue outstanding waits for k-tile 0 and not for their acknowledgements.
+  if (stores_behind == 4 * kEpiSweeps) lds_dma_wait_newest<4 * kEpiSweeps>();
+  else if (stores_behind == 8 * kEpiSweeps) lds_dma_wait_newest<8 * kEpiSweeps>();
+  else lds_dma_wait_all();
+  __syncthreads();      // k-tile 0 is everybody's; the last epilogue's readers of the staging area are done
   // k-tiles 1 (both operands) and 2 (A) travel while k-tile 0 is multiplied (zeros when there are
   // none).  A's tile 2 is issued last: the in-order counter then lets it stay in flight across the
   // first wait.
@@ -399,8 +448,24 @@ __global__ __launch_bounds__(kBigThreads) void gemm_mfma16_kernel(GemmArgs g) {
   }
   lds_dma_wait_all();   // the zero-fill loads past the end: the epilogue reuses the stages
 
-  big_tile_epilogue<T, ACT>(acc, lds, g, m0, n0);
-  __syncthreads();      // the epilogue's readers of LDS are done before the next tile's loads land
+  const int next_id = tile_id + gridDim.x;
+  requested = next_id < total;
+  stores_behind = big_tile_epilogue<T, ACT>(acc, lds + kEpiOff, g, m0, n0, [&] {
+    if (!requested) return;
+    int m1, n1;
+    tile_origin(next_id, m1, n1);
+    // The lane's offsets are worked out afresh from a thread index the compiler takes for a new
+    // value: shared with the main loop's loaders they would be kept across it, in registers it
+    // does not have.
+    int tid1 = threadIdx.x;
+    asm volatile("" : "+v"(tid1));
+    OperandLoader<T, A_KC> la1;
+    OperandLoader<T, B_KC> lb1;
+    la1.init(A, g.lda, m1, g.M, g.K, tid1);
+    lb1.init(B, g.ldb, n1, g.N, g.K, tid1);
+    la1.issue(0, a_ring);
+    lb1.issue(0, b_ring);
+  });
   }
 }
 
