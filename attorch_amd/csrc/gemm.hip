@@ -178,7 +178,7 @@ __device__ __forceinline__ uint4 read_frag(const char* tile, int outer_base, int
 // first loads or, on this architecture's single in-order memory counter, for this tile's stores.
 // Returns the number of global stores each lane issued after `prefetch_next` when that number is
 // the same for every lane (a full tile with 16-byte aligned rows), -1 otherwise.
-constexpr int kEpiRows = 64;                                   // rows per chunk
+constexpr int kEpiRows = BM / 4;                               // rows per chunk
 constexpr int kEpiStageBytes = kEpiRows * kEpiPitch;           // 33 792
 constexpr int kEpiBiasBytes = BN * 4;                          // the tile's bias values as floats, behind the chunk
 constexpr int kEpiSweeps = kEpiRows / (kBigThreads / 32);      // 16-byte stores per lane and chunk
@@ -197,8 +197,8 @@ __device__ __forceinline__ int big_tile_epilogue(f32x16 (&acc)[4][kBigNJ], char*
   //   m = wm*128 + i*32 + lane%32,  n = wn*kBigWaveN + j*32 + rg*8 + (lane/32)*4   (tile-local).
   // Storing that straight to memory touches 32 rows per instruction with 16 bytes each; instead
   // the rows go through LDS and leave whole: 32 lanes x 16 bytes = one 512-byte row segment per
-  // half-wave.  Chunk c holds rows 64 c .. 64 c + 63: row tiles 2 (c % 2), 2 (c % 2) + 1 of the
-  // four waves with wm = c / 2.
+  // half-wave.  Chunk c holds row tile c of every wave, so that all eight share the work of each
+  // chunk: rows 32 c .. 32 c + 31 of the upper and of the lower half of the tile.
   T* __restrict__ C = reinterpret_cast<T*>(g.c);
   T* __restrict__ P = reinterpret_cast<T*>(g.pre_act);
   const bool rows16 = ((g.ldc & 7) == 0) && aligned16_dev(C) && (n0 + BN <= g.N) &&
@@ -226,35 +226,29 @@ __device__ __forceinline__ int big_tile_epilogue(f32x16 (&acc)[4][kBigNJ], char*
     if (is_pre && !P) continue;   // uniform
     ++outputs;
 #pragma unroll
-    for (int c = 0; c < BM / kEpiRows; ++c) {
+    for (int c = 0; c < 4; ++c) {
       __syncthreads();            // previous readers of the staging area are done (and the bias is in place)
-      if (wm == (c >> 1)) {
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
+      for (int j = 0; j < NJ; ++j)
 #pragma unroll
-          for (int rg = 0; rg < 4; ++rg) {
-            const int nl = wn * kBigWaveN + j * 32 + rg * 8 + frag_half * 4;
-            const float4 bv = *reinterpret_cast<const float4*>(bias_tile + nl);
+        for (int rg = 0; rg < 4; ++rg) {
+          const int nl = wn * kBigWaveN + j * 32 + rg * 8 + frag_half * 4;
+          const float4 bv = *reinterpret_cast<const float4*>(bias_tile + nl);
+          float v[4] = {acc[c][j][rg * 4 + 0] + bv.x, acc[c][j][rg * 4 + 1] + bv.y, acc[c][j][rg * 4 + 2] + bv.z,
+                        acc[c][j][rg * 4 + 3] + bv.w};
+          if (ACT != AT_ACT_NONE && !is_pre) {
 #pragma unroll
-            for (int ii = 0; ii < 2; ++ii) {
-              const int i = (c & 1) * 2 + ii;
-              float v[4] = {acc[i][j][rg * 4 + 0] + bv.x, acc[i][j][rg * 4 + 1] + bv.y, acc[i][j][rg * 4 + 2] + bv.z,
-                            acc[i][j][rg * 4 + 3] + bv.w};
-              if (ACT != AT_ACT_NONE && !is_pre) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = act_forward(ACT, v[e], g.param);
-              }
-              store_f32<T, 4>(reinterpret_cast<T*>(stage + (ii * 32 + frag_row) * kEpiPitch) + nl, v);
-            }
+            for (int e = 0; e < 4; ++e) v[e] = act_forward(ACT, v[e], g.param);
           }
-      }
+          store_f32<T, 4>(reinterpret_cast<T*>(stage + (wm * 32 + frag_row) * kEpiPitch) + nl, v);
+        }
       __syncthreads();
       // 2 rows per wave and sweep, 32 lanes x 16 bytes per row
       const int rsub = tid >> 5, cseg = (tid & 31) * 8;
 #pragma unroll
       for (int r0 = 0; r0 < kEpiRows; r0 += kBigThreads / 32) {
         const int ml = r0 + rsub;
-        const int m = m0 + c * kEpiRows + ml;
+        const int m = m0 + (ml >> 5) * (BM / 2) + c * 32 + (ml & 31);
         if (m >= g.M) continue;
         if (rows16) {
           const uint4 v = *reinterpret_cast<const uint4*>(stage + ml * kEpiPitch + cseg * 2);
@@ -285,7 +279,7 @@ __device__ __forceinline__ int big_tile_epilogue(f32x16 (&acc)[4][kBigNJ], char*
       }
     }
   }
-  return exact ? outputs * (BM / kEpiRows) * kEpiSweeps : -1;
+  return exact ? outputs * 4 * kEpiSweeps : -1;
 }
 
 // ACT is the compile-time activation id of the epilogue (the act switch must fold away: the
