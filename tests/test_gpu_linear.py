@@ -106,6 +106,12 @@ HALF_DTYPES = [torch.float16, torch.bfloat16]
     ((2048, 512), 384),     # 128x128 tiles
     ((4096, 256), 256),     # 128x128 tiles, weight gradient split over the batch
     ((16384, 192), 320),    # split with a ragged last k-tile range
+    # 256x256 tiles walked by a grid smaller than their number (each workgroup takes two), with
+    # ragged last row and column tiles among full ones: forward, input gradient and weight
+    # gradient in turn
+    ((8100, 256), 4088),
+    ((8100, 4088), 520),
+    ((300, 8104), 4088),
 ])
 def test_linear_16bit_kernel_selection(shape, out_dim, act_func, dtype) -> None:
     run_case(shape, out_dim, True, act_func, dtype)
