@@ -73,12 +73,15 @@ typedef __attribute__((address_space(3))) void lds_void_t;
 // LDS image of one operand tile of a k-tile.
 //  * CONTRACT_CONTIG (memory [outer][k]): 256 rows x 128 bytes, 16-byte chunks XOR-swizzled by
 //    the row (lds_chunk_offset); fragments are plain 128-bit reads.
-//  * otherwise (memory [k][outer]): 64 k-rows x 512 bytes kept as loaded; every pair of rows
-//    is one contiguous KiB (one wave-wide load) followed by 64 bytes of padding, which
-//    spreads the 8 rows a transposing fragment read touches evenly over the banks.  (Without the
-//    padding, k-row r keeping chunk x at position x ^ 2 (r & 3), the tiles are 2 KB smaller
-//    but the product that reads both operands this way is 2.7 % slower.)
-constexpr int kPairPitch = 1024 + 64;
+//  * otherwise (memory [k][outer]): 64 k-rows x 512 bytes; every pair of rows is one KiB (one
+//    wave-wide load) followed by 128 bytes of padding, and inside the KiB the two rows alternate in
+//    pieces of 64 bytes (piece 2 c + r holds columns 32 c .. 32 c + 31 of row r of the pair).  A
+//    transposing fragment read takes 64 bytes from each of four consecutive k-rows per half-wave:
+//    the two rows of a pair then sit 64 bytes apart and consecutive pairs 128 bytes further, so
+//    the four pieces cover all 64 banks once.  (With the rows of a pair kept whole, 512 bytes
+//    apart, they share their banks: the counters showed every second LDS cycle of such reads as a
+//    bank conflict.)
+constexpr int kPairPitch = 1024 + 128;
 template <bool CONTRACT_CONTIG> constexpr int operand_tile_bytes() { return CONTRACT_CONTIG ? kTileBytes : 32 * kPairPitch; }
 
 template <typename T, bool CONTRACT_CONTIG>
@@ -108,10 +111,12 @@ struct OperandLoader {
       // up to the end of the 16-byte unit that holds the last element (rows start on such units,
       // and the range check drops a dword that is only partly inside)
       rsrc = make_buffer_rsrc(base, ((int64_t)(K_ - 1) * ld + ((outer_total + 7) & ~7)) * 2);
-      // load i of wave w fills k-rows 2q, 2q+1 (q = kBigLoads w + i); lane -> k-row 2q + lane/32, 8 columns at (lane%32)*8
-      const int krow = wave * (kBigLoads * 2) + (lane >> 5);  // + 2 i
+      // load i of wave w fills k-rows 2q, 2q+1 (q = kBigLoads w + i); the lane's 16 bytes land at
+      // 16 * lane of the KiB, i.e. in piece lane / 4: row (lane / 4) % 2 of the pair, columns
+      // 32 * (lane / 8) + 8 * (lane % 4) ...
+      const int krow = wave * (kBigLoads * 2) + ((lane >> 2) & 1);  // + 2 i
       k_lane = 0;
-      lane_off = (int)(((int64_t)krow * ld + outer0 + (lane & 31) * 8) * 2);
+      lane_off = (int)(((int64_t)krow * ld + outer0 + (lane >> 3) * 32 + (lane & 3) * 8) * 2);
       blk_step = (int)(2 * ld * 2);
       k_step = (int)(BK * ld * 2);
     }
@@ -159,9 +164,10 @@ __device__ __forceinline__ uint4 read_frag(const char* tile, int outer_base, int
     const int i = lane & 15, g = lane >> 4;
     const int col = outer_base + (g & 1) * 16 + (i & 3) * 4;
     const int krow = ks * 16 + (g >> 1) * 8 + (i >> 2);
-    const char* p0 = tile + (krow >> 1) * kPairPitch + (krow & 1) * 512 + col * 2;
+    const int in_piece = ((col >> 5) * 2) * 64 + (col & 31) * 2;   // + 64 for the odd row of a pair
+    const char* p0 = tile + (krow >> 1) * kPairPitch + (krow & 1) * 64 + in_piece;
     const int krow1 = krow + 4;
-    const char* p1 = tile + (krow1 >> 1) * kPairPitch + (krow1 & 1) * 512 + col * 2;
+    const char* p1 = tile + (krow1 >> 1) * kPairPitch + (krow1 & 1) * 64 + in_piece;
     typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
     const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p0);
     const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p1);
