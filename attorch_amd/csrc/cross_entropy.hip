@@ -204,23 +204,61 @@ __global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_k
 
   const float scale = wt / denom[0] * up;
   const float k = scale / s;
-#pragma unroll
-  for (int i = 0; i < CACHE_VECS; ++i) {
-    const int v = tid + i * kCeBlock;
-    if (i < n_iter && v < n_int) {
-      float f[VEC];
-      unpack16<T>(cache[i], f);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) f[j] *= k;
-      store_grad_vec<T, TO>(dv, v, f);
-    }
-  }
-  if (edge >= 0) dr[edge] = from_f32<TO>(edge_e * k);
-  // The target column gets softmax - 1: the lane that stored the column overwrites it (stores of
-  // one lane to one address stay in order).
   const int tv = (int)t - head_n;   // target position relative to the first interior element
-  const bool owner = (tv >= 0 && tv < n_int * VEC) ? ((tv / VEC) % kCeBlock == tid) : (edge == (int)t);
-  if (owner) dr[t] = from_f32<TO>(fmaf(__builtin_amdgcn_exp2f(fmaf(x_t, kLog2e, -m2)), k, -scale));
+  const float g_target = fmaf(__builtin_amdgcn_exp2f(fmaf(x_t, kLog2e, -m2)), k, -scale);   // softmax - 1, scaled
+  if constexpr (!std::is_same<T, TO>::value) {
+    // fp32 gradient of 16-bit logits.  A lane's 8 values are 32 bytes of the output; stored as they
+    // are, each of the two store instructions of a wave writes every other 16 bytes of 2 KB — half
+    // of every cache line.  The values change lanes through LDS first (2 KB per wave, nobody else's:
+    // no barrier, a wave's LDS operations complete in order), so that each instruction writes one
+    // contiguous KiB.
+    __shared__ float4 exchange[kCeBlock / 64][128];
+    const int lane = tid & 63, wave = tid >> 6;
+    float4* const mine = exchange[wave];
+#pragma unroll
+    for (int i = 0; i < CACHE_VECS; ++i) {
+      if (i < n_iter) {   // uniform
+        float f[VEC];
+        unpack16<T>(cache[i], f);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) f[j] *= k;
+        mine[2 * lane] = make_float4(f[0], f[1], f[2], f[3]);
+        mine[2 * lane + 1] = make_float4(f[4], f[5], f[6], f[7]);
+        const float4 lo = mine[lane], hi = mine[64 + lane];
+        const int v0 = wave * 64 + i * kCeBlock;   // the wave's first vector of this sweep
+        float4* out = reinterpret_cast<float4*>(dv + (int64_t)v0 * VEC);
+        if (v0 + (lane >> 1) < n_int) out[lane] = lo;
+        if (v0 + 32 + (lane >> 1) < n_int) out[64 + lane] = hi;
+      }
+    }
+    if (edge >= 0) dr[edge] = edge_e * k;
+    // The target column gets softmax - 1 from the lane that stored it (stores of one lane to one
+    // address stay in order): vector tv / 8 is number tv / 8 % 64 of its wave's group of 64, and
+    // 16-byte piece 2 (number % 32) + (tv % 8) / 4 of that group's lower or upper KiB.
+    const int target_vec = tv / VEC;
+    const bool owner = (tv >= 0 && tv < n_int * VEC)
+                           ? (tid == (((target_vec >> 6) & (kCeBlock / 64 - 1)) << 6 | (target_vec & 31) << 1 |
+                                      ((tv >> 2) & 1)))
+                           : (edge == (int)t);
+    if (owner) dr[t] = g_target;
+  } else {
+#pragma unroll
+    for (int i = 0; i < CACHE_VECS; ++i) {
+      const int v = tid + i * kCeBlock;
+      if (i < n_iter && v < n_int) {
+        float f[VEC];
+        unpack16<T>(cache[i], f);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) f[j] *= k;
+        store_grad_vec<T, TO>(dv, v, f);
+      }
+    }
+    if (edge >= 0) dr[edge] = from_f32<TO>(edge_e * k);
+    // The target column gets softmax - 1: the lane that stored the column overwrites it (stores of
+    // one lane to one address stay in order).
+    const bool owner = (tv >= 0 && tv < n_int * VEC) ? ((tv / VEC) % kCeBlock == tid) : (edge == (int)t);
+    if (owner) dr[t] = from_f32<TO>(g_target);
+  }
 }
 
 // Streaming kernel: any dtypes, any alignment, any width; the row is read twice (online
