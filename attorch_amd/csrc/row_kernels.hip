@@ -814,7 +814,10 @@ __global__ __launch_bounds__(1024) void softmax_fwd_stream_kernel(
   }
 }
 
-template <typename TDY, typename TY, typename TDX, int VEC, int ITERS>
+// PERSIST: the workgroup walks over row-blocks (grid sized to the chip) and requests the next
+// row-block before it reduces and stores the current one.  !PERSIST: one row-block per workgroup
+// and nothing requested ahead; the grid covers the rows.
+template <typename TDY, typename TY, typename TDX, int VEC, int ITERS, bool PERSIST>
 __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
     const TDY* __restrict__ dy, const TY* __restrict__ y, TDX* __restrict__ dx, int64_t batch,
     int feat, int64_t dys, int64_t ys, int64_t dxs, int neg, int log, int group_log2) {
@@ -843,8 +846,10 @@ __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
   auto step = [&](int64_t rb, RowSet& cur, RowSet& nxt) {
     const int64_t row = rb * rpb + rib;
     const bool valid = row < batch;
-    nxt.dy.load(dy, row + row_step, dys, row + row_step < batch, lane, group, chunks);
-    nxt.y.load(y, row + row_step, ys, row + row_step < batch, lane, group, chunks);
+    if (PERSIST) {
+      nxt.dy.load(dy, row + row_step, dys, row + row_step < batch, lane, group, chunks);
+      nxt.y.load(y, row + row_step, ys, row + row_step < batch, lane, group, chunks);
+    }
     RowCache<TDY, VEC, ITERS>& cdy = cur.dy;
     RowCache<TY, VEC, ITERS>& cy = cur.y;
     cdy.mask(valid, lane, group, chunks, 0.f);   // dy = 0 makes every product of the padding vanish
@@ -881,6 +886,10 @@ __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
       }
     }
   };
+  if (!PERSIST) {
+    step(blockIdx.x, set_a, set_b);
+    return;
+  }
 #pragma unroll 1
   for (int64_t rb = blockIdx.x; rb < row_blocks; rb += 2 * (int64_t)gridDim.x) {
     step(rb, set_a, set_b);
@@ -981,6 +990,15 @@ inline int resident_blocks(const void* fn, int block, size_t lds) {
   }
   known.emplace(key, n);
   return n;
+}
+
+// Whether a backward pass that holds two tensors per row runs one row-block per workgroup instead
+// of the persistent grid: when there is work for many rounds of workgroups, a workgroup that ends
+// behind its stores does better than one that loops (its next loads count as arrived only after
+// its own stores are acknowledged); with few row-blocks per resident workgroup the ramp of short
+// workgroups costs more than that.
+inline bool one_shot(int64_t row_blocks, unsigned persistent) {
+  return row_blocks >= (int64_t)persistent * 4 && row_blocks <= (int64_t)INT32_MAX;
 }
 
 // Grid of a persistent row kernel: no more workgroups than stay resident at once, and as even a
@@ -1273,11 +1291,16 @@ int at_softmax_bwd(const void* dy, const void* y, void* dx, int64_t batch, int64
     const int64_t row_blocks = cdiv64(batch, p.block >> p.group_log2);
 #define AT_SOFTMAX_BWD_LAUNCH(VV)                                                                        \
   AT_DISPATCH_ITERS4(p.iters, {                                                                          \
-    auto kernel = softmax_bwd_kernel<TDY, TY, TY, VV, ITERS>;                                            \
+    auto kernel = softmax_bwd_kernel<TDY, TY, TY, VV, ITERS, true>;                                      \
     const unsigned grid = persistent_grid((const void*)kernel, p.block, 0, row_blocks, 0);               \
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(p.block), 0, stream, (const TDY*)dy, (const TY*)y,       \
-                       (TY*)dx, batch, (int)feat, dy_stride, y_stride, dx_stride, neg, log,              \
-                       p.group_log2);                                                                    \
+    if (one_shot(row_blocks, grid))                                                                      \
+      hipLaunchKernelGGL((softmax_bwd_kernel<TDY, TY, TY, VV, ITERS, false>), dim3((unsigned)row_blocks), \
+                         dim3(p.block), 0, stream, (const TDY*)dy, (const TY*)y, (TY*)dx, batch,         \
+                         (int)feat, dy_stride, y_stride, dx_stride, neg, log, p.group_log2);             \
+    else                                                                                                 \
+      hipLaunchKernelGGL(kernel, dim3(grid), dim3(p.block), 0, stream, (const TDY*)dy, (const TY*)y,     \
+                         (TY*)dx, batch, (int)feat, dy_stride, y_stride, dx_stride, neg, log,            \
+                         p.group_log2);                                                                  \
   })
     if (vec != 1) { AT_SOFTMAX_BWD_LAUNCH(VECW); } else { AT_SOFTMAX_BWD_LAUNCH(1); }
 #undef AT_SOFTMAX_BWD_LAUNCH
