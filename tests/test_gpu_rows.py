@@ -17,7 +17,10 @@ SHAPES = [(96,), (768,), (8000,), (1, 8000), (4, 2000), (8, 1024), (32, 1024), (
           (8096, 32), (12288, 1), (2049, 2), (4097, 4), (8, 960, 196), (2048, 64, 16), (33, 4096),
           (7, 8200), (5, 12345), (3, 40000), (2, 70001),
           # more row-blocks than the persistent grids hold at once: several rows per workgroup
-          (100001, 40), (20000, 520), (600000, 8)]
+          (100001, 40), (20000, 520), (600000, 8),
+          # many row-blocks per resident workgroup and a ragged last one: the softmax backward runs
+          # one row-block per workgroup here
+          (70001, 512), (9001, 4096)]
 
 
 @pytest.mark.parametrize('dtype', DTYPES)
