@@ -675,7 +675,8 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(
 // Softmax family.
 // ------------------------------------------------------------------------------------------
 // MAXB: largest workgroup the instance is launched with (256 leaves the compiler 256 registers per lane).
-template <typename TX, typename TY, int VEC, int ITERS, int MAXB>
+// PERSIST as in softmax_bwd_kernel: false = one row-block per workgroup, nothing requested ahead.
+template <typename TX, typename TY, int VEC, int ITERS, int MAXB, bool PERSIST>
 __global__ __launch_bounds__(MAXB) void softmax_fwd_kernel(
     const TX* __restrict__ x, TY* __restrict__ y, int64_t batch, int feat, int64_t xs, int64_t ys,
     int neg, int log, int group_log2) {
@@ -706,7 +707,7 @@ __global__ __launch_bounds__(MAXB) void softmax_fwd_kernel(
   auto step = [&](int64_t rb, RowCache<TX, VEC, ITERS>& cur, RowCache<TX, VEC, ITERS>& nxt) {
     const int64_t row = rb * rpb + rib;
     const bool valid = row < batch;
-    nxt.load(x, row + row_step, xs, row + row_step < batch, lane, group, chunks);
+    if (PERSIST) nxt.load(x, row + row_step, xs, row + row_step < batch, lane, group, chunks);
     cur.mask(valid, lane, group, chunks, pad);
     __builtin_amdgcn_sched_barrier(0);
 
@@ -766,6 +767,10 @@ __global__ __launch_bounds__(MAXB) void softmax_fwd_kernel(
       }
     }
   };
+  if (!PERSIST) {
+    step(blockIdx.x, set_a, set_b);
+    return;
+  }
 #pragma unroll 1
   for (int64_t rb = blockIdx.x; rb < row_blocks; rb += 2 * (int64_t)gridDim.x) {
     step(rb, set_a, set_b);
@@ -1241,10 +1246,16 @@ int at_softmax_fwd(const void* x, void* y, int64_t batch, int64_t feat, int64_t 
     const int64_t row_blocks = cdiv64(batch, p.block >> p.group_log2);
 #define AT_SOFTMAX_FWD_LAUNCH(VV, MAXB)                                                                  \
   AT_DISPATCH_ITERS(p.iters, {                                                                           \
-    auto kernel = softmax_fwd_kernel<TX, TY, VV, ITERS, MAXB>;                                           \
+    auto kernel = softmax_fwd_kernel<TX, TY, VV, ITERS, MAXB, true>;                                     \
     const unsigned grid = persistent_grid((const void*)kernel, p.block, 0, row_blocks, 0);               \
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(p.block), 0, stream, (const TX*)x, (TY*)y, batch,        \
-                       (int)feat, x_stride, y_stride, neg, log, p.group_log2);                           \
+    /* eight chunks per lane (one wave per wide row) do slightly better with the look-ahead */          \
+    if (ITERS < 8 && one_shot(row_blocks, grid))                                                         \
+      hipLaunchKernelGGL((softmax_fwd_kernel<TX, TY, VV, ITERS, MAXB, false>), dim3((unsigned)row_blocks), \
+                         dim3(p.block), 0, stream, (const TX*)x, (TY*)y, batch, (int)feat, x_stride,     \
+                         y_stride, neg, log, p.group_log2);                                              \
+    else                                                                                                 \
+      hipLaunchKernelGGL(kernel, dim3(grid), dim3(p.block), 0, stream, (const TX*)x, (TY*)y, batch,      \
+                         (int)feat, x_stride, y_stride, neg, log, p.group_log2);                         \
   })
     if (p.block <= 256) {
       if (vec != 1) { AT_SOFTMAX_FWD_LAUNCH(VECW, 256); } else { AT_SOFTMAX_FWD_LAUNCH(1, 256); }
