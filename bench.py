@@ -38,22 +38,22 @@ PEAK_MFMA_FP32_TFLOPS = 157.3    # dense fp32 MFMA
 # the 256 MB Infinity Cache serves are included.  They belong to the kernel sources whose digest is
 # TRAFFIC_SOURCE_DIGEST: when the sources of the loaded library differ, `traffic` is reported as
 # null and the recorded figure moves to `traffic_recorded` (stale until the profile is redone).
-TRAFFIC_SOURCE_DIGEST = '0c7fed6243f1f4da'
+TRAFFIC_SOURCE_DIGEST = 'e909313204c9756c'
 MEASURED_TRAFFIC_BYTES = {
-    'c4_linear_fwd': 4597191370,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.0 GiB read, 1.0 GiB written
-    'c2_layer_norm': 362347041,       # norm_fwd + norm_bwd + reduce_partials
-    'c2_rms_norm': 361817088,
-    'c2_softmax': 335901798,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
-    'c2_act_dropout': 335783801,      # act_dropout forward + backward
-    'c2_glu': 268579864,              # glu forward + backward
-    'c2_mse': 335720622,              # p_loss forward + backward
-    'c3_cross_entropy': 1718046981,   # ce_row_kernel (ignored rows are not read)
-    'c3_cross_entropy_autocast': 2503235731,
-    'c3_nll_loss': 826900559,         # nll forward (a gather) + the single-pass gradient write
-    'c5_conv_channels_last': 389747843,     # the two weights-in-registers kernels + weight gradient + weight reorders, no copies
-    'c5_conv': 595395565,             # the same + 2 layout copies
-    'c5_batch_norm_channels_last': 568556758,
-    'c5_batch_norm': 565693202,       # stats + apply + backward reduce + backward apply
+    'c4_linear_fwd': 4611841360,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.0 GiB read, 1.0 GiB written
+    'c2_layer_norm': 362346310,       # norm_fwd + norm_bwd + reduce_partials
+    'c2_rms_norm': 361810981,
+    'c2_softmax': 335893353,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
+    'c2_act_dropout': 335783418,      # act_dropout forward + backward
+    'c2_glu': 268580377,              # glu forward + backward
+    'c2_mse': 335721550,              # p_loss forward + backward
+    'c3_cross_entropy': 1717820790,   # ce_row_kernel (ignored rows are not read)
+    'c3_cross_entropy_autocast': 2502925447,
+    'c3_nll_loss': 826885215,         # nll forward (a gather) + the single-pass gradient write
+    'c5_conv_channels_last': 389746743,     # the two weights-in-registers kernels + weight gradient + weight reorders, no copies
+    'c5_conv': 595395114,             # the same + 2 layout copies
+    'c5_batch_norm_channels_last': 568555867,
+    'c5_batch_norm': 565688757,       # stats + apply + backward reduce + backward apply
 }
 
 
