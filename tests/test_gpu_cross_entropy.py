@@ -213,6 +213,40 @@ def test_autocast_at_vocabulary_width() -> None:
     assert torch.equal(xd.grad, grad.half())
 
 
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_fp32_gradient_with_targets_at_every_kind_of_position(dtype) -> None:
+    # fp32 gradient of 16-bit logits: the values change lanes before they are stored, and the target
+    # column is patched by the lane that stored it.  Targets at the first and last elements of rows
+    # (which start at different offsets from a 16-byte boundary, the width being odd), at both
+    # halves of a 16-byte vector, and around the points where a wave's and a workgroup's share of
+    # the row ends.
+    from attorch_amd import _lib
+    lib = _lib.load()
+    vocab = 50257
+    picks = [0, 1, 3, 4, 6, 7, 8, 9, 15, 16, 255, 256, 259, 260, 511, 512, 515, 516, 4091, 4092, 4095, 4096, 4099,
+             4100, 8191, 8192, 32767, 32768, 50248, 50249, 50252, 50253, 50255, 50256]
+    rows = len(picks)
+    x = randn((rows, vocab), 4001, dtype, 2.0)
+    target = torch.tensor(picks, dtype=torch.int64)
+    logits_d, target_d = x.cuda(), target.cuda()
+    grad = torch.full((rows, vocab), float('nan'), dtype=torch.float32, device='cuda')
+    loss = torch.empty((), dtype=torch.float32, device='cuda')
+    ws_bytes = lib.at_cross_entropy_workspace_bytes(rows)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device='cuda')
+    _lib.check(lib.at_cross_entropy_fwd_bwd(
+        logits_d.data_ptr(), target_d.data_ptr(), None, loss.data_ptr(), grad.data_ptr(), ws.data_ptr(), ws_bytes,
+        rows, vocab, vocab, vocab, -100, _lib.dtype_id(dtype), 0, _lib.dtype_id(torch.float32),
+        _lib.dtype_id(torch.float32), _lib.stream_of(logits_d)), 'at_cross_entropy_fwd_bwd')
+    ref = oracle.cross_entropy_backward(torch.tensor(1.0), x, target, None, -100, torch.float32,
+                                        compute=torch.float64)
+    assert not torch.isnan(grad).any()
+    assert_close(grad * rows, ref * rows, torch.float32, 'input_grad', atol_scale=10)
+    at_target = grad.cpu()[torch.arange(rows), target]
+    assert torch.all(at_target < 0), 'softmax - 1 at every target column'
+    assert_close(at_target * rows, ref[torch.arange(rows), target] * rows, torch.float32, 'target columns',
+                 atol_scale=10)
+
+
 def test_empty_batch_gives_nan_loss_and_empty_gradient() -> None:
     x = torch.empty(0, 7, device='cuda', requires_grad=True)
     loss = attorch_amd.CrossEntropyLoss()(x, torch.empty(0, dtype=torch.int64, device='cuda'))
