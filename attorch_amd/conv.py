@@ -154,7 +154,9 @@ class Conv2dAutoGrad(torch.autograd.Function):
                 and lib.at_conv2d_fwd_leaves_nhwc(*dims, dtype, dtype) == 1)
         ctx.input_nhwc = workspace if keep else None
         if requires_grad:
-            ctx.save_for_backward(input, weight)
+            # under autocast the weight gradient reads the low-precision copy made above
+            # (conv_layer.py:150-151 casts the saved input again): keep that copy
+            ctx.save_for_backward(input_k if input_k.dtype is not input.dtype else input, weight)
 
         return output
 
@@ -183,8 +185,8 @@ class Conv2dAutoGrad(torch.autograd.Function):
             # channels-last gradients in and out; a product this path does not cover is left to
             # the channels-first code below
             grad_last = output_grad.to(output_dtype).contiguous(memory_format=torch.channels_last)
-            need_input = input.requires_grad
-            need_weight = weight.requires_grad
+            need_input = ctx.needs_input_grad[0]
+            need_weight = ctx.needs_input_grad[1]
             with _lib.device_guard(input):
                 n_bytes = lib.at_conv2d_nhwc_workspace_bytes(1, *dims, dtype) if need_input else 0
                 if n_bytes > 0:
@@ -223,7 +225,7 @@ class Conv2dAutoGrad(torch.autograd.Function):
                     weight_grad if weight_grad is not None else rest[1], bias_grad,
                     None, None, None, None, None)
         return Conv2dAutoGrad._backward_channels_first(
-            ctx, input, weight, output_grad, input.requires_grad, weight.requires_grad,
+            ctx, input, weight, output_grad, ctx.needs_input_grad[0], ctx.needs_input_grad[1],
             ctx.bias_requires_grad)
 
     @staticmethod

@@ -210,8 +210,8 @@ __global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_k
     // fp32 gradient of 16-bit logits.  A lane's 8 values are 32 bytes of the output; stored as they
     // are, each of the two store instructions of a wave writes every other 16 bytes of 2 KB — half
     // of every cache line.  The values change lanes through LDS first (2 KB per wave, nobody else's:
-    // no barrier, a wave's LDS operations complete in order), so that each instruction writes one
-    // contiguous KiB.
+    // no workgroup barrier, a wave's LDS operations complete in order; wave barriers keep the compiler
+    // from reordering them), so that each instruction writes one contiguous KiB.
     __shared__ float4 exchange[kCeBlock / 64][128];
     const int lane = tid & 63, wave = tid >> 6;
     float4* const mine = exchange[wave];
@@ -224,7 +224,9 @@ __global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_k
         for (int j = 0; j < VEC; ++j) f[j] *= k;
         mine[2 * lane] = make_float4(f[0], f[1], f[2], f[3]);
         mine[2 * lane + 1] = make_float4(f[4], f[5], f[6], f[7]);
+        __builtin_amdgcn_wave_barrier();   // compiler only: the reads below stay behind the writes above
         const float4 lo = mine[lane], hi = mine[64 + lane];
+        __builtin_amdgcn_wave_barrier();   // ... and ahead of the next sweep's writes
         const int v0 = wave * 64 + i * kCeBlock;   // the wave's first vector of this sweep
         float4* out = reinterpret_cast<float4*>(dv + (int64_t)v0 * VEC);
         if (v0 + (lane >> 1) < n_int) out[lane] = lo;

@@ -123,7 +123,7 @@ class LinearAutoGrad(torch.autograd.Function):
         if bias_k is not None and output_dtype != input.dtype:
             bias_k = bias_k.to(output_dtype)
         contract_dim = in_feat_dim
-        ctx.padded_weight = None
+        padded_weight = None
         if _pad_features(batch_dim, in_feat_dim, out_feat_dim, compute_dtype):
             # zeros along the contraction add nothing; padded output columns are never stored
             contract_dim = _round_up8(in_feat_dim)
@@ -131,11 +131,12 @@ class LinearAutoGrad(torch.autograd.Function):
             weight_k = _zero_pad(weight_k, contract_dim, _round_up8(out_feat_dim))
             if input.requires_grad:
                 # the input gradient multiplies by the same padded copy: keep it instead of
-                # padding the weight a second time
-                ctx.padded_weight = weight_k
+                # padding the weight a second time (one more weight-sized buffer alive between
+                # forward and backward; it travels with the saved tensors, so hooks see it)
+                padded_weight = weight_k
 
         output = torch.empty((batch_dim, out_feat_dim), device=input.device, dtype=output_dtype)
-        if save_pre_act and ctx.padded_weight is not None and out_feat_dim % 8:
+        if save_pre_act and padded_weight is not None and out_feat_dim % 8:
             # the saved pre-activation gets rows that start on 16-byte boundaries (row stride
             # rounded up, the spare columns zero): the kernels then write and later read it in
             # whole vectors
@@ -159,8 +160,18 @@ class LinearAutoGrad(torch.autograd.Function):
         ctx.act = act
         ctx.bias_requires_grad = False if bias is None else bias.requires_grad
         ctx.output_dtype = output_dtype
+        ctx.input_shape = input.shape
         if requires_grad:
-            ctx.save_for_backward(input, pre_act if save_pre_act else None, weight)
+            # Under autocast the low-precision copies made for the forward product are what the
+            # backward products read (linear_layer.py:152-155 casts them again there): keeping
+            # them costs one cast per operand and step instead of two.  Copies that were
+            # zero-padded are not kept (the padded weight aside): backward pads afresh.
+            cast = compute_dtype != input.dtype or compute_dtype != weight.dtype
+            keep_input = (input_k if cast and input_k.shape[1] == in_feat_dim and weight.requires_grad
+                          else flattened_input)
+            keep_weight = (weight_k if cast and weight_k.shape == weight.shape and input.requires_grad
+                           else weight)
+            ctx.save_for_backward(keep_input, pre_act if save_pre_act else None, keep_weight, padded_weight)
 
         return output.view(*input.shape[:-1], out_feat_dim)
 
@@ -173,18 +184,18 @@ class LinearAutoGrad(torch.autograd.Function):
         Gradients of the linear layer with respect to input, weight and bias.
         """
         lib = _lib.load()
-        input, pre_act, weight = ctx.saved_tensors
-        _lib.require_same_device('Linear backward', input, output_grad)
+        flattened_input, pre_act, weight, padded_weight = ctx.saved_tensors
+        _lib.require_same_device('Linear backward', flattened_input, output_grad)
         output_dtype = ctx.output_dtype
-        device = input.device
+        device = flattened_input.device
+        input_needs_grad, weight_needs_grad = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
 
         output_grad = _matrix(output_grad.flatten(0, -2))
-        flattened_input = input.flatten(0, -2)
         batch_dim, in_feat_dim = flattened_input.shape
         _, out_feat_dim = weight.shape
-        stream = _lib.stream_of(input)
+        stream = _lib.stream_of(flattened_input)
 
-        if (weight.requires_grad and output_dtype is torch.float32
+        if (weight_needs_grad and output_dtype is torch.float32
                 and output_grad.dtype is torch.float32 and flattened_input.dtype is torch.float32
                 and weight.dtype is torch.float32 and (pre_act is None or pre_act.dtype is torch.float32)
                 and lib.at_linear_bwd_small_supported(batch_dim, in_feat_dim, out_feat_dim,
@@ -195,11 +206,11 @@ class LinearAutoGrad(torch.autograd.Function):
             operands = [output_grad, input_mm, weight_mm] + ([] if pre_act_mm is None else [pre_act_mm])
             if all(t.data_ptr() % 16 == 0 and _lib.row_stride(t) % 4 == 0 for t in operands):
                 input_grad = (torch.empty((batch_dim, in_feat_dim), dtype=output_dtype, device=device)
-                              if input.requires_grad else None)
+                              if input_needs_grad else None)
                 weight_grad = torch.empty((in_feat_dim, out_feat_dim), dtype=output_dtype, device=device)
                 bias_grad = (torch.empty(out_feat_dim, dtype=output_dtype, device=device)
                              if ctx.bias_requires_grad else None)
-                with _lib.device_guard(input):
+                with _lib.device_guard(flattened_input):
                     _lib.check(lib.at_linear_bwd_small(
                         _lib.ptr(output_grad), _lib.ptr(pre_act_mm), _lib.ptr(input_mm), _lib.ptr(weight_mm),
                         _lib.ptr(input_grad), _lib.ptr(weight_grad), _lib.ptr(bias_grad), batch_dim,
@@ -210,12 +221,15 @@ class LinearAutoGrad(torch.autograd.Function):
                         0.0 if ctx.param is None else ctx.param, _lib.dtype_id(torch.float32), stream),
                         'at_linear_bwd_small')
                 if input_grad is not None:
-                    input_grad = input_grad.view_as(input)
+                    input_grad = input_grad.view(ctx.input_shape)
                 return input_grad, weight_grad, bias_grad, None
 
-        with _lib.device_guard(input):
+        with _lib.device_guard(flattened_input):
             bias_grad = None
             padded_cols = _round_up8(out_feat_dim)
+            # set only where this function itself allocates a gradient buffer whose rows are
+            # zero-padded to whole vectors; never inferred from a tensor's strides
+            padded_grad = None
             if ctx.act_func is None:
                 pre_act_grad = output_grad
             elif (pre_act.stride(0) == padded_cols and padded_cols != out_feat_dim
@@ -238,6 +252,7 @@ class LinearAutoGrad(torch.autograd.Function):
                     0.0 if ctx.param is None else ctx.param, _lib.dtype_id(pre_act.dtype),
                     _lib.dtype_id(pre_act.dtype), _lib.dtype_id(pre_act.dtype), stream), 'at_act_bwd')
                 pre_act_grad = pre_act_grad_p[:, :out_feat_dim]
+                padded_grad = pre_act_grad_p
                 if bias_grad_p is not None:
                     bias_grad = bias_grad_p[:out_feat_dim].clone()
             else:
@@ -265,15 +280,14 @@ class LinearAutoGrad(torch.autograd.Function):
             contract_dim = out_feat_dim
             if pad:
                 contract_dim = _round_up8(out_feat_dim)
-                if grad_mm.stride(0) == contract_dim and grad_mm.shape[1] != contract_dim:
-                    # a view of a buffer whose rows are padded with zeros already
-                    grad_mm = grad_mm.as_strided((batch_dim, contract_dim), (contract_dim, 1))
+                if padded_grad is not None and padded_grad.dtype is output_dtype:
+                    grad_mm = padded_grad
                 else:
                     grad_mm = _zero_pad(grad_mm, batch_dim, contract_dim)
             input_grad = weight_grad = None
-            if input.requires_grad:
-                if pad and ctx.padded_weight is not None and ctx.padded_weight.dtype is output_dtype:
-                    weight_mm = ctx.padded_weight
+            if input_needs_grad:
+                if pad and padded_weight is not None and padded_weight.dtype is output_dtype:
+                    weight_mm = padded_weight
                 else:
                     weight_mm = _matrix(weight.to(output_dtype))
                     if pad:
@@ -284,8 +298,8 @@ class LinearAutoGrad(torch.autograd.Function):
                     in_feat_dim, contract_dim, _lib.row_stride(grad_mm), _lib.row_stride(weight_mm),
                     _lib.row_stride(input_grad), _lib.dtype_id(output_dtype),
                     _lib.dtype_id(output_dtype), stream), 'at_linear_bwd_input')
-                input_grad = input_grad.view_as(input)
-            if weight.requires_grad:
+                input_grad = input_grad.view(ctx.input_shape)
+            if weight_needs_grad:
                 input_mm = _matrix(flattened_input.to(output_dtype))
                 if pad:
                     input_mm = _zero_pad(input_mm, batch_dim, _round_up8(in_feat_dim))

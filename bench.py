@@ -109,24 +109,39 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument('--calibrate-copy', action='store_true',
                         help='also run a plain 256 MiB -> 256 MiB device copy, the known-size kernel that '
                              'hardware byte counters of a profiling run are scaled by')
+    parser.add_argument('--detail-file', type=str,
+                        default=os.path.join(os.path.dirname(os.path.abspath(__file__)), 'gpurun_out',
+                                             'bench_detail.json'),
+                        help='where the full per-config record (module-level, torch-native, CPU figures) goes')
     return parser.parse_args()
 
 
-def gpu_time_ms(fn: Callable[[], None], iters: int, warmup: int = 2) -> float:
+def gpu_time_ms(fn: Callable[[], None], iters: int, warmup: int = 2, batches: int = 1) -> float:
     """
-    Average duration of fn's GPU work in ms, from HIP events recorded on the stream the
-    kernels are launched on (PyTorch's current stream).
+    Duration of fn's GPU work in ms, from HIP events recorded on the stream the kernels are
+    launched on (PyTorch's current stream).  `batches` event-bracketed groups of `iters` calls
+    are timed back to back and the median of the groups' means is returned (one group: its mean).
     """
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(iters):
-        fn()
-    stop.record()
+    events = [torch.cuda.Event(enable_timing=True) for _ in range(batches + 1)]
+    events[0].record()
+    for b in range(batches):
+        for _ in range(iters):
+            fn()
+        events[b + 1].record()
     torch.cuda.synchronize()
-    return start.elapsed_time(stop) / iters
+    times = sorted(events[b].elapsed_time(events[b + 1]) / iters for b in range(batches))
+    return times[len(times) // 2]
+
+
+def kernel_time_ms(fn: Callable[[], None]) -> float:
+    """
+    The protocol of the secondary configs, whatever --steps says: 10 warm-up calls, then 60 timed
+    calls in 6 event-bracketed groups of 10, median of the groups.
+    """
+    return gpu_time_ms(fn, 10, 10, 6)
 
 
 def wall_time_ms(fn: Callable[[], None], steps: int, warmup: int) -> float:
@@ -319,10 +334,11 @@ def bench_linear(cfg: str, steps: int, warmup: int, with_cpu: bool) -> Dict:
     kernels = {}
     for kname, fn in (('linear_fwd', k_fwd), ('act_bwd_with_bias_grad', k_act), ('linear_bwd_input', k_dx),
                       ('linear_bwd_weight', k_dw), ('colsum_unfused', k_db)):
-        kernels[kname] = gpu_time_ms(fn, iters)
+        kernels[kname] = kernel_time_ms(fn) if cfg == 'c1' else gpu_time_ms(fn, iters, 2, 3)
     gemm_flop = 2.0 * m * k * n
     fwd_tflops = gemm_flop / kernels['linear_fwd'] / 1e9
     out = {
+        'tag': f'{cfg} linear {str(dtype)[6:]} {act}',
         'workload': f'{cfg}: Linear {str(dtype)[6:]} fwd+bwd X[{m},{k}] W[{k},{n}] act={act}',
         'metric': 'Linear fwd+bwd TFLOP/s', 'value': flop / ms_step / 1e9, 'unit': 'TFLOP/s',
         'ms_per_step': ms_step,
@@ -340,6 +356,8 @@ def bench_linear(cfg: str, steps: int, warmup: int, with_cpu: bool) -> Dict:
         layer.bias.grad = None
         result.backward(dyd)
     out['module_level'] = module_times_ms(lambda _: layer(xin), mod_bwd, max(3, min(steps, 20)), warmup)
+    if cfg == 'c4' and MODULE_TIMINGS:
+        out['amp'] = bench_linear_autocast(m, k, n, act, x, w, b, dy, max(3, min(steps, 10)), warmup)
     # torch's own GPU path for the same step (vendor BLAS + separate bias/activation kernels)
     ref_layer = torch.nn.Linear(k, n, bias=True, device='cuda', dtype=dtype)
     ref_act = torch.nn.GELU(approximate='tanh') if act == 'geluapprox' else torch.nn.ReLU()
@@ -378,6 +396,38 @@ def bench_linear(cfg: str, steps: int, warmup: int, with_cpu: bool) -> Dict:
         out['cpu_functional'] = functional_cpu_entry(
             cpu_functional, 6.0 * rows * k * n / 1e12, 'TFLOP/s', f'first {rows} of {m} rows, full K and N', dtype)
     return out
+
+
+def bench_linear_autocast(m, k, n, act, x, w, b, dy, steps: int, warmup: int) -> Dict:
+    """
+    The c4 layer as the reference's examples run it (examples/utils.py:13-36, amp=True): float32
+    input and parameters, forward under torch.autocast(float16), float16 output, float32 gradients
+    on the leaves; beside it the same layer with float16 tensors throughout.
+    """
+    import attorch_amd
+    f16 = torch.float16
+    result = {}
+    for label, store in (('fp16_tensors', f16), ('autocast_fp16_over_fp32_tensors', torch.float32)):
+        layer = attorch_amd.Linear(k, n, bias=True, act_func=act, dtype=store)
+        with torch.no_grad():
+            layer.weight.copy_(w.cuda())
+            layer.bias.copy_(b.cuda())
+        xin = x.to(store).cuda().requires_grad_(True)
+        dyd = dy.to(f16).cuda()
+
+        def step():
+            xin.grad = None
+            layer.weight.grad = None
+            layer.bias.grad = None
+            with torch.autocast('cuda', dtype=f16, enabled=store is torch.float32):
+                y = layer(xin)
+            y.backward(dyd)
+        result['ms_per_step_' + label] = _r(wall_time_ms(step, steps, warmup), 5)
+        del layer, xin, dyd
+        torch.cuda.empty_cache()
+    result['autocast_over_fp16'] = _r(result['ms_per_step_autocast_fp16_over_fp32_tensors'] /
+                                      result['ms_per_step_fp16_tensors'], 4)
+    return result
 
 
 # ------------------------------------------------------------------------------------------
@@ -476,8 +526,8 @@ def bench_rows(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
     def ew3():
         i = nxt()
         torch.add(xs[i], dys[i], out=dxs[i])
-    stream_ref = {'read1_write1_gbs': 2 * tbytes / gpu_time_ms(ew2, iters, warmup) / 1e6,
-                  'read2_write1_gbs': 3 * tbytes / gpu_time_ms(ew3, iters, warmup) / 1e6}
+    stream_ref = {'read1_write1_gbs': 2 * tbytes / kernel_time_ms(ew2) / 1e6,
+                  'read2_write1_gbs': 3 * tbytes / kernel_time_ms(ew3) / 1e6}
     # standalone activation layer with fused dropout on the same buffers (GELU-tanh, p = 0.1)
     def act_f():
         i = nxt()
@@ -545,10 +595,11 @@ def bench_rows(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
     for name, f, bwd, cpu in (('LayerNorm', ln_f, ln_b, cpu_ln), ('RMSNorm', rms_f, rms_b, cpu_rms),
                               ('Softmax', sm_f, sm_b, cpu_sm(False)), ('LogSoftmax', lsm_f, lsm_b, cpu_sm(True)),
                               ('GELU(tanh)+Dropout(0.1) layer', act_f, act_b, cpu_act)):
-        ms_f = gpu_time_ms(f, iters, warmup)
-        ms_b = gpu_time_ms(bwd, iters, warmup)
+        ms_f = kernel_time_ms(f)
+        ms_b = kernel_time_ms(bwd)
         gbs = 5 * tbytes / (ms_f + ms_b) / 1e6
         entry = {
+            'tag': f'c2 {name}',
             'workload': f'c2: {name} bf16 fwd+bwd X[{rows_},{feat}]', 'metric': 'HBM GB/s', 'value': gbs,
             'unit': 'GB/s', 'ms_fwd': ms_f, 'ms_bwd': ms_b,
             'fwd_gbs': 2 * tbytes / ms_f / 1e6, 'bwd_gbs': 3 * tbytes / ms_b / 1e6,
@@ -598,10 +649,11 @@ def bench_rows(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
                                     rows_ * feat, 2, 1, 1.0, dt, dt, dt, st()), 'mse_bwd')
     for name, f, bwd, fwd_units, bwd_units in (('GLU(sigmoid) over the features', glu_f, glu_b, 1.5, 2.5),
                                                ('MSELoss(mean), input gradient', mse_f, mse_b, 2.0, 3.0)):
-        ms_f = gpu_time_ms(f, iters, warmup)
-        ms_b = gpu_time_ms(bwd, iters, warmup)
+        ms_f = kernel_time_ms(f)
+        ms_b = kernel_time_ms(bwd)
         gbs = (fwd_units + bwd_units) * tbytes / (ms_f + ms_b) / 1e6
         results.append({
+            'tag': f'c2-shaped {name.split("(")[0]}',
             'workload': f'c2-shaped: {name} bf16 fwd+bwd X[{rows_},{feat}]', 'metric': 'HBM GB/s', 'value': gbs,
             'unit': 'GB/s', 'ms_fwd': ms_f, 'ms_bwd': ms_b,
             'fwd_gbs': fwd_units * tbytes / ms_f / 1e6, 'bwd_gbs': bwd_units * tbytes / ms_b / 1e6,
@@ -670,9 +722,10 @@ def bench_cross_entropy(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
         return module_times_ms(fwd, bwd, iters, warmup)
 
     for label, wt in (('unweighted', None), ('class-weighted', weight)):
-        ms = gpu_time_ms(c_abi_step(wt, dt, dlogits, loss), iters, warmup)
+        ms = kernel_time_ms(c_abi_step(wt, dt, dlogits, loss))
         gbs = (read_bytes + tbytes) / ms / 1e6
         entry = {
+            'tag': f'c3 CE {label}',
             'workload': f'c3: CrossEntropyLoss fp16 fwd+bwd logits[{rows_},{feat}], 5% ignore_index, {label}',
             'metric': 'HBM GB/s', 'value': gbs, 'unit': 'GB/s', 'ms_fwd_bwd': ms,
             'algorithmic_bytes': int(read_bytes + tbytes),
@@ -705,9 +758,10 @@ def bench_cross_entropy(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
     # custom_fwd(cast_inputs=float32) semantics): T read, 2T written, still one pass.
     grad32 = torch.empty((rows_, feat), dtype=torch.float32, device='cuda')
     loss32 = torch.empty((), dtype=torch.float32, device='cuda')
-    ms = gpu_time_ms(c_abi_step(None, raw._lib.dtype_id(torch.float32), grad32, loss32), iters, warmup)
+    ms = kernel_time_ms(c_abi_step(None, raw._lib.dtype_id(torch.float32), grad32, loss32))
     gbs = (read_bytes + 2 * tbytes) / ms / 1e6
     results.append({
+        'tag': 'c3 CE autocast fp32 grad',
         'workload': f'c3 autocast: CrossEntropyLoss fp16 logits[{rows_},{feat}] -> fp32 loss and gradient, '
                     f'5% ignore_index, unweighted',
         'metric': 'HBM GB/s', 'value': gbs, 'unit': 'GB/s', 'ms_fwd_bwd': ms,
@@ -738,10 +792,11 @@ def bench_cross_entropy(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
         raw.check(lib.at_nll_loss_bwd(one.data_ptr(), tgt_valid.data_ptr(), weight.data_ptr(),
                                       sum_weights.data_ptr(), dlogp.data_ptr(), rows_, feat, 1, 1, dt, 0, dt,
                                       st()), 'nll_bwd')
-    ms_f = gpu_time_ms(nll_fwd, max(5, steps // 2), warmup)
-    ms_b = gpu_time_ms(nll_bwd, max(5, steps // 2), warmup)
+    ms_f = kernel_time_ms(nll_fwd)
+    ms_b = kernel_time_ms(nll_bwd)
     gbs = tbytes / (ms_f + ms_b) / 1e6
     results.append({
+        'tag': 'c3 NLL weighted',
         'workload': f'c3: NLLLoss fp16 fwd+bwd log-probabilities[{rows_},{feat}], class-weighted mean',
         'metric': 'HBM GB/s', 'value': gbs, 'unit': 'GB/s', 'ms_fwd': ms_f, 'ms_bwd': ms_b,
         'bwd_gbs': tbytes / ms_b / 1e6,
@@ -844,7 +899,7 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
         conv_f()
         counter[0] = i - 1
         conv_dyh()
-    t = {k_: gpu_time_ms(f, iters, warmup) for k_, f in (('conv_fwd', conv_f), ('conv_grad_to_channels_last', conv_dyh),
+    t = {k_: kernel_time_ms(f) for k_, f in (('conv_fwd', conv_f), ('conv_grad_to_channels_last', conv_dyh),
                                                         ('conv_bwd_input', conv_dx),
                                                         ('conv_bwd_weight', conv_dw), ('bn_fwd', bn_f),
                                                         ('bn_bwd', bn_b_))}
@@ -856,12 +911,14 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
     # residual gradient: 8 tensors
     bn_gbs = 8 * tbytes / (t['bn_fwd'] + t['bn_bwd']) / 1e6
     conv_entry = {
+        'tag': 'c5 conv NCHW',
         'workload': f'c5: Conv2d 3x3 s1 p1 bf16 fwd+bwd X[{n},{c},{h},{w_}] W[{c},{c},3,3]',
         'metric': 'conv TFLOP/s', 'value': conv_tf, 'unit': 'TFLOP/s', 'kernel_ms': {k_: t[k_] for k_ in t if 'conv' in k_},
         'roofline': {'bound': 'mfma', 'achieved': conv_tf, 'peak': PEAK_MFMA_16BIT_TFLOPS, 'unit': 'TFLOP/s',
                      'frac': conv_tf / PEAK_MFMA_16BIT_TFLOPS, **traffic_fields('c5_conv')},
     }
     bn_entry = {
+        'tag': 'c5 BN NCHW',
         'workload': f'c5: BatchNorm2d(train)+residual+ReLU bf16 fwd+bwd X[{n},{c},{h},{w_}]',
         'metric': 'HBM GB/s', 'value': bn_gbs, 'unit': 'GB/s', 'ms_fwd': t['bn_fwd'], 'ms_bwd': t['bn_bwd'],
         'roofline': {'bound': 'hbm', 'achieved': bn_gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
@@ -892,11 +949,12 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
         i = nxt()
         raw.check(lib.at_conv2d_bwd_weight_nhwc(dyl[i].data_ptr(), xl[i].data_ptr(), dwt.data_ptr(),
                                                 lwork.data_ptr(), lws[2], *dims, dt, st()), 'conv_dw_nhwc')
-    tl = {k_: gpu_time_ms(f, iters, warmup) for k_, f in (('conv_fwd', last_f), ('conv_bwd_input', last_dx),
+    tl = {k_: kernel_time_ms(f) for k_, f in (('conv_fwd', last_f), ('conv_bwd_input', last_dx),
                                                          ('conv_bwd_weight', last_dw))}
     last_ms = sum(tl.values())
     last_tf = 3 * gflop / last_ms
     conv_last_entry = {
+        'tag': 'c5 conv NHWC',
         'workload': f'c5 with channels-last tensors: Conv2d 3x3 s1 p1 bf16 fwd+bwd X[{n},{c},{h},{w_}] '
                     f'W[{c},{c},3,3], memory format torch.channels_last',
         'metric': 'conv TFLOP/s', 'value': last_tf, 'unit': 'TFLOP/s', 'kernel_ms': tl,
@@ -925,9 +983,10 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
     for i in range(nsets):
         counter[0] = i - 1
         bn_last_f()
-    tbl = {k_: gpu_time_ms(f, iters, warmup) for k_, f in (('bn_fwd', bn_last_f), ('bn_bwd', bn_last_b))}
+    tbl = {k_: kernel_time_ms(f) for k_, f in (('bn_fwd', bn_last_f), ('bn_bwd', bn_last_b))}
     bn_last_gbs = 8 * n * c * h * w_ * 2 / (tbl['bn_fwd'] + tbl['bn_bwd']) / 1e6
     bn_last_entry = {
+        'tag': 'c5 BN NHWC',
         'workload': f'c5 with channels-last tensors: BatchNorm2d(train)+residual+ReLU bf16 fwd+bwd X[{n},{c},{h},{w_}]',
         'metric': 'HBM GB/s', 'value': bn_last_gbs, 'unit': 'GB/s', 'ms_fwd': tbl['bn_fwd'], 'ms_bwd': tbl['bn_bwd'],
         'roofline': {'bound': 'hbm', 'achieved': bn_last_gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
@@ -1084,13 +1143,10 @@ def main() -> int:
         extra.extend(bench_cross_entropy(args.steps, args.warmup, with_cpu))
     if 'c5' in wanted:
         extra.extend(bench_conv_bn(args.steps, args.warmup, with_cpu))
-    line = {
-        'metric': 'Linear fwd+bwd TFLOP/s; norm/softmax/CE HBM GB/s; % of MI355X roofline',
-        'value': head['value'], 'unit': 'TFLOP/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
-        'ms_per_step': head['ms_per_step'], 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
-        'dtype': 'bf16', 'data': 'synthetic',
-        'config': {'workload': head['workload'], 'step': 'attorch_amd.Linear forward + backward (dX, dW, db)',
-                   'algorithmic_flop_per_step': 6 * 16384 * 4096 * 16384},
+    detail = {
+        'metric': METRIC, 'value': head['value'], 'unit': 'TFLOP/s', 'n_gpus': 1, 'steps': args.steps,
+        'warmup': args.warmup, 'ms_per_step': head['ms_per_step'],
+        'config': {'workload': head['workload']},
         'roofline': head['roofline'],
         'cpu_baseline': head.get('cpu_baseline'),
         'cpu_functional': head.get('cpu_functional'),
@@ -1098,10 +1154,68 @@ def main() -> int:
         'torch_native': head.get('torch_native'),
         'frac_of_peak_step': head['frac_of_peak_step'],
         'kernel_ms': head['kernel_ms'], 'kernel_tflops': head['kernel_tflops'],
+        'amp': head.get('amp'),
         'configs': extra,
     }
-    print(json.dumps(line))
+    # Everything measured goes to a file (--detail-file, by default gpurun_out/bench_detail.json
+    # beside this script); stdout carries only the one compact line.
+    try:
+        os.makedirs(os.path.dirname(os.path.abspath(args.detail_file)), exist_ok=True)
+        with open(args.detail_file, 'w') as fh:
+            fh.write(json.dumps(detail) + '\n')
+    except OSError as exc:
+        print(f'bench.py: detail file not written ({exc})', file=sys.stderr)
+    print(json.dumps(compact_line(args, head, extra)))
     return 0
+
+
+METRIC = 'Linear fwd+bwd TFLOP/s; norm/softmax/CE HBM GB/s; % of MI355X roofline'
+
+
+def _r(v, digits=4):
+    return None if v is None else float(f'{v:.{digits}g}')
+
+
+def compact_line(args, head: Dict, extra: List[Dict]) -> Dict:
+    """
+    The one JSON line a harness parses: the contract fields, the headline's roofline and CPU
+    baseline, and per secondary config its tag, value, unit, roofline fraction, measured traffic
+    and CPU baseline.  Kept well under 4 KB.
+    """
+    configs = []
+    for e in extra:
+        item = {'tag': e.get('tag', e['workload'][:40]), 'value': _r(e['value']), 'unit': e['unit'],
+                'frac': _r(e['roofline']['frac']), 'traffic': e['roofline'].get('traffic')}
+        if e.get('cpu_baseline') is not None:
+            item['cpu'] = _r(e['cpu_baseline']['value'])
+        if 'ms_per_step' in e:
+            item['ms_per_step'] = _r(e['ms_per_step'])
+        if 'frac_of_peak_step' in e:
+            item['frac_step'] = _r(e['frac_of_peak_step'])
+        configs.append(item)
+    roof = head['roofline']
+    cb = head.get('cpu_baseline')
+    line = {
+        'metric': METRIC,
+        'value': _r(head['value'], 6), 'unit': 'TFLOP/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'ms_per_step': _r(head['ms_per_step'], 6), 'higher_is_better': True, 'scaling': 'weak',
+        'vs_baseline': None, 'dtype': 'bf16', 'data': 'synthetic',
+        'config': {'workload': head['workload'], 'step': 'attorch_amd.Linear forward + backward (dX, dW, db)',
+                   'algorithmic_flop_per_step': 6 * 16384 * 4096 * 16384},
+        'roofline': {'bound': roof['bound'], 'achieved': _r(roof['achieved'], 6), 'peak': roof['peak'],
+                     'unit': roof['unit'], 'frac': _r(roof['frac']), 'traffic': roof.get('traffic'),
+                     'kernel': roof.get('kernel')},
+        'cpu_baseline': None if cb is None else {'value': _r(cb['value']), 'unit': cb['unit'], 'cores': cb['cores'],
+                                                 'kind': cb['kind'], 'sample': cb['sample']},
+        'frac_of_peak_step': _r(head['frac_of_peak_step']),
+        'kernel_ms': {k: _r(v) for k, v in head['kernel_ms'].items()},
+        'configs_note': 'per secondary config: value in unit, frac of its roofline, traffic = measured HBM bytes '
+                        'per fwd+bwd, cpu = oracle on the host cores (cpu_baseline.cores threads) in the same unit',
+        'configs': configs,
+    }
+    if head.get('amp') is not None:
+        line['amp'] = head['amp']
+    return line
 
 
 if __name__ == '__main__':

@@ -189,7 +189,10 @@ int at_cross_entropy_scale_grad(void* dlogits, const void* output_grad, int64_t 
  * held until the process ends), so batch is limited to at_cross_entropy_static_max_batch()
  * = 65536 rows; larger batches return AT_ERR_WORKSPACE.  Every call on a GPU shares that
  * GPU's array: calls that overlap in time on one GPU (two streams) race; calls ordered on one
- * stream do not.  Arguments and results otherwise as at_cross_entropy_fwd_bwd. */
+ * stream do not.  The first call on a device looks up the address of that array
+ * (hipGetDevice + hipGetSymbolAddress, no allocation): make it outside a graph capture; later
+ * calls are kernel launches only.  Arguments and results otherwise as
+ * at_cross_entropy_fwd_bwd. */
 int64_t at_cross_entropy_static_max_batch(void);
 
 int at_cross_entropy_fwd_bwd_static(const void* logits, const int64_t* target,

@@ -109,6 +109,11 @@ def test_c3_cross_entropy_fp16(weighted) -> None:
 
 
 def test_c4_linear_bf16_gelu() -> None:
+    """
+    Every element of the output, the saved pre-activation and the three gradients against the
+    oracle, which runs the whole 6.6 TFLOP step on the host in row blocks.  No reference value
+    depends on anything the device computed.
+    """
     m, k, n = 16384, 4096, 16384
     x, w, b = randn((m, k), 4001, BF16), randn((k, n), 4002, BF16, 0.02), torch.zeros(n, dtype=BF16)
     dy = randn((m, n), 4003, BF16)
@@ -116,20 +121,64 @@ def test_c4_linear_bf16_gelu() -> None:
     y = attorch_amd.LinearAutoGrad.apply(xd, wd, bd, 'geluapprox')
     pre_act = y.grad_fn.saved_tensors[1].detach()
     y.backward(dy.cuda())
+    y, dx, dw, db = y.detach(), xd.grad, wd.grad, bd.grad
 
-    rows = torch.cat([torch.arange(0, 48), torch.arange(8000, 8032), torch.arange(m - 48, m)])
-    y_ref, pre_ref = oracle.linear_forward(x[rows], w, b, 'geluapprox', None, BF16)
-    assert_close(y[rows.cuda()], y_ref, BF16, 'output rows')
-    assert_close(pre_act[rows.cuda()], pre_ref, BF16, 'pre_act rows')
-    # backward of the sampled rows from the device's own pre-activation
-    dx_ref, _, _ = oracle.linear_backward(dy[rows], x[rows], w, pre_act[rows.cuda()].cpu(), 'geluapprox', None, BF16)
-    assert_close(xd.grad[rows.cuda()], dx_ref, BF16, 'input_grad rows')
-    # weight gradient: a band of input features over the whole batch, and the bias gradient
-    dz = (dy.float() * oracle.act_grad(pre_act.cpu().float(), 'geluapprox')).to(BF16)
-    cols = torch.cat([torch.arange(0, 8), torch.arange(2048, 2056), torch.arange(k - 8, k)])
-    dw_ref = (x[:, cols].float().T @ dz.float()).to(BF16)
-    assert_close(wd.grad[cols.cuda()], dw_ref, BF16, 'weight_grad rows', batch_reduction=True)
-    assert_close(bd.grad, dz.float().sum(dim=0).to(BF16), BF16, 'bias_grad', batch_reduction=True)
+    wf = w.float()
+    dw_sum = torch.zeros((k, n), dtype=F32)
+    db_sum = torch.zeros(n, dtype=torch.float64)
+    block = 2048
+    for r0 in range(0, m, block):
+        rows = slice(r0, r0 + block)
+        y_ref, pre_ref = oracle.linear_forward(x[rows], w, b, 'geluapprox', None, BF16)
+        assert_close(y[rows], y_ref, BF16, f'output rows {r0}..')
+        assert_close(pre_act[rows], pre_ref, BF16, f'pre_act rows {r0}..')
+        dz = (dy[rows].float() * oracle.act_grad(pre_ref.float(), 'geluapprox')).to(BF16)
+        assert_close(dx[rows], (dz.float() @ wf.T).to(BF16), BF16, f'input_grad rows {r0}..')
+        dw_sum += x[rows].float().T @ dz.float()
+        db_sum += dz.double().sum(dim=0)
+    assert_close(dw, dw_sum.to(BF16), BF16, 'weight_grad', batch_reduction=True)
+    assert_close(db, db_sum.float().to(BF16), BF16, 'bias_grad', batch_reduction=True)
+
+
+def test_c4_linear_autocast_fp16() -> None:
+    """
+    The c4 layer the way the reference's examples run it: float32 input and parameters under
+    torch.autocast(float16).  Operands and bias are rounded to float16 for the product
+    (linear_kernels.py:161-163,171-172), output and saved pre-activation are float16, the
+    backward products run in float16 and autograd widens the gradients to float32.
+    One row of every 256-row tile (all columns) for the output, the pre-activation and the
+    input gradient; a band of output features over the whole batch for the weight and bias
+    gradients, its reference pre-activation computed on the host.
+    """
+    m, k, n = 16384, 4096, 16384
+    x, w, b = randn((m, k), 4011), randn((k, n), 4012, F32, 0.02), randn((n,), 4013, F32, 0.1)
+    dy = randn((m, n), 4014, F16)
+    xd, wd, bd = (t.cuda().requires_grad_(True) for t in (x, w, b))
+    with torch.autocast('cuda', dtype=F16):
+        y = attorch_amd.LinearAutoGrad.apply(xd, wd, bd, 'geluapprox')
+    assert y.dtype is F16
+    pre_act = y.grad_fn.saved_tensors[1].detach()
+    assert pre_act.dtype is F16
+    # the saved operands are the float16 copies the forward product read, not float32 tensors
+    assert y.grad_fn.saved_tensors[0].dtype is F16 and y.grad_fn.saved_tensors[2].dtype is F16
+    y.backward(dy.cuda())
+    assert xd.grad.dtype is F32 and wd.grad.dtype is F32 and bd.grad.dtype is F32
+
+    rows = torch.tensor([t * 256 + (t * 37) % 256 for t in range(m // 256)] + [0, m - 1])
+    y_ref, pre_ref = oracle.linear_forward(x[rows], w, b, 'geluapprox', None, F16)
+    assert_close(y[rows.cuda()], y_ref, F16, 'output rows')
+    assert_close(pre_act[rows.cuda()], pre_ref, F16, 'pre_act rows')
+    dx_ref, _, _ = oracle.linear_backward(dy[rows], x[rows], w, pre_ref, 'geluapprox', None, F16)
+    assert_close(xd.grad[rows.cuda()], dx_ref.float(), F16, 'input_grad rows')
+
+    cols = torch.cat([torch.arange(0, 8), torch.arange(8190, 8198), torch.arange(n - 8, n)])
+    x16, w16 = x.to(F16).float(), w[:, cols].to(F16).float()
+    pre_band = (x16 @ w16 + b[cols].to(F16).float()).to(F16)
+    dz_band = (dy[:, cols].float() * oracle.act_grad(pre_band.float(), 'geluapprox')).to(F16)
+    assert_close(wd.grad[:, cols.cuda()], (x16.T @ dz_band.float()).to(F16).float(), F16, 'weight_grad band',
+                 batch_reduction=True)
+    assert_close(bd.grad[cols.cuda()], dz_band.float().sum(dim=0).to(F16).float(), F16, 'bias_grad band',
+                 batch_reduction=True)
 
 
 def test_c5_conv_bn_residual_relu_bf16() -> None:

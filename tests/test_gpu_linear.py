@@ -301,3 +301,80 @@ def test_small_backward_declines_other_shapes() -> None:
     p = t.data_ptr()
     assert lib.at_linear_bwd_small(p, p, p, p, p, p, None, 512, 783, 256, 256, 256, 783, 256, 783, 256, 4, 0.0, f32,
                                    _lib.stream_of(t)) == -7                  # AT_ERR_UNSUPPORTED, nothing launched
+
+
+@pytest.mark.parametrize('dtype', HALF_DTYPES)
+@pytest.mark.parametrize('offset', [0, 7])
+@pytest.mark.parametrize('input_grad', [True, False])
+def test_padded_path_takes_a_column_slice_as_upstream_gradient(dtype, offset, input_grad) -> None:
+    """
+    16-bit layer whose output width is not a multiple of 8 (the zero-padded operand path), no
+    activation, and an upstream gradient that is a column slice of a wider tensor whose row
+    stride happens to equal the padded width — as the backward of a concatenation hands out.
+    What lies outside the slice (NaN here) must never be read as padding.
+    """
+    batch, in_dim, out_dim, wide = 512, 200, 1001, 1008
+    x = randn((batch, in_dim), 1, dtype)
+    w = randn((in_dim, out_dim), 2, dtype, in_dim ** -0.5)
+    b = randn((out_dim,), 3, dtype, 0.1)
+    dy = randn((batch, out_dim), 4, dtype)
+    holder = torch.full((batch, wide), float('nan'), dtype=dtype, device='cuda')
+    upstream = holder[:, offset:offset + out_dim]
+    upstream.copy_(dy)
+    assert upstream.stride(0) == wide and not upstream.is_contiguous()
+    xd, wd, bd = x.cuda().requires_grad_(input_grad), w.cuda().requires_grad_(True), b.cuda().requires_grad_(True)
+    y = attorch_amd.LinearAutoGrad.apply(xd, wd, bd, None)
+    y.backward(upstream)
+    dx_ref, dw_ref, db_ref = oracle.linear_backward(dy, x, w, None, None, None, dtype)
+    if input_grad:
+        assert_close(xd.grad, dx_ref, dtype, 'input_grad')
+    assert_close(wd.grad, dw_ref, dtype, 'weight_grad', batch_reduction=True)
+    assert_close(bd.grad, db_ref, dtype, 'bias_grad', batch_reduction=True)
+
+
+@pytest.mark.parametrize('amp_dtype', HALF_DTYPES)
+@pytest.mark.parametrize('act_func', [None, 'relu', 'geluapprox'])
+@pytest.mark.parametrize('shape, out_dim', [((512, 256), 512), ((2048, 768), 768), ((4, 100, 333), 77),
+                                            ((1024, 200), 1001), ((64, 96), 80)])
+def test_linear_under_autocast_with_fp32_parameters(shape, out_dim, act_func, amp_dtype) -> None:
+    """
+    The reference's default training mode (examples/utils.py:13-36, tests/test_linear_layer.py
+    amp=True): float32 input and parameters under torch.autocast.  Operands and bias are rounded
+    to the autocast dtype for the product (linear_kernels.py:161-163,171-172), output and
+    pre-activation have that dtype, and the gradients reach the float32 leaves as float32.
+    """
+    in_dim = shape[-1]
+    x = randn(shape, 1)
+    w = randn((in_dim, out_dim), 2, torch.float32, in_dim ** -0.5)
+    b = randn((out_dim,), 3, torch.float32, 0.1)
+    dy = randn((*shape[:-1], out_dim), 4, amp_dtype)
+    name, param = oracle.parse_act_func(act_func)
+    xd, wd, bd = (t.cuda().requires_grad_(True) for t in (x, w, b))
+    with torch.autocast('cuda', dtype=amp_dtype):
+        y = attorch_amd.LinearAutoGrad.apply(xd, wd, bd, act_func)
+    assert y.dtype is amp_dtype
+    # nothing float32 and operand-sized is kept for backward: the casts made for the forward
+    # product are (zero-padded layers keep the originals and pad afresh)
+    saved = y.grad_fn.saved_tensors
+    if in_dim % 8 == 0 and out_dim % 8 == 0:
+        assert saved[0].dtype is amp_dtype and saved[2].dtype is amp_dtype
+    pre_act = None if saved[1] is None else saved[1].detach().cpu()
+    y.backward(dy.cuda())
+    assert xd.grad.dtype is torch.float32 and wd.grad.dtype is torch.float32 and bd.grad.dtype is torch.float32
+    y_ref, pre_ref = oracle.linear_forward(x, w, b, name, param, amp_dtype)
+    assert_close(y, y_ref, amp_dtype, 'output')
+    if name is not None:
+        assert_close(pre_act, pre_ref, amp_dtype, 'pre_act')
+    dx_ref, dw_ref, db_ref = oracle.linear_backward(dy, x, w, pre_act, name, param, amp_dtype)
+    assert_close(xd.grad, dx_ref.float(), amp_dtype, 'input_grad')
+    assert_close(wd.grad, dw_ref.float(), amp_dtype, 'weight_grad', batch_reduction=True)
+    assert_close(bd.grad, db_ref.float(), amp_dtype, 'bias_grad', batch_reduction=True)
+    # a second backward pass through a retained graph reads the same saved casts
+    xd.grad = wd.grad = bd.grad = None
+    with torch.autocast('cuda', dtype=amp_dtype):
+        y2 = attorch_amd.LinearAutoGrad.apply(xd, wd, bd, act_func)
+    y2.backward(dy.cuda(), retain_graph=True)
+    first = wd.grad.clone()
+    wd.grad = None
+    y2.backward(dy.cuda())
+    torch.testing.assert_close(wd.grad, first, rtol=0, atol=0)
