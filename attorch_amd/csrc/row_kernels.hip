@@ -376,8 +376,12 @@ __global__ __launch_bounds__(1024) void norm_fwd_stream_kernel(
 // Norm backward over a persistent grid.  Each workgroup walks row-blocks with a grid stride;
 // each lane accumulates the parameter gradients of the columns it owns.
 //   part_w / part_b: [gridDim.x, feat] fp32 partial rows (null when not wanted).
-// Dynamic LDS: blockDim.x * VEC floats (only used when a workgroup holds several rows).
+// Dynamic LDS: blockDim.x * VEC * norm_bwd_fold_chunks(ITERS) floats (only used when a workgroup
+// holds several rows).
 // ------------------------------------------------------------------------------------------
+// Chunks per lane whose parameter gradients cross LDS in one round of the final fold.
+constexpr int norm_bwd_fold_chunks(int iters) { return iters <= 2 ? iters : 1; }
+
 template <bool LAYER, typename TDY, typename TX, typename TDX, typename TW, int VEC, int ITERS>
 // RMSNorm with at most two chunks per lane fits 128 registers, i.e. two workgroups per CU; the
 // LayerNorm instance (bias gradient accumulators on top) would spill there and runs one per CU.
@@ -536,35 +540,50 @@ __global__ __launch_bounds__(512, (ITERS <= 2 && !LAYER ? 4 : 1)) void norm_bwd_
   }
 
   if (!part_w && !part_b) return;
-  // Fold the row-groups of this workgroup together, then emit one partial row.
+  // Fold the row-groups of this workgroup together, then emit one partial row.  The values cross
+  // through LDS as red[value][thread]: consecutive lanes touch consecutive banks both when every
+  // lane writes and when the lanes of the first row-group read the other groups' values, and all
+  // chunks of a gradient (up to two per lane) share one pair of barriers.
+  constexpr int FOLD = norm_bwd_fold_chunks(ITERS);
   const int n_out = (part_w ? 1 : 0) + ((LAYER && part_b) ? 1 : 0);
   for (int which = 0; which < n_out; ++which) {
     const bool is_w = (which == 0 && part_w);
     float* part = is_w ? part_w : part_b;
 #pragma unroll
-    for (int it = 0; it < ITERS; ++it) {
-      const int c = lane + it * group;
-      float v[VEC];
+    for (int it0 = 0; it0 < ITERS; it0 += FOLD) {
+      float v[FOLD][VEC];
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) v[j] = (is_w || !LAYER) ? acc_w[it][j] : acc_b[LAYER ? it : 0][j];
+      for (int f = 0; f < FOLD; ++f)
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+          v[f][j] = (is_w || !LAYER) ? acc_w[it0 + f][j] : acc_b[LAYER ? it0 + f : 0][j];
       if (rpb > 1) {
         __syncthreads();
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) red[(rib * group + lane) * VEC + j] = v[j];
+        for (int f = 0; f < FOLD; ++f)
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) red[(f * VEC + j) * blockDim.x + threadIdx.x] = v[f][j];
         __syncthreads();
         if (rib == 0) {
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) {
-            float s = 0.f;
-            for (int r = 0; r < rpb; ++r) s += red[(r * group + lane) * VEC + j];
-            v[j] = s;
-          }
+          for (int f = 0; f < FOLD; ++f)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+              const float* col = red + (f * VEC + j) * blockDim.x + lane;
+              float s = 0.f;
+              for (int r = 0; r < rpb; ++r) s += col[r * group];
+              v[f][j] = s;
+            }
         }
       }
-      if (rib == 0 && c < chunks) {
-        float* dst = part + (int64_t)blockIdx.x * feat + (int64_t)c * VEC;
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) dst[j] = v[j];
+      for (int f = 0; f < FOLD; ++f) {
+        const int c = lane + (it0 + f) * group;
+        if (rib == 0 && c < chunks) {
+          float* dst = part + (int64_t)blockIdx.x * feat + (int64_t)c * VEC;
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) dst[j] = v[f][j];
+        }
       }
     }
   }
@@ -1136,8 +1155,8 @@ int norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd
       const int64_t row_blocks = cdiv64(batch, rpb);
 #define AT_NORM_BWD_LAUNCH(TW, VV)                                                                       \
   {                                                                                                      \
-    const size_t lds = rpb > 1 ? (size_t)p.block * VV * sizeof(float) : 0;                              \
     AT_DISPATCH_ITERS4(p.iters, {                                                                        \
+      const size_t lds = rpb > 1 ? (size_t)p.block * VV * norm_bwd_fold_chunks(ITERS) * sizeof(float) : 0; \
       auto kernel = norm_bwd_kernel<LAYER, TDY, TX, TDY, TW, VV, ITERS>;                                 \
       parts = (int)persistent_grid((const void*)kernel, p.block, lds, row_blocks, kMaxPartialRows);      \
       float* part_b = bias_grad ? part_w + (int64_t)parts * feat : nullptr;                              \

@@ -35,7 +35,8 @@ def _assert_mostly_close(actual, expected, rtol, atol, what, outliers=2e-3, low_
     bad = ((a - e).abs() / scale > atol + rtol * e.abs() / scale).float().mean().item()
     if low_precision is None:
         low_precision = actual.dtype is not torch.float32
-    limit = outliers if low_precision else 0.0
+    # small tensors: one element may miss whatever the fraction says
+    limit = max(outliers, 1.5 / max(1, a.numel())) if low_precision else 0.0
     assert bad <= limit, f'{what}: {bad:.5f} of the elements differ by more than the tolerance'
 
 
