@@ -2,9 +2,13 @@
 // gradient of the logits from ONE pass over the logits.
 //
 // HBM-bound: the algorithmic traffic is one read of the logits and one write of the gradient.
-// One 512-lane workgroup owns a row and keeps it in registers as raw 128-bit vectors
-// (CACHE_VECS per lane), so the three sweeps the math needs (max, sum of exponentials,
-// gradient) cost a single read.  Rows need not be 16-byte aligned (a vocabulary of 50257
+// One workgroup of 512 lanes (1024 for rows of more than 4096 vectors: twice the waves with half
+// the vectors each move the same bytes 4 % faster) owns a row and keeps it in registers as raw
+// 128-bit vectors (CACHE_VECS per lane), so the three sweeps the math needs (max, sum of
+// exponentials, gradient) cost a single read.  A workgroup ends with its row: on this
+// architecture a wave's loads are counted behind its own earlier stores, so a workgroup that walks
+// over several rows waits for the acknowledgement of one row's stores before the next row's loads
+// count as arrived (a persistent grid of resident workgroups measured 363 us against 300 us).  Rows need not be 16-byte aligned (a vocabulary of 50257
 // fp16 logits makes every other row start on an odd element): a row is addressed through
 // the 16-byte grid of its own address space, interior vectors move with 128-bit accesses and
 // only the first and last vector of a row fall back to guarded element accesses.  The
@@ -23,30 +27,38 @@
 namespace at_hip {
 namespace {
 
-constexpr int kCeBlock = 512;
+constexpr int kCeBlock = 512;         // lanes per row, rows of up to 4096 vectors
+constexpr int kCeWideBlock = 1024;    // lanes per row beyond that
+// The divisor of the mean is summed by kCeDenomParts workgroups, each over its share of the rows;
+// their partial sums sit at the start of the workspace and every reader adds them in index order.
+constexpr int kCeDenomParts = 16;
+constexpr int kCeDenomBlock = 512;
 
 __device__ __forceinline__ bool target_kept(int64_t t, int64_t ignore_index, int feat) {
   return t != ignore_index && t >= 0 && t < feat;
 }
 
-// denom = sum over kept rows of weight[target] (or the kept-row count).  Single workgroup so
-// the summation order is fixed.
-__global__ __launch_bounds__(1024) void ce_denominator_kernel(
+// denom_parts[p] = sum over the kept rows of share p of weight[target] (or their count).  The shares
+// and the order inside a workgroup are fixed, so the divisor is reproducible.
+__global__ __launch_bounds__(kCeDenomBlock) void ce_denominator_kernel(
     const int64_t* __restrict__ target, const void* __restrict__ weight, int wdt,
-    float* __restrict__ denom_out, int64_t batch, int feat, int64_t ignore_index) {
+    float* __restrict__ denom_parts, int64_t batch, int feat, int64_t ignore_index) {
   __shared__ float scratch[16];
+  const int64_t share = (batch + kCeDenomParts - 1) / kCeDenomParts;
+  const int64_t begin = (int64_t)blockIdx.x * share;
+  const int64_t end = begin + share < batch ? begin + share : batch;
   float s = 0.f;
   // targets first, then the weights they select: two rounds of independent loads per batch of
   // rows instead of a dependent pair per row (the pass is pure memory latency)
-  constexpr int U = 8;
-  for (int64_t base = threadIdx.x; base < batch; base += (int64_t)blockDim.x * U) {
+  constexpr int U = 4;
+  for (int64_t base = begin + threadIdx.x; base < end; base += (int64_t)kCeDenomBlock * U) {
     int64_t t[U];
     bool kept[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int64_t i = base + (int64_t)u * blockDim.x;
-      t[u] = i < batch ? target[i] : 0;
-      kept[u] = i < batch && target_kept(t[u], ignore_index, feat);
+      const int64_t i = base + (int64_t)u * kCeDenomBlock;
+      t[u] = i < end ? target[i] : 0;
+      kept[u] = i < end && target_kept(t[u], ignore_index, feat);
     }
     float w[U];
 #pragma unroll
@@ -54,8 +66,16 @@ __global__ __launch_bounds__(1024) void ce_denominator_kernel(
 #pragma unroll
     for (int u = 0; u < U; ++u) s += w[u];
   }
-  s = group_reduce(s, (int)blockDim.x, scratch, SumOp(), 0.f);
-  if (threadIdx.x == 0) denom_out[0] = s;
+  s = group_reduce(s, kCeDenomBlock, scratch, SumOp(), 0.f);
+  if (threadIdx.x == 0) denom_parts[blockIdx.x] = s;
+}
+
+// The divisor from its partial sums, added in index order (the pointer is uniform: scalar loads).
+__device__ __forceinline__ float ce_denominator(const float* __restrict__ denom_parts) {
+  float d = 0.f;
+#pragma unroll
+  for (int p = 0; p < kCeDenomParts; ++p) d += denom_parts[p];
+  return d;
 }
 
 __global__ __launch_bounds__(1024) void ce_finalize_kernel(
@@ -66,7 +86,7 @@ __global__ __launch_bounds__(1024) void ce_finalize_kernel(
 #pragma unroll 8
   for (int64_t i = threadIdx.x; i < batch; i += blockDim.x) s += row_loss[i];
   s = group_reduce(s, (int)blockDim.x, scratch, SumOp(), 0.f);
-  if (threadIdx.x == 0) store_scalar_f32(loss, out_dt, 0, s / denom[0]);
+  if (threadIdx.x == 0) store_scalar_f32(loss, out_dt, 0, s / ce_denominator(denom));
 }
 
 // Stores the 16 / sizeof(T) gradient values of interior vector v of a row; `base` is the address of
@@ -96,8 +116,9 @@ __device__ __forceinline__ bool read_upstream(const void* upstream, int gdt, int
 // A row is split into "interior" 16-byte vectors (fully inside the row, 128-bit accesses) and
 // at most 7 + 7 "edge" elements before the first and after the last interior vector, each
 // owned by one of the first 16 lanes and moved with element accesses.
-template <typename T, typename TO, int CACHE_VECS>
-__global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_kernel(
+// BLOCK lanes per row: 512 (three workgroups per CU) or 1024 (two workgroups per CU).
+template <typename T, typename TO, int CACHE_VECS, int BLOCK>
+__global__ __launch_bounds__(BLOCK, (BLOCK == kCeWideBlock ? 8 : 6)) void ce_row_kernel(
     const T* __restrict__ logits, const int64_t* __restrict__ target, const void* __restrict__ weight,
     int wdt, const float* __restrict__ denom, float* __restrict__ row_loss, TO* __restrict__ dlogits,
     int feat, int64_t xs, int64_t ds, int64_t ignore_index, const void* __restrict__ upstream, int gdt,
@@ -128,7 +149,7 @@ __global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_k
       float zero[VEC];
 #pragma unroll
       for (int j = 0; j < VEC; ++j) zero[j] = 0.f;
-      for (int v = tid; v < n_int; v += kCeBlock) store_grad_vec<T, TO>(dv, v, zero);
+      for (int v = tid; v < n_int; v += BLOCK) store_grad_vec<T, TO>(dv, v, zero);
       if (edge >= 0) dr[edge] = from_f32<TO>(0.f);
     }
     return;
@@ -136,7 +157,7 @@ __global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_k
 
   // Vectors per lane that this row really uses; uniform, so the unrolled sweeps below skip the
   // rest of the cache with scalar branches.
-  const int n_iter = (n_int + kCeBlock - 1) / kCeBlock;
+  const int n_iter = (n_int + BLOCK - 1) / BLOCK;
   constexpr float kLog2e = 1.4426950408889634f;
 
   // All loads of the row are issued back to back and without a branch (the register writes on the
@@ -149,14 +170,14 @@ __global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_k
   const uint4* const safe = reinterpret_cast<const uint4*>(xr - off);
 #pragma unroll
   for (int i = 0; i < CACHE_VECS; ++i) {
-    const int v = tid + i * kCeBlock;
+    const int v = tid + i * BLOCK;
     cache[i] = *(v < n_int ? xv + v : safe);
   }
   const float edge_x = to_f32(xr[edge >= 0 ? edge : 0]);
 #pragma unroll
   for (int i = 0; i < CACHE_VECS; ++i) {
     constexpr uint32_t P = Word<T>::kNegInf;
-    if (tid + i * kCeBlock >= n_int) cache[i] = make_uint4(P, P, P, P);
+    if (tid + i * BLOCK >= n_int) cache[i] = make_uint4(P, P, P, P);
   }
 
   float m = edge >= 0 ? edge_x : -INFINITY;
@@ -169,7 +190,7 @@ __global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_k
       for (int j = 0; j < VEC; ++j) m = fmaxf(m, f[j]);
     }
   }
-  m = group_reduce(m, kCeBlock, scratch, MaxOp(), -INFINITY);
+  m = group_reduce(m, BLOCK, scratch, MaxOp(), -INFINITY);
   // Keep the row cached as raw data: without this the compiler may keep widened fp32 copies
   // of every element alive across the sweeps.
 #pragma unroll
@@ -193,7 +214,7 @@ __global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_k
       cache[i] = pack16<T>(f);
     }
   }
-  s = group_reduce(s, kCeBlock, scratch, SumOp(), 0.f);
+  s = group_reduce(s, BLOCK, scratch, SumOp(), 0.f);
 #pragma unroll
   for (int i = 0; i < CACHE_VECS; ++i) keep_raw(cache[i]);
 
@@ -202,7 +223,7 @@ __global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_k
   if (tid == 0 && row_loss) row_loss[row] = (__logf(s) - x_t + m) * wt;
   if (!dr) return;
 
-  const float scale = wt / denom[0] * up;
+  const float scale = wt / ce_denominator(denom) * up;
   const float k = scale / s;
   const int tv = (int)t - head_n;   // target position relative to the first interior element
   const float g_target = fmaf(__builtin_amdgcn_exp2f(fmaf(x_t, kLog2e, -m2)), k, -scale);   // softmax - 1, scaled
@@ -212,7 +233,7 @@ __global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_k
     // of every cache line.  The values change lanes through LDS first (2 KB per wave, nobody else's:
     // no workgroup barrier, a wave's LDS operations complete in order; wave barriers keep the compiler
     // from reordering them), so that each instruction writes one contiguous KiB.
-    __shared__ float4 exchange[kCeBlock / 64][128];
+    __shared__ float4 exchange[BLOCK / 64][128];
     const int lane = tid & 63, wave = tid >> 6;
     float4* const mine = exchange[wave];
 #pragma unroll
@@ -227,7 +248,7 @@ __global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_k
         __builtin_amdgcn_wave_barrier();   // compiler only: the reads below stay behind the writes above
         const float4 lo = mine[lane], hi = mine[64 + lane];
         __builtin_amdgcn_wave_barrier();   // ... and ahead of the next sweep's writes
-        const int v0 = wave * 64 + i * kCeBlock;   // the wave's first vector of this sweep
+        const int v0 = wave * 64 + i * BLOCK;   // the wave's first vector of this sweep
         float4* out = reinterpret_cast<float4*>(dv + (int64_t)v0 * VEC);
         if (v0 + (lane >> 1) < n_int) out[lane] = lo;
         if (v0 + 32 + (lane >> 1) < n_int) out[64 + lane] = hi;
@@ -239,14 +260,14 @@ __global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_k
     // 16-byte piece 2 (number % 32) + (tv % 8) / 4 of that group's lower or upper KiB.
     const int target_vec = tv / VEC;
     const bool owner = (tv >= 0 && tv < n_int * VEC)
-                           ? (tid == (((target_vec >> 6) & (kCeBlock / 64 - 1)) << 6 | (target_vec & 31) << 1 |
+                           ? (tid == (((target_vec >> 6) & (BLOCK / 64 - 1)) << 6 | (target_vec & 31) << 1 |
                                       ((tv >> 2) & 1)))
                            : (edge == (int)t);
     if (owner) dr[t] = g_target;
   } else {
 #pragma unroll
     for (int i = 0; i < CACHE_VECS; ++i) {
-      const int v = tid + i * kCeBlock;
+      const int v = tid + i * BLOCK;
       if (i < n_iter && v < n_int) {
         float f[VEC];
         unpack16<T>(cache[i], f);
@@ -258,7 +279,7 @@ __global__ __launch_bounds__(kCeBlock, (CACHE_VECS <= 13 ? 6 : 4)) void ce_row_k
     if (edge >= 0) dr[edge] = from_f32<TO>(edge_e * k);
     // The target column gets softmax - 1: the lane that stored the column overwrites it (stores of
     // one lane to one address stay in order).
-    const bool owner = (tv >= 0 && tv < n_int * VEC) ? ((tv / VEC) % kCeBlock == tid) : (edge == (int)t);
+    const bool owner = (tv >= 0 && tv < n_int * VEC) ? ((tv / VEC) % BLOCK == tid) : (edge == (int)t);
     if (owner) dr[t] = from_f32<TO>(g_target);
   }
 }
@@ -294,7 +315,7 @@ __global__ __launch_bounds__(1024) void ce_row_stream_kernel(
   const float wt = weight ? load_scalar_f32(weight, wdt, t) : 1.f;
   if (threadIdx.x == 0 && row_loss) row_loss[row] = (__logf(s) - to_f32(xr[t]) + m) * wt;
   if (!dr) return;
-  const float scale = wt / denom[0] * up;
+  const float scale = wt / ce_denominator(denom) * up;
   const float k = scale / s;
   for (int c = threadIdx.x; c < feat; c += blockDim.x) {
     float g = __expf(to_f32(xr[c]) - m) * k;
@@ -368,23 +389,28 @@ int launch_ce_rows(const void* logits, const int64_t* target, const void* weight
     same_phase = (la % es) == 0 && (da % os) == 0 &&
                  ((int64_t)(da / os) - (int64_t)(la / es)) % unit == 0 && (dlogits_stride - logits_stride) % unit == 0;
   }
-  const bool cached = same_phase && max_vecs <= (int64_t)kCeBlock * 16 && (la % es) == 0;
+  const bool cached = same_phase && max_vecs <= (int64_t)kCeWideBlock * 8 && (la % es) == 0;
 
   return dispatch_one(logits_dtype, [&](auto* tp) -> int {
     typedef std::remove_pointer_t<decltype(tp)> T;
     auto run = [&](auto* top) -> int {
       typedef std::remove_pointer_t<decltype(top)> TO;
       if (cached) {
-        const int per_lane = (int)cdiv64(max_vecs, kCeBlock);
-#define AT_CE_LAUNCH(CV)                                                                              \
-  hipLaunchKernelGGL((ce_row_kernel<T, TO, CV>), dim3((unsigned)batch), dim3(kCeBlock), 0, stream,    \
-                     (const T*)logits, target, weight, weight_dtype, denom, row_loss, (TO*)dlogits,   \
+#define AT_CE_LAUNCH(CV, BLK)                                                                            \
+  hipLaunchKernelGGL((ce_row_kernel<T, TO, CV, BLK>), dim3((unsigned)batch), dim3(BLK), 0, stream,       \
+                     (const T*)logits, target, weight, weight_dtype, denom, row_loss, (TO*)dlogits,      \
                      (int)feat, logits_stride, dlogits_stride, ignore_index, upstream, grad_dtype, skip_if_one)
-        if (per_lane <= 2) AT_CE_LAUNCH(2);
-        else if (per_lane <= 4) AT_CE_LAUNCH(4);
-        else if (per_lane <= 8) AT_CE_LAUNCH(8);
-        else if (per_lane <= 13) AT_CE_LAUNCH(13);   // up to 13 vectors: registers for three workgroups per CU
-        else AT_CE_LAUNCH(16);
+        if (max_vecs > (int64_t)kCeBlock * 8) {
+          const int per_lane = (int)cdiv64(max_vecs, kCeWideBlock);   // 5 .. 8
+          if (per_lane <= 6) AT_CE_LAUNCH(6, kCeWideBlock);
+          else if (per_lane <= 7) AT_CE_LAUNCH(7, kCeWideBlock);
+          else AT_CE_LAUNCH(8, kCeWideBlock);
+        } else {
+          const int per_lane = (int)cdiv64(max_vecs, kCeBlock);
+          if (per_lane <= 2) AT_CE_LAUNCH(2, kCeBlock);
+          else if (per_lane <= 4) AT_CE_LAUNCH(4, kCeBlock);
+          else AT_CE_LAUNCH(8, kCeBlock);
+        }
 #undef AT_CE_LAUNCH
       } else {
         hipLaunchKernelGGL((ce_row_stream_kernel<T, TO>), dim3((unsigned)batch), dim3(1024), 0, stream,
@@ -417,10 +443,10 @@ int ce_fwd_bwd(const void* logits, const int64_t* target, const void* weight, vo
                int64_t ignore_index, int logits_dtype, int weight_dtype, int out_dtype, int loss_dtype,
                hipStream_t stream) {
   if (!dtype_valid(loss_dtype)) return AT_ERR_DTYPE;
-  float* denom = workspace;
-  float* row_loss = denom + 4;
-  hipLaunchKernelGGL(ce_denominator_kernel, dim3(1), dim3(1024), 0, stream, target, weight, weight_dtype,
-                     denom, batch, (int)feat, ignore_index);
+  float* denom = workspace;                  // kCeDenomParts partial sums
+  float* row_loss = denom + kCeDenomParts;
+  hipLaunchKernelGGL(ce_denominator_kernel, dim3(kCeDenomParts), dim3(kCeDenomBlock), 0, stream, target, weight,
+                     weight_dtype, denom, batch, (int)feat, ignore_index);
   int rc = launch_ce_rows(logits, target, weight, denom, row_loss, dlogits, batch, feat, logits_stride,
                           dlogits_stride, ignore_index, logits_dtype, weight_dtype, out_dtype, nullptr, 0, 0,
                           stream);
@@ -435,17 +461,17 @@ int ce_fwd_bwd(const void* logits, const int64_t* target, const void* weight, vo
 
 using namespace at_hip;
 
-// Workspace of at_cross_entropy_fwd_bwd_static: the divisor and one loss per row (65536 rows at
-// most, 256 KiB).  Device memory of the library itself: every GPU the library runs on holds its own
+// Workspace of at_cross_entropy_fwd_bwd_static: the divisor's partial sums and one loss per row
+// (65536 rows at most, 256 KiB).  Device memory of the library itself: every GPU the library runs on holds its own
 // copy until the process ends.  In host code this name is only a handle for hipGetSymbolAddress;
 // kernels receive the address that call returns for the current device.
-static __device__ __align__(256) float ce_static_scratch[4 + 65536];
+static __device__ __align__(256) float ce_static_scratch[kCeDenomParts + 65536];
 
 extern "C" {
 
 int64_t at_cross_entropy_workspace_bytes(int64_t batch) {
   if (batch < 0) return 0;
-  return (4 + batch) * (int64_t)sizeof(float);
+  return (kCeDenomParts + batch) * (int64_t)sizeof(float);
 }
 
 int at_cross_entropy_fwd_bwd(const void* logits, const int64_t* target, const void* weight, void* loss,

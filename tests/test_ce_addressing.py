@@ -9,11 +9,16 @@ inside the pages the tensor occupies (a load outside them is a GPU memory fault,
 import pytest
 
 SHAPES = [(12288, 1), (5, 7), (8096, 32), (48, 50257), (9, 12345), (4, 131075), (1, 8000), (3, 8),
-          (64, 33), (37, 129), (512, 4099), (2, 2), (7, 3)]
+          (64, 33), (37, 129), (512, 4099), (2, 2), (7, 3), (3, 32768), (3, 32776), (2, 65536), (2, 49153)]
 
 
-def check(batch, feat, elem_size, base, block=512, cache_vecs=16):
+def check(batch, feat, elem_size, base):
     vec = 16 // elem_size
+    # the launcher's choice: 512 lanes and up to 8 vectors per lane, 1024 lanes beyond 4096 vectors
+    max_vecs = -(-feat // vec)
+    block = 1024 if max_vecs > 512 * 8 else 512
+    per_lane = -(-max_vecs // block)
+    cache_vecs = next(c for c in ((6, 7, 8) if block == 1024 else (2, 4, 8)) if per_lane <= c) if max_vecs <= 8192 else 0
     first_page = base // 4096 * 4096
     end = base + batch * feat * elem_size
     last_page_end = (end + 4095) // 4096 * 4096
