@@ -48,6 +48,7 @@ PROTOTYPES = {
     'at_linear_bwd_input': (I, [P, P, P, L, L, L, L, L, L, I, I, P]),
     'at_linear_bwd_weight_workspace_bytes': (L, [L, L, L, I]),
     'at_linear_bwd_small_supported': (I, [L, L, L, I]),
+    'at_linear_bwd_wide_output_supported': (I, [L, L, L, I]),
     'at_linear_bwd_small': (I, [P, P, P, P, P, P, P, L, L, L, L, L, L, L, L, L, I, F, I, P]),
     'at_linear_bwd_weight': (I, [P, P, P, P, L, L, L, L, L, L, L, I, I, P]),
     'at_act_bwd_workspace_bytes': (L, [L, L]),

@@ -53,6 +53,7 @@ struct GemmArgs {
   float* partial;
   int kt_per_split;
   int ldw;
+  int round_dt;       // generic kernels: results are rounded to this dtype before they are stored (fp32: as they are)
 };
 
 constexpr int BM = 256, BN = 256, BK = 64;
@@ -188,9 +189,15 @@ constexpr int kEpiRows = BM / 4;                               // rows per chunk
 constexpr int kEpiStageBytes = kEpiRows * kEpiPitch;           // 33 792
 constexpr int kEpiBiasBytes = BN * 4;                          // the tile's bias values as floats, behind the chunk
 constexpr int kEpiSweeps = kEpiRows / (kBigThreads / 32);      // 16-byte stores per lane and chunk
-template <typename T, int ACT, typename Prefetch>
+// TO is T, or float for a product whose result is wanted in fp32 although the operands have 16 bits
+// (the backward products under autocast: autograd would widen the 16-bit result anyway): the tile
+// is staged rounded to T as always and widened by the store sweep, which then writes 1 KiB of a row
+// per wave and takes twice the sweeps.
+template <typename T, int ACT, typename TO, typename Prefetch>
 __device__ __forceinline__ int big_tile_epilogue(f32x16 (&acc)[4][kBigNJ], char* stage, const GemmArgs& g, int m0,
                                                  int n0, Prefetch&& prefetch_next) {
+  constexpr bool WIDE = !std::is_same<T, TO>::value;
+  static_assert(!WIDE || (std::is_same<TO, float>::value && ACT == AT_ACT_NONE), "fp32 results only without activation");
   constexpr int NJ = kBigNJ;
   // a thread index the compiler takes for a new value: what the epilogue derives from it is worked
   // out here and not kept in registers across the main loop
@@ -207,8 +214,9 @@ __device__ __forceinline__ int big_tile_epilogue(f32x16 (&acc)[4][kBigNJ], char*
   // chunk: rows 32 c .. 32 c + 31 of the upper and of the lower half of the tile.
   T* __restrict__ C = reinterpret_cast<T*>(g.c);
   T* __restrict__ P = reinterpret_cast<T*>(g.pre_act);
-  const bool rows16 = ((g.ldc & 7) == 0) && aligned16_dev(C) && (n0 + BN <= g.N) &&
-                      (!P || (((g.ldp & 7) == 0) && aligned16_dev(P)));
+  const bool rows16 = WIDE ? (((g.ldc & 3) == 0) && aligned16_dev(g.c) && (n0 + BN <= g.N))
+                           : (((g.ldc & 7) == 0) && aligned16_dev(C) && (n0 + BN <= g.N) &&
+                              (!P || (((g.ldp & 7) == 0) && aligned16_dev(P))));
   const bool exact = rows16 && m0 + BM <= g.M;
   float* const bias_tile = reinterpret_cast<float*>(stage + kEpiStageBytes);
   // the bias of the tile's columns goes to LDS before anything else: a global load further down
@@ -249,6 +257,28 @@ __device__ __forceinline__ int big_tile_epilogue(f32x16 (&acc)[4][kBigNJ], char*
           store_f32<T, 4>(reinterpret_cast<T*>(stage + (wm * 32 + frag_row) * kEpiPitch) + nl, v);
         }
       __syncthreads();
+      if constexpr (WIDE) {
+        // one row per wave and sweep: 64 lanes x 4 values, 16 bytes of fp32 each
+        float* __restrict__ Cw = reinterpret_cast<float*>(g.c);
+        const int rw = tid >> 6, cw = (tid & 63) * 4;
+#pragma unroll
+        for (int r0 = 0; r0 < kEpiRows; r0 += kBigThreads / 64) {
+          const int ml = r0 + rw;
+          const int m = m0 + (ml >> 5) * (BM / 2) + c * 32 + (ml & 31);
+          if (m >= g.M) continue;
+          float v[4];
+          load_f32<T, 4>(reinterpret_cast<const T*>(stage + ml * kEpiPitch) + cw, v);
+          float* out = Cw + (int64_t)m * g.ldc + n0 + cw;
+          if (rows16) {
+            *reinterpret_cast<float4*>(out) = make_float4(v[0], v[1], v[2], v[3]);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n0 + cw + e < g.N) out[e] = v[e];
+          }
+        }
+        continue;
+      }
       // 2 rows per wave and sweep, 32 lanes x 16 bytes per row
       const int rsub = tid >> 5, cseg = (tid & 31) * 8;
 #pragma unroll
@@ -285,12 +315,12 @@ __device__ __forceinline__ int big_tile_epilogue(f32x16 (&acc)[4][kBigNJ], char*
       }
     }
   }
-  return exact ? outputs * 4 * kEpiSweeps : -1;
+  return exact ? outputs * 4 * kEpiSweeps * (WIDE ? 2 : 1) : -1;
 }
 
 // ACT is the compile-time activation id of the epilogue (the act switch must fold away: the
 // epilogue is fully unrolled over the accumulator registers).
-template <typename T, bool A_MC, bool B_KC, int ACT>
+template <typename T, bool A_MC, bool B_KC, int ACT, typename TO = T>
 __global__ __launch_bounds__(kBigThreads) void gemm_mfma16_kernel(GemmArgs g) {
   constexpr bool A_KC = !A_MC;
   constexpr int kATile = operand_tile_bytes<A_KC>(), kBTile = operand_tile_bytes<B_KC>();
@@ -450,7 +480,7 @@ __global__ __launch_bounds__(kBigThreads) void gemm_mfma16_kernel(GemmArgs g) {
 
   const int next_id = tile_id + gridDim.x;
   requested = next_id < total;
-  stores_behind = big_tile_epilogue<T, ACT>(acc, lds + kEpiOff, g, m0, n0, [&] {
+  stores_behind = big_tile_epilogue<T, ACT, TO>(acc, lds + kEpiOff, g, m0, n0, [&] {
     if (!requested) return;
     int m1, n1;
     tile_origin(next_id, m1, n1);
@@ -548,7 +578,8 @@ __device__ __forceinline__ uint4 read_frag_mid(const char* tile, int outer_base,
   }
 }
 
-template <typename T, bool A_MC, bool B_KC, bool SPLIT>
+// TO as in big_tile_epilogue: T, or float for the value rounded to T and widened (no activation).
+template <typename T, bool A_MC, bool B_KC, bool SPLIT, typename TO = T>
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_mid16_kernel(GemmArgs g) {
   constexpr bool A_KC = !A_MC;
   __shared__ __attribute__((aligned(1024))) char lds[kMidLds];
@@ -664,6 +695,29 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_mid16_kernel(GemmArgs g)
     }
     return;
   }
+  if constexpr (!std::is_same<T, TO>::value) {
+    float* __restrict__ Cw = reinterpret_cast<float*>(g.c);
+    const bool rows16w = ((g.ldc & 3) == 0) && aligned16_dev(Cw) && (n0 + MT <= g.N);
+    for (int r0 = 0; r0 < MT; r0 += 16) {
+      const int ml = r0 + rsub, m = m0 + ml;
+      if (m >= g.M) continue;
+      float v[8];
+      *reinterpret_cast<float4*>(v) = *reinterpret_cast<const float4*>(stage + ml * kMidEpiPitch + cseg);
+      *reinterpret_cast<float4*>(v + 4) = *reinterpret_cast<const float4*>(stage + ml * kMidEpiPitch + cseg + 4);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = to_f32(from_f32<T>(v[e]));
+      float* out = Cw + (int64_t)m * g.ldc + n0 + cseg;
+      if (rows16w) {
+        *reinterpret_cast<float4*>(out) = *reinterpret_cast<const float4*>(v);
+        *reinterpret_cast<float4*>(out + 4) = *reinterpret_cast<const float4*>(v + 4);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (n0 + cseg + e < g.N) out[e] = v[e];
+      }
+    }
+    return;
+  }
   T* __restrict__ C = reinterpret_cast<T*>(g.c);
   T* __restrict__ P = g.act != AT_ACT_NONE ? reinterpret_cast<T*>(g.pre_act) : nullptr;
   const bool rows16 = ((g.ldc & 7) == 0) && aligned16_dev(C) && (n0 + MT <= g.N) &&
@@ -699,9 +753,10 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_mid16_kernel(GemmArgs g)
   }
 }
 
-// C[m][n] = sum over the splits of partial[s][m][n], rounded once.  One lane per 8 columns.
-template <typename T>
-__global__ __launch_bounds__(256) void gemm_split_finish_kernel(const float* __restrict__ partial, T* __restrict__ C,
+// C[m][n] = sum over the splits of partial[s][m][n], rounded once to T.  One lane per 8 columns.
+// TO = T, or float for the rounded value widened (as in big_tile_epilogue).
+template <typename T, typename TO = T>
+__global__ __launch_bounds__(256) void gemm_split_finish_kernel(const float* __restrict__ partial, TO* __restrict__ C,
                                                                 int M, int N, int ldw, int64_t ldc, int splits) {
   const int segs = ldw / 8;
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -719,13 +774,18 @@ __global__ __launch_bounds__(256) void gemm_split_finish_kernel(const float* __r
     acc[4] += hi.x; acc[5] += hi.y; acc[6] += hi.z; acc[7] += hi.w;
     src += (int64_t)M * ldw;
   }
-  T* out = C + (int64_t)m * ldc + n;
-  if (n + 8 <= N && (ldc & 7) == 0 && aligned16_dev(C)) {
-    store_f32<T, 8>(out, acc);
+  TO* out = C + (int64_t)m * ldc + n;
+  if constexpr (!std::is_same<T, TO>::value) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = to_f32(from_f32<T>(acc[e]));
+  }
+  constexpr int kPer = 16 / (int)sizeof(TO);   // elements per 16 bytes of output
+  if (n + 8 <= N && (ldc % kPer) == 0 && aligned16_dev(C)) {
+    store_f32<TO, 8>(out, acc);
   } else {
 #pragma unroll
     for (int e = 0; e < 8; ++e)
-      if (n + e < N) out[e] = from_f32<T>(acc[e]);
+      if (n + e < N) out[e] = from_f32<TO>(acc[e]);
   }
 }
 
@@ -942,6 +1002,13 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g) {
   }
 }
 
+// v rounded to a 16-bit dtype and widened again (fp32: v itself).
+__device__ __forceinline__ float round_through(float v, int dt) {
+  if (dt == AT_DTYPE_F16) return to_f32(from_f32<f16_t>(v));
+  if (dt == AT_DTYPE_BF16) return to_f32(from_f32<bf16_t>(v));
+  return v;
+}
+
 // Epilogue of the generic kernels: one 32x32 accumulator tile per wave (register r of a lane =
 // C[m = lane % 32][n = (r / 4) * 8 + (lane / 32) * 4 + r % 4]) goes through a wave-private block
 // of LDS (32 rows of 36 floats) and is finished in a rolled loop, so that the run-time activation
@@ -985,7 +1052,7 @@ __device__ __forceinline__ void wave_tile_epilogue(const f32x16& acc, float* blo
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e)
-      if (n + e < g.N) C[(int64_t)m * g.ldc + n + e] = from_f32<TO>(v[e]);
+      if (n + e < g.N) C[(int64_t)m * g.ldc + n + e] = from_f32<TO>(round_through(v[e], g.round_dt));
   }
 }
 
@@ -997,6 +1064,7 @@ struct SimpleArgs {
   int M, N, K;
   int64_t sam, sak, sbk, sbn, ldc, ldp;
   int act; float param; int bias_dt;
+  int round_dt;   // results are rounded to this dtype before they are stored (fp32: as they are)
 };
 
 template <typename TI, typename TO>
@@ -1820,10 +1888,13 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
   if (M == 0) return AT_OK;
 
   const bool a_contig_k = layout != kDw, b_contig_k = layout == kDx;
+  // A backward product of 16-bit operands may be asked for in fp32: the value rounded to the operand
+  // dtype, widened (what the 16-bit product followed by autograd's cast to an fp32 leaf gives).
+  const bool wide = layout != kFwd && in_dt != AT_DTYPE_F32 && out_dt == AT_DTYPE_F32;
   // 16-byte loads need aligned rows; an operand whose rows run along the contraction index also
   // needs K in whole vectors (the other layout reads whole rows of k, and what a vector picks up
   // past M or N only reaches outputs that are not stored).
-  bool fast = in_dt != AT_DTYPE_F32 && out_dt == in_dt && aligned16(a) && aligned16(b) && (lda % 8) == 0 &&
+  bool fast = in_dt != AT_DTYPE_F32 && (out_dt == in_dt || wide) && aligned16(a) && aligned16(b) && (lda % 8) == 0 &&
               (ldb % 8) == 0;
   if (a_contig_k || b_contig_k) fast = fast && (K % 8) == 0;
   // buffer descriptors address each operand with 32-bit byte offsets below 2 GiB
@@ -1834,7 +1905,7 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
 
   const int64_t big_tiles = cdiv64(M, BM) * cdiv64(N, BN);
   if (fast && prefer_mid_tiles(M, N)) {
-    GemmArgs g{a, b, c, pre_act, bias, (int)M, (int)N, (int)K, lda, ldb, ldc, ldp, act, param, bias_dt, nullptr, 0, 0};
+    GemmArgs g{a, b, c, pre_act, bias, (int)M, (int)N, (int)K, lda, ldb, ldc, ldp, act, param, bias_dt, nullptr, 0, 0, AT_DTYPE_F32};
     const unsigned grid = (unsigned)(cdiv64(M, MT) * cdiv64(N, MT));
     int splits = 1;
     if (layout == kDw && workspace) {
@@ -1853,12 +1924,18 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
           hipLaunchKernelGGL((gemm_mid16_kernel<T, true, false, true>), dim3(grid, splits), dim3(kGemmThreads), 0,
                              stream, g);
           const int64_t items = M * (g.ldw / 8);
-          hipLaunchKernelGGL((gemm_split_finish_kernel<T>), dim3((unsigned)cdiv64(items, 256)), dim3(256), 0, stream,
-                             (const float*)workspace, (T*)c, (int)M, (int)N, g.ldw, ldc, splits);
+          if (wide)
+            hipLaunchKernelGGL((gemm_split_finish_kernel<T, float>), dim3((unsigned)cdiv64(items, 256)), dim3(256), 0,
+                               stream, (const float*)workspace, (float*)c, (int)M, (int)N, g.ldw, ldc, splits);
+          else
+            hipLaunchKernelGGL((gemm_split_finish_kernel<T>), dim3((unsigned)cdiv64(items, 256)), dim3(256), 0, stream,
+                               (const float*)workspace, (T*)c, (int)M, (int)N, g.ldw, ldc, splits);
         } else if (layout == kDx) {
-          hipLaunchKernelGGL((gemm_mid16_kernel<T, false, true, false>), dim3(grid), dim3(kGemmThreads), 0, stream, g);
+          if (wide) hipLaunchKernelGGL((gemm_mid16_kernel<T, false, true, false, float>), dim3(grid), dim3(kGemmThreads), 0, stream, g);
+          else hipLaunchKernelGGL((gemm_mid16_kernel<T, false, true, false>), dim3(grid), dim3(kGemmThreads), 0, stream, g);
         } else if (layout == kDw) {
-          hipLaunchKernelGGL((gemm_mid16_kernel<T, true, false, false>), dim3(grid), dim3(kGemmThreads), 0, stream, g);
+          if (wide) hipLaunchKernelGGL((gemm_mid16_kernel<T, true, false, false, float>), dim3(grid), dim3(kGemmThreads), 0, stream, g);
+          else hipLaunchKernelGGL((gemm_mid16_kernel<T, true, false, false>), dim3(grid), dim3(kGemmThreads), 0, stream, g);
         } else {
           hipLaunchKernelGGL((gemm_mid16_kernel<T, false, false, false>), dim3(grid), dim3(kGemmThreads), 0, stream, g);
         }
@@ -1868,7 +1945,7 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
   }
 
   if (fast) {
-    GemmArgs g{a, b, c, pre_act, bias, (int)M, (int)N, (int)K, lda, ldb, ldc, ldp, act, param, bias_dt, nullptr, 0, 0};
+    GemmArgs g{a, b, c, pre_act, bias, (int)M, (int)N, (int)K, lda, ldb, ldc, ldp, act, param, bias_dt, nullptr, 0, 0, AT_DTYPE_F32};
     // one workgroup per CU at a time (LDS): a grid of that many walks the tiles itself
     const int64_t resident = (int64_t)device_cu_count() / 8 * 8;
     const unsigned grid = (unsigned)(big_tiles > resident && resident > 0 ? resident : big_tiles);
@@ -1878,9 +1955,11 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
         return AT_ERR_DTYPE;
       } else {
         if (layout == kDx) {
-          hipLaunchKernelGGL((gemm_mfma16_kernel<T, false, true, AT_ACT_NONE>), dim3(grid), dim3(kBigThreads), 0, stream, g);
+          if (wide) hipLaunchKernelGGL((gemm_mfma16_kernel<T, false, true, AT_ACT_NONE, float>), dim3(grid), dim3(kBigThreads), 0, stream, g);
+          else hipLaunchKernelGGL((gemm_mfma16_kernel<T, false, true, AT_ACT_NONE>), dim3(grid), dim3(kBigThreads), 0, stream, g);
         } else if (layout == kDw) {
-          hipLaunchKernelGGL((gemm_mfma16_kernel<T, true, false, AT_ACT_NONE>), dim3(grid), dim3(kBigThreads), 0, stream, g);
+          if (wide) hipLaunchKernelGGL((gemm_mfma16_kernel<T, true, false, AT_ACT_NONE, float>), dim3(grid), dim3(kBigThreads), 0, stream, g);
+          else hipLaunchKernelGGL((gemm_mfma16_kernel<T, true, false, AT_ACT_NONE>), dim3(grid), dim3(kBigThreads), 0, stream, g);
         } else {
           switch (act) {
 #define AT_FWD_CASE(ID) case ID: hipLaunchKernelGGL((gemm_mfma16_kernel<T, false, false, ID>), dim3(grid), dim3(kBigThreads), 0, stream, g); break;
@@ -1948,7 +2027,7 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
   if (in_dt == AT_DTYPE_F32 && out_dt == AT_DTYPE_F32 && aligned16(a) && aligned16(b) && (lda % 4) == 0 &&
       (ldb % 4) == 0 && (!(a_contig_k || b_contig_k) || (K % 4) == 0) && M >= 32 && N >= 32 &&
       (a_contig_k ? M : K) * lda * 4 < ((int64_t)1 << 31) && (b_contig_k ? N : K) * ldb * 4 < ((int64_t)1 << 31)) {
-    GemmArgs g{a, b, c, pre_act, bias, (int)M, (int)N, (int)K, lda, ldb, ldc, ldp, act, param, bias_dt, nullptr, 0, 0};
+    GemmArgs g{a, b, c, pre_act, bias, (int)M, (int)N, (int)K, lda, ldb, ldc, ldp, act, param, bias_dt, nullptr, 0, 0, AT_DTYPE_F32};
     // outputs with fewer 64x64 tiles than CUs: 32x32 tiles, the contraction shared by the waves
     if (cdiv64(M, 64) * cdiv64(N, 64) < device_cu_count() && K >= 128 && (M % 4) == 0 && (N % 4) == 0) {
       const unsigned grid = (unsigned)(cdiv64(M, 32) * cdiv64(N, 32));
@@ -1996,7 +2075,7 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
 
   SimpleArgs s{a, b, c, pre_act, bias, (int)M, (int)N, (int)K,
                a_contig_k ? lda : 1, a_contig_k ? 1 : lda, b_contig_k ? 1 : ldb, b_contig_k ? ldb : 1,
-               ldc, ldp, act, param, bias_dt};
+               ldc, ldp, act, param, bias_dt, wide ? in_dt : AT_DTYPE_F32};
   return dispatch_dtype(in_dt, [&](auto* ti) -> int {
     typedef std::remove_pointer_t<decltype(ti)> TI;
     return dispatch_dtype(out_dt, [&](auto* to) -> int {
@@ -2048,6 +2127,18 @@ int at_linear_bwd_input(const void* pre_act_grad, const void* weight, void* inpu
   return run_gemm(kDx, pre_act_grad, weight, input_grad, nullptr, nullptr, batch, in_feat, out_feat,
                   grad_stride, weight_stride, input_grad_stride, 0, AT_ACT_NONE, 0.f, in_dtype, 0, out_dtype,
                   (hipStream_t)stream);
+}
+
+int at_linear_bwd_wide_output_supported(int64_t batch, int64_t in_feat, int64_t out_feat, int dtype) {
+  if (dtype != AT_DTYPE_F16 && dtype != AT_DTYPE_BF16) return 0;
+  // the conditions under which run_gemm takes a tiled 16-bit kernel for dX = dZ W^T and dW = X^T dZ
+  // when every row stride equals the row's extent
+  if ((in_feat % 8) || (out_feat % 8)) return 0;
+  if (batch < 64 || in_feat < 64 || out_feat < 64) return 0;
+  if (batch * in_feat < (int64_t)MT * MT || in_feat * out_feat < (int64_t)MT * MT) return 0;
+  const int64_t limit = (int64_t)1 << 31;
+  if (batch * out_feat * 2 >= limit || in_feat * out_feat * 2 >= limit || batch * in_feat * 2 >= limit) return 0;
+  return 1;
 }
 
 int at_linear_bwd_small_supported(int64_t batch, int64_t in_feat, int64_t out_feat, int dtype) {

@@ -161,6 +161,7 @@ class LinearAutoGrad(torch.autograd.Function):
         ctx.bias_requires_grad = False if bias is None else bias.requires_grad
         ctx.output_dtype = output_dtype
         ctx.input_shape = input.shape
+        ctx.leaf_dtypes = (input.dtype, weight.dtype)
         if requires_grad:
             # Under autocast the low-precision copies made for the forward product are what the
             # backward products read (linear_layer.py:152-155 casts them again there): keeping
@@ -284,6 +285,14 @@ class LinearAutoGrad(torch.autograd.Function):
                     grad_mm = padded_grad
                 else:
                     grad_mm = _zero_pad(grad_mm, batch_dim, contract_dim)
+            # Gradients of float32 tensors that took part in 16-bit products (autocast): the
+            # kernels write the 16-bit result widened to float32 themselves, which spares
+            # autograd's cast pass over each gradient.
+            wide = (not pad and output_dtype is not torch.float32 and batch_dim > 0
+                    and bool(lib.at_linear_bwd_wide_output_supported(batch_dim, in_feat_dim, out_feat_dim,
+                                                                     _lib.dtype_id(output_dtype))))
+            input_grad_dtype = torch.float32 if wide and ctx.leaf_dtypes[0] is torch.float32 else output_dtype
+            weight_grad_dtype = torch.float32 if wide and ctx.leaf_dtypes[1] is torch.float32 else output_dtype
             input_grad = weight_grad = None
             if input_needs_grad:
                 if pad and padded_weight is not None and padded_weight.dtype is output_dtype:
@@ -292,18 +301,18 @@ class LinearAutoGrad(torch.autograd.Function):
                     weight_mm = _matrix(weight.to(output_dtype))
                     if pad:
                         weight_mm = _zero_pad(weight_mm, in_feat_dim, contract_dim)
-                input_grad = torch.empty((batch_dim, in_feat_dim), dtype=output_dtype, device=device)
+                input_grad = torch.empty((batch_dim, in_feat_dim), dtype=input_grad_dtype, device=device)
                 _lib.check(lib.at_linear_bwd_input(
                     _lib.ptr(grad_mm), _lib.ptr(weight_mm), _lib.ptr(input_grad), batch_dim,
                     in_feat_dim, contract_dim, _lib.row_stride(grad_mm), _lib.row_stride(weight_mm),
                     _lib.row_stride(input_grad), _lib.dtype_id(output_dtype),
-                    _lib.dtype_id(output_dtype), stream), 'at_linear_bwd_input')
+                    _lib.dtype_id(input_grad_dtype), stream), 'at_linear_bwd_input')
                 input_grad = input_grad.view(ctx.input_shape)
             if weight_needs_grad:
                 input_mm = _matrix(flattened_input.to(output_dtype))
                 if pad:
                     input_mm = _zero_pad(input_mm, batch_dim, _round_up8(in_feat_dim))
-                weight_grad = torch.empty((in_feat_dim, out_feat_dim), dtype=output_dtype,
+                weight_grad = torch.empty((in_feat_dim, out_feat_dim), dtype=weight_grad_dtype,
                                           device=device)
                 if batch_dim == 0:
                     weight_grad.zero_()
@@ -317,7 +326,7 @@ class LinearAutoGrad(torch.autograd.Function):
                         _lib.ptr(workspace), workspace_bytes, batch_dim,
                         in_feat_dim, out_feat_dim, _lib.row_stride(input_mm), _lib.row_stride(grad_mm),
                         _lib.row_stride(weight_grad), _lib.dtype_id(output_dtype),
-                        _lib.dtype_id(output_dtype), stream), 'at_linear_bwd_weight')
+                        _lib.dtype_id(weight_grad_dtype), stream), 'at_linear_bwd_weight')
             if ctx.bias_requires_grad and bias_grad is None:
                 bias_grad = torch.empty(out_feat_dim, dtype=pre_act_grad.dtype, device=device)
                 if batch_dim == 0:

@@ -665,6 +665,83 @@ def bench_rows(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
     return results
 
 
+def bench_rows_tall() -> List[Dict]:
+    """
+    The c2 layers on eight times the rows ([65536, 4096] bf16, 512 MiB per tensor): the kernels
+    run for a quarter of a millisecond, so what they reach here is their bandwidth without the
+    launch and ramp-up cost that weighs on the 25-50 us launches of c2 itself.
+    """
+    raw = Raw()
+    lib = raw.lib
+    rows_, feat, dtype = 65536, 4096, torch.bfloat16
+    dt = raw._lib.dtype_id(dtype)
+    nsets = 2
+    xs = [gen((rows_, feat), 2401 + i, dtype).cuda() for i in range(nsets)]
+    dys = [gen((rows_, feat), 2411 + i, dtype).cuda() for i in range(nsets)]
+    ys = [torch.empty_like(xs[0]) for _ in range(nsets)]
+    dxs = [torch.empty_like(xs[0]) for _ in range(nsets)]
+    w = gen((feat,), 2201, dtype, 0.1, 1.0).cuda()
+    b = gen((feat,), 2202, dtype, 0.1).cuda()
+    mean, rstd = torch.empty(rows_, device='cuda'), torch.empty(rows_, device='cuda')
+    dwg, dbg = torch.empty(feat, device='cuda'), torch.empty(feat, device='cuda')
+    wsb = lib.at_norm_bwd_workspace_bytes(rows_, feat, 2)
+    ws = torch.empty(wsb, dtype=torch.uint8, device='cuda')
+    tbytes = rows_ * feat * 2
+    st = raw.stream
+    counter = [0]
+
+    def nxt():
+        counter[0] = (counter[0] + 1) % nsets
+        return counter[0]
+
+    def ln_f():
+        i = nxt()
+        raw.check(lib.at_layer_norm_fwd(xs[i].data_ptr(), w.data_ptr(), b.data_ptr(), mean.data_ptr(),
+                                        rstd.data_ptr(), ys[i].data_ptr(), rows_, feat, feat, feat, 1e-5, dt, dt,
+                                        dt, st()), 'ln_fwd')
+
+    def ln_b():
+        i = nxt()
+        raw.check(lib.at_layer_norm_bwd(dys[i].data_ptr(), xs[i].data_ptr(), mean.data_ptr(), rstd.data_ptr(),
+                                        w.data_ptr(), dxs[i].data_ptr(), dwg.data_ptr(), dbg.data_ptr(),
+                                        ws.data_ptr(), wsb, rows_, feat, feat, feat, feat, dt, dt, dt, dt, st()),
+                  'ln_bwd')
+
+    def rms_f():
+        i = nxt()
+        raw.check(lib.at_rms_norm_fwd(xs[i].data_ptr(), w.data_ptr(), rstd.data_ptr(), ys[i].data_ptr(), rows_,
+                                      feat, feat, feat, 1e-5, dt, dt, dt, st()), 'rms_fwd')
+
+    def rms_b():
+        i = nxt()
+        raw.check(lib.at_rms_norm_bwd(dys[i].data_ptr(), xs[i].data_ptr(), rstd.data_ptr(), w.data_ptr(),
+                                      dxs[i].data_ptr(), dwg.data_ptr(), ws.data_ptr(), wsb, rows_, feat, feat,
+                                      feat, feat, dt, dt, dt, dt, st()), 'rms_bwd')
+
+    def sm_f():
+        i = nxt()
+        raw.check(lib.at_softmax_fwd(xs[i].data_ptr(), ys[i].data_ptr(), rows_, feat, feat, feat, 0, 0, dt, dt,
+                                     st()), 'softmax_fwd')
+
+    def sm_b():
+        i = nxt()
+        raw.check(lib.at_softmax_bwd(dys[i].data_ptr(), ys[i].data_ptr(), dxs[i].data_ptr(), rows_, feat, feat,
+                                     feat, feat, 0, 0, dt, dt, dt, st()), 'softmax_bwd')
+    results = []
+    for name, f, bwd in (('LayerNorm', ln_f, ln_b), ('RMSNorm', rms_f, rms_b), ('Softmax', sm_f, sm_b)):
+        ms_f, ms_b = gpu_time_ms(f, 5, 3, 3), gpu_time_ms(bwd, 5, 3, 3)
+        gbs = 5 * tbytes / (ms_f + ms_b) / 1e6
+        results.append({
+            'tag': f'c2x8 {name}',
+            'workload': f'c2 shape with eight times the rows: {name} bf16 fwd+bwd X[{rows_},{feat}]',
+            'metric': 'HBM GB/s', 'value': gbs, 'unit': 'GB/s', 'ms_fwd': ms_f, 'ms_bwd': ms_b,
+            'fwd_gbs': 2 * tbytes / ms_f / 1e6, 'bwd_gbs': 3 * tbytes / ms_b / 1e6,
+            'roofline': {'bound': 'hbm', 'achieved': gbs, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                         'frac': gbs / PEAK_HBM_GBS, 'traffic': None},
+        })
+    return results
+
+
 # ------------------------------------------------------------------------------------------
 # c3: CrossEntropy fp16 [8192, 50257]
 # ------------------------------------------------------------------------------------------
@@ -1139,6 +1216,7 @@ def main() -> int:
         extra.append(bench_linear('c1', max(args.steps, 50), args.warmup, with_cpu))
     if 'c2' in wanted:
         extra.extend(bench_rows(args.steps, args.warmup, with_cpu))
+        extra.extend(bench_rows_tall())
     if 'c3' in wanted:
         extra.extend(bench_cross_entropy(args.steps, args.warmup, with_cpu))
     if 'c5' in wanted:

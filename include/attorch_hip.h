@@ -310,6 +310,15 @@ int at_linear_bwd_input(const void* pre_act_grad, const void* weight, void* inpu
                         int64_t weight_stride, int64_t input_grad_stride, int in_dtype,
                         int out_dtype, at_stream_t stream);
 
+/* The two backward products take out_dtype = fp32 with 16-bit operands: the result is the product
+ * rounded to the operand dtype and then widened, i.e. what the reference's 16-bit products under
+ * torch.autocast (attorch/linear_layer.py:152-155) give once autograd has cast them to a float32
+ * leaf — written in one pass instead of a 16-bit store and a cast kernel.  The tiled kernels do
+ * this in their epilogue; at_linear_bwd_wide_output_supported tells (1 / 0) whether both products
+ * of a layer with contiguous, 16-byte aligned operands of these extents run on them (otherwise
+ * the generic kernels still give the same values, only slower than a 16-bit result plus a cast). */
+int at_linear_bwd_wide_output_supported(int64_t batch, int64_t in_feat, int64_t out_feat, int dtype);
+
 /* Scratch for at_linear_bwd_weight: with it, a weight gradient whose [in_feat, out_feat] tile
  * grid is small next to the GPU is computed in several slices of the batch at once (fp32 partial
  * sums, added in a fixed order); so is the weight gradient of a layer with at most 16 output

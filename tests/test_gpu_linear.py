@@ -378,3 +378,42 @@ def test_linear_under_autocast_with_fp32_parameters(shape, out_dim, act_func, am
     wd.grad = None
     y2.backward(dy.cuda())
     torch.testing.assert_close(wd.grad, first, rtol=0, atol=0)
+
+
+@pytest.mark.parametrize('dtype', HALF_DTYPES)
+@pytest.mark.parametrize('batch, in_dim, out_dim', [
+    (8100, 520, 4088),     # 256x256 tiles with ragged edges (input gradient) / 128x128 tiles
+    (4096, 256, 256),      # 128x128 tiles, weight gradient split over the batch
+    (2048, 512, 384),      # 128x128 tiles
+    (300, 264, 520),       # generic kernel (small problem)
+    (1000, 1000, 1000),
+])
+def test_backward_products_write_fp32_like_a_cast_of_the_16bit_result(batch, in_dim, out_dim, dtype) -> None:
+    """
+    C ABI: at_linear_bwd_input / at_linear_bwd_weight with 16-bit operands and out_dtype = fp32 give
+    exactly the 16-bit result widened (the product is rounded to the operand dtype first), whichever
+    kernel serves the shape.
+    """
+    from attorch_amd import _lib
+    lib = _lib.load()
+    did, f32 = _lib.dtype_id(dtype), _lib.dtype_id(torch.float32)
+    x = randn((batch, in_dim), 1, dtype).cuda()
+    w = randn((in_dim, out_dim), 2, dtype, in_dim ** -0.5).cuda()
+    dz = randn((batch, out_dim), 3, dtype).cuda()
+    stream = _lib.stream_of(x)
+    workspace_bytes = lib.at_linear_bwd_weight_workspace_bytes(batch, in_dim, out_dim, did)
+    workspace = torch.empty(max(workspace_bytes, 16), dtype=torch.uint8, device='cuda')
+    results = {}
+    for out_dtype, oid in ((dtype, did), (torch.float32, f32)):
+        dx = torch.full((batch, in_dim), float('nan'), dtype=out_dtype, device='cuda')
+        dw = torch.full((in_dim, out_dim), float('nan'), dtype=out_dtype, device='cuda')
+        _lib.check(lib.at_linear_bwd_input(dz.data_ptr(), w.data_ptr(), dx.data_ptr(), batch, in_dim, out_dim,
+                                           out_dim, out_dim, in_dim, did, oid, stream), 'at_linear_bwd_input')
+        _lib.check(lib.at_linear_bwd_weight(x.data_ptr(), dz.data_ptr(), dw.data_ptr(), workspace.data_ptr(),
+                                            workspace_bytes, batch, in_dim, out_dim, in_dim, out_dim, out_dim,
+                                            did, oid, stream), 'at_linear_bwd_weight')
+        results[out_dtype] = (dx, dw)
+    for narrow, wide, what in zip(results[dtype], results[torch.float32], ('input_grad', 'weight_grad')):
+        assert wide.dtype is torch.float32
+        assert torch.equal(narrow.float(), wide), what
+    assert_close(results[dtype][0], dz.double().cpu() @ w.double().cpu().T, dtype, 'input_grad')
