@@ -376,11 +376,11 @@ __global__ __launch_bounds__(1024) void norm_fwd_stream_kernel(
 // Norm backward over a persistent grid.  Each workgroup walks row-blocks with a grid stride;
 // each lane accumulates the parameter gradients of the columns it owns.
 //   part_w / part_b: [gridDim.x, feat] fp32 partial rows (null when not wanted).
-// Dynamic LDS: blockDim.x * VEC * norm_bwd_fold_chunks(ITERS) floats (only used when a workgroup
-// holds several rows).
+// Dynamic LDS: (blockDim.x - lanes per row) * VEC * ITERS floats per parameter gradient (only used
+// when a workgroup holds several rows; at most 57 KB: rows of more than two chunks per lane take
+// the whole workgroup).
 // ------------------------------------------------------------------------------------------
-// Chunks per lane whose parameter gradients cross LDS in one round of the final fold.
-constexpr int norm_bwd_fold_chunks(int iters) { return iters <= 2 ? iters : 1; }
+constexpr bool norm_bwd_fused_tail(bool layer, int iters) { return layer || iters > 2; }
 
 template <bool LAYER, typename TDY, typename TX, typename TDX, typename TW, int VEC, int ITERS>
 // RMSNorm with at most two chunks per lane fits 128 registers, i.e. two workgroups per CU; the
@@ -395,6 +395,10 @@ __global__ __launch_bounds__(512, (ITERS <= 2 && !LAYER ? 4 : 1)) void norm_bwd_
   // With few chunks per lane the normalised input and the scaled gradient of the first sweep stay
   // in registers as fp32 for the second; otherwise the second sweep recomputes them.
   constexpr bool KEEP = ITERS * VEC <= 16;
+  // Whether the parameter gradients leave inside the workgroup's last row-block (see `step`) or
+  // behind the loop.  The instances held to 128 registers (two workgroups per CU) spill in their
+  // main loop with the former and keep the latter.
+  constexpr bool FUSED_TAIL = norm_bwd_fused_tail(LAYER, ITERS);
   __shared__ float slots[2][16][2];
   extern __shared__ float red[];
   const int group = 1 << group_log2;
@@ -438,10 +442,17 @@ __global__ __launch_bounds__(512, (ITERS <= 2 && !LAYER ? 4 : 1)) void norm_bwd_
     t.x.load(x, row, xs, v, lane, group, chunks);
   };
   fetch(set_a, (int64_t)blockIdx.x * rpb + rib);
-  auto step = [&](int64_t rb, RowSet& cur, RowSet& nxt) {
+  // LAST: the workgroup's last row-block.  Nothing is requested ahead, and the parameter gradients,
+  // complete after its first sweep, leave in front of its stores instead of behind the loop: a
+  // barrier at the end of the kernel would first wait for the acknowledgement of the last stores.
+  // The row-groups after the first hand their sums over through LDS as red[value][thread - group]
+  // (consecutive lanes, consecutive banks), published by the barrier of the row sums; the first
+  // row-group adds them up in a fixed order and writes the workgroup's partial row.
+  auto step = [&](int64_t rb, RowSet& cur, RowSet& nxt, auto last_tag) {
+    constexpr bool LAST = decltype(last_tag)::value;
     const int64_t row = rb * rpb + rib;
     const bool valid = row < batch;
-    fetch(nxt, row + row_step);
+    if (!LAST) fetch(nxt, row + row_step);
     RowCache<TDY, VEC, ITERS>& cdy = cur.dy;
     RowCache<TX, VEC, ITERS>& cx = cur.x;
     const float mean = cur.mean, rstd = cur.rstd;
@@ -490,8 +501,46 @@ __global__ __launch_bounds__(512, (ITERS <= 2 && !LAYER ? 4 : 1)) void norm_bwd_
       // one chunk at a time: keeps the widened temporaries of a single chunk live, not of all
       __builtin_amdgcn_sched_barrier(0);
     }
+    const int n_out = (part_w ? 1 : 0) + ((LAYER && part_b) ? 1 : 0);
+    const int others = blockDim.x - group;   // lanes of the row-groups 1 .. rpb - 1
+    if (LAST && FUSED_TAIL && rib > 0) {
+      for (int which = 0; which < n_out; ++which) {
+        const bool is_w = (which == 0 && part_w);
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+          for (int j = 0; j < VEC; ++j)
+            red[((which * ITERS + it) * VEC + j) * others + (threadIdx.x - group)] =
+                (is_w || !LAYER) ? acc_w[it][j] : acc_b[LAYER ? it : 0][j];
+      }
+    }
     group_sum2(s1, s2, group, slots, parity);
     parity ^= 1;
+    if (LAST && FUSED_TAIL && n_out > 0) {
+      if (rpb > 1 && group <= kWave) __syncthreads();   // the row sums of such groups pass no barrier of their own
+      if (rib == 0) {
+        for (int which = 0; which < n_out; ++which) {
+          const bool is_w = (which == 0 && part_w);
+          float* part = (is_w ? part_w : part_b) + (int64_t)blockIdx.x * feat;
+#pragma unroll
+          for (int it = 0; it < ITERS; ++it) {
+            const int c = lane + it * group;
+            float v[VEC];
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+              float sum = (is_w || !LAYER) ? acc_w[it][j] : acc_b[LAYER ? it : 0][j];
+              const float* col = red + ((which * ITERS + it) * VEC + j) * others + lane;
+              for (int r = 1; r < rpb; ++r) sum += col[(r - 1) * group];
+              v[j] = sum;
+            }
+            if (c < chunks) {
+#pragma unroll
+              for (int j = 0; j < VEC; ++j) part[(int64_t)c * VEC + j] = v[j];
+            }
+          }
+        }
+      }
+    }
     // the input gradient is rstd * (g - (h * s1 + s2) / feat); rstd / feat folded into the sums
     s1 *= inv_feat * rstd;
     s2 = LAYER ? s2 * inv_feat * rstd : 0.f;
@@ -533,56 +582,70 @@ __global__ __launch_bounds__(512, (ITERS <= 2 && !LAYER ? 4 : 1)) void norm_bwd_
       }
     }
   };
+  const int64_t stride = gridDim.x;
+  if constexpr (FUSED_TAIL) {
+    // every workgroup has at least one row-block (the grid is no larger than their number)
 #pragma unroll 1
-  for (int64_t rb = blockIdx.x; rb < row_blocks; rb += 2 * (int64_t)gridDim.x) {
-    step(rb, set_a, set_b);
-    if (rb + gridDim.x < row_blocks) step(rb + gridDim.x, set_b, set_a);
+    for (int64_t rb = blockIdx.x;; rb += 2 * stride) {
+      if (rb + stride >= row_blocks) {
+        step(rb, set_a, set_b, std::true_type());
+        break;
+      }
+      step(rb, set_a, set_b, std::false_type());
+      if (rb + 2 * stride >= row_blocks) {
+        step(rb + stride, set_b, set_a, std::true_type());
+        break;
+      }
+      step(rb + stride, set_b, set_a, std::false_type());
+    }
+  } else {
+#pragma unroll 1
+    for (int64_t rb = blockIdx.x; rb < row_blocks; rb += 2 * stride) {
+      step(rb, set_a, set_b, std::false_type());
+      if (rb + stride < row_blocks) step(rb + stride, set_b, set_a, std::false_type());
+    }
   }
 
-  if (!part_w && !part_b) return;
-  // Fold the row-groups of this workgroup together, then emit one partial row.  The values cross
-  // through LDS as red[value][thread]: consecutive lanes touch consecutive banks both when every
-  // lane writes and when the lanes of the first row-group read the other groups' values, and all
-  // chunks of a gradient (up to two per lane) share one pair of barriers.
-  constexpr int FOLD = norm_bwd_fold_chunks(ITERS);
-  const int n_out = (part_w ? 1 : 0) + ((LAYER && part_b) ? 1 : 0);
-  for (int which = 0; which < n_out; ++which) {
-    const bool is_w = (which == 0 && part_w);
-    float* part = is_w ? part_w : part_b;
+  if (FUSED_TAIL || (!part_w && !part_b)) return;
+  // Behind the loop: fold the row-groups of this workgroup together, then emit one partial row.
+  // Same hand-over through LDS, with a pair of barriers of its own.
+  {
+    const int n_out = (part_w ? 1 : 0) + ((LAYER && part_b) ? 1 : 0);
+    const int others = blockDim.x - group;
+    if (rpb > 1) {
+      __syncthreads();
+      if (rib > 0) {
+        for (int which = 0; which < n_out; ++which) {
+          const bool is_w = (which == 0 && part_w);
 #pragma unroll
-    for (int it0 = 0; it0 < ITERS; it0 += FOLD) {
-      float v[FOLD][VEC];
+          for (int it = 0; it < ITERS; ++it)
 #pragma unroll
-      for (int f = 0; f < FOLD; ++f)
-#pragma unroll
-        for (int j = 0; j < VEC; ++j)
-          v[f][j] = (is_w || !LAYER) ? acc_w[it0 + f][j] : acc_b[LAYER ? it0 + f : 0][j];
-      if (rpb > 1) {
-        __syncthreads();
-#pragma unroll
-        for (int f = 0; f < FOLD; ++f)
-#pragma unroll
-          for (int j = 0; j < VEC; ++j) red[(f * VEC + j) * blockDim.x + threadIdx.x] = v[f][j];
-        __syncthreads();
-        if (rib == 0) {
-#pragma unroll
-          for (int f = 0; f < FOLD; ++f)
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) {
-              const float* col = red + (f * VEC + j) * blockDim.x + lane;
-              float s = 0.f;
-              for (int r = 0; r < rpb; ++r) s += col[r * group];
-              v[f][j] = s;
-            }
+            for (int j = 0; j < VEC; ++j)
+              red[((which * ITERS + it) * VEC + j) * others + (threadIdx.x - group)] =
+                  (is_w || !LAYER) ? acc_w[it][j] : acc_b[LAYER ? it : 0][j];
         }
       }
+      __syncthreads();
+    }
+    if (rib == 0) {
+      for (int which = 0; which < n_out; ++which) {
+        const bool is_w = (which == 0 && part_w);
+        float* part = (is_w ? part_w : part_b) + (int64_t)blockIdx.x * feat;
 #pragma unroll
-      for (int f = 0; f < FOLD; ++f) {
-        const int c = lane + (it0 + f) * group;
-        if (rib == 0 && c < chunks) {
-          float* dst = part + (int64_t)blockIdx.x * feat + (int64_t)c * VEC;
+        for (int it = 0; it < ITERS; ++it) {
+          const int c = lane + it * group;
+          float v[VEC];
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) dst[j] = v[f][j];
+          for (int j = 0; j < VEC; ++j) {
+            float sum = (is_w || !LAYER) ? acc_w[it][j] : acc_b[LAYER ? it : 0][j];
+            const float* col = red + ((which * ITERS + it) * VEC + j) * others + lane;
+            for (int r = 1; r < rpb; ++r) sum += col[(r - 1) * group];
+            v[j] = sum;
+          }
+          if (c < chunks) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) part[(int64_t)c * VEC + j] = v[j];
+          }
         }
       }
     }
@@ -1156,7 +1219,7 @@ int norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd
 #define AT_NORM_BWD_LAUNCH(TW, VV)                                                                       \
   {                                                                                                      \
     AT_DISPATCH_ITERS4(p.iters, {                                                                        \
-      const size_t lds = rpb > 1 ? (size_t)p.block * VV * norm_bwd_fold_chunks(ITERS) * sizeof(float) : 0; \
+      const size_t lds = rpb > 1 ? (size_t)(p.block - (1 << p.group_log2)) * VV * ITERS * n_grads * sizeof(float) : 0; \
       auto kernel = norm_bwd_kernel<LAYER, TDY, TX, TDY, TW, VV, ITERS>;                                 \
       parts = (int)persistent_grid((const void*)kernel, p.block, lds, row_blocks, kMaxPartialRows);      \
       float* part_b = bias_grad ? part_w + (int64_t)parts * feat : nullptr;                              \
