@@ -100,7 +100,7 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument('--gpus', type=int, default=1)
     parser.add_argument('--steps', type=int, default=20)
     parser.add_argument('--warmup', type=int, default=5)
-    parser.add_argument('--configs', type=str, default='c1,c2,c3,c5',
+    parser.add_argument('--configs', type=str, default='c1,c2,c2x8,c3,c5',
                         help='secondary configs to measure besides the headline (c4); "none" skips them')
     parser.add_argument('--no-cpu', action='store_true', help='skip the CPU baselines')
     parser.add_argument('--no-modules', action='store_true',
@@ -1216,6 +1216,7 @@ def main() -> int:
         extra.append(bench_linear('c1', max(args.steps, 50), args.warmup, with_cpu))
     if 'c2' in wanted:
         extra.extend(bench_rows(args.steps, args.warmup, with_cpu))
+    if 'c2x8' in wanted:
         extra.extend(bench_rows_tall())
     if 'c3' in wanted:
         extra.extend(bench_cross_entropy(args.steps, args.warmup, with_cpu))

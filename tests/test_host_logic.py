@@ -142,7 +142,7 @@ def test_argument_errors_without_gpu() -> None:
     assert lib.at_linear_bwd_weight_workspace_bytes(16384, 8192, 8192, 2) == 0
     assert lib.at_linear_bwd_weight(None, p, p, None, 0, 4, 8, 8, 8, 8, 8, 0, 0, None) == -1
     assert lib.at_norm_bwd_workspace_bytes(16, 8, 2) == 16 * 8 * 4 * 2
-    assert lib.at_cross_entropy_workspace_bytes(10) == 56
+    assert lib.at_cross_entropy_workspace_bytes(10) == (16 + 10) * 4   # 16 partial sums of the divisor + one loss per row
 
 
 def test_get_output_dtype_policy(monkeypatch) -> None:
@@ -229,3 +229,40 @@ def test_row_stride_of_extent_one_dimensions() -> None:
     weight = torch.zeros(63, 1).T.contiguous()            # shape [1, 63], stride(0) stays 1
     assert tuple(weight.shape) == (1, 63) and _lib.row_stride(weight) == 63
     assert _lib.row_stride(torch.zeros(0, 7)) == 7
+
+
+def test_bench_final_line_stays_compact() -> None:
+    """
+    bench.py ends with one JSON line that a harness reads from the tail of stdout: with every
+    secondary config present it must stay far below 8 KB and carry the contract fields, the
+    roofline and the CPU baseline of the headline and one compact record per secondary config.
+    """
+    import argparse
+    import json
+    import bench
+    head = {
+        'value': 1169.123456, 'ms_per_step': 5.6412345,
+        'workload': 'c4: Linear bfloat16 fwd+bwd X[16384,4096] W[4096,16384] act=geluapprox',
+        'roofline': {'bound': 'mfma', 'kernel': 'linear_fwd (GEMM + bias + activation epilogue)', 'achieved': 1147.2,
+                     'peak': 2500.0, 'unit': 'TFLOP/s', 'frac': 0.459, 'traffic': 4611841360},
+        'cpu_baseline': {'value': 0.51, 'unit': 'TFLOP/s', 'cores': 16, 'kind': 'port',
+                         'sample': 'first 2048 of 16384 rows, full K and N, oracle fwd+bwd in fp32 compute'},
+        'frac_of_peak_step': 0.468,
+        'kernel_ms': {'linear_fwd': 1.9, 'act_bwd_with_bias_grad': 0.28, 'linear_bwd_input': 1.7,
+                      'linear_bwd_weight': 1.7, 'colsum_unfused': 0.1},
+        'amp': {'ms_per_step_fp16_tensors': 5.8, 'ms_per_step_autocast_fp16_over_fp32_tensors': 6.0,
+                'autocast_over_fp16': 1.03},
+    }
+    entry = {'tag': 'c2 GELU(tanh)+Dropout(0.1) layer', 'workload': 'x' * 200, 'value': 4234.123456, 'unit': 'GB/s',
+             'roofline': {'frac': 0.5234567, 'traffic': 362346310, 'note': 'y' * 300},
+             'cpu_baseline': {'value': 1.5167704445, 'unit': 'GB/s', 'cores': 16}, 'module_level': {'note': 'z' * 500}}
+    line = bench.compact_line(argparse.Namespace(steps=20, warmup=5), head, [dict(entry) for _ in range(24)])
+    text = json.dumps(line)
+    assert len(text) < 6000
+    for key in ('metric', 'value', 'unit', 'n_gpus', 'steps', 'warmup', 'ms_per_step', 'higher_is_better', 'scaling',
+                'vs_baseline', 'dtype', 'data', 'config', 'roofline', 'cpu_baseline'):
+        assert key in line, key
+    assert line['vs_baseline'] is None and line['n_gpus'] == 1
+    assert set(line['roofline']) >= {'bound', 'achieved', 'peak', 'unit', 'frac', 'traffic'}
+    assert set(line['cpu_baseline']) >= {'value', 'unit', 'cores', 'kind', 'sample'}
+    assert len(line['configs']) == 24 and all('frac' in c and 'tag' in c for c in line['configs'])
