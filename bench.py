@@ -1,21 +1,29 @@
 """
 Benchmark of the attorch layer-kernel hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs c4,c2,...] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs c1,c2,c2x8,c3,c5] [--no-cpu]
+                    [--detail-file PATH]
 
 A "step" is one forward + backward pass of the headline workload over one batch of synthetic
 input that is already resident in HBM: attorch_amd.Linear with fused GELU(tanh), bf16,
 X[16384, 4096] x W[4096, 16384] (BASELINE config 4, the configuration the 70 %-of-MFMA-peak
-target is quoted on).  One JSON line is printed; besides the contract fields it carries
+target is quoted on).  stdout ends with ONE compact JSON line (a few KB); besides the contract
+fields it carries
   roofline      the dominant kernel (the forward MFMA GEMM with its fused epilogue) against
                 the MI355X dense bf16 MFMA peak, timed with HIP events on the launch stream
   cpu_baseline  the CPU oracle of the same workload on a bounded sample of rows, timed on
                 this host's cores (a reported baseline, not a target)
+  amp           the same step with float32 tensors under torch.autocast(float16) against the
+                step on float16 tensors
   configs       the other BASELINE configs (c1 Linear fp32, c2 LayerNorm / RMSNorm / Softmax
-                / LogSoftmax, c3 CrossEntropy, c5 Conv2d + BatchNorm2d), each as absolute
-                throughput, fraction of its roofline and CPU baseline.
+                / LogSoftmax, c2x8 the same layers on eight times the rows, c3 CrossEntropy,
+                c5 Conv2d + BatchNorm2d), each as tag, absolute throughput, fraction of its
+                roofline, measured HBM traffic and CPU baseline.
+The full record (module-level and torch-native timings, CPU functional baselines, notes) is
+written to --detail-file (gpurun_out/bench_detail.json beside this script by default).
 Buffers of the bandwidth-bound configs are rotated over several sets so the 256 MB Infinity
-Cache cannot serve them.
+Cache cannot serve them.  Secondary configs are timed with 10 warm-up and 60 timed calls (median
+of 6 groups of 10) whatever --steps says.
 """
 
 import argparse
@@ -38,22 +46,22 @@ PEAK_MFMA_FP32_TFLOPS = 157.3    # dense fp32 MFMA
 # the 256 MB Infinity Cache serves are included.  They belong to the kernel sources whose digest is
 # TRAFFIC_SOURCE_DIGEST: when the sources of the loaded library differ, `traffic` is reported as
 # null and the recorded figure moves to `traffic_recorded` (stale until the profile is redone).
-TRAFFIC_SOURCE_DIGEST = 'e909313204c9756c'
+TRAFFIC_SOURCE_DIGEST = '7e3a79c42e599137'
 MEASURED_TRAFFIC_BYTES = {
-    'c4_linear_fwd': 4611841360,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.0 GiB read, 1.0 GiB written
-    'c2_layer_norm': 362346310,       # norm_fwd + norm_bwd + reduce_partials
-    'c2_rms_norm': 361810981,
-    'c2_softmax': 335893353,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
-    'c2_act_dropout': 335783418,      # act_dropout forward + backward
-    'c2_glu': 268580377,              # glu forward + backward
-    'c2_mse': 335721550,              # p_loss forward + backward
-    'c3_cross_entropy': 1717820790,   # ce_row_kernel (ignored rows are not read)
-    'c3_cross_entropy_autocast': 2502925447,
-    'c3_nll_loss': 826885215,         # nll forward (a gather) + the single-pass gradient write
-    'c5_conv_channels_last': 389746743,     # the two weights-in-registers kernels + weight gradient + weight reorders, no copies
-    'c5_conv': 595395114,             # the same + 2 layout copies
-    'c5_batch_norm_channels_last': 568555867,
-    'c5_batch_norm': 565688757,       # stats + apply + backward reduce + backward apply
+    'c4_linear_fwd': 5010981602,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.7 GiB read, 1.0 GiB written
+    'c2_layer_norm': 362245971,       # norm_fwd + norm_bwd + reduce_partials
+    'c2_rms_norm': 361808996,
+    'c2_softmax': 335901415,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
+    'c2_act_dropout': 335781498,      # act_dropout forward + backward
+    'c2_glu': 268578777,              # glu forward + backward
+    'c2_mse': 335721326,              # p_loss forward + backward
+    'c3_cross_entropy': 1683540255,   # ce_row_kernel (ignored rows are not read)
+    'c3_cross_entropy_autocast': 2436772378,
+    'c3_nll_loss': 826898518,         # nll forward (a gather) + the single-pass gradient write
+    'c5_conv_channels_last': 389752029,     # the two weights-in-registers kernels + weight gradient + weight reorders, no copies
+    'c5_conv': 595399947,             # the same + 2 layout copies
+    'c5_batch_norm_channels_last': 568554857,
+    'c5_batch_norm': 565700194,       # stats + apply + backward reduce + backward apply
 }
 
 
