@@ -16,7 +16,9 @@ from .helpers import DTYPES, assert_close, compute_dtype, randn
 pytestmark = pytest.mark.gpu
 
 SHAPES = [(1, 8000), (4, 2000), (8, 1024), (32, 1024), (2048, 768), (6144, 256), (8096, 32), (12288, 1),
-          (5, 7), (48, 50257), (9, 12345), (4, 131075)]
+          (5, 7), (48, 50257), (9, 12345), (4, 131075),
+          # rows of more than 4096 vectors: 1024 lanes per row with 6, 7 or 8 vectors each
+          (6, 20001), (5, 32768), (3, 65536), (3, 57003)]
 
 
 def make_targets(batch, feat, seed, ignore_fraction):
