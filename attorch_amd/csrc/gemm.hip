@@ -521,8 +521,11 @@ struct MidLoader {
   i32x4 rsrc;
   int lane_off, blk_step, k_step, K;
 
-  __device__ __forceinline__ void init(const T* base, int64_t ld, int outer0, int outer_total, int K_) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int tid;   // thread index inside the four waves that load a tile together
+
+  __device__ __forceinline__ void init(const T* base, int64_t ld, int outer0, int outer_total, int K_, int tid_) {
+    tid = tid_;
+    const int lane = tid & 63, wave = tid >> 6;
     K = K_;
     if (CONTRACT_CONTIG) {
       rsrc = make_buffer_rsrc(base, ((int64_t)(outer_total - 1) * ld + K_) * 2);
@@ -539,7 +542,7 @@ struct MidLoader {
     }
   }
   __device__ __forceinline__ void issue(int kt, char* tile) const {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = tid & 63, wave = tid >> 6;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int q = wave * 4 + i;
@@ -550,7 +553,8 @@ struct MidLoader {
         const int k = kt * BK + chunk * 8;
         off = k < K ? lane_off + i * blk_step + k * 2 : kOobOffset;
       } else {
-        off = lane_off + i * blk_step + kt * k_step;
+        // k-rows at or past K lie past the end of the buffer and read as zeros
+        off = kt * BK < K ? lane_off + i * blk_step + kt * k_step : kOobOffset;
       }
       lds_dma_16(rsrc, off, tile + q * 1024);
     }
@@ -579,10 +583,17 @@ __device__ __forceinline__ uint4 read_frag_mid(const char* tile, int outer_base,
 }
 
 // TO as in big_tile_epilogue: T, or float for the value rounded to T and widened (no activation).
-template <typename T, bool A_MC, bool B_KC, bool SPLIT, typename TO = T>
-__global__ __launch_bounds__(kGemmThreads, 2) void gemm_mid16_kernel(GemmArgs g) {
+// KG = 2: for problems with at most one tile per CU.  The workgroup has eight waves in two groups
+// of four; each group multiplies every other k-tile of the same output tile from LDS stages of its
+// own, and the two sets of accumulators are added while the tile is staged for the epilogue.  A CU
+// then has two waves per SIMD to cover each other's waits, as it has with two workgroups of four.
+template <typename T, bool A_MC, bool B_KC, bool SPLIT, typename TO = T, int KG = 1>
+__global__ __launch_bounds__(kGemmThreads * KG, KG == 1 ? 2 : 1) void gemm_mid16_kernel(GemmArgs g) {
   constexpr bool A_KC = !A_MC;
-  __shared__ __attribute__((aligned(1024))) char lds[kMidLds];
+  static_assert(KG == 1 || (KG == 2 && !SPLIT), "one or two k-groups; no k-groups inside a split of the contraction");
+  constexpr int kStagesBytes = KG * 2 * kMidStage;
+  constexpr int kEpiBytes = KG * MT * kMidEpiPitch * 4;
+  __shared__ __attribute__((aligned(1024))) char lds[kStagesBytes > kEpiBytes ? kStagesBytes : kEpiBytes];
   const T* __restrict__ A = reinterpret_cast<const T*>(g.a);
   const T* __restrict__ B = reinterpret_cast<const T*>(g.b);
 
@@ -604,8 +615,10 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_mid16_kernel(GemmArgs g)
   const int m0 = (first_m + in_group % gsz) * MT;
   const int n0 = (in_group / gsz) * MT;
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) & 3;
+  const int kgroup = KG == 1 ? 0 : (int)(threadIdx.x >> 8);
   const int wm = wave >> 1, wn = wave & 1;
+  char* const stages = lds + kgroup * 2 * kMidStage;   // this k-group's two stages
 
   f32x16 acc[2][2];
 #pragma unroll
@@ -617,24 +630,27 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_mid16_kernel(GemmArgs g)
 
   MidLoader<T, A_KC> la;
   MidLoader<T, B_KC> lb;
-  la.init(A, g.lda, m0, g.M, g.K);
-  lb.init(B, g.ldb, n0, g.N, g.K);
+  la.init(A, g.lda, m0, g.M, g.K, threadIdx.x & 255);
+  lb.init(B, g.ldb, n0, g.N, g.K, threadIdx.x & 255);
   int kt0 = 0, KT = (g.K + BK - 1) / BK;
   if (SPLIT) {
     kt0 = blockIdx.y * g.kt_per_split;
     KT = kt0 + g.kt_per_split < KT ? kt0 + g.kt_per_split : KT;   // the host leaves no split empty
   }
-  la.issue(kt0, lds);
-  lb.issue(kt0, lds + kMidTileBytes);
+  // k-group q takes k-tiles kt0 + q, kt0 + q + KG, ...; both groups make the same number of steps (a
+  // k-tile past the end reads as zeros), so every wave passes every barrier
+  kt0 += kgroup;
+  la.issue(kt0, stages);
+  lb.issue(kt0, stages + kMidTileBytes);
   lds_dma_wait_all();
   __syncthreads();
 
-  for (int kt = kt0; kt < KT; ++kt) {
-    const char* cur = lds + ((kt - kt0) & 1) * kMidStage;
-    char* nxt = lds + (((kt - kt0) & 1) ^ 1) * kMidStage;
-    if (kt + 1 < KT) {
-      la.issue(kt + 1, nxt);
-      lb.issue(kt + 1, nxt + kMidTileBytes);
+  for (int kt = kt0, step = 0; kt - kgroup < KT; kt += KG, ++step) {
+    const char* cur = stages + (step & 1) * kMidStage;
+    char* nxt = stages + ((step & 1) ^ 1) * kMidStage;
+    if (kt - kgroup + KG < KT) {
+      la.issue(kt + KG, nxt);
+      lb.issue(kt + KG, nxt + kMidTileBytes);
     }
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
@@ -657,14 +673,15 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_mid16_kernel(GemmArgs g)
   // ---- epilogue: accumulators (+ bias) -> LDS as fp32 -> rows of 8 columns per lane ----
   // A lane holds, for tile (i, j) and register group rg, C[m][n .. n+3] with
   //   m = wm*64 + i*32 + lane%32,  n = wn*64 + j*32 + rg*8 + (lane/32)*4   (tile-local).
-  float* stage = reinterpret_cast<float*>(lds);
+  float* stage = reinterpret_cast<float*>(lds) + kgroup * MT * kMidEpiPitch;   // k-group 1 stages its sums behind group 0's
+  const bool with_bias = g.bias && kgroup == 0;
 #pragma unroll
   for (int j = 0; j < 2; ++j)
 #pragma unroll
     for (int rg = 0; rg < 4; ++rg) {
       const int nl = wn * 64 + j * 32 + rg * 8 + (lane >> 5) * 4;
       float bv[4] = {0.f, 0.f, 0.f, 0.f};
-      if (g.bias) {
+      if (with_bias) {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
           if (n0 + nl + e < g.N) bv[e] = load_scalar_f32(g.bias, g.bias_dt, n0 + nl + e);
@@ -681,8 +698,20 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_mid16_kernel(GemmArgs g)
       }
     }
   __syncthreads();
-  // 256 lanes: 16 rows per sweep, 16 lanes x 8 columns per row
+  // 16 rows per sweep and k-group, 16 lanes x 8 columns per row; the sums of the k-groups are added here
   const int rsub = threadIdx.x >> 4, cseg = (threadIdx.x & 15) * 8;
+  constexpr int kSweepRows = 16 * KG;
+  auto load8 = [&](int ml, float (&v)[8]) {
+    const float* src = reinterpret_cast<const float*>(lds) + ml * kMidEpiPitch + cseg;
+    *reinterpret_cast<float4*>(v) = *reinterpret_cast<const float4*>(src);
+    *reinterpret_cast<float4*>(v + 4) = *reinterpret_cast<const float4*>(src + 4);
+    if (KG == 2) {
+      const float4 lo = *reinterpret_cast<const float4*>(src + MT * kMidEpiPitch);
+      const float4 hi = *reinterpret_cast<const float4*>(src + MT * kMidEpiPitch + 4);
+      v[0] += lo.x; v[1] += lo.y; v[2] += lo.z; v[3] += lo.w;
+      v[4] += hi.x; v[5] += hi.y; v[6] += hi.z; v[7] += hi.w;
+    }
+  };
   if (SPLIT) {
     // partial tile as fp32; ldw is a multiple of 8, so whole segments stay inside the row
     float* part = g.partial + (int64_t)blockIdx.y * g.M * g.ldw;
@@ -698,12 +727,11 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_mid16_kernel(GemmArgs g)
   if constexpr (!std::is_same<T, TO>::value) {
     float* __restrict__ Cw = reinterpret_cast<float*>(g.c);
     const bool rows16w = ((g.ldc & 3) == 0) && aligned16_dev(Cw) && (n0 + MT <= g.N);
-    for (int r0 = 0; r0 < MT; r0 += 16) {
+    for (int r0 = 0; r0 < MT; r0 += kSweepRows) {
       const int ml = r0 + rsub, m = m0 + ml;
       if (m >= g.M) continue;
       float v[8];
-      *reinterpret_cast<float4*>(v) = *reinterpret_cast<const float4*>(stage + ml * kMidEpiPitch + cseg);
-      *reinterpret_cast<float4*>(v + 4) = *reinterpret_cast<const float4*>(stage + ml * kMidEpiPitch + cseg + 4);
+      load8(ml, v);
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[e] = to_f32(from_f32<T>(v[e]));
       float* out = Cw + (int64_t)m * g.ldc + n0 + cseg;
@@ -722,12 +750,11 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_mid16_kernel(GemmArgs g)
   T* __restrict__ P = g.act != AT_ACT_NONE ? reinterpret_cast<T*>(g.pre_act) : nullptr;
   const bool rows16 = ((g.ldc & 7) == 0) && aligned16_dev(C) && (n0 + MT <= g.N) &&
                       (!P || (((g.ldp & 7) == 0) && aligned16_dev(P)));
-  for (int r0 = 0; r0 < MT; r0 += 16) {
+  for (int r0 = 0; r0 < MT; r0 += kSweepRows) {
     const int ml = r0 + rsub, m = m0 + ml;
     if (m >= g.M) continue;
     float v[8];
-    *reinterpret_cast<float4*>(v) = *reinterpret_cast<const float4*>(stage + ml * kMidEpiPitch + cseg);
-    *reinterpret_cast<float4*>(v + 4) = *reinterpret_cast<const float4*>(stage + ml * kMidEpiPitch + cseg + 4);
+    load8(ml, v);
     if (P) {
       T* out = P + (int64_t)m * g.ldp + n0 + cseg;
       if (rows16) {
@@ -1845,14 +1872,17 @@ enum Layout { kFwd = 0, kDx = 1, kDw = 2 };
 
 // Tile choice for a problem the 16-bit kernels can address.  One workgroup of the 256x256
 // kernel occupies a CU, so its time goes in whole rounds of one tile per CU; the 128x128 kernel
-// runs two workgroups per CU at about 65 % of the other's rate (measured: one round of 512
-// tiles takes 0.65 of a round of 256 large ones).
+// runs two workgroups per CU, a full round of 512 tiles taking about 0.7 of a round of 256 large
+// ones (measured over fourteen layer shapes, 0.65-0.74).  Its rounds are whole too — a last round
+// costs a round even when few tiles are left — unless that last round has at most one workgroup
+// per CU, which then has the CU to itself (0.6 of a round).
 inline bool prefer_mid_tiles(int64_t M, int64_t N) {
   const int64_t cus = device_cu_count();
   const double big = (double)cdiv64(cdiv64(M, BM) * cdiv64(N, BN), cus);
-  double mid = (double)(cdiv64(M, MT) * cdiv64(N, MT)) / (double)(2 * cus);
-  if (mid < 0.6) mid = 0.6;
-  return mid * 0.65 < big;
+  const int64_t tiles = cdiv64(M, MT) * cdiv64(N, MT);
+  const int64_t full = tiles / (2 * cus), rest = tiles - full * 2 * cus;
+  const double mid = 0.7 * ((double)full + (rest == 0 ? 0.0 : rest <= cus ? 0.6 : 1.0));
+  return mid < big;
 }
 
 // Number of splits of the contraction for the weight gradient (a [in, out] tile grid that is
@@ -1912,6 +1942,7 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
       splits = dw_split_count(M, N, K);
       if (workspace_bytes < (int64_t)splits * M * dw_partial_pitch(N) * 4) splits = 1;
     }
+    const bool two_groups = splits == 1 && (int64_t)grid <= device_cu_count() && cdiv64(K, BK) >= 4;
     return dispatch_dtype(in_dt, [&](auto* tp) -> int {
       typedef std::remove_pointer_t<decltype(tp)> T;
       if constexpr (std::is_same<T, float>::value) {
@@ -1930,6 +1961,14 @@ int run_gemm(Layout layout, const void* a, const void* b, void* c, void* pre_act
           else
             hipLaunchKernelGGL((gemm_split_finish_kernel<T>), dim3((unsigned)cdiv64(items, 256)), dim3(256), 0, stream,
                                (const float*)workspace, (T*)c, (int)M, (int)N, g.ldw, ldc, splits);
+        } else if (two_groups) {
+          // at most one tile per CU: eight waves per tile, two k-groups (see the kernel)
+#define AT_MID2(AMC, BKC, TOUT) \
+  hipLaunchKernelGGL((gemm_mid16_kernel<T, AMC, BKC, false, TOUT, 2>), dim3(grid), dim3(2 * kGemmThreads), 0, stream, g)
+          if (layout == kDx) { if (wide) AT_MID2(false, true, float); else AT_MID2(false, true, T); }
+          else if (layout == kDw) { if (wide) AT_MID2(true, false, float); else AT_MID2(true, false, T); }
+          else AT_MID2(false, false, T);
+#undef AT_MID2
         } else if (layout == kDx) {
           if (wide) hipLaunchKernelGGL((gemm_mid16_kernel<T, false, true, false, float>), dim3(grid), dim3(kGemmThreads), 0, stream, g);
           else hipLaunchKernelGGL((gemm_mid16_kernel<T, false, true, false>), dim3(grid), dim3(kGemmThreads), 0, stream, g);

@@ -106,6 +106,7 @@ HALF_DTYPES = [torch.float16, torch.bfloat16]
     ((2048, 512), 384),     # 128x128 tiles
     ((4096, 256), 256),     # 128x128 tiles, weight gradient split over the batch
     ((16384, 192), 320),    # split with a ragged last k-tile range
+    ((1000, 520), 776),     # 128x128 tiles, fewer than CUs: two k-groups per tile, an odd number of k-tiles
     # 256x256 tiles walked by a grid smaller than their number (each workgroup takes two), with
     # ragged last row and column tiles among full ones: forward, input gradient and weight
     # gradient in turn
@@ -387,6 +388,7 @@ def test_linear_under_autocast_with_fp32_parameters(shape, out_dim, act_func, am
     (2048, 512, 384),      # 128x128 tiles
     (300, 264, 520),       # generic kernel (small problem)
     (1000, 1000, 1000),
+    (1000, 520, 776),      # two k-groups per tile, an odd number of k-tiles
 ])
 def test_backward_products_write_fp32_like_a_cast_of_the_16bit_result(batch, in_dim, out_dim, dtype) -> None:
     """
