@@ -779,6 +779,269 @@ __global__ __launch_bounds__(256, 2) void conv_igemm_stationary_kernel(IgemmArgs
 }
 
 // ------------------------------------------------------------------------------------------
+// Forward / input-gradient kernel for channels-last 3x3 layers with stride 1 and padding 1 over 64
+// contraction channels: weights resident in registers, image rows in a ring of LDS slots.
+// ------------------------------------------------------------------------------------------
+// The image is cut into bands of 28 output columns and each band into steps of 8 output rows.  A
+// workgroup (4 waves = 2 halves of 64 output channels x 2 groups of 4 rows) walks down a range of
+// consecutive steps.  A 32-pixel MFMA operand is a piece of ONE image row (28 columns used), so the
+// fragment of input row y, column shift kw serves the taps (0, kw), (1, kw) and (2, kw) of the
+// output rows y + 1, y and y - 1: 72 fragment reads feed the 144 MFMAs of a wave and step, half of
+// what pixel tiles cut from the flattened image need.  Rows live in 18 slots of 30 pixels x 128
+// bytes (band + one neighbour column each side, zeros outside the image by way of out-of-range
+// loads): the 10 rows of the step being multiplied and the at most 8 or 9 new ones of the next
+// step, requested a whole step ahead; a step keeps the two bottom rows of the step before.  The
+// 16-byte chunks of a pixel are XORed with (pixel / 2) % 8, which spreads any 16 consecutive
+// pixels over all banks (no bank conflicts measured).  Rows above and below the image are never
+// loaded: their fragments are read from 128 bytes of zeros.  Outputs leave straight from the
+// accumulators (see the epilogue) as buffer stores with out-of-range offsets for what must not be
+// written, always 8 per wave and step: the in-order memory counter then lets the wave wait for its
+// row loads (issued before those stores) without waiting for the stores themselves.  One barrier
+// per step, no LDS staging of the output.
+constexpr int kRingBand = 28;                           // output columns per band
+constexpr int kRingCols = kRingBand + 2;                // window columns
+constexpr int kRingRow = kRingCols * 128;               // bytes per slot
+constexpr int kRingSlots = 18;
+constexpr int kRingStep = 8;                            // output rows per step
+constexpr int kRingRows = kRingSlots * kRingRow + 4 * 128;   // + what lanes 28..31 read past the last slot
+constexpr int kRingZero = kRingRows + CBN * 4;          // 128 bytes of zeros, 128-byte aligned
+constexpr int kRingLds = kRingZero + 128;
+constexpr int kRingRowChunks = kRingCols * 8;           // 16-byte chunks per slot
+constexpr int kRingStores = 8;                          // stores per wave and step
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+struct RingArgs {
+  int bands, steps_per_strip, total_steps;
+  int64_t out_bytes;
+  FastDiv div_steps, div_bands;
+};
+
+template <typename T>
+__device__ __forceinline__ uint2 pack4(const float (&v)[4]) {
+  union { uint2 raw; T e[4]; } u;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) u.e[e] = from_f32<T>(v[e]);
+  return u.raw;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256, 2) void conv_igemm_ring_kernel(IgemmArgs g, RingArgs ra) {
+  __shared__ __attribute__((aligned(1024))) char lds[kRingLds];
+  float* const bias_tile = reinterpret_cast<float*>(lds + kRingRows);
+  const int grp = blockIdx.z;
+  const int n0 = blockIdx.y * CBN;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int wn = wave & 1, wr = wave >> 1;
+
+  // Ranges of steps are cut in an order in which workgroups b and b + grid / 2 are neighbours:
+  // those two share a CU (the second half of the grid is placed once every CU has one workgroup,
+  // measurably later), and when the steps do not divide evenly the one that starts first gets the
+  // longer range.
+  const int half = (int)gridDim.x >> 1;   // the grid is even
+  const int bx = (int)blockIdx.x;
+  const int v = bx < half ? 2 * bx + 1 : 2 * (bx - half);
+  int q = (int)(((int64_t)v * ra.total_steps) / (int)gridDim.x);
+  const int q_end = (int)(((int64_t)(v + 1) * ra.total_steps) / (int)gridDim.x);
+  if (q >= q_end) return;
+
+  auto decode = [&](int qq, int& n, int& b, int& s) {
+    const int strip = fast_div(qq, ra.div_steps);
+    s = qq - strip * ra.steps_per_strip;
+    n = fast_div(strip, ra.div_bands);
+    b = strip - n * ra.bands;
+  };
+  const i32x4 rin = make_buffer_rsrc(g.act, g.act_bytes);
+
+  // Requests the rows step qq needs and the step before it (same strip) does not hold; `fresh`:
+  // nothing is held.  Returns the strip's anchor: image row r lives in slot (anchor + r) % 18.
+  int next_slot = 0;
+  auto issue_rows = [&](int qq, bool fresh, int anchor_prev) -> int {
+    int n, b, s;
+    decode(qq, n, b, s);
+    const int y0 = s * kRingStep;
+    const int r_hi = y0 + kRingStep < g.IH ? y0 + kRingStep : g.IH - 1;
+    int r_lo, anchor;
+    if (fresh || s == 0) {
+      r_lo = y0 > 0 ? y0 - 1 : 0;
+      anchor = ((next_slot - r_lo) % kRingSlots + kRingSlots) % kRingSlots;
+    } else {
+      r_lo = y0 + 1;
+      anchor = anchor_prev;
+    }
+    // what a lane fetches of a row: LDS chunk c = 64 j + lane is position c % 8 of window pixel
+    // c / 8 and holds the pixel's chunk (c % 8) ^ (pixel / 2) % 8.  Recomputed per call on purpose
+    // (the empty asm hides that only the band changes): kept across the main loop it would take
+    // registers from it.
+    int lane_v = lane;
+    asm volatile("" : "+v"(lane_v));
+    int loff[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = j * 64 + lane_v;
+      const int px = c >> 3, chunk = (c ^ (px >> 1)) & 7;
+      const int col = b * kRingBand + px - 1;
+      const bool ok = px < kRingCols && (unsigned)col < (unsigned)g.IW;
+      loff[j] = ok ? (px - 1) * g.Ctot * 2 + chunk * 16 : kOobOffset;
+    }
+    for (int r = r_lo + wave; r <= r_hi; r += 4) {
+      const int slot = (anchor + r) % kRingSlots;
+      const unsigned row_off = (unsigned)((((n * g.IH + r) * g.IW + b * kRingBand) * g.Ctot + grp * g.Cg) * 2);
+      char* const dst = lds + slot * kRingRow;
+#pragma unroll
+      for (int j = 0; j < 3; ++j) lds_dma_16(rin, (int)((unsigned)loff[j] + row_off), dst + j * 1024);
+      if (lane_v < kRingRowChunks - 192) lds_dma_16(rin, (int)((unsigned)loff[3] + row_off), dst + 3072);
+    }
+    if (r_hi >= r_lo) next_slot = (anchor + r_hi + 1) % kRingSlots;
+    return anchor;
+  };
+
+  int anchor_cur = issue_rows(q, true, 0);
+  if (threadIdx.x < 32) reinterpret_cast<uint32_t*>(lds + kRingZero)[threadIdx.x] = 0u;
+  if (g.bias && threadIdx.x < CBN)
+    bias_tile[threadIdx.x] =
+        n0 + (int)threadIdx.x < g.Og ? load_scalar_f32(g.bias, g.bias_dt, grp * g.Og + n0 + threadIdx.x) : 0.f;
+
+  // this wave's weights: fragment-major, 36 fragments of 64 lanes x 16 bytes
+  const int ntiles32 = (g.Og + 31) >> 5;
+  const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(
+      g.wf, 0, (int)((int64_t)gridDim.z * ntiles32 * g.K * 64), 0x00020000);
+  const int wrow = ((grp * ntiles32 + (n0 >> 5) + wn) * (g.K >> 4)) * 1024 + lane * 16;
+  uint4 wreg[36];
+#pragma unroll
+  for (int i = 0; i < 36; ++i)
+    wreg[i] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rw, wrow, i * 1024, 0));
+  const __amdgpu_buffer_rsrc_t rout = __builtin_amdgcn_make_buffer_rsrc(g.out, 0, (int)ra.out_bytes, 0x00020000);
+  const int Otot = g.Og * (int)gridDim.z;
+
+  bool first = true;
+  for (; q < q_end; ++q) {
+    int n, b, s;
+    decode(q, n, b, s);
+    // the rows of this step were requested before the stores of the step before
+    if (first) lds_dma_wait_all();
+    else lds_dma_wait_newest<kRingStores>();
+    __syncthreads();   // everybody's rows are there; nobody reads the rows of the step before any more
+    int anchor_next = anchor_cur;
+
+    const int y = s * kRingStep + wr * 4;   // this wave's first output row
+    // fragment address of (input row i, column shift kw, k-step kc): (row_base[i] + t[kw]) ^ (kc << 5);
+    // the row bases are wave-uniform and multiples of 128, the XOR only touches bits 5-6.  A row
+    // above or below the image reads the 128 zero bytes instead (every lane the same 16).
+    int row_base[6], t[3];
+    bool inside[6];
+    {
+      int lane_v = lane;
+      asm volatile("" : "+v"(lane_v));
+#pragma unroll
+      for (int kw = 0; kw < 3; ++kw) {
+        const int px = (lane_v & 31) + kw;
+        t[kw] = px * 128 + ((((lane_v >> 5) ^ (px >> 1)) & 7) << 4);
+      }
+#pragma unroll
+      for (int i = 0; i < 6; ++i) {
+        const int r = y - 1 + i;
+        inside[i] = (unsigned)r < (unsigned)g.IH;
+        row_base[i] = ((anchor_cur + (inside[i] ? r : 0)) % kRingSlots) * kRingRow;
+      }
+    }
+    f32x16 acc[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[r][e] = 0.f;
+
+    // fragment f = (input row i, column shift kw, k-step kc), fetched three fragments ahead
+    {
+      constexpr int kFrags = 72, kAhead = 3, kSplit = 12;
+      uint4 af[kAhead + 1];
+      auto fetch = [&](int f) {
+        const int i = f / 12, kw = (f % 12) / 4, kc = f % 4;
+        const int at = inside[i] ? row_base[i] + t[kw] : kRingZero;
+        af[f % (kAhead + 1)] = *reinterpret_cast<const uint4*>(lds + (at ^ (kc << 5)));
+      };
+#pragma unroll
+      for (int f = 0; f < kAhead; ++f) fetch(f);
+      auto run = [&](auto from, auto to) {
+#pragma unroll
+        for (int f = decltype(from)::value; f < decltype(to)::value; ++f) {
+          __builtin_amdgcn_sched_barrier(0);
+          if (f + kAhead < kFrags) fetch(f + kAhead);
+          const int i = f / 12, kw = (f % 12) / 4, kc = f % 4;
+          const uint4 a = af[f % (kAhead + 1)];
+#pragma unroll
+          for (int kh = 0; kh < 3; ++kh) {
+            const int r = i - kh;
+            if (r < 0 || r > 3) continue;
+            // operands this way round: a lane ends up with 4 consecutive channels of one pixel
+            acc[r] = Mfma16<T>::run(wreg[(kh * 3 + kw) * 4 + kc], a, acc[r]);
+          }
+        }
+      };
+      // the next step's rows are requested behind the first MFMAs, whose run time covers the address
+      // arithmetic of the requests
+      run(std::integral_constant<int, 0>{}, std::integral_constant<int, kSplit>{});
+      __builtin_amdgcn_sched_barrier(0);
+      if (q + 1 < q_end) anchor_next = issue_rows(q + 1, false, anchor_cur);
+      run(std::integral_constant<int, kSplit>{}, std::integral_constant<int, kFrags>{});
+    }
+
+    // ---- outputs ----
+    // A lane holds channels rg*8 + (lane/32)*4 .. +3 of pixel lane % 32 of each of its 4 rows.
+    // Exchanging the packed values of an even and an odd register group between the two halves
+    // of the wave (v_permlane32_swap) leaves lane (pixel, 0) with channels 16 p .. 16 p + 7 and
+    // lane (pixel, 1) with 16 p + 8 .. 16 p + 15: 16 bytes per lane, 32 contiguous bytes per pixel
+    // and store, without a trip through LDS.
+    {
+      int lane_v = lane;
+      asm volatile("" : "+v"(lane_v));
+      const int ch0 = wn * 32 + (lane_v >> 5) * 4;
+      float bv[4][4];
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        float4 t4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (g.bias) t4 = *reinterpret_cast<const float4*>(bias_tile + ch0 + rg * 8);
+        bv[rg][0] = t4.x; bv[rg][1] = t4.y; bv[rg][2] = t4.z; bv[rg][3] = t4.w;
+      }
+      const int x = lane_v & 31, xg = b * kRingBand + x;
+      const int chs = wn * 32 + (lane_v >> 5) * 8;   // + 16 p: first of the lane's 8 channels after the exchange
+      bool ook[2];
+      unsigned ooff[2];
+#pragma unroll
+      for (int p = 0; p < 2; ++p) {
+        ook[p] = x < kRingBand && xg < g.OW && n0 + chs + 16 * p < g.Og;
+        ooff[p] = (unsigned)(((n * g.IH) * g.OW + xg) * Otot + grp * g.Og + n0 + chs + 16 * p) * 2u;
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const bool row_ok = y + r < g.IH;
+        const unsigned row_off = (unsigned)((y + r) * g.OW * Otot * 2);
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+          uint2 part[2];
+#pragma unroll
+          for (int k = 0; k < 2; ++k) {
+            const int rg = 2 * p + k;
+            float o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = acc[r][rg * 4 + e] + bv[rg][e];
+            part[k] = pack4<T>(o);
+          }
+          const auto sx = __builtin_amdgcn_permlane32_swap(part[0].x, part[1].x, false, false);
+          const auto sy = __builtin_amdgcn_permlane32_swap(part[0].y, part[1].y, false, false);
+          u32x4 d;
+          d[0] = sx[0]; d[1] = sy[0]; d[2] = sx[1]; d[3] = sy[1];
+          __builtin_amdgcn_raw_buffer_store_b128(d, rout, ook[p] && row_ok ? (int)(ooff[p] + row_off) : kOobOffset, 0, 0);
+        }
+      }
+    }
+    anchor_cur = anchor_next;
+    first = false;
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // Weight-gradient kernel.
 // ------------------------------------------------------------------------------------------
 // Operand tile in LDS: 64 pixel rows x 128 bytes (64 channels) as loaded, the 16-byte chunk
@@ -1288,13 +1551,31 @@ int run_igemm(IgemmArgs g, const void* w, const ConvProblem& p, int flip, int cg
     const int64_t tiles_m = cdiv64(g.M, CBM);
     const int stat_grid = device_cu_count() * 2 / 8 * 8;
     const bool stationary = resident && g.tiles_per_tap == 1 && g.KT == 9 && stat_grid >= 8 && tiles_m >= 4 * stat_grid;
-    if (resident) {
+    // rows in a ring of LDS slots: channels-last 3x3 layers with stride 1 and padding 1, bands of 28
+    // columns that waste little of the 32-pixel operands, and at least one step of 8 rows for
+    // every resident workgroup
+    RingArgs ra{};
+    ra.bands = (int)cdiv64(g.IW, kRingBand);
+    ra.steps_per_strip = (int)cdiv64(g.IH, kRingStep);
+    const int64_t ring_steps = n_img * ra.bands * ra.steps_per_strip;
+    const bool ring = g.out_last && g.tiles_per_tap == 1 && g.KT == 9 && g.KW == 3 && g.sh == 1 && g.sw == 1 &&
+                      g.ph == 1 && g.pw == 1 && OH == g.IH && g.OW == g.IW && stat_grid >= 8 &&
+                      ring_steps >= stat_grid && ring_steps < INT32_MAX && g.IW * 5 >= ra.bands * 32 * 4 &&
+                      g.Og % 8 == 0 && (reinterpret_cast<uintptr_t>(g.out) & 15u) == 0;
+    if (resident || ring) {
       const int ntiles = (g.Og + 31) / 32;
       const int64_t chunks = (int64_t)groups * ntiles * (g.K / 16) * 64;
       hipLaunchKernelGGL((conv_weight_frags_direct_kernel<T>), dim3((unsigned)cdiv64(chunks, 256)), dim3(256), 0,
                          stream, (const T*)w, (T*)g.wf, cg_real, g.Cg, g.Og, (int)(p.KH * p.KW), flip, ntiles,
                          chunks);
-      if (stationary) {
+      if (ring) {
+        ra.total_steps = (int)ring_steps;
+        ra.out_bytes = (int64_t)g.M * g.Og * groups * 2;
+        ra.div_steps = make_fastdiv(ra.steps_per_strip);
+        ra.div_bands = make_fastdiv(ra.bands);
+        const dim3 rgrid((unsigned)stat_grid, (unsigned)g.nbn, (unsigned)groups);
+        hipLaunchKernelGGL((conv_igemm_ring_kernel<T>), rgrid, dim3(256), 0, stream, g, ra);
+      } else if (stationary) {
         const dim3 sgrid((unsigned)stat_grid, (unsigned)g.nbn, (unsigned)groups);
         if (g.out_last)
           hipLaunchKernelGGL((conv_igemm_stationary_kernel<T, true, 9>), sgrid, dim3(256), 0, stream, g, (int)tiles_m);

@@ -164,6 +164,8 @@ def test_conv_matrix_core_path_agrees_with_generic_kernel(dtype) -> None:
     (90, 64, 55, 55, 128, 1, 1, True),     # last tile partly empty, two channel tiles
     (96, 128, 56, 56, 128, 1, 2, False),   # two groups
     (100, 64, 57, 57, 40, 1, 1, True),     # element stores, channel tile partly empty
+    (128, 64, 56, 56, 64, 1, 1, True),     # the benchmark's layer at its batch size
+    (140, 64, 30, 84, 40, 1, 1, False),    # wide, short images; channel tile partly empty
 ])
 def test_conv_window_kernel_agrees_with_generic_kernel_at_size(n, c, h, w, o, pad, groups, bias, dtype) -> None:
     """
@@ -381,6 +383,11 @@ CHANNELS_LAST_CASES = [
     ((2, 128, 9, 8), 64, (1, 1), (1, 1), (0, 0), 1),
     ((1, 64, 12, 10), 64, (5, 3), (1, 1), (2, 0), 1),
     ((2, 32, 14, 14), 64, (3, 3), (1, 1), (1, 1), 1),      # 32 input channels: the forward product falls back
+    # enough steps of 8 rows x 28 columns for every resident workgroup: image rows in a ring of LDS slots
+    ((74, 64, 56, 28), 64, (3, 3), (1, 1), (1, 1), 1),     # one band
+    ((44, 64, 30, 84), 48, (3, 3), (1, 1), (1, 1), 1),     # three bands, 6 rows in the last step, 48 output channels
+    ((30, 64, 57, 52), 72, (3, 3), (1, 1), (1, 1), 1),     # last band 24 columns, one row in the last step, two channel tiles
+    ((38, 128, 56, 56), 128, (3, 3), (1, 1), (1, 1), 2),   # two groups
 ]
 
 
@@ -447,7 +454,8 @@ def test_channel_sum(batch, feat, spatial, dtype) -> None:
     assert_close(out, x.double().sum((0, 2)).cpu(), dtype, 'channel sum', batch_reduction=True)
 
 
-@pytest.mark.parametrize('shape, out_dim, bias', [((88, 64, 56, 56), 64, True), ((90, 64, 55, 55), 40, False)])
+@pytest.mark.parametrize('shape, out_dim, bias', [((88, 64, 56, 56), 64, True), ((90, 64, 55, 55), 40, False),
+                                                  ((128, 64, 56, 56), 64, True), ((100, 64, 57, 56), 40, False)])
 def test_conv2d_weights_resident_kernel_same_on_both_layouts(shape, out_dim, bias) -> None:
     # batch sizes at which a workgroup walks over several tiles with the weights in registers
     dtype = torch.bfloat16
