@@ -23,6 +23,8 @@ P, I, L, F, U = c_void_p, c_int, c_int64, c_float, ctypes.c_uint32
 PROTOTYPES = {
     'at_version': (I, []),
     'at_error_string': (ctypes.c_char_p, [I]),
+    'at_mfma_probe': (I, [L, I, P, P]),
+    'at_mfma_probe_flop': (L, [L]),
     'at_rms_norm_fwd': (I, [P, P, P, P, L, L, L, L, F, I, I, I, P]),
     'at_rms_norm_bwd': (I, [P, P, P, P, P, P, P, L, L, L, L, L, L, I, I, I, I, P]),
     'at_norm_bwd_workspace_bytes': (L, [L, L, I]),

@@ -1196,6 +1196,31 @@ def bench_conv_bn(steps: int, warmup: int, with_cpu: bool) -> List[Dict]:
     return [conv_entry, conv_last_entry, bn_entry, bn_last_entry]
 
 
+def mfma_probe() -> Dict:
+    """
+    What the matrix cores sustain without any memory traffic (at_mfma_probe: bf16 32x32x16 MFMAs
+    back to back on every CU, operands in registers), once with a constant operand pair and once
+    with operands that change from MFMA to MFMA as in a real product.  The second figure is the
+    ceiling an MFMA-bound kernel on real data can reach on this device (it is power-limited); the
+    first reaches the published peak.  Median of 5 launches of about 10 ms each.
+    """
+    from attorch_amd import _lib
+    lib = _lib.load()
+    scratch = torch.zeros(4, dtype=torch.uint8, device='cuda')
+    stream = torch.cuda.current_stream().cuda_stream
+    iters = 4000
+    flop = lib.at_mfma_probe_flop(iters)
+    out = {}
+    for name, rnd in (('constant_operands', 0), ('changing_operands', 1)):
+        def launch() -> None:
+            _lib.check(lib.at_mfma_probe(iters, rnd, scratch.data_ptr(), stream), 'at_mfma_probe')
+        ms = gpu_time_ms(launch, 1, 2, 5)
+        out[name] = flop / ms / 1e9
+    return {'unit': 'TFLOP/s', 'tflops_constant_operands': out['constant_operands'],
+            'tflops_changing_operands': out['changing_operands'],
+            'note': 'bf16 MFMA 32x32x16 from registers, no memory traffic; changing operands = ceiling for real data'}
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
@@ -1218,6 +1243,8 @@ def main() -> int:
         torch.cuda.synchronize()
         del src, dst
     head = bench_linear('c4', args.steps, args.warmup, with_cpu)
+    head['mfma_probe'] = mfma_probe()
+    head['frac_of_mfma_probe_step'] = head['value'] / head['mfma_probe']['tflops_changing_operands']
     extra: List[Dict] = []
     wanted = [] if args.configs == 'none' else args.configs.split(',')
     if 'c1' in wanted:
@@ -1242,6 +1269,8 @@ def main() -> int:
         'frac_of_peak_step': head['frac_of_peak_step'],
         'kernel_ms': head['kernel_ms'], 'kernel_tflops': head['kernel_tflops'],
         'amp': head.get('amp'),
+        'mfma_probe': head.get('mfma_probe'),
+        'frac_of_mfma_probe_step': head.get('frac_of_mfma_probe_step'),
         'configs': extra,
     }
     # Everything measured goes to a file (--detail-file, by default gpurun_out/bench_detail.json
@@ -1302,6 +1331,13 @@ def compact_line(args, head: Dict, extra: List[Dict]) -> Dict:
     }
     if head.get('amp') is not None:
         line['amp'] = head['amp']
+    if head.get('mfma_probe') is not None:
+        probe = head['mfma_probe']
+        line['mfma_probe'] = {'unit': 'TFLOP/s', 'constant_operands': _r(probe['tflops_constant_operands']),
+                              'changing_operands': _r(probe['tflops_changing_operands']),
+                              'step_over_changing': _r(head['frac_of_mfma_probe_step']),
+                              'note': 'register-resident bf16 MFMAs, no memory traffic: the device sustains the '
+                                      'published peak only with constant operands'}
     return line
 
 

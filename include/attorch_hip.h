@@ -76,6 +76,17 @@ int at_version(void);
 /* Static description of a return code of this library (never null). */
 const char* at_error_string(int code);
 
+/* Measurement aid with no counterpart in the reference: v_mfma_f32_32x32x16_bf16 back to back on
+ * every CU (two workgroups of four waves each), operands and accumulators in registers, no memory
+ * traffic.  random_operands != 0: the operands are pseudo-random values in [-1, 1) that change
+ * from one MFMA to the next, as in a real product; 0: one constant pair.  The caller times the
+ * launch; at_mfma_probe_flop(iters) is the arithmetic it performs.  scratch4: 4 writable bytes of
+ * device memory (never written in practice).  The rate with changing operands is what the matrix
+ * cores of this device sustain under their power limit; the nominal peak is only reached with
+ * constant operands. */
+int at_mfma_probe(int64_t iters, int random_operands, void* scratch4, at_stream_t stream);
+int64_t at_mfma_probe_flop(int64_t iters);
+
 /* ------------------------------------------------------------------------------------------
  * RMSNorm — replaces rms_norm_forward_kernel / rms_norm_backward_kernel,
  * attorch/rms_norm_kernels.py:21-88 and :98-193, launched from attorch/rms_norm_layer.py:68-75
