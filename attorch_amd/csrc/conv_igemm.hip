@@ -1191,7 +1191,7 @@ __global__ __launch_bounds__(256) void conv_dw_kernel(DwArgs g) {
 constexpr int kRowsWinMax = 208;                              // window pixels at most
 constexpr int kRowsSlots = 36;                                // wave-wide loads per k-tile: 8 + 26 + 2 spare
 constexpr int kRowsStage = kRowsSlots * 1024;                 // dY tile, then the window (+ spare rows)
-constexpr int kRowsStages = 4;                                // k-tiles in LDS: one multiplied, three in flight
+constexpr int kRowsStages = 4;                                // k-tiles in LDS: a pair multiplied, a pair in flight
 
 struct DwRowsArgs {
   const void* dy;     // [N*OH*OW][Otot]
@@ -1315,30 +1315,37 @@ __global__ __launch_bounds__(kRowsWaves * 64) void conv_dw_rows_kernel(DwRowsArg
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][t][e] = 0.f;
 
-#pragma unroll
-  for (int d = 0; d < kRowsStages - 1; ++d) issue(t_begin + d, lds + d * kRowsStage);
+  // k-tiles are multiplied in pairs between barriers: while the pair in stages {0, 1} (or {2, 3}) is
+  // multiplied, the next pair travels into the other two stages.  One barrier, one wait for loads
+  // and one ramp-up of the fragment reads per two k-tiles.
+  issue(t_begin, lds);
+  issue(t_begin + 1, lds + kRowsStage);
   typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-  for (int t = t_begin; t < t_end; ++t) {
-    const int st = (t - t_begin) % kRowsStages;
-    // loads are answered in order: all but the two younger k-tiles' loads of this wave are done
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kRowsStages - 2) * (kRowsSlots / kRowsWaves)) : "memory");
-    __syncthreads();   // k-tile t is in LDS for everybody, and nobody reads k-tile t - 1 any more
-    issue(t + kRowsStages - 1, lds + ((st + kRowsStages - 1) % kRowsStages) * kRowsStage);
-    const char* cur = lds + st * kRowsStage;
-    auto frag = [&](const int (&rel)[2]) {
-      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(cur + rel[0]));
-      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(cur + rel[1]));
-      const uint2 x0 = __builtin_bit_cast(uint2, lo), x1 = __builtin_bit_cast(uint2, hi);
-      return make_uint4(x0.x, x0.y, x1.x, x1.y);
-    };
+  for (int t = t_begin; t < t_end; t += 2) {
+    const int half = ((t - t_begin) >> 1) & 1;
+    lds_dma_wait_all();
+    __syncthreads();   // this pair is in LDS for everybody, and nobody reads the pair before any more
+    issue(t + 2, lds + ((half ^ 1) * 2) * kRowsStage);
+    issue(t + 3, lds + ((half ^ 1) * 2 + 1) * kRowsStage);
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-      const uint4 a0 = frag(a_rel[kk][0]), a1 = frag(a_rel[kk][1]);
+    for (int u = 0; u < 2; ++u) {
+      if (t + u >= t_end) break;   // uniform
+      const char* cur = lds + (half * 2 + u) * kRowsStage;
+      auto frag = [&](const int (&rel)[2]) {
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(cur + rel[0]));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(cur + rel[1]));
+        const uint2 x0 = __builtin_bit_cast(uint2, lo), x1 = __builtin_bit_cast(uint2, hi);
+        return make_uint4(x0.x, x0.y, x1.x, x1.y);
+      };
 #pragma unroll
-      for (int kw = 0; kw < 3; ++kw) {
-        const uint4 b = frag(b_rel[kk][kw]);
-        acc[0][kw] = Mfma16<T>::run(a0, b, acc[0][kw]);
-        acc[1][kw] = Mfma16<T>::run(a1, b, acc[1][kw]);
+      for (int kk = 0; kk < 2; ++kk) {
+        const uint4 a0 = frag(a_rel[kk][0]), a1 = frag(a_rel[kk][1]);
+#pragma unroll
+        for (int kw = 0; kw < 3; ++kw) {
+          const uint4 b = frag(b_rel[kk][kw]);
+          acc[0][kw] = Mfma16<T>::run(a0, b, acc[0][kw]);
+          acc[1][kw] = Mfma16<T>::run(a1, b, acc[1][kw]);
+        }
       }
     }
   }

@@ -49,3 +49,33 @@ def test_layers_run_on_the_current_stream() -> None:
     side.synchronize()
     for e, g in zip(expected, got):
         torch.testing.assert_close(g, e, rtol=0, atol=0)
+
+
+def test_matrix_core_probe_runs_and_counts_its_work() -> None:
+    """
+    at_mfma_probe launches on the given stream and returns; at_mfma_probe_flop is 2 workgroups x 4
+    waves per CU x iters x 64 MFMAs of 32 x 32 x 16.  Changing operands must not come out faster
+    than a constant pair by more than measurement noise.
+    """
+    from attorch_amd import _lib
+    lib = _lib.load()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    iters = 500
+    assert lib.at_mfma_probe_flop(iters) == cus * 2 * 4 * iters * 64 * 2 * 32 * 32 * 16
+    assert lib.at_mfma_probe_flop(0) == 0
+    scratch = torch.zeros(4, dtype=torch.uint8, device='cuda')
+    stream = torch.cuda.current_stream().cuda_stream
+    assert lib.at_mfma_probe(iters, 0, None, stream) == -1          # null scratch
+    assert lib.at_mfma_probe(0, 0, scratch.data_ptr(), stream) == -2
+    times = []
+    for rnd in (0, 1):
+        for _ in range(2):
+            _lib.check(lib.at_mfma_probe(iters, rnd, scratch.data_ptr(), stream), 'probe')
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        _lib.check(lib.at_mfma_probe(iters, rnd, scratch.data_ptr(), stream), 'probe')
+        end.record()
+        torch.cuda.synchronize()
+        times.append(start.elapsed_time(end))
+    assert scratch.sum().item() == 0
+    assert times[1] > 0.9 * times[0]
