@@ -201,7 +201,9 @@ class LinearAutoGrad(torch.autograd.Function):
                 and weight.dtype is torch.float32 and (pre_act is None or pre_act.dtype is torch.float32)
                 and lib.at_linear_bwd_small_supported(batch_dim, in_feat_dim, out_feat_dim,
                                                       _lib.dtype_id(torch.float32))):
-            # small fp32 layer: activation gradient, both products and the bias sum in one launch
+            # small fp32 layer: activation gradient, both products and the bias sum in one launch.
+            # The kernel always forms the weight gradient (a workgroup's tile of it is what its
+            # waves share), so a frozen weight takes the separate launches below instead.
             input_mm, weight_mm = _matrix(flattened_input), _matrix(weight)
             pre_act_mm = None if ctx.act_func is None else _matrix(pre_act)
             operands = [output_grad, input_mm, weight_mm] + ([] if pre_act_mm is None else [pre_act_mm])
