@@ -574,7 +574,7 @@ int at_channel_sum(const void* x, void* out, int64_t batch, int64_t feat, int64_
  * act = AT_ACT_NONE gives plain dropout (input may then be null in bwd).  drop_p = 0 disables
  * dropout (pass 0 outside training).  A dropped element is exactly zero, kept ones are scaled
  * by 1 / (1 - drop_p) (dropout_kernels.py:26-27).  The mask is a pure function of (seed,
- * element index) — Philox4x32-10 (16 bits per element), not Triton's generator, so masks differ from the
+ * element index) — Philox4x32-7 (16 bits per element), not Triton's generator, so masks differ from the
  * reference's for equal seeds; forward and backward of one call pair agree.
  * ------------------------------------------------------------------------------------------ */
 int at_act_dropout_fwd(const void* input, void* output, int64_t size, int act, float param,
