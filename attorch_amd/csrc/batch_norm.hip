@@ -137,50 +137,51 @@ __global__ __launch_bounds__(kBnBlock) void bn_stats_kernel(const T* __restrict_
   }
 }
 
-// Statistics of channel c for an apply workgroup.  Every thread of the workgroup calls this.
-//   part != nullptr: wave 0 merges the P partial (count, mean, M2) triples with three sums over the
-//     wave (total count; count-weighted mean; M2 plus count * squared distance of each partial
-//     mean from the merged one) — the same order in every workgroup, so all of them get the same
-//     bits — and the result travels through LDS; `count` receives the number of elements.
+// Statistics of channel c for an apply workgroup.  Every thread calls this.
+//   part != nullptr: every wave merges the P partial (count, mean, M2) triples by itself with three
+//     sums over its lanes (total count; count-weighted mean; M2 plus count * squared distance of
+//     each partial mean from the merged one) — the same order in every wave of every workgroup, so
+//     all of them get the same bits, and no barrier or LDS is needed; `count` receives the number
+//     of elements.
 //   part == nullptr: the running statistics (evaluation mode).
 __device__ __forceinline__ void channel_stats(const float* __restrict__ part, int P, int c,
                                               const void* __restrict__ running_mean,
-                                              const void* __restrict__ running_var, int rdt,
-                                              float* smem /* 4 floats */, float& mean, float& var, float& count) {
+                                              const void* __restrict__ running_var, int rdt, float& mean,
+                                              float& var, float& count) {
   if (!part) {
     mean = load_scalar_f32(running_mean, rdt, c);
     var = load_scalar_f32(running_var, rdt, c);
     count = 0.f;
     return;
   }
-  __syncthreads();   // previous readers of smem are done
-  if (threadIdx.x < 64) {
-    float n = 0.f, nm = 0.f;
-    for (int p = threadIdx.x; p < P; p += 64) {
-      const float* src = part + ((int64_t)c * P + p) * 3;
-      n += src[0];
-      nm += src[0] * src[1];
+  const int lane = threadIdx.x & 63;
+  // the lane's first triple stays in registers for the second sum (with up to 64 splits nothing
+  // is read twice)
+  float n = 0.f, nm = 0.f, first[3] = {0.f, 0.f, 0.f};
+  for (int p = lane; p < P; p += 64) {
+    const float* src = part + ((int64_t)c * P + p) * 3;
+    const float pn = src[0], pm = src[1], pq = src[2];
+    if (p == lane) {
+      first[0] = pn; first[1] = pm; first[2] = pq;
     }
-    n = wave_reduce(n, 64, SumOp());
-    nm = wave_reduce(nm, 64, SumOp());
-    const float m = nm / n;
-    float m2 = 0.f;
-    for (int p = threadIdx.x; p < P; p += 64) {
-      const float* src = part + ((int64_t)c * P + p) * 3;
-      const float d = src[1] - m;
-      m2 += src[2] + src[0] * d * d;
-    }
-    m2 = wave_reduce(m2, 64, SumOp());
-    if (threadIdx.x == 0) {
-      smem[0] = m;
-      smem[1] = m2 / n;
-      smem[2] = n;
-    }
+    n += pn;
+    nm += pn * pm;
   }
-  __syncthreads();
-  mean = smem[0];
-  var = smem[1];
-  count = smem[2];
+  n = wave_reduce(n, 64, SumOp());
+  nm = wave_reduce(nm, 64, SumOp());
+  const float m = nm / n;
+  float m2 = 0.f;
+  for (int p = lane; p < P; p += 64) {
+    const float* src = part + ((int64_t)c * P + p) * 3;
+    const bool cached = p == lane;
+    const float pn = cached ? first[0] : src[0], pm = cached ? first[1] : src[1], pq = cached ? first[2] : src[2];
+    const float d = pm - m;
+    m2 += pq + pn * d * d;
+  }
+  m2 = wave_reduce(m2, 64, SumOp());
+  mean = m;
+  var = m2 / n;
+  count = n;
 }
 
 // y = act(w * (x - mean) * inv_std + b (+ residual)); one workgroup per slice of a plane.
@@ -194,7 +195,6 @@ __global__ __launch_bounds__(kBnBlock) void bn_apply_kernel(
     void* __restrict__ running_mean, void* __restrict__ running_var, int rdt, int update_running,
     float momentum, float eps, const void* __restrict__ w, const void* __restrict__ b, int wdt, int C, int S,
     float param, int64_t total_planes) {
-  __shared__ float smem[4];
   const int sp = S / VEC;
   const int step = gridDim.y * kBnBlock;
   for (int64_t plane = blockIdx.x; plane < total_planes; plane += gridDim.x) {
@@ -218,7 +218,7 @@ __global__ __launch_bounds__(kBnBlock) void bn_apply_kernel(
     };
     issue(i0 < sp ? i0 : 0);
     float mean, var, count;
-    channel_stats(part, P, c, running_mean, running_var, rdt, smem, mean, var, count);
+    channel_stats(part, P, c, running_mean, running_var, rdt, mean, var, count);
     const float inv_std = rsqrtf(var + eps);
     if (plane < C && blockIdx.y == 0 && threadIdx.x == 0) {
       if (mean_out) mean_out[c] = mean;
@@ -561,10 +561,9 @@ __global__ __launch_bounds__(64) void bn_last_finalize_kernel(
     const float* __restrict__ part, int P, float* __restrict__ stat, float* __restrict__ mean_out,
     float* __restrict__ inv_std_out, void* __restrict__ running_mean, void* __restrict__ running_var, int rdt,
     int update_running, float momentum, float eps, int C) {
-  __shared__ float smem[4];
   const int c = blockIdx.x;
   float mean, var, count;
-  channel_stats(part, P, c, running_mean, running_var, rdt, smem, mean, var, count);
+  channel_stats(part, P, c, running_mean, running_var, rdt, mean, var, count);
   if (threadIdx.x != 0) return;
   const float inv_std = rsqrtf(var + eps);
   stat[c] = mean;

@@ -511,7 +511,6 @@ constexpr int MT = 128;                          // tile edge
 constexpr int kMidTileBytes = MT * BK * 2;       // one operand tile, 16 KiB
 constexpr int kMidStage = 2 * kMidTileBytes;
 constexpr int kMidEpiPitch = MT + 4;             // floats per row of the staged output tile
-constexpr int kMidLds = 2 * kMidStage > MT * kMidEpiPitch * 4 ? 2 * kMidStage : MT * kMidEpiPitch * 4;
 
 // LDS image of an operand tile stored [k][outer] in memory: 64 k-rows x 256 bytes as loaded,
 // four rows per KiB (one wave-wide load), the 16-byte chunk index XORed with 4 * (k-row % 4) so
@@ -1214,7 +1213,6 @@ struct SplitShape {
 // wave 0's reads of the fold area, so wave 0 alone may go on using smem.
 template <bool A_MC, bool B_KC, int TK, int DZ, bool COLSUM>
 __device__ __forceinline__ f32x16 split_tile(const SplitTile& t, float* smem, float* colsum_out) {
-  constexpr int TM = 32;
   constexpr int NV = TK * 8 / kSplitThreads;   // 16-byte vectors per lane, operand and k-tile
   static_assert(NV >= 1 && (TK / 2) % kSplitWaves == 0, "k-tile too small for the workgroup");
   static_assert(!COLSUM || (DZ == 2 && !B_KC && TK % 16 == 0), "column sums are taken from a [k][n] tile");
