@@ -109,7 +109,7 @@ __global__ __launch_bounds__(kBnBlock) void bn_stats_kernel(const T* __restrict_
   __shared__ Welford smem[kBnBlock / 64];
   const int c = blockIdx.x, p = blockIdx.y;
   Welford acc{0.f, 0.f, 0.f};
-  constexpr int U = 4;
+  constexpr int U = 8;   // all of a workgroup's chunks in one round of loads at the usual sizes
   RawVec<T, VEC> raw[U];
   for_channel_chunks_batched<VEC, U>(
       c, p, P, N, C, S, [&](int u, int64_t off) { raw[u].load(x + off); },
