@@ -46,22 +46,22 @@ PEAK_MFMA_FP32_TFLOPS = 157.3    # dense fp32 MFMA
 # the 256 MB Infinity Cache serves are included.  They belong to the kernel sources whose digest is
 # TRAFFIC_SOURCE_DIGEST: when the sources of the loaded library differ, `traffic` is reported as
 # null and the recorded figure moves to `traffic_recorded` (stale until the profile is redone).
-TRAFFIC_SOURCE_DIGEST = 'f4ea7f9079ba5b2b'
+TRAFFIC_SOURCE_DIGEST = '3441afcc72367e05'
 MEASURED_TRAFFIC_BYTES = {
-    'c4_linear_fwd': 4639369477,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.7 GiB read, 1.0 GiB written
-    'c2_layer_norm': 362249339,       # norm_fwd + norm_bwd + reduce_partials
-    'c2_rms_norm': 361808236,
-    'c2_softmax': 335902407,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
-    'c2_act_dropout': 335781338,      # act_dropout forward + backward
-    'c2_glu': 268579113,              # glu forward + backward
-    'c2_mse': 335720558,              # p_loss forward + backward
-    'c3_cross_entropy': 1683512285,   # ce_row_kernel (ignored rows are not read)
-    'c3_cross_entropy_autocast': 2436824554,
-    'c3_nll_loss': 826899159,         # nll forward (a gather) + the single-pass gradient write
-    'c5_conv_channels_last': 397630567,     # the two ring kernels + weight gradient + weight reorders, no copies
-    'c5_conv': 595352378,             # the same + 2 layout copies
-    'c5_batch_norm_channels_last': 568532977,
-    'c5_batch_norm': 581423153,       # stats + apply + backward reduce + backward apply
+    'c4_linear_fwd': 4493092605,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.7 GiB read, 1.0 GiB written
+    'c2_layer_norm': 362251943,       # norm_fwd + norm_bwd + reduce_partials
+    'c2_rms_norm': 361814478,
+    'c2_softmax': 335907377,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
+    'c2_act_dropout': 335776322,      # act_dropout forward + backward
+    'c2_glu': 268584124,              # glu forward + backward
+    'c2_mse': 335729072,              # p_loss forward + backward
+    'c3_cross_entropy': 1683529308,   # ce_row_kernel (ignored rows are not read)
+    'c3_cross_entropy_autocast': 2436837245,
+    'c3_nll_loss': 826897725,         # nll forward (a gather) + the single-pass gradient write
+    'c5_conv_channels_last': 397622066,     # the two ring kernels + weight gradient + weight reorders, no copies
+    'c5_conv': 595379362,             # the same + 2 layout copies
+    'c5_batch_norm_channels_last': 568580636,
+    'c5_batch_norm': 591969192,       # stats + apply + backward reduce + backward apply
 }
 
 
