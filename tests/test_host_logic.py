@@ -256,6 +256,9 @@ def test_bench_final_line_stays_compact() -> None:
     entry = {'tag': 'c2 GELU(tanh)+Dropout(0.1) layer', 'workload': 'x' * 200, 'value': 4234.123456, 'unit': 'GB/s',
              'roofline': {'frac': 0.5234567, 'traffic': 362346310, 'note': 'y' * 300},
              'cpu_baseline': {'value': 1.5167704445, 'unit': 'GB/s', 'cores': 16}, 'module_level': {'note': 'z' * 500}}
+    head['mfma_probe'] = {'unit': 'TFLOP/s', 'tflops_constant_operands': 2465.123, 'tflops_changing_operands': 1797.456,
+                          'note': 'n' * 200}
+    head['frac_of_mfma_probe_step'] = 0.6534
     line = bench.compact_line(argparse.Namespace(steps=20, warmup=5), head, [dict(entry) for _ in range(24)])
     text = json.dumps(line)
     assert len(text) < 6000
@@ -266,3 +269,12 @@ def test_bench_final_line_stays_compact() -> None:
     assert set(line['roofline']) >= {'bound', 'achieved', 'peak', 'unit', 'frac', 'traffic'}
     assert set(line['cpu_baseline']) >= {'value', 'unit', 'cores', 'kind', 'sample'}
     assert len(line['configs']) == 24 and all('frac' in c and 'tag' in c for c in line['configs'])
+
+
+def test_recorded_traffic_belongs_to_the_kernel_sources_in_the_tree() -> None:
+    """
+    bench.py reports the measured HBM traffic of its kernels only while the kernel sources have the
+    digest the measurements were recorded for; a source change without a new measurement shows here.
+    """
+    import bench
+    assert bench.kernel_source_digest() == bench.TRAFFIC_SOURCE_DIGEST
