@@ -7,10 +7,12 @@ forward + backward step measured as one.  Prints one JSON line per block and bac
 ms_fwd, ms_bwd and ms_fwd_bwd.
 
     python -m examples.run_blocks [--dtype bf16|fp16|fp32] [--amp] [--amp-dtype fp16|bf16] [--iters N]
+                                  [--channels-last]
 
 --amp keeps parameters and inputs in float32 and runs the forward pass under torch.autocast, as
 the reference's examples do by default; --dtype then only names the storage dtype of the non-AMP
-runs and is ignored.
+runs and is ignored.  --channels-last hands the ResNet block its image in torch.channels_last
+memory format: Conv2d and BatchNorm2d of attorch_amd then work on that layout without copies.
 """
 
 import argparse
@@ -66,6 +68,8 @@ def main() -> int:
                         help='float32 parameters and inputs, forward under torch.autocast')
     parser.add_argument('--amp-dtype', default='fp16', choices=['fp16', 'bf16'])
     parser.add_argument('--iters', type=int, default=20)
+    parser.add_argument('--channels-last', action='store_true',
+                        help='ResNet block input in torch.channels_last memory format')
     args = parser.parse_args()
     if not torch.cuda.is_available():
         print('examples.run_blocks: no HIP device visible.', file=sys.stderr)
@@ -86,9 +90,13 @@ def main() -> int:
     t = torch.randint(0, 10, (4096,), generator=gen).cuda()
     cases.append(('MLP 784-2048-2048-10, batch 4096', make(MLPClassifier, 784, 2048, 2, 10),
                   lambda m: m(x, t)))
-    img = torch.randn(64, 64, 56, 56, generator=gen).to('cuda', dtype).requires_grad_(True)
-    cases.append(('ResNet basic block 64->64, X[64,64,56,56]', make(BasicBlock, 64, 64),
-                  lambda m: m(img).float().square().mean()))
+    img = torch.randn(64, 64, 56, 56, generator=gen).to('cuda', dtype)
+    if args.channels_last:
+        img = img.contiguous(memory_format=torch.channels_last)
+    img.requires_grad_(True)
+    cases.append(('ResNet basic block 64->64, X[64,64,56,56]' + (' channels-last' if args.channels_last else ''),
+                  make(BasicBlock, 64, 64),
+                  lambda m: m(img)))   # the block's output itself: its random upstream gradient keeps its memory format
     tok = torch.randint(0, 8192, (8, 512), generator=gen).cuda()
     cases.append(('GPT block x2, dim 1024, 16 heads, vocab 8192, tokens [8,512]',
                   make(TinyGPT, 8192, 2, 1024, 16), lambda m: m(tok, return_loss=True)))
