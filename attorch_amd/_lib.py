@@ -213,3 +213,22 @@ def row_stride(tensor: Tensor) -> int:
         return max(int(tensor.shape[1]), 1)
     return int(tensor.stride(0))
 
+
+def in_memory_format(tensor: Tensor, memory_format: torch.memory_format) -> Tensor:
+    """
+    `tensor.contiguous(memory_format=...)`, with the library's tiled transpose for the one case the
+    layers meet on their hot path: a 16-bit NCHW-contiguous device tensor wanted channels-last
+    (an upstream gradient that some other operator produced in the default format).
+    """
+    if tensor.is_contiguous(memory_format=memory_format):
+        return tensor
+    if (memory_format is torch.channels_last and tensor.dim() == 4 and tensor.is_cuda
+            and tensor.dtype in (torch.float16, torch.bfloat16) and tensor.is_contiguous() and tensor.numel() > 0
+            and tensor.shape[0] <= 65535):
+        batch, feat, height, width = tensor.shape
+        out = torch.empty_like(tensor, memory_format=torch.channels_last)
+        with device_guard(tensor):
+            check(load().at_nchw_to_nhwc(ptr(tensor), ptr(out), batch, feat, height * width, dtype_id(tensor.dtype),
+                                         stream_of(tensor)), 'at_nchw_to_nhwc')
+        return out
+    return tensor.contiguous(memory_format=memory_format)

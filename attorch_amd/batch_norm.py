@@ -107,7 +107,7 @@ class BatchNormAutoGrad(torch.autograd.Function):
         forward_entry = (lib.at_batch_norm_fwd_nhwc if ctx.rows_of_features
                          else lib.at_batch_norm_fwd)
         input_k = input.contiguous(memory_format=layout)
-        residual_k = (pre_act_add.to(input.dtype).contiguous(memory_format=layout)
+        residual_k = (_lib.in_memory_format(pre_act_add.to(input.dtype), layout)
                       if add_pre_act else None)
         output = torch.empty_like(input_k)
         pre_act = torch.empty_like(input_k) if save_pre_act else None
@@ -159,7 +159,7 @@ class BatchNormAutoGrad(torch.autograd.Function):
         batch_dim, feat_dim, spatial_dim = _dims(input)
         device = input.device
 
-        output_grad_k = output_grad.to(input.dtype).contiguous(memory_format=ctx.layout)
+        output_grad_k = _lib.in_memory_format(output_grad.to(input.dtype), ctx.layout)
         backward_entry = (lib.at_batch_norm_bwd_nhwc if ctx.rows_of_features
                           else lib.at_batch_norm_bwd)
         input_grad = torch.empty_like(input)

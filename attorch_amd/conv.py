@@ -184,7 +184,7 @@ class Conv2dAutoGrad(torch.autograd.Function):
         if ctx.channels_last:
             # channels-last gradients in and out; a product this path does not cover is left to
             # the channels-first code below
-            grad_last = output_grad.to(output_dtype).contiguous(memory_format=torch.channels_last)
+            grad_last = _lib.in_memory_format(output_grad.to(output_dtype), torch.channels_last)
             need_input = ctx.needs_input_grad[0]
             need_weight = ctx.needs_input_grad[1]
             with _lib.device_guard(input):

@@ -549,3 +549,27 @@ def test_batch_norm_channels_last_eval_and_block() -> None:
     names = ('output', 'input_grad', 'eval output', 'conv weight_grad', 'bn weight_grad')
     for name, first, second in zip(names, *results):
         assert_close(second, first.cpu(), dtype, name, batch_reduction='weight_grad' in name)
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_channels_last_layers_take_an_upstream_gradient_in_the_default_format(dtype) -> None:
+    """
+    A channels-last Conv2d / BatchNorm2d whose upstream gradient arrives NCHW-contiguous (another
+    operator produced it) converts it with the library's transpose: same gradients, bit for bit, as
+    with a channels-last upstream gradient.
+    """
+    x = randn((6, 64, 20, 24), 1, dtype).cuda().contiguous(memory_format=torch.channels_last)
+    w = randn((64, 64, 3, 3), 2, dtype, 576 ** -0.5).cuda()
+    res = randn((6, 64, 20, 24), 5, dtype).cuda().contiguous(memory_format=torch.channels_last)
+    dy = randn((6, 64, 20, 24), 3, dtype).cuda()
+    assert dy.is_contiguous() and not dy.is_contiguous(memory_format=torch.channels_last)
+    results = []
+    for grad in (dy, dy.contiguous(memory_format=torch.channels_last)):
+        xd, wd, rd = x.clone().requires_grad_(True), w.clone().requires_grad_(True), res.clone().requires_grad_(True)
+        bn = attorch_amd.BatchNorm2d(64, act_func='relu', device='cuda', dtype=dtype)
+        y = bn(attorch_amd.Conv2dAutoGrad.apply(xd, wd, None, 1, 1, 1, 1, 1), rd)
+        assert y.is_contiguous(memory_format=torch.channels_last)
+        y.backward(grad)
+        results.append((xd.grad, wd.grad, rd.grad, bn.weight.grad, bn.bias.grad))
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
