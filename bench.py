@@ -20,7 +20,8 @@ fields it carries
                 c5 Conv2d + BatchNorm2d), each as tag, absolute throughput, fraction of its
                 roofline, measured HBM traffic and CPU baseline.
 The full record (module-level and torch-native timings, CPU functional baselines, notes) is
-written to --detail-file (gpurun_out/bench_detail.json beside this script by default).
+written to --detail-file (bench_detail.json in the run-output folder beside this script by
+default).
 Buffers of the bandwidth-bound configs are rotated over several sets so the 256 MB Infinity
 Cache cannot serve them.  Secondary configs are timed with 10 warm-up and 60 timed calls (median
 of 6 groups of 10) whatever --steps says.
@@ -1273,8 +1274,7 @@ def main() -> int:
         'frac_of_mfma_probe_step': head.get('frac_of_mfma_probe_step'),
         'configs': extra,
     }
-    # Everything measured goes to a file (--detail-file, by default gpurun_out/bench_detail.json
-    # beside this script); stdout carries only the one compact line.
+    # Everything measured goes to a file (--detail-file); stdout carries only the one compact line.
     try:
         os.makedirs(os.path.dirname(os.path.abspath(args.detail_file)), exist_ok=True)
         with open(args.detail_file, 'w') as fh:
