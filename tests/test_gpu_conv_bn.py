@@ -477,7 +477,11 @@ def test_conv2d_weights_resident_kernel_same_on_both_layouts(shape, out_dim, bia
 
 
 @pytest.mark.parametrize('dtype', DTYPES)
-@pytest.mark.parametrize('shape', [(4, 64, 7, 7), (2, 96, 5, 6), (3, 8, 4, 4), (5, 24, 3, 5), (2, 2048, 2, 3), (2, 4104, 3, 2)])
+@pytest.mark.parametrize('shape', [(4, 64, 7, 7), (2, 96, 5, 6), (3, 8, 4, 4), (5, 24, 3, 5), (2, 2048, 2, 3), (2, 4104, 3, 2),
+                                   # every power of two of 16-byte chunks per row up to a wave's 64, over enough
+                                   # rows for several rounds of loads per lane
+                                   (16, 512, 9, 9), (8, 256, 7, 9), (8, 128, 14, 14), (6, 32, 31, 17),
+                                   (32, 16, 12, 10), (9, 64, 33, 35)])
 @pytest.mark.parametrize('affine, residual, act_func', [(True, True, 'relu'), (False, False, None),
                                                         (True, False, 'silu'), (True, True, 'leaky_relu_0.01')])
 def test_batch_norm_channels_last(shape, dtype, affine, residual, act_func) -> None:
