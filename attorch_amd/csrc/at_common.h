@@ -82,26 +82,6 @@ __device__ __forceinline__ void store_f32(T* __restrict__ p, const float (&v)[N]
   }
 }
 
-// store_f32 for outputs nobody reads again soon (whole activations streamed out once): the
-// non-temporal hint keeps them from displacing the inputs still being read from the caches.
-template <typename T, int N>
-__device__ __forceinline__ void store_f32_stream(T* __restrict__ p, const float (&v)[N]) {
-  typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
-  constexpr int BYTES = N * (int)sizeof(T);
-  if constexpr (BYTES % 16 == 0) {
-    constexpr int PER = 16 / (int)sizeof(T);
-#pragma unroll
-    for (int j = 0; j < N / PER; ++j) {
-      union { u32x4_t r; T e[PER]; } u;
-#pragma unroll
-      for (int i = 0; i < PER; ++i) u.e[i] = from_f32<T>(v[j * PER + i]);
-      __builtin_nontemporal_store(u.r, reinterpret_cast<u32x4_t*>(p) + j);
-    }
-  } else {
-    store_f32<T, N>(p, v);
-  }
-}
-
 // Parameter vectors (weight / bias) may be stored in a dtype different from the
 // activations; they are small and cache resident, so a runtime dtype switch is enough.
 template <int N>

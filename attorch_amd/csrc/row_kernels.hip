@@ -19,8 +19,6 @@
 namespace at_hip {
 namespace {
 
-template <int ITERS> constexpr int cache_len() { return ITERS > 0 ? ITERS : 1; }
-
 // Makes an index opaque to the optimiser.  Parameter vectors do not depend on the row, so inside
 // a row loop the compiler would hoist their loads out of the loop and keep them (widened to
 // fp32) in registers for the whole kernel; an opaque index ties each load to its iteration.
