@@ -223,3 +223,56 @@ def test_c5_conv_bn_residual_relu_bf16() -> None:
     assert_close(wdv.grad, dw_ref.to(BF16), BF16, 'batch_norm weight_grad', batch_reduction=True)
     assert_close(bdv.grad, db_ref.to(BF16), BF16, 'batch_norm bias_grad', batch_reduction=True)
     assert_close(rd.grad, dres_ref, BF16, 'batch_norm residual_grad')
+
+
+def test_batch_norm_of_2_gib_and_more() -> None:
+    """
+    The passes that sum over a channel read tensors below 2 GiB through a buffer resource; from
+    that size on they keep plain pointers.  [2, 16, 8200, 4100] bf16 is 2.15 GB: residual and
+    ReLU fused, forward and backward.  The device's own batch_norm in float32 is the checker at
+    this size (the CPU oracle would take minutes on a billion elements); tolerances of bf16.
+    """
+    dtype = torch.bfloat16
+    shape = (2, 16, 8200, 4100)
+    assert shape[0] * shape[1] * shape[2] * shape[3] * 2 >= 1 << 31
+    gen = torch.Generator(device='cuda').manual_seed(11)
+    x = torch.randn(shape, device='cuda', dtype=dtype, generator=gen).mul_(1.5).add_(0.25).requires_grad_(True)
+    res = torch.randn(shape, device='cuda', dtype=dtype, generator=gen).requires_grad_(True)
+    dy = torch.randn(shape, device='cuda', dtype=dtype, generator=gen)
+    w = (1 + 0.1 * torch.randn(16, device='cuda', generator=gen)).to(dtype).requires_grad_(True)
+    b = (0.1 * torch.randn(16, device='cuda', generator=gen)).to(dtype).requires_grad_(True)
+    rm, rv = torch.zeros(16, device='cuda', dtype=dtype), torch.ones(16, device='cuda', dtype=dtype)
+    out = attorch_amd.BatchNormAutoGrad.apply(x, True, w, b, rm, rv, 0.1, 1e-5, True, res, 'relu')
+    out.backward(dy)
+
+    xr, rr = x.detach().float().requires_grad_(True), res.detach().float().requires_grad_(True)
+    wr, br = w.detach().float().requires_grad_(True), b.detach().float().requires_grad_(True)
+    rm_ref, rv_ref = torch.zeros(16, device='cuda'), torch.ones(16, device='cuda')
+    pre = torch.nn.functional.batch_norm(xr, rm_ref, rv_ref, wr, br, True, 0.1, 1e-5) + rr
+    ref = torch.relu(pre)
+    ref.backward(dy.float())
+    rtol, atol = 2e-2, 2e-2
+    # Where the pre-activation is within float32 rounding of zero, the two sides may land on
+    # different sides of the ReLU and differ by a whole gradient: a few in a million elements,
+    # left out of the gradient comparison.
+    boundary = pre.detach().abs() <= 1e-4
+    assert boundary.sum().item() < 1e-4 * boundary.numel()
+    del pre
+
+    def check(actual, expected, what, skip=None):
+        wrong = (actual.float() - expected).abs() > atol + rtol * expected.abs()
+        if skip is not None:
+            wrong &= ~skip
+        bad = wrong.sum().item()
+        assert bad == 0, f'{what}: {bad} elements out of tolerance'
+
+    check(out, ref.detach(), 'output')
+    del ref
+    check(x.grad, xr.grad, 'input_grad', boundary)
+    check(res.grad, rr.grad, 'residual_grad', boundary)
+    scale = max(1.0, wr.grad.abs().max().item())
+    check(w.grad / scale, wr.grad / scale, 'weight_grad')
+    scale = max(1.0, br.grad.abs().max().item())
+    check(b.grad / scale, br.grad / scale, 'bias_grad')
+    check(rm, rm_ref, 'running_mean')
+    check(rv, rv_ref, 'running_var')
