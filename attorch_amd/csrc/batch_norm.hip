@@ -225,6 +225,8 @@ __global__ __launch_bounds__(kBnBlock) void bn_apply_kernel(
     float param, int64_t total_planes) {
   const int sp = S / VEC;
   const int step = gridDim.y * kBnBlock;
+  int merged_c = -1;   // the channel whose statistics the workgroup holds (planes a multiple of C apart share it)
+  float mean = 0.f, var = 0.f, count = 0.f;
   for (int64_t plane = blockIdx.x; plane < total_planes; plane += gridDim.x) {
     const int c = (int)(plane % C);
     const int64_t base = plane * (int64_t)S;
@@ -245,8 +247,10 @@ __global__ __launch_bounds__(kBnBlock) void bn_apply_kernel(
       }
     };
     issue(i0 < sp ? i0 : 0);
-    float mean, var, count;
-    channel_stats(part, P, c, running_mean, running_var, rdt, mean, var, count);
+    if (c != merged_c) {   // uniform
+      merged_c = c;
+      channel_stats(part, P, c, running_mean, running_var, rdt, mean, var, count);
+    }
     const float inv_std = rsqrtf(var + eps);
     if (plane < C && blockIdx.y == 0 && threadIdx.x == 0) {
       if (mean_out) mean_out[c] = mean;
@@ -357,6 +361,8 @@ __global__ __launch_bounds__(kBnBlock) void bn_bwd_apply_kernel(
   __shared__ float smem[2];
   const int sp = S / VEC;
   const int step = gridDim.y * kBnBlock;
+  int summed_c = -1;   // the channel whose sums the workgroup holds (planes a multiple of C apart share it)
+  float s1 = 0.f, s2 = 0.f;
   for (int64_t plane = blockIdx.x; plane < total_planes; plane += gridDim.x) {
     const int c = (int)(plane % C);
     const int64_t base = plane * (int64_t)S;
@@ -375,22 +381,26 @@ __global__ __launch_bounds__(kBnBlock) void bn_bwd_apply_kernel(
       }
     };
     issue(i0 < sp ? i0 : 0);   // in flight while the partial sums of the channel are added up
-    __syncthreads();   // previous readers of smem are done
-    if (threadIdx.x < 64) {
-      float s1 = 0.f, s2 = 0.f;
-      for (int p = threadIdx.x; p < P; p += 64) {
-        s1 += part[((int64_t)c * P + p) * 2];
-        s2 += part[((int64_t)c * P + p) * 2 + 1];
+    if (c != summed_c) {       // uniform
+      summed_c = c;
+      __syncthreads();   // previous readers of smem are done
+      if (threadIdx.x < 64) {
+        float a1 = 0.f, a2 = 0.f;
+        for (int p = threadIdx.x; p < P; p += 64) {
+          a1 += part[((int64_t)c * P + p) * 2];
+          a2 += part[((int64_t)c * P + p) * 2 + 1];
+        }
+        a1 = wave_reduce(a1, 64, SumOp());
+        a2 = wave_reduce(a2, 64, SumOp());
+        if (threadIdx.x == 0) {
+          smem[0] = a1;
+          smem[1] = a2;
+        }
       }
-      s1 = wave_reduce(s1, 64, SumOp());
-      s2 = wave_reduce(s2, 64, SumOp());
-      if (threadIdx.x == 0) {
-        smem[0] = s1;
-        smem[1] = s2;
-      }
+      __syncthreads();
+      s1 = smem[0];
+      s2 = smem[1];
     }
-    __syncthreads();
-    const float s1 = smem[0], s2 = smem[1];
     if (plane < C && blockIdx.y == 0 && threadIdx.x == 0) {
       if (weight_grad) weight_grad[c] = s1;
       if (bias_grad) bias_grad[c] = s2;
@@ -450,13 +460,15 @@ inline int bn_splits(int64_t N, int C) {
   return (int)want;
 }
 
-inline void apply_grid(int64_t planes, int S, int vec, dim3* grid) {
+// Grid of an apply pass: x walks over the planes with at most per_cu workgroups for every CU
+// (a workgroup then loops over planes), y splits long planes.
+inline void apply_grid(int64_t planes, int S, int vec, int per_cu, dim3* grid) {
   const int sp = S / vec;
   int gy = (int)cdiv64(sp, kBnBlock * 2);
   if (gy < 1) gy = 1;
   if (gy > 64) gy = 64;
   int64_t gx = planes;
-  const int64_t cap = (int64_t)device_cu_count() * 64;
+  const int64_t cap = (int64_t)device_cu_count() * per_cu;
   if (gx > cap) gx = cap;
   *grid = dim3((unsigned)gx, (unsigned)gy);
 }
@@ -1006,7 +1018,7 @@ int at_batch_norm_fwd(const void* input, const void* weight, const void* bias, f
     const float* part_in = batch_stats ? part : nullptr;   // null: the apply pass reads the running statistics
     dim3 grid;
     const int64_t planes = batch * feat;
-    apply_grid(planes, S, vec_ok ? VEC : 1, &grid);
+    apply_grid(planes, S, vec_ok ? VEC : 1, 64, &grid);
     if (vec_ok) {
       AT_BN_ACT_SWITCH(act, hipLaunchKernelGGL((bn_apply_kernel<T, VEC, ACT>), grid, dim3(kBnBlock), 0, stream,
                                                (const T*)input, (const T*)pre_act_add, (T*)pre_act, (T*)output,
@@ -1072,7 +1084,10 @@ int at_batch_norm_bwd(const void* output_grad, const void* pre_act, const void* 
     }
     dim3 grid;
     const int64_t planes = batch * feat;
-    apply_grid(planes, S, vec_ok ? VEC : 1, &grid);
+    // Two planes per workgroup at c5's size, of one channel when the grid is a multiple of C: the
+    // channel's sums are then added up once for both (c5: 72 -> 69 us for the backward pass; the
+    // forward pass is best at one plane each).
+    apply_grid(planes, S, vec_ok ? VEC : 1, 16, &grid);
     const float count = (float)(batch * spatial);
     if (vec_ok)
       hipLaunchKernelGGL((bn_bwd_apply_kernel<T, VEC>), grid, dim3(kBnBlock), 0, stream, (const T*)g_for_apply,

@@ -47,22 +47,22 @@ PEAK_MFMA_FP32_TFLOPS = 157.3    # dense fp32 MFMA
 # the 256 MB Infinity Cache serves are included.  They belong to the kernel sources whose digest is
 # TRAFFIC_SOURCE_DIGEST: when the sources of the loaded library differ, `traffic` is reported as
 # null and the recorded figure moves to `traffic_recorded` (stale until the profile is redone).
-TRAFFIC_SOURCE_DIGEST = 'e9a4acd88e64ce28'
+TRAFFIC_SOURCE_DIGEST = 'b7c36b63ee36f715'
 MEASURED_TRAFFIC_BYTES = {
-    'c4_linear_fwd': 4691189595,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.7 GiB read, 1.0 GiB written
-    'c2_layer_norm': 362248594,       # norm_fwd + norm_bwd + reduce_partials
-    'c2_rms_norm': 361810912,
-    'c2_softmax': 335902473,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
-    'c2_act_dropout': 335771421,      # act_dropout forward + backward
-    'c2_glu': 268579657,              # glu forward + backward
-    'c2_mse': 335722062,              # p_loss forward + backward
-    'c3_cross_entropy': 1683549449,   # ce_row_kernel (ignored rows are not read)
-    'c3_cross_entropy_autocast': 2436770295,
-    'c3_nll_loss': 826900072,         # nll forward (a gather) + the single-pass gradient write
-    'c5_conv_channels_last': 397503273,     # the two ring kernels + weight gradient + weight reorders, no copies
-    'c5_conv': 595350726,             # the same + 2 layout copies
-    'c5_batch_norm_channels_last': 567960039,
-    'c5_batch_norm': 565835679,       # stats + apply + backward reduce + backward apply
+    'c4_linear_fwd': 4705493680,      # gemm_mfma16_kernel<bf16, ..., GELU-tanh>: 3.7 GiB read, 1.0 GiB written
+    'c2_layer_norm': 362246782,       # norm_fwd + norm_bwd + reduce_partials
+    'c2_rms_norm': 361809038,
+    'c2_softmax': 335901896,          # softmax_fwd + softmax_bwd (same kernels for log-softmax)
+    'c2_act_dropout': 335771228,      # act_dropout forward + backward
+    'c2_glu': 268579817,              # glu forward + backward
+    'c2_mse': 335723406,              # p_loss forward + backward
+    'c3_cross_entropy': 1683527018,   # ce_row_kernel (ignored rows are not read)
+    'c3_cross_entropy_autocast': 2436782254,
+    'c3_nll_loss': 826899934,         # nll forward (a gather) + the single-pass gradient write
+    'c5_conv_channels_last': 397515918,     # the two ring kernels + weight gradient + weight reorders, no copies
+    'c5_conv': 595354072,             # the same + 2 layout copies
+    'c5_batch_norm_channels_last': 567988040,
+    'c5_batch_norm': 565877886,       # stats + apply + backward reduce + backward apply
 }
 
 
